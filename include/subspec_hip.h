@@ -1,0 +1,117 @@
+/*
+ * C ABI of libsubspec_hip.so: hand-written gfx950 (MI355X) kernels for the speculative-decoding
+ * hot path of NYCU-EDgeAi/subspec.  Plain pointers and sizes only; every pointer named "device"
+ * is device memory owned by the caller, every call is asynchronous on `stream` (a hipStream_t
+ * passed as void*, NULL = the default stream) and allocates nothing.
+ *
+ * Return value: 0 on success, a negative SUBSPEC_ERR_* otherwise; subspec_last_error() then
+ * returns a human-readable message (thread-local).
+ *
+ * Each entry point cites the reference interface it replaces (paths relative to the reference).
+ */
+#ifndef SUBSPEC_HIP_H
+#define SUBSPEC_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SUBSPEC_ABI_VERSION 1
+
+/* element types of logits / probabilities / KV / activations */
+#define SUBSPEC_F32 0
+#define SUBSPEC_F16 1
+#define SUBSPEC_BF16 2
+
+#define SUBSPEC_OK 0
+#define SUBSPEC_ERR_ARG (-1)       /* bad shape / dtype / alignment / null pointer */
+#define SUBSPEC_ERR_WORKSPACE (-2) /* workspace too small */
+#define SUBSPEC_ERR_HIP (-3)       /* a HIP runtime call failed */
+#define SUBSPEC_ERR_LIMIT (-4)     /* size beyond what the kernels are built for */
+
+/* verify_method / threshold_method as in generator_kwargs (configs/methods/subspec_sd_lossy.yaml:20-31) */
+#define SUBSPEC_VERIFY_EXACT 0
+#define SUBSPEC_VERIFY_LOSSY 1
+#define SUBSPEC_GATE_ENTROPY 0
+#define SUBSPEC_GATE_PROB 1
+
+/* How the normalized entropy of 16-bit rows is evaluated.
+ *  GUARD : one fp32 pass; rows whose entropy lies within 2% of the threshold are re-evaluated
+ *          with the reference's per-element rounding (p, log p and p*log p each rounded to the
+ *          row dtype), so gate decisions match the reference.
+ *  ALWAYS: every row uses the per-element rounding; node_entropy is then the value the
+ *          reference computes. */
+#define SUBSPEC_ENTROPY_GUARD 0
+#define SUBSPEC_ENTROPY_ALWAYS 1
+
+#define SUBSPEC_MAX_TREE_NODES 256
+
+int subspec_abi_version(void);
+const char* subspec_last_error(void);
+
+/* ------------------------------------------------------------------------------------------
+ * Tree verification, fused: softmax statistics, first-index argmax of the rounded probabilities,
+ * normalized entropy, p[parent(i), token(i)] for every node, then the greedy walk or the lossy
+ * bottom-up DP, longest-path extraction and bonus token -- three kernel launches, no host sync.
+ *
+ * Replaces  verify_tree            specdecodes/models/utils/tree_verify.py:8-163
+ *           lossy_bottom_up_verify specdecodes/models/utils/lossy_tree_verify.py:9-343
+ *           _sample_token(return_probs=True) + .cpu()   specdecodes/models/generators/base.py:109-139,
+ *                                                       tree_verify.py:51-52,117-118
+ *           _verify_step           specdecodes/models/generators/classic_sd.py:111-116
+ * for the greedy (do_sample=False) target.
+ *
+ * logits      device, [batch, rows, vocab] contiguous, element type `dtype`; row r of a tree is
+ *             the target distribution at original node r + skip_nodes.
+ * token_ids   device int32 [batch, n_nodes]   token of every node of the WHOLE tree
+ * parents     device int32 [batch, n_nodes]   parent index, -1 for the root; parent < child
+ * root        context node to start from (original indexing)
+ * eos_token_id  < 0 : none
+ * out_tokens  device int64 [batch, n_nodes + 1]  accepted tokens followed by the bonus token
+ * out_ctx     device int64 [batch, n_nodes + 1]  context node (original indexing) of each token
+ *                                               = the KV rows to keep
+ * out_counts  device int32 [batch, 4]  {emitted, accept_len, total_len, status}; status != 0
+ *                                      means the tree broke a precondition (see verify.hip)
+ * node_target / node_entropy / node_child_prob   device [batch, rows] (int64 / float / float):
+ *             argmax token, normalized entropy and p[parent(i), token(i)] per scored node
+ *             (what the reference's diagnostics are computed from); node_entropy is only
+ *             written for the entropy gate.
+ */
+size_t subspec_tree_verify_workspace(int64_t batch, int64_t rows, int64_t vocab, int dtype);
+
+int subspec_tree_verify(const void* logits, int dtype, int64_t batch, int64_t rows, int64_t vocab,
+                        const int32_t* token_ids, const int32_t* parents, int64_t n_nodes,
+                        int32_t root, int32_t skip_nodes, int64_t eos_token_id,
+                        int verify_method, int threshold_method, double threshold, int32_t window_size,
+                        int entropy_policy,
+                        void* workspace, size_t workspace_bytes,
+                        int64_t* out_tokens, int64_t* out_ctx, int32_t* out_counts,
+                        int64_t* node_target, float* node_entropy, float* node_child_prob,
+                        void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * KV-cache compaction after verification: for every slab (one [seq, row_bytes] matrix: one
+ * layer x {K,V} x batch x kv-head), row offset+j <- row offset+ctx[j] for j < count, with
+ * gather-then-scatter semantics; rows outside [offset, offset+count) are untouched.
+ *
+ * Replaces  KVManager.reorder_cache_with_offset -> TreeStaticCache.reorder_cache_with_offset
+ *           specdecodes/models/utils/cache_utils.py:55-56,166-208 (and :85-103 for the dynamic cache).
+ *
+ * slab_ptrs   device array of n_slabs base pointers, or NULL when the slabs are
+ *             base + i * slab_stride_bytes
+ * ctx         device int64 [>= count]  (e.g. out_ctx of subspec_tree_verify)
+ * count_dev   device int32*, number of rows to move read on the device (e.g. &out_counts[0]);
+ *             NULL -> use count_host.  max_count bounds both (<= SUBSPEC_MAX_TREE_NODES).
+ */
+int subspec_kv_compact(void* base, void* const* slab_ptrs, int64_t n_slabs, int64_t slab_stride_bytes,
+                       int64_t seq_len, int64_t row_bytes, int64_t offset,
+                       const int64_t* ctx, const int32_t* count_dev, int32_t count_host, int32_t max_count,
+                       void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SUBSPEC_HIP_H */

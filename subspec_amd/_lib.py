@@ -1,0 +1,66 @@
+"""ctypes binding of libsubspec_hip.so (the C ABI declared in include/subspec_hip.h).
+
+The library is built in-tree by ``python -m subspec_amd.build`` (or ``__graft_entry__.build()``).
+There is no CPU fallback: if the library is missing, ``lib()`` raises.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+import re
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "lib", "libsubspec_hip.so")
+HEADER = os.path.join(os.path.dirname(HERE), "include", "subspec_hip.h")
+
+F32, F16, BF16 = 0, 1, 2
+VERIFY_EXACT, VERIFY_LOSSY = 0, 1
+GATE_ENTROPY, GATE_PROB = 0, 1
+ENTROPY_GUARD, ENTROPY_ALWAYS = 0, 1
+MAX_TREE_NODES = 256
+
+_lib = None
+
+_p, _i32, _i64, _f64, _sz = C.c_void_p, C.c_int32, C.c_int64, C.c_double, C.c_size_t
+_SIGNATURES = {
+    "subspec_abi_version": (C.c_int, []),
+    "subspec_last_error": (C.c_char_p, []),
+    "subspec_tree_verify_workspace": (_sz, [_i64, _i64, _i64, C.c_int]),
+    "subspec_tree_verify": (C.c_int, [_p, C.c_int, _i64, _i64, _i64, _p, _p, _i64, _i32, _i32, _i64,
+                                      C.c_int, C.c_int, _f64, _i32, C.c_int, _p, _sz,
+                                      _p, _p, _p, _p, _p, _p, _p]),
+    "subspec_kv_compact": (C.c_int, [_p, _p, _i64, _i64, _i64, _i64, _i64, _p, _p, _i32, _i32, _p]),
+}
+
+
+class SubspecHipError(RuntimeError):
+    pass
+
+
+def declared_symbols():
+    """Names of all functions declared in include/subspec_hip.h."""
+    with open(HEADER) as f:
+        text = re.sub(r"/\*.*?\*/", "", f.read(), flags=re.S)
+    return sorted(set(re.findall(r"\b(subspec_[a-z0-9_]+)\s*\(", text)))
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise SubspecHipError(
+                f"{LIB_PATH} not found: build it with `python -m subspec_amd.build` "
+                "(hipcc, gfx950). There is no CPU fallback.")
+        handle = C.CDLL(LIB_PATH)
+        for name, (res, args) in _SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.restype, fn.argtypes = res, args
+        _lib = handle
+    return _lib
+
+
+def check(code: int, what: str) -> None:
+    if code != 0:
+        msg = lib().subspec_last_error().decode("utf-8", "replace")
+        kind = ValueError if code in (-1, -4) else SubspecHipError
+        raise kind(f"{what}: {msg} (code {code})")

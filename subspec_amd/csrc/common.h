@@ -1,0 +1,144 @@
+// Shared helpers for the gfx950 kernels of the speculative-decoding hot path.
+// Wavefront size is 64 everywhere; nothing here is written for 32-wide execution.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+#include <math.h>
+
+#include "../../include/subspec_hip.h"
+
+namespace subspec {
+
+constexpr int kWave = 64;
+
+// ---------------------------------------------------------------- error reporting (host)
+void set_error(const char* fmt, ...);
+#define SUBSPEC_FAIL(code, ...)            \
+  do {                                     \
+    ::subspec::set_error(__VA_ARGS__);     \
+    return (code);                         \
+  } while (0)
+#define SUBSPEC_CHECK_HIP(expr)                                                              \
+  do {                                                                                       \
+    hipError_t e_ = (expr);                                                                  \
+    if (e_ != hipSuccess) SUBSPEC_FAIL(SUBSPEC_ERR_HIP, "%s failed: %s", #expr, hipGetErrorString(e_)); \
+  } while (0)
+
+inline size_t dtype_size(int dtype) { return dtype == SUBSPEC_F32 ? 4 : 2; }
+inline bool dtype_ok(int dtype) { return dtype == SUBSPEC_F32 || dtype == SUBSPEC_F16 || dtype == SUBSPEC_BF16; }
+inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+
+// ---------------------------------------------------------------- element types
+struct bf16_t { uint16_t bits; };
+struct f16_t { uint16_t bits; };
+
+__device__ __forceinline__ float bf16_bits_to_float(uint32_t b) { return __uint_as_float(b << 16); }
+__device__ __forceinline__ float f16_bits_to_float(uint32_t b) {
+  union { uint16_t u; _Float16 h; } c;
+  c.u = (uint16_t)b;
+  return (float)c.h;
+}
+// round-to-nearest-even to bfloat16, result widened back to float (NaN kept as NaN)
+__device__ __forceinline__ float round_bf16(float x) {
+  uint32_t u = __float_as_uint(x);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return x;
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return __uint_as_float(u & 0xffff0000u);
+}
+__device__ __forceinline__ float round_f16(float x) { return (float)(_Float16)x; }
+
+template <int DT> struct Elem;
+template <> struct Elem<SUBSPEC_F32> {
+  using storage = float;
+  static constexpr int kBytes = 4;
+  static __device__ __forceinline__ float load(const void* p, int64_t i) { return ((const float*)p)[i]; }
+  static __device__ __forceinline__ float round(float x) { return x; }
+  static __device__ __forceinline__ void store(void* p, int64_t i, float v) { ((float*)p)[i] = v; }
+  static __device__ __forceinline__ float min_normal() { return 1.17549435e-38f; }
+};
+template <> struct Elem<SUBSPEC_F16> {
+  using storage = uint16_t;
+  static constexpr int kBytes = 2;
+  static __device__ __forceinline__ float load(const void* p, int64_t i) { return f16_bits_to_float(((const uint16_t*)p)[i]); }
+  static __device__ __forceinline__ float round(float x) { return round_f16(x); }
+  static __device__ __forceinline__ void store(void* p, int64_t i, float v) {
+    union { uint16_t u; _Float16 h; } c;
+    c.h = (_Float16)v;
+    ((uint16_t*)p)[i] = c.u;
+  }
+  static __device__ __forceinline__ float min_normal() { return 6.103515625e-05f; }
+};
+template <> struct Elem<SUBSPEC_BF16> {
+  using storage = uint16_t;
+  static constexpr int kBytes = 2;
+  static __device__ __forceinline__ float load(const void* p, int64_t i) { return bf16_bits_to_float(((const uint16_t*)p)[i]); }
+  static __device__ __forceinline__ float round(float x) { return round_bf16(x); }
+  static __device__ __forceinline__ void store(void* p, int64_t i, float v) {
+    ((uint16_t*)p)[i] = (uint16_t)(__float_as_uint(round_bf16(v)) >> 16);
+  }
+  static __device__ __forceinline__ float min_normal() { return 1.17549435e-38f; }
+};
+
+// ---------------------------------------------------------------- wave / block reductions
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, kWave));
+  return v;
+}
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+  return v;
+}
+__device__ __forceinline__ int wave_min_i(int v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = min(v, __shfl_xor(v, o, kWave));
+  return v;
+}
+
+// Block-wide reductions over THREADS threads; `scratch` holds at least THREADS/64 words and may
+// be reused after the call returns (each helper ends with a barrier).
+template <int THREADS>
+__device__ __forceinline__ float block_max(float v, float* scratch) {
+  constexpr int W = THREADS / kWave;
+  v = wave_max(v);
+  if ((threadIdx.x & (kWave - 1)) == 0) scratch[threadIdx.x / kWave] = v;
+  __syncthreads();
+  float r = scratch[0];
+#pragma unroll
+  for (int i = 1; i < W; ++i) r = fmaxf(r, scratch[i]);
+  __syncthreads();
+  return r;
+}
+// Sum in a fixed order (wave butterfly, then waves 0..W-1) so results do not depend on timing.
+template <int THREADS>
+__device__ __forceinline__ float block_sum(float v, float* scratch) {
+  constexpr int W = THREADS / kWave;
+  v = wave_sum(v);
+  if ((threadIdx.x & (kWave - 1)) == 0) scratch[threadIdx.x / kWave] = v;
+  __syncthreads();
+  float r = scratch[0];
+#pragma unroll
+  for (int i = 1; i < W; ++i) r += scratch[i];
+  __syncthreads();
+  return r;
+}
+template <int THREADS>
+__device__ __forceinline__ int block_min_i(int v, int* scratch) {
+  constexpr int W = THREADS / kWave;
+  v = wave_min_i(v);
+  if ((threadIdx.x & (kWave - 1)) == 0) scratch[threadIdx.x / kWave] = v;
+  __syncthreads();
+  int r = scratch[0];
+#pragma unroll
+  for (int i = 1; i < W; ++i) r = min(r, scratch[i]);
+  __syncthreads();
+  return r;
+}
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+}  // namespace subspec

@@ -1,0 +1,584 @@
+// Fused tree verification for gfx950.
+//
+// Launch sequence (all on the caller's stream, no host synchronisation):
+//   1. row_partial_kernel  - grid (slices, batch*rows), 512 threads.  A workgroup streams its
+//      slice of one logits row with 16-byte loads, several per thread in flight, and reduces it in
+//      a single pass to (sum exp, sum t*exp, max, first index of the max); the row is read from
+//      HBM exactly once.  HBM-bound: algorithmic bytes = rows * vocab * sizeof(dtype).
+//   2. row_exact_kernel    - same grid; exits at once unless the row needs the reference's
+//      per-element rounding (entropy within the guard band of the threshold, fp16 rows, or a
+//      possible tie between *rounded* probabilities at the row maximum).
+//   3. tree_accept_kernel  - one workgroup per tree: combines the partials, gathers
+//      p[parent(i), token(i)], runs the greedy walk or the bottom-up DP on the <= 256 nodes in LDS
+//      and writes the accepted path, contexts and bonus token.
+//
+// Semantics follow the reference's verify_tree / lossy_bottom_up_verify
+// (specdecodes/models/utils/tree_verify.py:49-163, lossy_tree_verify.py:66-168,247-291):
+// argmax is the FIRST index whose probability, rounded to the logits dtype, equals the rounded
+// row maximum; the normalized entropy of a 16-bit row is sum(entr(p)) with p, log p and p*log p
+// each rounded to that dtype, the sum rounded once, divided by float(ln V) and rounded again.
+#include "common.h"
+#include <algorithm>
+
+namespace subspec {
+
+constexpr int kRowThreads = 512;
+constexpr int kMaxSplits = 64;
+constexpr int kTailThreads = 256;
+
+// per (row, slice): reference point of the exponentials, sum exp2(t), sum t*exp2(t) with
+// t = (x - ref) * log2(e), true maximum of the slice and the first index holding it
+struct Part1 { float ref; float s; float u; float m; int32_t idx; int32_t pad[3]; };
+struct Part2 { float esum; int32_t tie_idx; };
+
+// ------------------------------------------------------------------ packed register tiles
+template <int DT, int VEC> struct Tile;
+template <> struct Tile<SUBSPEC_F32, 4> {
+  float4 r;
+  __device__ __forceinline__ void load(const void* p, int64_t i) { r = *(const float4*)((const float*)p + i); }
+  __device__ __forceinline__ void fill_neg_inf() { r = make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY); }
+  __device__ __forceinline__ float get(int k) const { return k == 0 ? r.x : k == 1 ? r.y : k == 2 ? r.z : r.w; }
+  __device__ __forceinline__ void fence() { asm volatile("" : "+v"(r.x), "+v"(r.y), "+v"(r.z), "+v"(r.w)); }
+};
+template <> struct Tile<SUBSPEC_F32, 1> {
+  float r;
+  __device__ __forceinline__ void load(const void* p, int64_t i) { r = ((const float*)p)[i]; }
+  __device__ __forceinline__ void fill_neg_inf() { r = -INFINITY; }
+  __device__ __forceinline__ float get(int) const { return r; }
+  __device__ __forceinline__ void fence() { asm volatile("" : "+v"(r)); }
+};
+template <int DT> struct Tile16x8 {
+  uint4 r;
+  __device__ __forceinline__ void load(const void* p, int64_t i) { r = *(const uint4*)((const uint16_t*)p + i); }
+  __device__ __forceinline__ void fill_neg_inf() {
+    const uint32_t w = DT == SUBSPEC_BF16 ? 0xff80ff80u : 0xfc00fc00u;
+    r = make_uint4(w, w, w, w);
+  }
+  __device__ __forceinline__ float get(int k) const {
+    const uint32_t w = (k >> 1) == 0 ? r.x : (k >> 1) == 1 ? r.y : (k >> 1) == 2 ? r.z : r.w;
+    if (DT == SUBSPEC_BF16) return (k & 1) ? __uint_as_float(w & 0xffff0000u) : __uint_as_float(w << 16);
+    return f16_bits_to_float((k & 1) ? (w >> 16) : (w & 0xffffu));
+  }
+  // Makes the packed registers opaque to the optimiser so that the unpacked floats of one pass
+  // are not kept alive for the next one (that would double the register footprint of the slice).
+  __device__ __forceinline__ void fence() { asm volatile("" : "+v"(r.x), "+v"(r.y), "+v"(r.z), "+v"(r.w)); }
+};
+template <> struct Tile<SUBSPEC_BF16, 8> : Tile16x8<SUBSPEC_BF16> {};
+template <> struct Tile<SUBSPEC_F16, 8> : Tile16x8<SUBSPEC_F16> {};
+template <int DT> struct Tile16x1 {
+  uint16_t r;
+  __device__ __forceinline__ void load(const void* p, int64_t i) { r = ((const uint16_t*)p)[i]; }
+  __device__ __forceinline__ void fill_neg_inf() { r = DT == SUBSPEC_BF16 ? 0xff80 : 0xfc00; }
+  __device__ __forceinline__ float get(int) const {
+    return DT == SUBSPEC_BF16 ? bf16_bits_to_float(r) : f16_bits_to_float(r);
+  }
+  __device__ __forceinline__ void fence() { uint32_t w = r; asm volatile("" : "+v"(w)); r = (uint16_t)w; }
+};
+template <> struct Tile<SUBSPEC_BF16, 1> : Tile16x1<SUBSPEC_BF16> {};
+template <> struct Tile<SUBSPEC_F16, 1> : Tile16x1<SUBSPEC_F16> {};
+
+// ------------------------------------------------------------------ kernel 1: one pass over HBM
+// sum exp and sum t*exp of one tile relative to the reference `mb = -ref * log2(e)`;
+// t is clamped so that exp2(t) == 0 implies t * exp2(t) == 0 (x may be -inf).
+template <int DT, int VEC>
+__device__ __forceinline__ float tile_accumulate(const Tile<DT, VEC>& t, float mb, float (&s)[2], float (&u)[2]) {
+  float x[VEC];
+#pragma unroll
+  for (int k = 0; k < VEC; ++k) x[k] = t.get(k);
+  float tmax = x[0];
+#pragma unroll
+  for (int k = 1; k < VEC; ++k) tmax = fmaxf(tmax, x[k]);
+#pragma unroll
+  for (int k = 0; k < VEC; ++k) {
+    const float tt = fmaxf(fmaf(x[k], kLog2e, mb), -200.f);
+    const float e = __builtin_amdgcn_exp2f(tt);
+    s[k & 1] += e;
+    u[k & 1] = fmaf(tt, e, u[k & 1]);
+  }
+  return tmax;
+}
+
+template <int DT, int VEC, int U>
+__global__ __launch_bounds__(kRowThreads) void row_partial_kernel(
+    const void* __restrict__ logits, int64_t vocab, int splits, int64_t chunk, Part1* __restrict__ part) {
+  __shared__ float red_f[kRowThreads / kWave];
+  __shared__ int red_i[kRowThreads / kWave];
+  const int64_t row = blockIdx.y;
+  const int c = blockIdx.x;
+  const int tid = threadIdx.x;
+  const int64_t c0 = (int64_t)c * chunk;
+  const int64_t n = min(chunk, vocab - c0);           // elements of this slice (a multiple of VEC)
+  const int64_t base = row * vocab + c0;
+  const int64_t ntiles = n / VEC;
+
+  // Reference point for the exponentials: the largest value among the first tile of every
+  // thread.  It is at most the true maximum; the slice is redone against the true maximum in the
+  // (pathological) case that the two are so far apart that exp2 could overflow.
+  float ref;
+  {
+    Tile<DT, VEC> t0;
+    if (tid < ntiles) t0.load(logits, base + (int64_t)tid * VEC); else t0.fill_neg_inf();
+    float r = t0.get(0);
+#pragma unroll
+    for (int k = 1; k < VEC; ++k) r = fmaxf(r, t0.get(k));
+    ref = block_max<kRowThreads>(r, red_f);
+    if (ref == -INFINITY) ref = -1e30f;
+  }
+
+  float vmax = -INFINITY;
+  int64_t best_tile = 0;
+  float s[2], u[2];
+  for (int pass = 0; pass < 2; ++pass) {
+    const float mb = -ref * kLog2e;
+    s[0] = s[1] = u[0] = u[1] = 0.f;
+    for (int64_t j0 = tid; j0 < ntiles; j0 += (int64_t)kRowThreads * U) {
+      Tile<DT, VEC> t[U];
+#pragma unroll
+      for (int i = 0; i < U; ++i) {
+        const int64_t j = j0 + (int64_t)i * kRowThreads;
+        if (j < ntiles) t[i].load(logits, base + j * VEC); else t[i].fill_neg_inf();
+      }
+#pragma unroll
+      for (int i = 0; i < U; ++i) {
+        const float tmax = tile_accumulate<DT, VEC>(t[i], mb, s, u);
+        if (tmax > vmax) { vmax = tmax; best_tile = j0 + (int64_t)i * kRowThreads; }
+      }
+    }
+    if (pass == 1) break;
+    const float m_true = block_max<kRowThreads>(vmax, red_f);
+    if (!((m_true - ref) * kLog2e > 100.f)) break;    // workgroup-uniform
+    ref = m_true;
+  }
+  const float m = block_max<kRowThreads>(vmax, red_f);
+
+  int idx = 0x7fffffff;
+  if (vmax == m && m != -INFINITY) {                  // first index of the maximum inside this thread's tiles
+    Tile<DT, VEC> tb;
+    tb.load(logits, base + best_tile * VEC);
+#pragma unroll
+    for (int k = VEC - 1; k >= 0; --k)
+      if (tb.get(k) == m) idx = (int)(c0 + best_tile * VEC + k);
+  }
+  const float ssum = block_sum<kRowThreads>(s[0] + s[1], red_f);
+  const float usum = block_sum<kRowThreads>(u[0] + u[1], red_f);
+  idx = block_min_i<kRowThreads>(idx, red_i);
+  if (tid == 0) part[row * splits + c] = Part1{ref, ssum, usum, m, idx, 0, 0, 0};
+}
+
+// ------------------------------------------------------------------ combining the slices of a row
+struct RowStat {
+  float m, S, h;        // row max, sum exp(x - m), normalized entropy from the fp32 pass
+  float pmax;           // max probability rounded to the row dtype
+  int first_idx;        // first index holding the max logit
+  bool need_emu;        // entropy must be re-evaluated with per-element rounding
+  bool need_tie;        // rounded probabilities of distinct logits may tie with the max
+};
+
+struct VerifyParams {
+  int64_t vocab;
+  int splits;
+  int64_t chunk;
+  int gate_entropy;     // 1 when the entropy gate is active (lossy + entropy)
+  int entropy_policy;
+  float theta;
+  float ln_vocab;       // float(ln V), or 1 when V == 1 (lossy_tree_verify.py:68)
+};
+
+template <int DT>
+__device__ __forceinline__ float finish_entropy(float H, float ln_vocab) {
+  // sum rounded to the row dtype, divided by float(ln V), rounded again
+  return Elem<DT>::round(Elem<DT>::round(H) / ln_vocab);
+}
+
+template <int DT>
+__device__ RowStat combine_row(const Part1* __restrict__ p, const VerifyParams& vp) {
+  RowStat r;
+  float m = -INFINITY;
+  for (int c = 0; c < vp.splits; ++c) m = fmaxf(m, p[c].m);
+  float S = 0.f, U = 0.f;
+  int first = 0x7fffffff;
+  for (int c = 0; c < vp.splits; ++c) {
+    if (p[c].m == -INFINITY) continue;
+    const float d = fmaxf((p[c].ref - m) * kLog2e, -200.f);   // ref <= slice max <= m
+    const float w = __builtin_amdgcn_exp2f(d);
+    S = fmaf(p[c].s, w, S);
+    U = fmaf(fmaf(d, p[c].s, p[c].u), w, U);
+    if (p[c].m == m) first = min(first, p[c].idx);
+  }
+  r.m = m;
+  r.S = S;
+  r.first_idx = first;
+  r.pmax = Elem<DT>::round(1.0f / S);
+  const float H = logf(S) - kLn2 * U / S;
+  r.h = finish_entropy<DT>(H, vp.ln_vocab);
+  const float h_raw = H / vp.ln_vocab;
+  r.need_emu = false;
+  if (vp.gate_entropy && DT != SUBSPEC_F32) {
+    const float band = 0.02f * fabsf(vp.theta) + 1e-3f;
+    r.need_emu = vp.entropy_policy == SUBSPEC_ENTROPY_ALWAYS || DT == SUBSPEC_F16 ||
+                 fabsf(h_raw - vp.theta) <= band;
+  }
+  // Two distinct logits of the row dtype differ by >= 2 ulp-of-one when |max| >= 2, so their
+  // probabilities differ by more than one ulp and cannot round to the same value unless the
+  // rounded maximum is subnormal.
+  r.need_tie = !(fabsf(m) >= 2.0f && (1.0f / S) >= Elem<DT>::min_normal());
+  return r;
+}
+
+// probability of logit x in a row, as the reference stores it: exp(x - m) / S rounded to dtype
+template <int DT>
+__device__ __forceinline__ float rounded_prob(float x, float m, float S) {
+  return Elem<DT>::round(expf(x - m) / S);
+}
+
+// ------------------------------------------------------------------ kernel 2: rare exact pass
+template <int DT>
+__global__ __launch_bounds__(kRowThreads) void row_exact_kernel(
+    const void* __restrict__ logits, VerifyParams vp, const Part1* __restrict__ part1,
+    Part2* __restrict__ part2) {
+  __shared__ float red_f[kRowThreads / kWave];
+  __shared__ int red_i[kRowThreads / kWave];
+  const int64_t row = blockIdx.y;
+  const int c = blockIdx.x;
+  const RowStat rs = combine_row<DT>(part1 + row * vp.splits, vp);
+  if (!rs.need_emu && !rs.need_tie) return;           // uniform across the workgroup
+  const int64_t c0 = (int64_t)c * vp.chunk;
+  const int64_t n = min(vp.chunk, vp.vocab - c0);
+  const int64_t base = row * vp.vocab + c0;
+  float acc = 0.f;
+  int tie = 0x7fffffff;
+  for (int64_t i = threadIdx.x; i < n; i += kRowThreads) {
+    const float x = Elem<DT>::load(logits, base + i);
+    const float p = rounded_prob<DT>(x, rs.m, rs.S);
+    if (rs.need_emu && p > 0.f) acc += Elem<DT>::round(-p * Elem<DT>::round(logf(p)));
+    if (p == rs.pmax && tie == 0x7fffffff) tie = (int)(c0 + i);
+  }
+  acc = block_sum<kRowThreads>(acc, red_f);
+  tie = block_min_i<kRowThreads>(tie, red_i);
+  if (threadIdx.x == 0) part2[row * vp.splits + c] = Part2{acc, tie};
+}
+
+// ------------------------------------------------------------------ kernel 3: per-tree tail
+struct TreeParams {
+  int64_t rows, n_nodes;
+  int root, skip;
+  int64_t eos;
+  int method, gate;
+  double theta;
+  int window;
+};
+
+template <int DT>
+__global__ __launch_bounds__(kTailThreads) void tree_accept_kernel(
+    const void* __restrict__ logits, VerifyParams vp, TreeParams tp,
+    const Part1* __restrict__ part1, const Part2* __restrict__ part2,
+    const int32_t* __restrict__ token_ids, const int32_t* __restrict__ parents,
+    int64_t* __restrict__ out_tokens, int64_t* __restrict__ out_ctx, int32_t* __restrict__ out_counts,
+    int64_t* __restrict__ node_target, float* __restrict__ node_entropy, float* __restrict__ node_child_prob) {
+  constexpr int N = SUBSPEC_MAX_TREE_NODES;
+  __shared__ float sm_m[N], sm_S[N], sm_h[N], sm_cp[N];
+  __shared__ int sm_tgt[N], sm_tok[N], sm_par[N];
+  __shared__ short sm_head[N], sm_next[N], sm_best_next[N], sm_best_len[N], sm_exact_after[N];
+  __shared__ int sm_status;
+
+  const int b = blockIdx.x;
+  const int tid = threadIdx.x;
+  const int rows = (int)tp.rows, n_nodes = (int)tp.n_nodes, skip = tp.skip;
+  const bool lossy = tp.method == SUBSPEC_VERIFY_LOSSY;
+  token_ids += (int64_t)b * n_nodes;
+  parents += (int64_t)b * n_nodes;
+  if (tid == 0) sm_status = 0;
+  __syncthreads();
+
+  // ---- per scored row: max, sum, argmax token, entropy
+  if (tid < rows) {
+    const int64_t grow = (int64_t)b * rows + tid;
+    const RowStat rs = combine_row<DT>(part1 + grow * vp.splits, vp);
+    int tgt = rs.first_idx;
+    float h = rs.h;
+    if (rs.need_emu || rs.need_tie) {
+      float H = 0.f;
+      int tie = 0x7fffffff;
+      for (int c = 0; c < vp.splits; ++c) {
+        H += part2[grow * vp.splits + c].esum;
+        tie = min(tie, part2[grow * vp.splits + c].tie_idx);
+      }
+      if (rs.need_tie && tie != 0x7fffffff) tgt = tie;
+      if (rs.need_emu) h = finish_entropy<DT>(H, vp.ln_vocab);
+    }
+    sm_m[tid] = rs.m;
+    sm_S[tid] = rs.S;
+    sm_tgt[tid] = tgt;
+    sm_h[tid] = h;
+    node_target[grow] = tgt;
+    if (vp.gate_entropy) node_entropy[grow] = h;
+  }
+  if (tid < n_nodes) {
+    sm_tok[tid] = token_ids[tid];
+    const int p = parents[tid];
+    sm_par[tid] = p;
+    if (p >= tid) atomicOr(&sm_status, 2);            // precondition: parents precede children
+  }
+  __syncthreads();
+
+  // ---- p[parent(i), token(i)] for every node whose parent row was scored
+  if (tid < n_nodes) {
+    float cp = -1.f;
+    const int p = sm_par[tid];
+    if (p >= 0) {
+      int rp = p - skip;
+      if (rp < 0 && !lossy) rp += rows;                // the exact walk indexes rows like a python list
+      const int tk = sm_tok[tid];
+      if (rp >= 0 && rp < rows && tk >= 0 && tk < vp.vocab) {
+        const float x = Elem<DT>::load(logits, ((int64_t)b * rows + rp) * vp.vocab + sm_tok[tid]);
+        cp = rounded_prob<DT>(x, sm_m[rp], sm_S[rp]);
+      }
+    }
+    sm_cp[tid] = cp;
+    const int local = tid - skip;
+    if (local >= 0 && local < rows) node_child_prob[(int64_t)b * rows + local] = cp;
+  }
+  __syncthreads();
+  if (tid != 0) return;
+
+  out_tokens += (int64_t)b * (n_nodes + 1);
+  out_ctx += (int64_t)b * (n_nodes + 1);
+  int emitted = 0, accept = 0, total = 0;
+
+  if (!lossy) {
+    // ---------------- greedy walk in original indexing (tree_verify.py:49-106)
+    for (int i = 0; i < n_nodes; ++i) sm_head[i] = -1;
+    for (int i = n_nodes - 1; i >= 1; --i) {
+      const int p = sm_par[i];
+      if (p >= 0 && p < n_nodes) { sm_next[i] = sm_head[p]; sm_head[p] = (short)i; }
+    }
+    int cur = tp.root;
+    int bonus = -1;
+    bool bad = cur < 0 || cur >= n_nodes;
+    auto row_of = [&](int node) { int r = node - skip; if (r < 0) r += rows; return r; };
+    while (!bad && sm_head[cur] >= 0) {
+      ++total;
+      const int r = row_of(cur);
+      if (r < 0 || r >= rows) { bad = true; break; }
+      const int t = sm_tgt[r];
+      int hit = -1;
+      for (int c = sm_head[cur]; c >= 0; c = sm_next[c])
+        if (sm_tok[c] == t) { hit = c; break; }
+      if (hit < 0) { bonus = t; break; }
+      ++accept;
+      out_tokens[emitted] = t;
+      out_ctx[emitted] = cur;
+      ++emitted;
+      if (tp.eos >= 0 && (int64_t)t == tp.eos) break;
+      cur = hit;
+      if (sm_head[cur] < 0) break;
+      if (sm_head[cur] - skip >= rows) break;          // children were not scored in this call
+    }
+    if (!bad && (emitted == 0 || tp.eos < 0 || out_tokens[emitted - 1] != tp.eos)) {
+      if (bonus < 0) {
+        const int r = row_of(cur);
+        if (r < 0 || r >= rows) bad = true; else bonus = sm_tgt[r];
+      }
+      if (!bad) { out_tokens[emitted] = bonus; out_ctx[emitted] = cur; ++emitted; }
+    }
+    if (bad) sm_status |= 1;
+  } else {
+    // ---------------- bottom-up DP in local indexing (lossy_tree_verify.py:112-168)
+    const int nl = min(rows, n_nodes - skip);
+    if (nl <= 0) {
+      out_tokens[0] = rows > 0 ? sm_tgt[0] : 0;
+      out_ctx[0] = tp.root;
+      emitted = 1;
+    } else {
+      int root = tp.root - skip;
+      if (root < 0 || root >= nl) root = 0;
+      for (int i = 0; i < nl; ++i) { sm_head[i] = -1; sm_best_next[i] = -1; sm_best_len[i] = 0; sm_exact_after[i] = 0; }
+      for (int i = nl - 1; i >= 0; --i) {
+        const int p = sm_par[i + skip] - skip;
+        if (p >= 0 && p < nl && p != i) { sm_next[i] = sm_head[p]; sm_head[p] = (short)i; }
+      }
+      const bool use_entropy = tp.gate == SUBSPEC_GATE_ENTROPY;
+      const int need = max(0, tp.window);
+      for (int u = nl - 1; u >= 0; --u) {
+        if (sm_head[u] < 0) continue;
+        const int tgt = sm_tgt[u];
+        int best_exact = -1;
+        for (int c = sm_head[u]; c >= 0; c = sm_next[c])
+          if (sm_tok[c + skip] == tgt) best_exact = max(best_exact, (int)sm_exact_after[c]);
+        if (best_exact >= 0) sm_exact_after[u] = (short)(1 + best_exact);
+        int pick = -1, pick_len = 0;
+        bool pick_exact = false;
+        float pick_p = -1.f;
+        const bool gate_blocks_u = use_entropy && ((double)sm_h[u] >= tp.theta);
+        for (int c = sm_head[u]; c >= 0; c = sm_next[c]) {
+          const bool is_exact = sm_tok[c + skip] == tgt;
+          float p = -1.f;
+          if (!is_exact) {
+            if (sm_exact_after[c] < need) continue;
+            if (gate_blocks_u) continue;
+            p = sm_cp[c + skip];
+            if (!use_entropy && (double)p < tp.theta) continue;
+          }
+          const int len = 1 + sm_best_len[c];
+          if (len > pick_len) { pick = c; pick_len = len; pick_exact = is_exact; pick_p = p; }
+          else if (len == pick_len) {
+            if (is_exact && !pick_exact) { pick = c; pick_exact = true; pick_p = p; }
+            else if (!is_exact && !pick_exact && p > pick_p) { pick = c; pick_p = p; }
+          }
+        }
+        if (pick >= 0 && pick_len > 0) { sm_best_next[u] = (short)pick; sm_best_len[u] = (short)pick_len; }
+      }
+      int ctx = root;
+      while (true) {                                   // lossy_tree_verify.py:247-286
+        const int nxt = sm_best_next[ctx];
+        if (nxt < 0) break;
+        const int t = sm_tok[nxt + skip];
+        out_tokens[emitted] = t;
+        out_ctx[emitted] = ctx + skip;
+        ++emitted;
+        if (tp.eos >= 0 && (int64_t)t == tp.eos) break;
+        ctx = nxt;
+      }
+      accept = emitted;
+      if (emitted == 0 || tp.eos < 0 || out_tokens[emitted - 1] != tp.eos) {
+        out_tokens[emitted] = sm_tgt[ctx];
+        out_ctx[emitted] = ctx + skip;
+        ++emitted;
+      }
+      total = emitted;
+    }
+  }
+  out_counts[b * 4 + 0] = emitted;
+  out_counts[b * 4 + 1] = accept;
+  out_counts[b * 4 + 2] = total;
+  out_counts[b * 4 + 3] = sm_status;
+}
+
+// ------------------------------------------------------------------ host side
+struct Plan { int vec, splits; int64_t chunk; };
+
+// Slices per row: enough workgroups to cover the chip several times over when there are few
+// rows, one slice per row when there are many; a slice is a whole number of 512-thread tiles.
+static bool make_plan(const void* logits, int dtype, int64_t total_rows, int64_t vocab, Plan* pl) {
+  const int vec_full = dtype == SUBSPEC_F32 ? 4 : 8;
+  const bool aligned = (vocab % vec_full == 0) && ((uintptr_t)logits % 16 == 0);
+  pl->vec = aligned ? vec_full : 1;
+  const int64_t quantum = (int64_t)kRowThreads * pl->vec;
+  int64_t splits = (2048 + total_rows - 1) / total_rows;
+  splits = std::min<int64_t>(splits, std::max<int64_t>(1, vocab / 8192));
+  splits = std::max<int64_t>(1, std::min<int64_t>(splits, kMaxSplits));
+  int64_t chunk = (vocab + splits - 1) / splits;
+  chunk = (chunk + quantum - 1) / quantum * quantum;
+  splits = (vocab + chunk - 1) / chunk;
+  if (splits > kMaxSplits) return false;
+  pl->splits = (int)splits;
+  pl->chunk = chunk;
+  return true;
+}
+
+template <int DT, int VEC>
+static void launch_partial(const Plan& pl, dim3 grid, hipStream_t st, const void* logits, int64_t vocab, Part1* p1) {
+  hipLaunchKernelGGL((row_partial_kernel<DT, VEC, 4>), grid, dim3(kRowThreads), 0, st, logits, vocab, pl.splits,
+                     pl.chunk, p1);
+}
+
+template <int DT>
+static int run_verify(const void* logits, int64_t batch, int64_t rows, int64_t vocab, const Plan& pl,
+                      const VerifyParams& vp, const TreeParams& tp, Part1* p1, Part2* p2,
+                      const int32_t* token_ids, const int32_t* parents, int64_t* out_tokens, int64_t* out_ctx,
+                      int32_t* out_counts, int64_t* node_target, float* node_entropy, float* node_child_prob,
+                      hipStream_t st) {
+  const dim3 grid(pl.splits, (unsigned)(batch * rows));
+  if (pl.vec == 1) launch_partial<DT, 1>(pl, grid, st, logits, vocab, p1);
+  else launch_partial<DT, (DT == SUBSPEC_F32 ? 4 : 8)>(pl, grid, st, logits, vocab, p1);
+  hipLaunchKernelGGL((row_exact_kernel<DT>), grid, dim3(kRowThreads), 0, st, logits, vp, p1, p2);
+  hipLaunchKernelGGL((tree_accept_kernel<DT>), dim3((unsigned)batch), dim3(kTailThreads), 0, st, logits, vp, tp,
+                     p1, p2, token_ids, parents, out_tokens, out_ctx, out_counts, node_target, node_entropy,
+                     node_child_prob);
+  SUBSPEC_CHECK_HIP(hipGetLastError());
+  return SUBSPEC_OK;
+}
+
+}  // namespace subspec
+
+using namespace subspec;
+
+extern "C" size_t subspec_tree_verify_workspace(int64_t batch, int64_t rows, int64_t vocab, int dtype) {
+  (void)vocab; (void)dtype;
+  if (batch <= 0 || rows <= 0) return 256;
+  const size_t n = (size_t)batch * rows * kMaxSplits;
+  return align_up(n * sizeof(Part1), 256) + align_up(n * sizeof(Part2), 256);
+}
+
+extern "C" int subspec_tree_verify(const void* logits, int dtype, int64_t batch, int64_t rows, int64_t vocab,
+                                   const int32_t* token_ids, const int32_t* parents, int64_t n_nodes,
+                                   int32_t root, int32_t skip_nodes, int64_t eos_token_id,
+                                   int verify_method, int threshold_method, double threshold, int32_t window_size,
+                                   int entropy_policy, void* workspace, size_t workspace_bytes,
+                                   int64_t* out_tokens, int64_t* out_ctx, int32_t* out_counts,
+                                   int64_t* node_target, float* node_entropy, float* node_child_prob,
+                                   void* stream) {
+  if (!dtype_ok(dtype)) SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "tree_verify: unknown dtype %d", dtype);
+  if (!logits || !token_ids || !parents || !workspace || !out_tokens || !out_ctx || !out_counts || !node_target ||
+      !node_entropy || !node_child_prob)
+    SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "tree_verify: null pointer argument");
+  if (batch <= 0 || rows <= 0 || vocab <= 0 || n_nodes <= 0)
+    SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "tree_verify: batch=%lld rows=%lld vocab=%lld n_nodes=%lld must be positive",
+                 (long long)batch, (long long)rows, (long long)vocab, (long long)n_nodes);
+  if (rows > SUBSPEC_MAX_TREE_NODES || n_nodes > SUBSPEC_MAX_TREE_NODES)
+    SUBSPEC_FAIL(SUBSPEC_ERR_LIMIT, "tree_verify: rows=%lld / n_nodes=%lld exceed the %d-node limit",
+                 (long long)rows, (long long)n_nodes, SUBSPEC_MAX_TREE_NODES);
+  if (vocab >= (int64_t)1 << 31 || batch * rows > 65535)
+    SUBSPEC_FAIL(SUBSPEC_ERR_LIMIT, "tree_verify: vocab=%lld or batch*rows=%lld too large", (long long)vocab,
+                 (long long)(batch * rows));
+  if (verify_method != SUBSPEC_VERIFY_EXACT && verify_method != SUBSPEC_VERIFY_LOSSY)
+    SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "tree_verify: unsupported verify_method %d", verify_method);
+  if (threshold_method != SUBSPEC_GATE_ENTROPY && threshold_method != SUBSPEC_GATE_PROB)
+    SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "tree_verify: unsupported threshold_method %d", threshold_method);
+  if (skip_nodes < 0 || skip_nodes >= n_nodes + rows)
+    SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "tree_verify: skip_nodes=%d out of range", skip_nodes);
+  if (workspace_bytes < subspec_tree_verify_workspace(batch, rows, vocab, dtype))
+    SUBSPEC_FAIL(SUBSPEC_ERR_WORKSPACE, "tree_verify: workspace of %zu bytes is smaller than the %zu required",
+                 workspace_bytes, subspec_tree_verify_workspace(batch, rows, vocab, dtype));
+  if ((uintptr_t)workspace % 16 != 0) SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "tree_verify: workspace must be 16-byte aligned");
+  if ((uintptr_t)logits % dtype_size(dtype) != 0) SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "tree_verify: logits misaligned");
+
+  Plan pl;
+  if (!make_plan(logits, dtype, batch * rows, vocab, &pl))
+    SUBSPEC_FAIL(SUBSPEC_ERR_LIMIT, "tree_verify: vocab=%lld needs more than %d slices per row", (long long)vocab,
+                 kMaxSplits);
+  const size_t n = (size_t)batch * rows * kMaxSplits;
+  Part1* p1 = (Part1*)workspace;
+  Part2* p2 = (Part2*)((char*)workspace + align_up(n * sizeof(Part1), 256));
+
+  VerifyParams vp;
+  vp.vocab = vocab;
+  vp.splits = pl.splits;
+  vp.chunk = pl.chunk;
+  vp.gate_entropy = (verify_method == SUBSPEC_VERIFY_LOSSY && threshold_method == SUBSPEC_GATE_ENTROPY) ? 1 : 0;
+  vp.entropy_policy = entropy_policy;
+  vp.theta = (float)threshold;
+  vp.ln_vocab = vocab > 1 ? (float)log((double)vocab) : 1.0f;
+  TreeParams tp;
+  tp.rows = rows;
+  tp.n_nodes = n_nodes;
+  tp.root = root;
+  tp.skip = skip_nodes;
+  tp.eos = eos_token_id;
+  tp.method = verify_method;
+  tp.gate = threshold_method;
+  tp.theta = threshold;
+  tp.window = window_size;
+  hipStream_t st = (hipStream_t)stream;
+  switch (dtype) {
+    case SUBSPEC_F32:
+      return run_verify<SUBSPEC_F32>(logits, batch, rows, vocab, pl, vp, tp, p1, p2, token_ids, parents, out_tokens,
+                                     out_ctx, out_counts, node_target, node_entropy, node_child_prob, st);
+    case SUBSPEC_F16:
+      return run_verify<SUBSPEC_F16>(logits, batch, rows, vocab, pl, vp, tp, p1, p2, token_ids, parents, out_tokens,
+                                     out_ctx, out_counts, node_target, node_entropy, node_child_prob, st);
+    default:
+      return run_verify<SUBSPEC_BF16>(logits, batch, rows, vocab, pl, vp, tp, p1, p2, token_ids, parents, out_tokens,
+                                      out_ctx, out_counts, node_target, node_entropy, node_child_prob, st);
+  }
+}

@@ -1,0 +1,133 @@
+"""Thin torch-tensor front ends of the C ABI: pointer extraction, shape checks, output allocation.
+
+torch is used for device memory and the current stream only; all arithmetic happens in
+libsubspec_hip.so.
+"""
+from __future__ import annotations
+
+from typing import Dict, Optional
+
+import torch
+
+from . import _lib as L
+
+_DT = {torch.float32: L.F32, torch.float16: L.F16, torch.bfloat16: L.BF16}
+
+
+def _dtype_code(t: torch.Tensor) -> int:
+    try:
+        return _DT[t.dtype]
+    except KeyError:
+        raise ValueError(f"unsupported dtype {t.dtype}; expected float32, float16 or bfloat16") from None
+
+
+def _require_gpu(*tensors: torch.Tensor) -> torch.device:
+    dev = tensors[0].device
+    for t in tensors:
+        if t.device.type != "cuda":
+            raise L.SubspecHipError("the HIP kernels need device tensors (no CPU fallback)")
+        if t.device != dev:
+            raise ValueError("all tensors must live on the same device")
+    return dev
+
+
+def _stream(dev: torch.device) -> int:
+    return torch.cuda.current_stream(dev).cuda_stream
+
+
+def tree_verify(
+    logits: torch.Tensor,            # [B, rows, V] or [rows, V]
+    token_ids: torch.Tensor,         # int32 [B, n] or [n], device
+    parents: torch.Tensor,           # int32 [B, n] or [n], device
+    *,
+    root: int = 0,
+    skip_nodes: int = 0,
+    eos_token_id: Optional[int] = None,
+    verify_method: str = "exact",
+    threshold_method: str = "prob",
+    threshold: float = 0.0,
+    window_size: int = 1,
+    exact_entropy: bool = False,
+    workspace: Optional[torch.Tensor] = None,
+) -> Dict[str, torch.Tensor]:
+    """Runs the fused verifier; everything stays on the device (no synchronisation here).
+
+    Returns device tensors: ``tokens`` / ``contexts`` int64 [B, n+1], ``counts`` int32 [B, 4]
+    (emitted, accept_len, total_len, status) and the per-node ``target`` int64 / ``entropy`` /
+    ``child_prob`` float32 [B, rows].
+    """
+    if logits.dim() == 2:
+        logits = logits.unsqueeze(0)
+    if token_ids.dim() == 1:
+        token_ids, parents = token_ids.unsqueeze(0), parents.unsqueeze(0)
+    if logits.dim() != 3 or token_ids.dim() != 2 or parents.shape != token_ids.shape:
+        raise ValueError("expected logits [B, rows, V] and token_ids / parents [B, n]")
+    dev = _require_gpu(logits, token_ids, parents)
+    B, rows, V = logits.shape
+    n = token_ids.shape[1]
+    if token_ids.shape[0] != B:
+        raise ValueError(f"batch mismatch: logits {B} vs tree arrays {token_ids.shape[0]}")
+    method = {"exact": L.VERIFY_EXACT, "lossy": L.VERIFY_LOSSY}.get(str(verify_method or "exact").strip().lower())
+    if method is None:
+        raise ValueError(f"Unsupported verify_method: {verify_method!r} (supported: 'exact', 'lossy')")
+    gate = {"entropy": L.GATE_ENTROPY, "prob": L.GATE_PROB}.get(str(threshold_method or "entropy").strip().lower())
+    if gate is None:
+        raise ValueError(f"Unsupported threshold_method: {threshold_method!r} (supported: 'entropy', 'prob')")
+    logits = logits.contiguous()
+    token_ids = token_ids.to(torch.int32).contiguous()
+    parents = parents.to(torch.int32).contiguous()
+    lib = L.lib()
+    need = lib.subspec_tree_verify_workspace(B, rows, V, _dtype_code(logits))
+    if workspace is None:
+        workspace = torch.empty(need, dtype=torch.uint8, device=dev)
+    out = {
+        "tokens": torch.empty((B, n + 1), dtype=torch.int64, device=dev),
+        "contexts": torch.empty((B, n + 1), dtype=torch.int64, device=dev),
+        "counts": torch.empty((B, 4), dtype=torch.int32, device=dev),
+        "target": torch.empty((B, rows), dtype=torch.int64, device=dev),
+        "entropy": torch.zeros((B, rows), dtype=torch.float32, device=dev),
+        "child_prob": torch.empty((B, rows), dtype=torch.float32, device=dev),
+    }
+    code = lib.subspec_tree_verify(
+        logits.data_ptr(), _dtype_code(logits), B, rows, V, token_ids.data_ptr(), parents.data_ptr(), n,
+        int(root), int(skip_nodes), -1 if eos_token_id is None else int(eos_token_id),
+        method, gate, float(threshold), int(window_size),
+        L.ENTROPY_ALWAYS if exact_entropy else L.ENTROPY_GUARD,
+        workspace.data_ptr(), workspace.numel() * workspace.element_size(),
+        out["tokens"].data_ptr(), out["contexts"].data_ptr(), out["counts"].data_ptr(),
+        out["target"].data_ptr(), out["entropy"].data_ptr(), out["child_prob"].data_ptr(), _stream(dev))
+    L.check(code, "subspec_tree_verify")
+    return out
+
+
+def kv_compact_(
+    cache: torch.Tensor,             # [..., seq, head_dim], contiguous; every leading index is a slab
+    contexts: torch.Tensor,          # int64 device tensor, kept rows relative to `offset`
+    offset: int,
+    count: Optional[int] = None,
+    count_dev: Optional[torch.Tensor] = None,
+    max_count: Optional[int] = None,
+) -> torch.Tensor:
+    """In place: ``cache[..., offset + j, :] = cache[..., offset + contexts[j], :]`` for j < count."""
+    dev = _require_gpu(cache, contexts)
+    if not cache.is_contiguous():
+        raise ValueError("kv_compact_: cache must be contiguous")
+    if contexts.dtype != torch.int64 or not contexts.is_contiguous():
+        raise ValueError("kv_compact_: contexts must be a contiguous int64 tensor")
+    seq, hd = cache.shape[-2], cache.shape[-1]
+    row_bytes = hd * cache.element_size()
+    n_slabs = cache.numel() // (seq * hd)
+    if count_dev is None:
+        count = int(contexts.numel()) if count is None else int(count)
+    else:
+        _require_gpu(count_dev)
+        if count_dev.dtype != torch.int32:
+            raise ValueError("kv_compact_: count_dev must be int32")
+        count = 0
+    if max_count is None:
+        max_count = min(int(contexts.numel()), L.MAX_TREE_NODES) if count_dev is not None else count
+    code = L.lib().subspec_kv_compact(
+        cache.data_ptr(), None, n_slabs, seq * row_bytes, seq, row_bytes, int(offset), contexts.data_ptr(),
+        None if count_dev is None else count_dev.data_ptr(), count, int(max_count), _stream(dev))
+    L.check(code, "subspec_kv_compact")
+    return cache
