@@ -111,6 +111,28 @@ int subspec_kv_compact(void* base, void* const* slab_ptrs, int64_t n_slabs, int6
                        const int64_t* ctx, const int32_t* count_dev, int32_t count_host, int32_t max_count,
                        void* stream);
 
+/* ------------------------------------------------------------------------------------------
+ * Top-k draft-tree expansion: per batch item the global top-k over (leaves x vocab) of
+ * round_dtype(probs[b, l, v] * parent_probs[b, l]), sorted by value descending and, among equal
+ * values, flat index (l * vocab + v) ascending.
+ *
+ * Replaces  DraftModelBase.topk_sampling -> _topk_flatten   specdecodes/models/draft_models/base.py:268-305
+ *           (and its graph twin _topk_flatten_for_graph :307-323): torch.mul into a full-size buffer
+ *           followed by torch.topk over the flattened row.
+ *
+ * probs          device [batch, leaves, vocab] contiguous, element type `dtype`
+ * parent_probs   device [batch, leaves], same dtype
+ * k              1 <= k <= min(vocab, 64)   (the reference clamps k to vocab on the host)
+ * token_ids      device int64 [batch, k]    flat index %  vocab
+ * topk_probs     device `dtype` [batch, k]
+ * parent_indices device int64 [batch, k]    flat index // vocab
+ */
+size_t subspec_topk_expand_workspace(int64_t batch, int64_t leaves, int64_t vocab, int32_t k);
+
+int subspec_topk_expand(const void* probs, const void* parent_probs, int dtype, int64_t batch, int64_t leaves,
+                        int64_t vocab, int32_t k, void* workspace, size_t workspace_bytes,
+                        int64_t* token_ids, void* topk_probs, int64_t* parent_indices, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -40,13 +40,8 @@ __device__ __forceinline__ float f16_bits_to_float(uint32_t b) {
   c.u = (uint16_t)b;
   return (float)c.h;
 }
-// round-to-nearest-even to bfloat16, result widened back to float (NaN kept as NaN)
-__device__ __forceinline__ float round_bf16(float x) {
-  uint32_t u = __float_as_uint(x);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return x;
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return __uint_as_float(u & 0xffff0000u);
-}
+// round-to-nearest-even to bfloat16, result widened back to float (v_cvt_pk_bf16_f32 on gfx950)
+__device__ __forceinline__ float round_bf16(float x) { return (float)(__bf16)x; }
 __device__ __forceinline__ float round_f16(float x) { return (float)(_Float16)x; }
 
 template <int DT> struct Elem;

@@ -1,0 +1,327 @@
+// Top-k draft-tree expansion for gfx950: global top-k over (leaves x vocab) of
+// round(p[l, v] * parent_prob[l]) with the canonical tie rule (value descending, flat index
+// ascending), fused into one pass over the probabilities.
+//
+// Follows DraftModelBase.topk_sampling / _topk_flatten
+// (specdecodes/models/draft_models/base.py:268-305): buf = sampled_probs * parent_probs[..., None]
+// rounded to the tensor dtype; topk(buf.view(B, L*V), min(k, V), sorted=True); token = idx % V,
+// parent = idx // V.  torch.topk leaves the order of equal values unspecified; this kernel fixes it
+// to the lowest flat index first.
+//
+//   1. topk_slice_kernel - grid (slices, B*L), 512 threads.  A workgroup streams its slice of one
+//      row once.  The k-th largest of 512 per-thread maxima over a 16K-element sample gives a
+//      threshold; afterwards every element costs unpack + multiply + round + compare, and the few
+//      survivors go to a candidate list in LDS that is pruned to the slice's exact top-k in
+//      (key, index) order.  HBM-bound: algorithmic bytes = B * L * V * sizeof(dtype).
+//   2. topk_merge_kernel - one workgroup per batch item ranks the <= slices*L*k candidates and
+//      writes values, token ids and parent indices in sorted order.
+#include "common.h"
+#include <algorithm>
+
+namespace subspec {
+
+constexpr int kTopkThreads = 512;
+constexpr int kTopkCap = 4608;          // candidate slots per workgroup: one 4096-element group + 512
+constexpr int kTopkPruneAt = 512;
+constexpr int kTopkMaxK = 64;
+constexpr int kTopkMaxSlices = 64;
+constexpr int kMergeThreads = 1024;
+constexpr int kMergeCap = 4096;
+
+// (key, flat index) as one integer that sorts like "larger key first, then smaller index first"
+__device__ __forceinline__ uint64_t pack_candidate(float key, uint32_t flat) {
+  uint32_t b = __float_as_uint(key);
+  b ^= (b & 0x80000000u) ? 0xffffffffu : 0x80000000u;
+  return ((uint64_t)b << 32) | (uint64_t)(0xffffffffu - flat);
+}
+__device__ __forceinline__ float candidate_key(uint64_t c) {
+  uint32_t b = (uint32_t)(c >> 32);
+  b ^= (b & 0x80000000u) ? 0x80000000u : 0xffffffffu;
+  return __uint_as_float(b);
+}
+__device__ __forceinline__ uint32_t candidate_flat(uint64_t c) { return 0xffffffffu - (uint32_t)c; }
+
+template <int DT, int VEC> struct PTile;
+template <> struct PTile<SUBSPEC_F32, 4> {
+  float4 r;
+  __device__ __forceinline__ void load(const void* p, int64_t i) { r = *(const float4*)((const float*)p + i); }
+  __device__ __forceinline__ float get(int k) const { return k == 0 ? r.x : k == 1 ? r.y : k == 2 ? r.z : r.w; }
+};
+template <> struct PTile<SUBSPEC_F32, 1> {
+  float r;
+  __device__ __forceinline__ void load(const void* p, int64_t i) { r = ((const float*)p)[i]; }
+  __device__ __forceinline__ float get(int) const { return r; }
+};
+template <int DT> struct PTile16x8 {
+  uint4 r;
+  __device__ __forceinline__ void load(const void* p, int64_t i) { r = *(const uint4*)((const uint16_t*)p + i); }
+  __device__ __forceinline__ float get(int k) const {
+    const uint32_t w = (k >> 1) == 0 ? r.x : (k >> 1) == 1 ? r.y : (k >> 1) == 2 ? r.z : r.w;
+    if (DT == SUBSPEC_BF16) return (k & 1) ? __uint_as_float(w & 0xffff0000u) : __uint_as_float(w << 16);
+    return f16_bits_to_float((k & 1) ? (w >> 16) : (w & 0xffffu));
+  }
+};
+template <> struct PTile<SUBSPEC_BF16, 8> : PTile16x8<SUBSPEC_BF16> {};
+template <> struct PTile<SUBSPEC_F16, 8> : PTile16x8<SUBSPEC_F16> {};
+template <int DT> struct PTile16x1 {
+  uint16_t r;
+  __device__ __forceinline__ void load(const void* p, int64_t i) { r = ((const uint16_t*)p)[i]; }
+  __device__ __forceinline__ float get(int) const {
+    return DT == SUBSPEC_BF16 ? bf16_bits_to_float(r) : f16_bits_to_float(r);
+  }
+};
+template <> struct PTile<SUBSPEC_BF16, 1> : PTile16x1<SUBSPEC_BF16> {};
+template <> struct PTile<SUBSPEC_F16, 1> : PTile16x1<SUBSPEC_F16> {};
+
+// k-th best (0-based rank k-1) of `count` packed candidates in LDS by counting; every thread calls.
+// Returns 0 (below every candidate) when count < k.  `out` is a one-word LDS scratch.
+template <int THREADS>
+__device__ uint64_t kth_best(const uint64_t* list, int count, int k, uint64_t* out) {
+  if (threadIdx.x == 0) *out = 0;
+  __syncthreads();
+  for (int i = threadIdx.x; i < count; i += THREADS) {
+    const uint64_t mine = list[i];
+    int rank = 0;
+    for (int j = 0; j < count; ++j) rank += list[j] > mine;
+    if (rank == k - 1) *out = mine;                    // packed values are distinct (distinct indices)
+  }
+  __syncthreads();
+  const uint64_t r = *out;
+  __syncthreads();
+  return r;
+}
+
+// Keeps only candidates >= cut (all of them when cut == 0).  Every thread calls.
+template <int THREADS>
+__device__ int prune_list(uint64_t* list, int count, uint64_t cut, int* counter) {
+  uint64_t keep[(kTopkCap + THREADS - 1) / THREADS];
+  int nkeep = 0;
+#pragma unroll
+  for (int s = 0; s < (kTopkCap + THREADS - 1) / THREADS; ++s) {
+    const int i = threadIdx.x + s * THREADS;
+    keep[s] = 0;
+    if (i < count && list[i] >= cut && list[i] != 0) { keep[s] = list[i]; ++nkeep; }
+  }
+  if (threadIdx.x == 0) *counter = 0;
+  __syncthreads();
+#pragma unroll
+  for (int s = 0; s < (kTopkCap + THREADS - 1) / THREADS; ++s)
+    if (keep[s] != 0) list[atomicAdd(counter, 1)] = keep[s];
+  __syncthreads();
+  (void)nkeep;
+  return *counter;
+}
+
+template <int DT, int VEC>
+__global__ __launch_bounds__(kTopkThreads) void topk_slice_kernel(
+    const void* __restrict__ probs, const void* __restrict__ parent_probs, int64_t vocab, int leaves, int splits,
+    int64_t chunk, int k, uint64_t* __restrict__ cand, int32_t* __restrict__ cand_count) {
+  __shared__ uint64_t list[kTopkCap];
+  __shared__ uint64_t sample[kTopkThreads];
+  __shared__ uint64_t kth_slot;
+  __shared__ int count, overflow;
+
+  const int64_t row = blockIdx.y;                      // b * leaves + l
+  const int c = blockIdx.x;
+  const int tid = threadIdx.x;
+  const int leaf = (int)(row % leaves);
+  const int64_t c0 = (int64_t)c * chunk;
+  const int64_t n = min(chunk, vocab - c0);
+  const int64_t base = row * vocab + c0;
+  const int64_t ntiles = n / VEC;
+  const float q = Elem<DT>::load(parent_probs, row);
+  const uint32_t flat0 = (uint32_t)((int64_t)leaf * vocab + c0);
+
+  // ---- threshold from a sample: k-th largest of the per-thread maxima over the first 4 tiles
+  float smax = -INFINITY;
+  uint32_t sflat = 0;
+  bool sany = false;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int64_t j = tid + (int64_t)i * kTopkThreads;
+    if (j < ntiles) {
+      PTile<DT, VEC> t;
+      t.load(probs, base + j * VEC);
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        const float key = Elem<DT>::round(t.get(e) * q);
+        if (!sany || key > smax) { smax = key; sflat = flat0 + (uint32_t)(j * VEC + e); sany = true; }
+      }
+    }
+  }
+  sample[tid] = sany ? pack_candidate(smax, sflat) : 0;
+  if (tid == 0) { count = 0; overflow = 0; }
+  __syncthreads();
+  uint64_t tau = kth_best<kTopkThreads>(sample, kTopkThreads, k, &kth_slot);
+  float tau_key = tau ? candidate_key(tau) : -INFINITY;
+
+  // ---- stream the slice; survivors go to the LDS list
+  const int64_t ngroups = (ntiles + kTopkThreads - 1) / kTopkThreads;
+  bool careful = false;
+  for (;;) {
+    for (int64_t g = 0; g < ngroups; ++g) {
+      const int64_t j = g * kTopkThreads + tid;
+      if (j < ntiles) {
+        PTile<DT, VEC> t;
+        t.load(probs, base + j * VEC);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+          const float key = Elem<DT>::round(t.get(e) * q);
+          if (key >= tau_key) {
+            const uint64_t pc = pack_candidate(key, flat0 + (uint32_t)(j * VEC + e));
+            if (pc >= tau) {
+              const int slot = atomicAdd(&count, 1);
+              if (slot < kTopkCap) list[slot] = pc; else overflow = 1;
+            }
+          }
+        }
+      }
+      if (careful) {
+        // per-group bookkeeping: the list never loses an entry because it is pruned to <= k
+        // whenever fewer than one group's worth of free slots remain
+        __syncthreads();
+        const int cnt = count;
+        __syncthreads();                               // nobody appends before everyone has read it
+        if (cnt > kTopkPruneAt) {
+          tau = kth_best<kTopkThreads>(list, cnt, k, &kth_slot);
+          tau_key = candidate_key(tau);
+          prune_list<kTopkThreads>(list, cnt, tau, &count);
+        }
+      }
+    }
+    __syncthreads();
+    if (!overflow) break;                              // workgroup-uniform
+    // too many survivors for the list (heavy ties or adversarial order): start over, pruning
+    // after every group so that nothing is dropped
+    careful = true;
+    __syncthreads();
+    if (tid == 0) { count = 0; overflow = 0; }
+    __syncthreads();
+  }
+
+  // ---- exact top-k of the slice in (key, index) order
+  int cnt = min(count, kTopkCap);
+  tau = kth_best<kTopkThreads>(list, cnt, k, &kth_slot);
+  cnt = prune_list<kTopkThreads>(list, cnt, tau, &count);
+  const int64_t slot0 = (row * splits + c) * kTopkMaxK;
+  for (int i = tid; i < cnt; i += kTopkThreads) cand[slot0 + i] = list[i];
+  if (tid == 0) cand_count[row * splits + c] = cnt;
+}
+
+template <int DT>
+__global__ __launch_bounds__(kMergeThreads) void topk_merge_kernel(
+    const uint64_t* __restrict__ cand, const int32_t* __restrict__ cand_count, int64_t vocab, int leaves, int splits,
+    int k, int64_t* __restrict__ token_ids, void* __restrict__ topk_probs, int64_t* __restrict__ parent_indices) {
+  __shared__ uint64_t list[kMergeCap];
+  __shared__ int total;
+  const int b = blockIdx.x;
+  if (threadIdx.x == 0) total = 0;
+  __syncthreads();
+  const int lists = leaves * splits;
+  for (int s = threadIdx.x; s < lists * kTopkMaxK; s += kMergeThreads) {
+    const int li = s / kTopkMaxK, i = s % kTopkMaxK;
+    const int64_t g = (int64_t)b * lists + li;
+    if (i < cand_count[g]) list[atomicAdd(&total, 1)] = cand[g * kTopkMaxK + i];
+  }
+  __syncthreads();
+  const int cnt = total;
+  for (int i = threadIdx.x; i < cnt; i += kMergeThreads) {
+    const uint64_t mine = list[i];
+    int rank = 0;
+    for (int j = 0; j < cnt; ++j) rank += list[j] > mine;
+    if (rank < k) {
+      const uint32_t flat = candidate_flat(mine);
+      token_ids[(int64_t)b * k + rank] = flat % vocab;
+      parent_indices[(int64_t)b * k + rank] = flat / vocab;
+      Elem<DT>::store(topk_probs, (int64_t)b * k + rank, candidate_key(mine));
+    }
+  }
+}
+
+struct TopkPlan { int vec, splits; int64_t chunk; };
+
+static bool topk_plan(const void* probs, int dtype, int64_t rows, int64_t vocab, int k, int leaves, TopkPlan* pl) {
+  const int vec_full = dtype == SUBSPEC_F32 ? 4 : 8;
+  const bool aligned = (vocab % vec_full == 0) && ((uintptr_t)probs % 16 == 0);
+  pl->vec = aligned ? vec_full : 1;
+  const int64_t quantum = (int64_t)kTopkThreads * pl->vec;
+  int64_t splits = (1024 + rows - 1) / rows;
+  splits = std::min<int64_t>(splits, std::max<int64_t>(1, vocab / 16384));
+  splits = std::min<int64_t>(splits, std::max<int64_t>(1, kMergeCap / ((int64_t)leaves * k)));
+  splits = std::max<int64_t>(1, std::min<int64_t>(splits, kTopkMaxSlices));
+  int64_t chunk = (vocab + splits - 1) / splits;
+  chunk = (chunk + quantum - 1) / quantum * quantum;
+  splits = (vocab + chunk - 1) / chunk;
+  pl->splits = (int)splits;
+  pl->chunk = chunk;
+  return (int64_t)leaves * splits * k <= kMergeCap;
+}
+
+template <int DT>
+static int run_topk(const void* probs, const void* parent_probs, int64_t batch, int leaves, int64_t vocab, int k,
+                    const TopkPlan& pl, uint64_t* cand, int32_t* cand_count, int64_t* token_ids, void* topk_probs,
+                    int64_t* parent_indices, hipStream_t st) {
+  const dim3 grid(pl.splits, (unsigned)(batch * leaves));
+  if (pl.vec == 1)
+    hipLaunchKernelGGL((topk_slice_kernel<DT, 1>), grid, dim3(kTopkThreads), 0, st, probs, parent_probs, vocab, leaves,
+                       pl.splits, pl.chunk, k, cand, cand_count);
+  else
+    hipLaunchKernelGGL((topk_slice_kernel<DT, (DT == SUBSPEC_F32 ? 4 : 8)>), grid, dim3(kTopkThreads), 0, st, probs,
+                       parent_probs, vocab, leaves, pl.splits, pl.chunk, k, cand, cand_count);
+  hipLaunchKernelGGL((topk_merge_kernel<DT>), dim3((unsigned)batch), dim3(kMergeThreads), 0, st, cand, cand_count,
+                     vocab, leaves, pl.splits, k, token_ids, topk_probs, parent_indices);
+  SUBSPEC_CHECK_HIP(hipGetLastError());
+  return SUBSPEC_OK;
+}
+
+}  // namespace subspec
+
+using namespace subspec;
+
+extern "C" size_t subspec_topk_expand_workspace(int64_t batch, int64_t leaves, int64_t vocab, int32_t k) {
+  (void)vocab; (void)k;
+  if (batch <= 0 || leaves <= 0) return 256;
+  const size_t lists = (size_t)batch * leaves * kTopkMaxSlices;
+  return align_up(lists * kTopkMaxK * sizeof(uint64_t), 256) + align_up(lists * sizeof(int32_t), 256);
+}
+
+extern "C" int subspec_topk_expand(const void* probs, const void* parent_probs, int dtype, int64_t batch,
+                                   int64_t leaves, int64_t vocab, int32_t k, void* workspace, size_t workspace_bytes,
+                                   int64_t* token_ids, void* topk_probs, int64_t* parent_indices, void* stream) {
+  if (!dtype_ok(dtype)) SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "topk_expand: unknown dtype %d", dtype);
+  if (!probs || !parent_probs || !workspace || !token_ids || !topk_probs || !parent_indices)
+    SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "topk_expand: null pointer argument");
+  if (batch <= 0 || leaves <= 0 || vocab <= 0 || k <= 0)
+    SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "topk_expand: batch=%lld leaves=%lld vocab=%lld k=%d must be positive",
+                 (long long)batch, (long long)leaves, (long long)vocab, k);
+  if (k > vocab) SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "topk_expand: k=%d exceeds vocab=%lld (clamp k on the host)", k, (long long)vocab);
+  if (k > kTopkMaxK) SUBSPEC_FAIL(SUBSPEC_ERR_LIMIT, "topk_expand: k=%d exceeds the limit of %d", k, kTopkMaxK);
+  if (leaves * vocab >= ((int64_t)1 << 32) || batch * leaves > 65535)
+    SUBSPEC_FAIL(SUBSPEC_ERR_LIMIT, "topk_expand: leaves*vocab=%lld or batch*leaves=%lld too large",
+                 (long long)(leaves * vocab), (long long)(batch * leaves));
+  if (workspace_bytes < subspec_topk_expand_workspace(batch, leaves, vocab, k))
+    SUBSPEC_FAIL(SUBSPEC_ERR_WORKSPACE, "topk_expand: workspace of %zu bytes is smaller than the %zu required",
+                 workspace_bytes, subspec_topk_expand_workspace(batch, leaves, vocab, k));
+  if ((uintptr_t)workspace % 16 != 0) SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "topk_expand: workspace must be 16-byte aligned");
+  if ((uintptr_t)probs % dtype_size(dtype) != 0 || (uintptr_t)parent_probs % dtype_size(dtype) != 0)
+    SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "topk_expand: misaligned input");
+  TopkPlan pl;
+  if (!topk_plan(probs, dtype, batch * leaves, vocab, k, (int)leaves, &pl))
+    SUBSPEC_FAIL(SUBSPEC_ERR_LIMIT, "topk_expand: leaves=%lld x k=%d candidates exceed the merge capacity",
+                 (long long)leaves, k);
+  const size_t lists = (size_t)batch * leaves * kTopkMaxSlices;
+  uint64_t* cand = (uint64_t*)workspace;
+  int32_t* cand_count = (int32_t*)((char*)workspace + align_up(lists * kTopkMaxK * sizeof(uint64_t), 256));
+  hipStream_t st = (hipStream_t)stream;
+  switch (dtype) {
+    case SUBSPEC_F32:
+      return run_topk<SUBSPEC_F32>(probs, parent_probs, batch, (int)leaves, vocab, k, pl, cand, cand_count, token_ids,
+                                   topk_probs, parent_indices, st);
+    case SUBSPEC_F16:
+      return run_topk<SUBSPEC_F16>(probs, parent_probs, batch, (int)leaves, vocab, k, pl, cand, cand_count, token_ids,
+                                   topk_probs, parent_indices, st);
+    default:
+      return run_topk<SUBSPEC_BF16>(probs, parent_probs, batch, (int)leaves, vocab, k, pl, cand, cand_count,
+                                    token_ids, topk_probs, parent_indices, st);
+  }
+}

@@ -131,3 +131,35 @@ def kv_compact_(
         None if count_dev is None else count_dev.data_ptr(), count, int(max_count), _stream(dev))
     L.check(code, "subspec_kv_compact")
     return cache
+
+
+def topk_expand(sampled_probs: torch.Tensor, parent_probs: torch.Tensor, k: int,
+                workspace: Optional[torch.Tensor] = None):
+    """Global top-k over (leaves x vocab) of ``round(sampled_probs * parent_probs[..., None])``.
+
+    ``sampled_probs`` [B, L, V], ``parent_probs`` [B, L] (same dtype).  Returns
+    ``(token_ids int64 [B, k], topk_probs dtype [B, k], parent_indices int64 [B, k])`` on the device,
+    sorted by value descending, equal values by flat index ascending.
+    """
+    if sampled_probs.dim() != 3 or parent_probs.shape != sampled_probs.shape[:2]:
+        raise ValueError("expected sampled_probs [B, L, V] and parent_probs [B, L]")
+    if parent_probs.dtype != sampled_probs.dtype:
+        raise ValueError("sampled_probs and parent_probs must share a dtype")
+    dev = _require_gpu(sampled_probs, parent_probs)
+    B, Lv, V = sampled_probs.shape
+    k = min(int(k), int(V))
+    sampled_probs = sampled_probs.contiguous()
+    parent_probs = parent_probs.contiguous()
+    lib = L.lib()
+    need = lib.subspec_topk_expand_workspace(B, Lv, V, k)
+    if workspace is None:
+        workspace = torch.empty(need, dtype=torch.uint8, device=dev)
+    token_ids = torch.empty((B, k), dtype=torch.int64, device=dev)
+    parents = torch.empty((B, k), dtype=torch.int64, device=dev)
+    vals = torch.empty((B, k), dtype=sampled_probs.dtype, device=dev)
+    code = lib.subspec_topk_expand(
+        sampled_probs.data_ptr(), parent_probs.data_ptr(), _dtype_code(sampled_probs), B, Lv, V, k,
+        workspace.data_ptr(), workspace.numel() * workspace.element_size(),
+        token_ids.data_ptr(), vals.data_ptr(), parents.data_ptr(), _stream(dev))
+    L.check(code, "subspec_topk_expand")
+    return token_ids, vals, parents

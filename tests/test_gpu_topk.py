@@ -1,0 +1,88 @@
+"""GPU parity: top-k draft-tree expansion through the C ABI against the oracle.
+Bar: values, token ids and parent indices bit-exact under the canonical tie rule
+(value descending, flat index ascending)."""
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+from oracle import topk as ot
+from subspec_amd import ops
+
+DEV = "cuda:0"
+
+
+def _check(probs, parent, k):
+    tok, val, par = ops.topk_expand(probs.to(DEV), parent.to(DEV), k)
+    torch.cuda.synchronize()
+    e_tok, e_val, e_par = ot.topk_expand(probs, parent, k)
+    assert torch.equal(val.cpu(), e_val), (val.cpu(), e_val)
+    assert torch.equal(tok.cpu(), e_tok)
+    assert torch.equal(par.cpu(), e_par)
+    return tok.cpu(), val.cpu(), par.cpu()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_small_shapes_ragged_vocab(dtype):
+    g = torch.Generator().manual_seed(1)
+    for B, L, V, k in ((1, 1, 9, 9), (2, 3, 17, 5), (3, 4, 1001, 16), (1, 8, 5000, 8), (2, 10, 32000, 10),
+                       (4, 1, 40960, 64), (1, 6, 777, 6)):
+        print("topk", dtype, B, L, V, k, flush=True)
+        probs = torch.softmax(torch.randn(B, L, V, generator=g) * 3, -1).to(dtype)
+        parent = torch.rand(B, L, generator=g).to(dtype)
+        _check(probs, parent, k)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_heavy_ties_and_adversarial_order(dtype):
+    V = 40000
+    # fewer non-zero entries than k: the rest must be the lowest flat indices holding zero
+    probs = torch.zeros(1, 3, V, dtype=dtype)
+    probs[0, 1, 77] = 0.5
+    probs[0, 2, 5] = 0.25
+    parent = torch.tensor([[1.0, 0.5, 1.0]], dtype=dtype)
+    tok, val, par = _check(probs, parent, 8)
+    assert par.tolist()[0][:2] == [1, 2] or val.tolist()[0][0] == 0.25
+    # constant rows: every element ties
+    _check(torch.full((2, 2, V), 0.001, dtype=dtype), torch.ones(2, 2, dtype=dtype), 16)
+    # ascending order: every new element beats the running threshold
+    asc = (torch.arange(V, dtype=torch.float32) / V).to(dtype).view(1, 1, V)
+    _check(asc, torch.ones(1, 1, dtype=dtype), 16)
+    # descending order
+    _check(asc.flip(-1).contiguous(), torch.ones(1, 1, dtype=dtype), 16)
+
+
+def test_config2_rows_bf16_full_vocab():
+    g = torch.Generator().manual_seed(2)
+    V = 152064
+    logits = (torch.randn(48, 1, V, generator=g) * (torch.rand(48, 1, 1, generator=g) * 2.5 + 0.5)).to(torch.bfloat16)
+    probs = torch.softmax(logits, -1)
+    parent = torch.rand(48, 1, generator=g).to(torch.bfloat16)
+    tok, val, par = _check(probs, parent, 16)
+    # same values as the reference's literal torch.topk call (its index order within ties is unspecified)
+    t_tok, t_val, t_par = ot.topk_expand_torch(probs, parent, 16)
+    assert torch.equal(val, t_val)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+def test_draft_step_shape_full_vocab(dtype):
+    # one draft step of the real pipeline: batch 1, k leaves, temperature-sharpened distribution
+    g = torch.Generator().manual_seed(3)
+    V = 152064
+    probs = torch.softmax((torch.randn(1, 8, V, generator=g) * 2).to(dtype) / 0.2, -1)
+    parent = torch.rand(1, 8, generator=g).to(dtype)
+    _check(probs, parent, 8)
+    root = torch.softmax((torch.randn(1, 1, V, generator=g) * 2).to(dtype) / 0.2, -1)
+    _check(root, torch.ones(1, 1, dtype=dtype), 8)
+
+
+def test_argument_errors():
+    p = torch.rand(1, 1, 128, device=DEV)
+    with pytest.raises(ValueError):
+        ops.topk_expand(p, torch.ones(1, 2, device=DEV), 4)
+    with pytest.raises(ValueError):
+        ops.topk_expand(p, torch.ones(1, 1, device=DEV, dtype=torch.bfloat16), 4)
+    with pytest.raises(ValueError):
+        ops.topk_expand(p, torch.ones(1, 1, device=DEV), 100)       # k beyond the kernel's limit
+    tok, val, par = ops.topk_expand(torch.rand(1, 1, 5, device=DEV), torch.ones(1, 1, device=DEV), 50)
+    assert tok.shape == (1, 5)                                     # k clamps to the vocabulary
