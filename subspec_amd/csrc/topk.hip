@@ -157,45 +157,58 @@ __global__ __launch_bounds__(kTopkThreads) void topk_slice_kernel(
 
   // ---- stream the slice; survivors go to the LDS list
   const int64_t ngroups = (ntiles + kTopkThreads - 1) / kTopkThreads;
-  bool careful = false;
-  for (;;) {
+  auto scan_tile = [&](const PTile<DT, VEC>& t, int64_t j) {
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+      const float key = Elem<DT>::round(t.get(e) * q);
+      if (key >= tau_key) {
+        const uint64_t pc = pack_candidate(key, flat0 + (uint32_t)(j * VEC + e));
+        if (pc >= tau) {
+          const int slot = atomicAdd(&count, 1);
+          if (slot < kTopkCap) list[slot] = pc; else overflow = 1;
+        }
+      }
+    }
+  };
+  // fast path: four tiles per thread in flight, no bookkeeping between groups
+  constexpr int U = 4;
+  for (int64_t g0 = 0; g0 < ngroups; g0 += U) {
+    PTile<DT, VEC> t[U];
+#pragma unroll
+    for (int i = 0; i < U; ++i) {
+      const int64_t j = (g0 + i) * kTopkThreads + tid;
+      if (j < ntiles) t[i].load(probs, base + j * VEC);
+    }
+#pragma unroll
+    for (int i = 0; i < U; ++i) {
+      const int64_t j = (g0 + i) * kTopkThreads + tid;
+      if (j < ntiles) scan_tile(t[i], j);
+    }
+  }
+  __syncthreads();
+  if (overflow) {                                      // workgroup-uniform
+    // too many survivors for the list (heavy ties or adversarial order): start over, one group
+    // at a time, pruning to the best k whenever fewer than a group's worth of slots remain, so
+    // that nothing is ever dropped
+    __syncthreads();
+    if (tid == 0) { count = 0; overflow = 0; }
+    __syncthreads();
     for (int64_t g = 0; g < ngroups; ++g) {
       const int64_t j = g * kTopkThreads + tid;
       if (j < ntiles) {
         PTile<DT, VEC> t;
         t.load(probs, base + j * VEC);
-#pragma unroll
-        for (int e = 0; e < VEC; ++e) {
-          const float key = Elem<DT>::round(t.get(e) * q);
-          if (key >= tau_key) {
-            const uint64_t pc = pack_candidate(key, flat0 + (uint32_t)(j * VEC + e));
-            if (pc >= tau) {
-              const int slot = atomicAdd(&count, 1);
-              if (slot < kTopkCap) list[slot] = pc; else overflow = 1;
-            }
-          }
-        }
+        scan_tile(t, j);
       }
-      if (careful) {
-        // per-group bookkeeping: the list never loses an entry because it is pruned to <= k
-        // whenever fewer than one group's worth of free slots remain
-        __syncthreads();
-        const int cnt = count;
-        __syncthreads();                               // nobody appends before everyone has read it
-        if (cnt > kTopkPruneAt) {
-          tau = kth_best<kTopkThreads>(list, cnt, k, &kth_slot);
-          tau_key = candidate_key(tau);
-          prune_list<kTopkThreads>(list, cnt, tau, &count);
-        }
+      __syncthreads();
+      const int cnt = count;
+      __syncthreads();                                 // nobody appends before everyone has read it
+      if (cnt > kTopkPruneAt) {
+        tau = kth_best<kTopkThreads>(list, cnt, k, &kth_slot);
+        tau_key = candidate_key(tau);
+        prune_list<kTopkThreads>(list, cnt, tau, &count);
       }
     }
-    __syncthreads();
-    if (!overflow) break;                              // workgroup-uniform
-    // too many survivors for the list (heavy ties or adversarial order): start over, pruning
-    // after every group so that nothing is dropped
-    careful = true;
-    __syncthreads();
-    if (tid == 0) { count = 0; overflow = 0; }
     __syncthreads();
   }
 

@@ -5,9 +5,11 @@
 //      slice of one logits row with 16-byte loads, several per thread in flight, and reduces it in
 //      a single pass to (sum exp, sum t*exp, max, first index of the max); the row is read from
 //      HBM exactly once.  HBM-bound: algorithmic bytes = rows * vocab * sizeof(dtype).
-//   2. row_exact_kernel    - same grid; exits at once unless the row needs the reference's
-//      per-element rounding (entropy within the guard band of the threshold, fp16 rows, or a
-//      possible tie between *rounded* probabilities at the row maximum).
+//   2. exact pass          - only for rows that need the reference's per-element rounding
+//      (entropy within the guard band of the threshold, fp16 rows, or a possible tie between
+//      *rounded* probabilities at the row maximum): run by the same workgroup right after step 1
+//      when a row is one slice, otherwise by row_exact_kernel (same grid, exits at once for
+//      rows that do not need it).
 //   3. tree_accept_kernel  - one workgroup per tree: combines the partials, gathers
 //      p[parent(i), token(i)], runs the greedy walk or the bottom-up DP on the <= 256 nodes in LDS
 //      and writes the accepted path, contexts and bonus token.
@@ -24,7 +26,7 @@ namespace subspec {
 
 constexpr int kRowThreads = 512;
 constexpr int kMaxSplits = 64;
-constexpr int kTailThreads = 256;
+constexpr int kTailThreads = 64;
 
 // per (row, slice): reference point of the exponentials, sum exp2(t), sum t*exp2(t) with
 // t = (x - ref) * log2(e), true maximum of the slice and the first index holding it
@@ -76,94 +78,6 @@ template <int DT> struct Tile16x1 {
 };
 template <> struct Tile<SUBSPEC_BF16, 1> : Tile16x1<SUBSPEC_BF16> {};
 template <> struct Tile<SUBSPEC_F16, 1> : Tile16x1<SUBSPEC_F16> {};
-
-// ------------------------------------------------------------------ kernel 1: one pass over HBM
-// sum exp and sum t*exp of one tile relative to the reference `mb = -ref * log2(e)`;
-// t is clamped so that exp2(t) == 0 implies t * exp2(t) == 0 (x may be -inf).
-template <int DT, int VEC>
-__device__ __forceinline__ float tile_accumulate(const Tile<DT, VEC>& t, float mb, float (&s)[2], float (&u)[2]) {
-  float x[VEC];
-#pragma unroll
-  for (int k = 0; k < VEC; ++k) x[k] = t.get(k);
-  float tmax = x[0];
-#pragma unroll
-  for (int k = 1; k < VEC; ++k) tmax = fmaxf(tmax, x[k]);
-#pragma unroll
-  for (int k = 0; k < VEC; ++k) {
-    const float tt = fmaxf(fmaf(x[k], kLog2e, mb), -200.f);
-    const float e = __builtin_amdgcn_exp2f(tt);
-    s[k & 1] += e;
-    u[k & 1] = fmaf(tt, e, u[k & 1]);
-  }
-  return tmax;
-}
-
-template <int DT, int VEC, int U>
-__global__ __launch_bounds__(kRowThreads) void row_partial_kernel(
-    const void* __restrict__ logits, int64_t vocab, int splits, int64_t chunk, Part1* __restrict__ part) {
-  __shared__ float red_f[kRowThreads / kWave];
-  __shared__ int red_i[kRowThreads / kWave];
-  const int64_t row = blockIdx.y;
-  const int c = blockIdx.x;
-  const int tid = threadIdx.x;
-  const int64_t c0 = (int64_t)c * chunk;
-  const int64_t n = min(chunk, vocab - c0);           // elements of this slice (a multiple of VEC)
-  const int64_t base = row * vocab + c0;
-  const int64_t ntiles = n / VEC;
-
-  // Reference point for the exponentials: the largest value among the first tile of every
-  // thread.  It is at most the true maximum; the slice is redone against the true maximum in the
-  // (pathological) case that the two are so far apart that exp2 could overflow.
-  float ref;
-  {
-    Tile<DT, VEC> t0;
-    if (tid < ntiles) t0.load(logits, base + (int64_t)tid * VEC); else t0.fill_neg_inf();
-    float r = t0.get(0);
-#pragma unroll
-    for (int k = 1; k < VEC; ++k) r = fmaxf(r, t0.get(k));
-    ref = block_max<kRowThreads>(r, red_f);
-    if (ref == -INFINITY) ref = -1e30f;
-  }
-
-  float vmax = -INFINITY;
-  int64_t best_tile = 0;
-  float s[2], u[2];
-  for (int pass = 0; pass < 2; ++pass) {
-    const float mb = -ref * kLog2e;
-    s[0] = s[1] = u[0] = u[1] = 0.f;
-    for (int64_t j0 = tid; j0 < ntiles; j0 += (int64_t)kRowThreads * U) {
-      Tile<DT, VEC> t[U];
-#pragma unroll
-      for (int i = 0; i < U; ++i) {
-        const int64_t j = j0 + (int64_t)i * kRowThreads;
-        if (j < ntiles) t[i].load(logits, base + j * VEC); else t[i].fill_neg_inf();
-      }
-#pragma unroll
-      for (int i = 0; i < U; ++i) {
-        const float tmax = tile_accumulate<DT, VEC>(t[i], mb, s, u);
-        if (tmax > vmax) { vmax = tmax; best_tile = j0 + (int64_t)i * kRowThreads; }
-      }
-    }
-    if (pass == 1) break;
-    const float m_true = block_max<kRowThreads>(vmax, red_f);
-    if (!((m_true - ref) * kLog2e > 100.f)) break;    // workgroup-uniform
-    ref = m_true;
-  }
-  const float m = block_max<kRowThreads>(vmax, red_f);
-
-  int idx = 0x7fffffff;
-  if (vmax == m && m != -INFINITY) {                  // first index of the maximum inside this thread's tiles
-    Tile<DT, VEC> tb;
-    tb.load(logits, base + best_tile * VEC);
-#pragma unroll
-    for (int k = VEC - 1; k >= 0; --k)
-      if (tb.get(k) == m) idx = (int)(c0 + best_tile * VEC + k);
-  }
-  const float ssum = block_sum<kRowThreads>(s[0] + s[1], red_f);
-  const float usum = block_sum<kRowThreads>(u[0] + u[1], red_f);
-  idx = block_min_i<kRowThreads>(idx, red_i);
-  if (tid == 0) part[row * splits + c] = Part1{ref, ssum, usum, m, idx, 0, 0, 0};
-}
 
 // ------------------------------------------------------------------ combining the slices of a row
 struct RowStat {
@@ -231,17 +145,14 @@ __device__ __forceinline__ float rounded_prob(float x, float m, float S) {
   return Elem<DT>::round(expf(x - m) / S);
 }
 
-// ------------------------------------------------------------------ kernel 2: rare exact pass
+// ------------------------------------------------------------------ rare exact pass over one slice
+// Re-reads the slice (normally still in L2) and evaluates what the reference evaluates element by
+// element: the entropy terms with p, log p and p*log p rounded to the row dtype, and the first
+// index whose rounded probability equals the rounded maximum.
 template <int DT>
-__global__ __launch_bounds__(kRowThreads) void row_exact_kernel(
-    const void* __restrict__ logits, VerifyParams vp, const Part1* __restrict__ part1,
-    Part2* __restrict__ part2) {
-  __shared__ float red_f[kRowThreads / kWave];
-  __shared__ int red_i[kRowThreads / kWave];
-  const int64_t row = blockIdx.y;
-  const int c = blockIdx.x;
-  const RowStat rs = combine_row<DT>(part1 + row * vp.splits, vp);
-  if (!rs.need_emu && !rs.need_tie) return;           // uniform across the workgroup
+__device__ __forceinline__ void row_exact_body(const void* __restrict__ logits, const VerifyParams& vp,
+                                               const RowStat& rs, int64_t row, int c, float* red_f, int* red_i,
+                                               Part2* __restrict__ part2) {
   const int64_t c0 = (int64_t)c * vp.chunk;
   const int64_t n = min(vp.chunk, vp.vocab - c0);
   const int64_t base = row * vp.vocab + c0;
@@ -258,7 +169,124 @@ __global__ __launch_bounds__(kRowThreads) void row_exact_kernel(
   if (threadIdx.x == 0) part2[row * vp.splits + c] = Part2{acc, tie};
 }
 
+// Separate launch, used when a row is split over several workgroups (the slices of a row must all
+// be reduced before any of them knows the row's statistics).
+template <int DT>
+__global__ __launch_bounds__(kRowThreads) void row_exact_kernel(
+    const void* __restrict__ logits, VerifyParams vp, const Part1* __restrict__ part1,
+    Part2* __restrict__ part2) {
+  __shared__ float red_f[kRowThreads / kWave];
+  __shared__ int red_i[kRowThreads / kWave];
+  const int64_t row = blockIdx.y;
+  const RowStat rs = combine_row<DT>(part1 + row * vp.splits, vp);
+  if (!rs.need_emu && !rs.need_tie) return;           // uniform across the workgroup
+  row_exact_body<DT>(logits, vp, rs, row, blockIdx.x, red_f, red_i, part2);
+}
+
+// ------------------------------------------------------------------ kernel 1: one pass over HBM
+// sum exp and sum t*exp of one tile relative to the reference `mb = -ref * log2(e)`;
+// t is clamped so that exp2(t) == 0 implies t * exp2(t) == 0 (x may be -inf).
+template <int DT, int VEC>
+__device__ __forceinline__ float tile_accumulate(const Tile<DT, VEC>& t, float mb, float (&s)[2], float (&u)[2]) {
+  float x[VEC];
+#pragma unroll
+  for (int k = 0; k < VEC; ++k) x[k] = t.get(k);
+  float tmax = x[0];
+#pragma unroll
+  for (int k = 1; k < VEC; ++k) tmax = fmaxf(tmax, x[k]);
+#pragma unroll
+  for (int k = 0; k < VEC; ++k) {
+    const float tt = fmaxf(fmaf(x[k], kLog2e, mb), -200.f);
+    const float e = __builtin_amdgcn_exp2f(tt);
+    s[k & 1] += e;
+    u[k & 1] = fmaf(tt, e, u[k & 1]);
+  }
+  return tmax;
+}
+
+template <int DT, int VEC, int U>
+__global__ __launch_bounds__(kRowThreads) void row_partial_kernel(
+    const void* __restrict__ logits, VerifyParams vp, Part1* __restrict__ part, Part2* __restrict__ part2) {
+  const int64_t vocab = vp.vocab, chunk = vp.chunk;
+  const int splits = vp.splits;
+  __shared__ float red_f[kRowThreads / kWave];
+  __shared__ int red_i[kRowThreads / kWave];
+  const int64_t row = blockIdx.y;
+  const int c = blockIdx.x;
+  const int tid = threadIdx.x;
+  const int64_t c0 = (int64_t)c * chunk;
+  const int64_t n = min(chunk, vocab - c0);           // elements of this slice (a multiple of VEC)
+  const int64_t base = row * vocab + c0;
+  const int64_t ntiles = n / VEC;
+
+  // Reference point for the exponentials: the largest value among the first tile of every
+  // thread.  It is at most the true maximum; the slice is redone against the true maximum in the
+  // (pathological) case that the two are so far apart that exp2 could overflow.
+  float ref;
+  {
+    Tile<DT, VEC> t0;
+    if (tid < ntiles) t0.load(logits, base + (int64_t)tid * VEC); else t0.fill_neg_inf();
+    float r = t0.get(0);
+#pragma unroll
+    for (int k = 1; k < VEC; ++k) r = fmaxf(r, t0.get(k));
+    ref = block_max<kRowThreads>(r, red_f);
+    if (ref == -INFINITY) ref = -1e30f;
+  }
+
+  float vmax = -INFINITY;
+  int64_t best_tile = 0;
+  float s[2], u[2];
+  for (int pass = 0; pass < 2; ++pass) {
+    const float mb = -ref * kLog2e;
+    s[0] = s[1] = u[0] = u[1] = 0.f;
+    for (int64_t j0 = tid; j0 < ntiles; j0 += (int64_t)kRowThreads * U) {
+      Tile<DT, VEC> t[U];
+#pragma unroll
+      for (int i = 0; i < U; ++i) {
+        const int64_t j = j0 + (int64_t)i * kRowThreads;
+        if (j < ntiles) t[i].load(logits, base + j * VEC); else t[i].fill_neg_inf();
+      }
+#pragma unroll
+      for (int i = 0; i < U; ++i) {
+        const float tmax = tile_accumulate<DT, VEC>(t[i], mb, s, u);
+        if (tmax > vmax) { vmax = tmax; best_tile = j0 + (int64_t)i * kRowThreads; }
+      }
+    }
+    if (pass == 1) break;
+    const float m_true = block_max<kRowThreads>(vmax, red_f);
+    if (!((m_true - ref) * kLog2e > 100.f)) break;    // workgroup-uniform
+    ref = m_true;
+  }
+  const float m = block_max<kRowThreads>(vmax, red_f);
+
+  int idx = 0x7fffffff;
+  if (vmax == m && m != -INFINITY) {                  // first index of the maximum inside this thread's tiles
+    Tile<DT, VEC> tb;
+    tb.load(logits, base + best_tile * VEC);
+#pragma unroll
+    for (int k = VEC - 1; k >= 0; --k)
+      if (tb.get(k) == m) idx = (int)(c0 + best_tile * VEC + k);
+  }
+  const float ssum = block_sum<kRowThreads>(s[0] + s[1], red_f);
+  const float usum = block_sum<kRowThreads>(u[0] + u[1], red_f);
+  idx = block_min_i<kRowThreads>(idx, red_i);
+  const Part1 mine{ref, ssum, usum, m, idx, {0, 0, 0}};
+  if (tid == 0) part[row * splits + c] = mine;
+  if (splits == 1) {
+    // the workgroup holds the statistics of the whole row: decide here whether the row needs the
+    // exact pass and run it while the row is still in cache
+    const RowStat rs = combine_row<DT>(&mine, vp);
+    if (rs.need_emu || rs.need_tie) row_exact_body<DT>(logits, vp, rs, row, 0, red_f, red_i, part2);
+  }
+}
+
 // ------------------------------------------------------------------ kernel 3: per-tree tail
+// One wavefront per tree.  Lane l owns nodes l, l+64, l+128, l+192 in registers; the tree is
+// walked with ballots (greedy walk) or reduced bottom-up in lockstep (lossy DP): nodes are visited
+// from the last to the first, the visited node's finished state is broadcast with readlane and
+// the lane owning its parent folds it in.  Choosing a child is a lexicographic maximum over
+// (path length, exact match, probability of a lossy child, lower index), which is exactly the
+// update rule of lossy_tree_verify.py:148-164 and does not depend on the visiting order.
 struct TreeParams {
   int64_t rows, n_nodes;
   int root, skip;
@@ -268,190 +296,230 @@ struct TreeParams {
   int window;
 };
 
-template <int DT>
+
+__device__ __forceinline__ int bcast_i(int v, int lane) { return __builtin_amdgcn_readlane(v, lane); }
+__device__ __forceinline__ uint64_t bcast_u64(uint64_t v, int lane) {
+  const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)v, lane);
+  const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(v >> 32), lane);
+  return ((uint64_t)hi << 32) | lo;
+}
+template <typename T, int kSlots>
+__device__ __forceinline__ T pick_slot(const T (&a)[kSlots], int slot) {
+  T r = a[0];
+#pragma unroll
+  for (int s = 1; s < kSlots; ++s) r = (slot == s) ? a[s] : r;
+  return r;
+}
+
+// kSlots = nodes per lane (1, 2 or 4: trees of up to 64, 128, 256 nodes); LOSSY selects the
+// verifier.  Both are compile-time so that the common 64-node case stays a few hundred
+// instructions: a single wavefront pays for every instruction-cache miss it takes.
+template <int DT, int kSlots, bool LOSSY>
 __global__ __launch_bounds__(kTailThreads) void tree_accept_kernel(
     const void* __restrict__ logits, VerifyParams vp, TreeParams tp,
     const Part1* __restrict__ part1, const Part2* __restrict__ part2,
     const int32_t* __restrict__ token_ids, const int32_t* __restrict__ parents,
     int64_t* __restrict__ out_tokens, int64_t* __restrict__ out_ctx, int32_t* __restrict__ out_counts,
     int64_t* __restrict__ node_target, float* __restrict__ node_entropy, float* __restrict__ node_child_prob) {
-  constexpr int N = SUBSPEC_MAX_TREE_NODES;
-  __shared__ float sm_m[N], sm_S[N], sm_h[N], sm_cp[N];
-  __shared__ int sm_tgt[N], sm_tok[N], sm_par[N];
-  __shared__ short sm_head[N], sm_next[N], sm_best_next[N], sm_best_len[N], sm_exact_after[N];
-  __shared__ int sm_status;
+  constexpr int N = kSlots * kWave;
+  __shared__ float sm_m[N], sm_S[N], sm_h[N];
+  __shared__ int sm_tgt[N], sm_par[N], sm_ea[N];
+  __shared__ unsigned long long sm_best[N];
 
   const int b = blockIdx.x;
-  const int tid = threadIdx.x;
+  const int lane = threadIdx.x;
   const int rows = (int)tp.rows, n_nodes = (int)tp.n_nodes, skip = tp.skip;
-  const bool lossy = tp.method == SUBSPEC_VERIFY_LOSSY;
+  constexpr bool lossy = LOSSY;
   token_ids += (int64_t)b * n_nodes;
   parents += (int64_t)b * n_nodes;
-  if (tid == 0) sm_status = 0;
-  __syncthreads();
-
-  // ---- per scored row: max, sum, argmax token, entropy
-  if (tid < rows) {
-    const int64_t grow = (int64_t)b * rows + tid;
-    const RowStat rs = combine_row<DT>(part1 + grow * vp.splits, vp);
-    int tgt = rs.first_idx;
-    float h = rs.h;
-    if (rs.need_emu || rs.need_tie) {
-      float H = 0.f;
-      int tie = 0x7fffffff;
-      for (int c = 0; c < vp.splits; ++c) {
-        H += part2[grow * vp.splits + c].esum;
-        tie = min(tie, part2[grow * vp.splits + c].tie_idx);
-      }
-      if (rs.need_tie && tie != 0x7fffffff) tgt = tie;
-      if (rs.need_emu) h = finish_entropy<DT>(H, vp.ln_vocab);
-    }
-    sm_m[tid] = rs.m;
-    sm_S[tid] = rs.S;
-    sm_tgt[tid] = tgt;
-    sm_h[tid] = h;
-    node_target[grow] = tgt;
-    if (vp.gate_entropy) node_entropy[grow] = h;
-  }
-  if (tid < n_nodes) {
-    sm_tok[tid] = token_ids[tid];
-    const int p = parents[tid];
-    sm_par[tid] = p;
-    if (p >= tid) atomicOr(&sm_status, 2);            // precondition: parents precede children
-  }
-  __syncthreads();
-
-  // ---- p[parent(i), token(i)] for every node whose parent row was scored
-  if (tid < n_nodes) {
-    float cp = -1.f;
-    const int p = sm_par[tid];
-    if (p >= 0) {
-      int rp = p - skip;
-      if (rp < 0 && !lossy) rp += rows;                // the exact walk indexes rows like a python list
-      const int tk = sm_tok[tid];
-      if (rp >= 0 && rp < rows && tk >= 0 && tk < vp.vocab) {
-        const float x = Elem<DT>::load(logits, ((int64_t)b * rows + rp) * vp.vocab + sm_tok[tid]);
-        cp = rounded_prob<DT>(x, sm_m[rp], sm_S[rp]);
-      }
-    }
-    sm_cp[tid] = cp;
-    const int local = tid - skip;
-    if (local >= 0 && local < rows) node_child_prob[(int64_t)b * rows + local] = cp;
-  }
-  __syncthreads();
-  if (tid != 0) return;
-
   out_tokens += (int64_t)b * (n_nodes + 1);
   out_ctx += (int64_t)b * (n_nodes + 1);
-  int emitted = 0, accept = 0, total = 0;
+  int status = 0;
 
-  if (!lossy) {
-    // ---------------- greedy walk in original indexing (tree_verify.py:49-106)
-    for (int i = 0; i < n_nodes; ++i) sm_head[i] = -1;
-    for (int i = n_nodes - 1; i >= 1; --i) {
-      const int p = sm_par[i];
-      if (p >= 0 && p < n_nodes) { sm_next[i] = sm_head[p]; sm_head[p] = (short)i; }
+  // ---- per scored row: max, sum, argmax token, entropy
+#pragma unroll
+  for (int s = 0; s < kSlots; ++s) {
+    const int r = s * kWave + lane;
+    if (r < rows) {
+      const int64_t grow = (int64_t)b * rows + r;
+      const RowStat rs = combine_row<DT>(part1 + grow * vp.splits, vp);
+      int tgt = rs.first_idx;
+      float h = rs.h;
+      if (rs.need_emu || rs.need_tie) {
+        float H = 0.f;
+        int tie = 0x7fffffff;
+        for (int c = 0; c < vp.splits; ++c) {
+          H += part2[grow * vp.splits + c].esum;
+          tie = min(tie, part2[grow * vp.splits + c].tie_idx);
+        }
+        if (rs.need_tie && tie != 0x7fffffff) tgt = tie;
+        if (rs.need_emu) h = finish_entropy<DT>(H, vp.ln_vocab);
+      }
+      sm_m[r] = rs.m;
+      sm_S[r] = rs.S;
+      sm_tgt[r] = tgt;
+      sm_h[r] = h;
+      node_target[grow] = tgt;
+      if (vp.gate_entropy) node_entropy[grow] = h;
     }
+  }
+  __syncthreads();
+
+  // ---- per node: token, parent, p[parent(i), token(i)]
+  int tok[kSlots], par[kSlots];
+  float cp[kSlots];
+#pragma unroll
+  for (int s = 0; s < kSlots; ++s) {
+    const int i = s * kWave + lane;
+    tok[s] = -1;
+    par[s] = -2;                                       // matches no node
+    cp[s] = -1.f;
+    if (i < n_nodes) {
+      tok[s] = token_ids[i];
+      par[s] = parents[i];
+      if (par[s] >= i) status |= 2;                    // precondition: parents precede children
+      if (par[s] >= 0) {
+        int rp = par[s] - skip;
+        if (rp < 0 && !lossy) rp += rows;              // the exact walk indexes rows like a python list
+        if (rp >= 0 && rp < rows && tok[s] >= 0 && tok[s] < vp.vocab) {
+          const float x = Elem<DT>::load(logits, ((int64_t)b * rows + rp) * vp.vocab + tok[s]);
+          cp[s] = rounded_prob<DT>(x, sm_m[rp], sm_S[rp]);
+        }
+      }
+      const int local = i - skip;
+      if (local >= 0 && local < rows) node_child_prob[(int64_t)b * rows + local] = cp[s];
+    }
+  }
+  status = __any(status != 0) ? 2 : 0;
+
+  int emitted = 0, accept = 0, total = 0;
+  auto emit = [&](int64_t token, int ctx) {
+    if (lane == 0) { out_tokens[emitted] = token; out_ctx[emitted] = ctx; }
+    ++emitted;
+  };
+  int64_t last_token = -1;
+
+  if constexpr (!LOSSY) {
+    // ---------------- greedy walk in original indexing (tree_verify.py:49-106)
+    auto row_of = [&](int node) { int r = node - skip; if (r < 0) r += rows; return r; };
+    auto first_child = [&](int node, int want_tok, bool match_tok) {
+      int found = -1;
+#pragma unroll
+      for (int s = kSlots - 1; s >= 0; --s) {
+        const uint64_t m = __ballot(par[s] == node && (!match_tok || tok[s] == want_tok));
+        if (m) found = s * kWave + __builtin_ctzll(m);
+      }
+      return found;
+    };
     int cur = tp.root;
     int bonus = -1;
     bool bad = cur < 0 || cur >= n_nodes;
-    auto row_of = [&](int node) { int r = node - skip; if (r < 0) r += rows; return r; };
-    while (!bad && sm_head[cur] >= 0) {
+    while (!bad && first_child(cur, 0, false) >= 0) {
       ++total;
       const int r = row_of(cur);
       if (r < 0 || r >= rows) { bad = true; break; }
       const int t = sm_tgt[r];
-      int hit = -1;
-      for (int c = sm_head[cur]; c >= 0; c = sm_next[c])
-        if (sm_tok[c] == t) { hit = c; break; }
+      const int hit = first_child(cur, t, true);
       if (hit < 0) { bonus = t; break; }
       ++accept;
-      out_tokens[emitted] = t;
-      out_ctx[emitted] = cur;
-      ++emitted;
+      emit(t, cur);
+      last_token = t;
       if (tp.eos >= 0 && (int64_t)t == tp.eos) break;
       cur = hit;
-      if (sm_head[cur] < 0) break;
-      if (sm_head[cur] - skip >= rows) break;          // children were not scored in this call
+      const int kid = first_child(cur, 0, false);
+      if (kid < 0) break;
+      if (kid - skip >= rows) break;                   // children were not scored in this call
     }
-    if (!bad && (emitted == 0 || tp.eos < 0 || out_tokens[emitted - 1] != tp.eos)) {
+    if (!bad && (emitted == 0 || tp.eos < 0 || last_token != tp.eos)) {
       if (bonus < 0) {
         const int r = row_of(cur);
         if (r < 0 || r >= rows) bad = true; else bonus = sm_tgt[r];
       }
-      if (!bad) { out_tokens[emitted] = bonus; out_ctx[emitted] = cur; ++emitted; }
+      if (!bad) emit(bonus, cur);
     }
-    if (bad) sm_status |= 1;
+    if (bad) status |= 1;
   } else {
     // ---------------- bottom-up DP in local indexing (lossy_tree_verify.py:112-168)
     const int nl = min(rows, n_nodes - skip);
     if (nl <= 0) {
-      out_tokens[0] = rows > 0 ? sm_tgt[0] : 0;
-      out_ctx[0] = tp.root;
-      emitted = 1;
+      emit(rows > 0 ? sm_tgt[0] : 0, tp.root);
     } else {
       int root = tp.root - skip;
       if (root < 0 || root >= nl) root = 0;
-      for (int i = 0; i < nl; ++i) { sm_head[i] = -1; sm_best_next[i] = -1; sm_best_len[i] = 0; sm_exact_after[i] = 0; }
-      for (int i = nl - 1; i >= 0; --i) {
-        const int p = sm_par[i + skip] - skip;
-        if (p >= 0 && p < nl && p != i) { sm_next[i] = sm_head[p]; sm_head[p] = (short)i; }
-      }
       const bool use_entropy = tp.gate == SUBSPEC_GATE_ENTROPY;
       const int need = max(0, tp.window);
-      for (int u = nl - 1; u >= 0; --u) {
-        if (sm_head[u] < 0) continue;
-        const int tgt = sm_tgt[u];
-        int best_exact = -1;
-        for (int c = sm_head[u]; c >= 0; c = sm_next[c])
-          if (sm_tok[c + skip] == tgt) best_exact = max(best_exact, (int)sm_exact_after[c]);
-        if (best_exact >= 0) sm_exact_after[u] = (short)(1 + best_exact);
-        int pick = -1, pick_len = 0;
-        bool pick_exact = false;
-        float pick_p = -1.f;
-        const bool gate_blocks_u = use_entropy && ((double)sm_h[u] >= tp.theta);
-        for (int c = sm_head[u]; c >= 0; c = sm_next[c]) {
-          const bool is_exact = sm_tok[c + skip] == tgt;
-          float p = -1.f;
-          if (!is_exact) {
-            if (sm_exact_after[c] < need) continue;
-            if (gate_blocks_u) continue;
-            p = sm_cp[c + skip];
-            if (!use_entropy && (double)p < tp.theta) continue;
-          }
-          const int len = 1 + sm_best_len[c];
-          if (len > pick_len) { pick = c; pick_len = len; pick_exact = is_exact; pick_p = p; }
-          else if (len == pick_len) {
-            if (is_exact && !pick_exact) { pick = c; pick_exact = true; pick_p = p; }
-            else if (!is_exact && !pick_exact && p > pick_p) { pick = c; pick_p = p; }
+      // Level-parallel reduction: all nodes of one depth fold themselves into their parents at
+      // once with LDS atomic max, deepest level first (a node's own state is final once every
+      // deeper level has been folded).
+      int pl[kSlots], depth[kSlots];                   // parent in local indexing (-1: none in the slice)
+      int max_depth = 0;
+#pragma unroll
+      for (int s = 0; s < kSlots; ++s) {
+        const int li = s * kWave + lane - skip;
+        pl[s] = -1;
+        depth[s] = 0;
+        if (s * kWave + lane < N) { sm_ea[s * kWave + lane] = 0; sm_best[s * kWave + lane] = 0; }
+        if (li >= 1 && li < nl) {
+          const int p = par[s] - skip;
+          if (p >= 0 && p < nl && p < li) pl[s] = p;
+        }
+        if (li >= 0 && li < nl) sm_par[li] = pl[s];
+      }
+      __syncthreads();
+#pragma unroll
+      for (int s = 0; s < kSlots; ++s) {
+        int d = 0;
+        for (int c = pl[s]; c >= 0; c = sm_par[c]) ++d;
+        depth[s] = d;
+        max_depth = max(max_depth, d);
+      }
+#pragma unroll
+      for (int o = 32; o > 0; o >>= 1) max_depth = max(max_depth, __shfl_xor(max_depth, o, kWave));
+      for (int d = max_depth; d >= 1; --d) {
+#pragma unroll
+        for (int s = 0; s < kSlots; ++s) {
+          if (depth[s] == d && pl[s] >= 0) {
+            const int li = s * kWave + lane - skip;
+            const int p = pl[s];
+            const bool ex = tok[s] == sm_tgt[p];
+            const int ea = sm_ea[li];
+            const int blen = (int)(sm_best[li] >> 54);
+            const bool gate_blocks = use_entropy ? ((double)sm_h[p] >= tp.theta) : ((double)cp[s] < tp.theta);
+            const bool admissible = ex || (ea >= need && !gate_blocks);
+            if (ex) atomicMax(&sm_ea[p], 1 + ea);
+            if (admissible) {
+              const uint32_t pb = ex ? 0u : __float_as_uint(fmaxf(cp[s], 0.f));
+              const unsigned long long key = ((unsigned long long)(1 + blen) << 54) | ((unsigned long long)ex << 53) |
+                                             ((unsigned long long)pb << 21) | ((unsigned long long)(511 - li) << 12) | 1ull;
+              atomicMax(&sm_best[p], key);
+            }
           }
         }
-        if (pick >= 0 && pick_len > 0) { sm_best_next[u] = (short)pick; sm_best_len[u] = (short)pick_len; }
+        __syncthreads();
       }
       int ctx = root;
       while (true) {                                   // lossy_tree_verify.py:247-286
-        const int nxt = sm_best_next[ctx];
-        if (nxt < 0) break;
-        const int t = sm_tok[nxt + skip];
-        out_tokens[emitted] = t;
-        out_ctx[emitted] = ctx + skip;
-        ++emitted;
+        const unsigned long long bk = sm_best[ctx];
+        if (bk == 0) break;
+        const int nxt = 511 - (int)((bk >> 12) & 0x1ff);
+        const int on = nxt + skip;
+        const int t = bcast_i(pick_slot<int, kSlots>(tok, on >> 6), on & (kWave - 1));
+        emit(t, ctx + skip);
+        last_token = t;
         if (tp.eos >= 0 && (int64_t)t == tp.eos) break;
         ctx = nxt;
       }
       accept = emitted;
-      if (emitted == 0 || tp.eos < 0 || out_tokens[emitted - 1] != tp.eos) {
-        out_tokens[emitted] = sm_tgt[ctx];
-        out_ctx[emitted] = ctx + skip;
-        ++emitted;
-      }
+      if (emitted == 0 || tp.eos < 0 || last_token != tp.eos) emit(sm_tgt[ctx], ctx + skip);
       total = emitted;
     }
   }
-  out_counts[b * 4 + 0] = emitted;
-  out_counts[b * 4 + 1] = accept;
-  out_counts[b * 4 + 2] = total;
-  out_counts[b * 4 + 3] = sm_status;
+  if (lane == 0) {
+    out_counts[b * 4 + 0] = emitted;
+    out_counts[b * 4 + 1] = accept;
+    out_counts[b * 4 + 2] = total;
+    out_counts[b * 4 + 3] = status;
+  }
 }
 
 // ------------------------------------------------------------------ host side
@@ -477,9 +545,8 @@ static bool make_plan(const void* logits, int dtype, int64_t total_rows, int64_t
 }
 
 template <int DT, int VEC>
-static void launch_partial(const Plan& pl, dim3 grid, hipStream_t st, const void* logits, int64_t vocab, Part1* p1) {
-  hipLaunchKernelGGL((row_partial_kernel<DT, VEC, 4>), grid, dim3(kRowThreads), 0, st, logits, vocab, pl.splits,
-                     pl.chunk, p1);
+static void launch_partial(dim3 grid, hipStream_t st, const void* logits, const VerifyParams& vp, Part1* p1, Part2* p2) {
+  hipLaunchKernelGGL((row_partial_kernel<DT, VEC, 4>), grid, dim3(kRowThreads), 0, st, logits, vp, p1, p2);
 }
 
 template <int DT>
@@ -489,12 +556,20 @@ static int run_verify(const void* logits, int64_t batch, int64_t rows, int64_t v
                       int32_t* out_counts, int64_t* node_target, float* node_entropy, float* node_child_prob,
                       hipStream_t st) {
   const dim3 grid(pl.splits, (unsigned)(batch * rows));
-  if (pl.vec == 1) launch_partial<DT, 1>(pl, grid, st, logits, vocab, p1);
-  else launch_partial<DT, (DT == SUBSPEC_F32 ? 4 : 8)>(pl, grid, st, logits, vocab, p1);
-  hipLaunchKernelGGL((row_exact_kernel<DT>), grid, dim3(kRowThreads), 0, st, logits, vp, p1, p2);
-  hipLaunchKernelGGL((tree_accept_kernel<DT>), dim3((unsigned)batch), dim3(kTailThreads), 0, st, logits, vp, tp,
-                     p1, p2, token_ids, parents, out_tokens, out_ctx, out_counts, node_target, node_entropy,
-                     node_child_prob);
+  if (pl.vec == 1) launch_partial<DT, 1>(grid, st, logits, vp, p1, p2);
+  else launch_partial<DT, (DT == SUBSPEC_F32 ? 4 : 8)>(grid, st, logits, vp, p1, p2);
+  if (pl.splits > 1) hipLaunchKernelGGL((row_exact_kernel<DT>), grid, dim3(kRowThreads), 0, st, logits, vp, p1, p2);
+  const int64_t widest = std::max<int64_t>(rows, tp.n_nodes);
+  const int slots = widest <= kWave ? 1 : widest <= 2 * kWave ? 2 : 4;
+  const bool lossy = tp.method == SUBSPEC_VERIFY_LOSSY;
+#define SUBSPEC_LAUNCH_TAIL(SLOTS, LOSSY)                                                                        \
+  hipLaunchKernelGGL((tree_accept_kernel<DT, SLOTS, LOSSY>), dim3((unsigned)batch), dim3(kTailThreads), 0, st,    \
+                     logits, vp, tp, p1, p2, token_ids, parents, out_tokens, out_ctx, out_counts, node_target,   \
+                     node_entropy, node_child_prob)
+  if (slots == 1) { if (lossy) SUBSPEC_LAUNCH_TAIL(1, true); else SUBSPEC_LAUNCH_TAIL(1, false); }
+  else if (slots == 2) { if (lossy) SUBSPEC_LAUNCH_TAIL(2, true); else SUBSPEC_LAUNCH_TAIL(2, false); }
+  else { if (lossy) SUBSPEC_LAUNCH_TAIL(4, true); else SUBSPEC_LAUNCH_TAIL(4, false); }
+#undef SUBSPEC_LAUNCH_TAIL
   SUBSPEC_CHECK_HIP(hipGetLastError());
   return SUBSPEC_OK;
 }
