@@ -9,10 +9,12 @@
 // to the lowest flat index first.
 //
 //   1. topk_slice_kernel - grid (slices, B*L), 512 threads.  A workgroup streams its slice of one
-//      row once.  The k-th largest of 512 per-thread maxima over a 16K-element sample gives a
-//      threshold; afterwards every element costs unpack + multiply + round + compare, and the few
-//      survivors go to a candidate list in LDS that is pruned to the slice's exact top-k in
-//      (key, index) order.  HBM-bound: algorithmic bytes = B * L * V * sizeof(dtype).
+//      row once.  A lower bound of the slice's k-th best is taken from the per-thread maxima of a
+//      16K-element sample; 16-bit rows are then screened eight elements at a time with packed
+//      unsigned maxima against the bit pattern of that bound, and the few survivors go to a
+//      candidate list in LDS.  Two checkpoints tighten the bound to the exact k-th best so far; at
+//      the end the list is pruned to the slice's exact top-k in (key, index) order.
+//      HBM-bound: algorithmic bytes = B * L * V * sizeof(dtype).
 //   2. topk_merge_kernel - one workgroup per batch item ranks the <= slices*L*k candidates and
 //      writes values, token ids and parent indices in sorted order.
 #include "common.h"
@@ -21,8 +23,8 @@
 namespace subspec {
 
 constexpr int kTopkThreads = 512;
-constexpr int kTopkCap = 4608;          // candidate slots per workgroup: one 4096-element group + 512
-constexpr int kTopkPruneAt = 512;
+constexpr int kTopkCap = 1024;          // candidate slots per workgroup
+constexpr int kTopkPruneAt = 512;       // careful mode prunes above this; one step adds at most 512
 constexpr int kTopkMaxK = 64;
 constexpr int kTopkMaxSlices = 64;
 constexpr int kMergeThreads = 1024;
@@ -40,6 +42,26 @@ __device__ __forceinline__ float candidate_key(uint64_t c) {
   return __uint_as_float(b);
 }
 __device__ __forceinline__ uint32_t candidate_flat(uint64_t c) { return 0xffffffffu - (uint32_t)c; }
+
+typedef unsigned short u16x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pk_max_u16(uint32_t a, uint32_t b) {
+  return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(u16x2_t, a), __builtin_bit_cast(u16x2_t, b)));
+}
+
+// Smallest non-negative 16-bit pattern u whose key round(value(u) * q) reaches tau_key.  Keys
+// grow with u for q > 0, so "key >= tau_key" can be tested on the raw bits with an unsigned
+// compare; patterns with the sign bit set compare high and are sorted out by the precise test.
+template <int DT>
+__device__ __forceinline__ uint32_t min_pattern_reaching(float q, float tau_key) {
+  if (!(q > 0.f)) return 0;
+  uint32_t lo = 0, hi = DT == SUBSPEC_BF16 ? 0x7f80u : 0x7c00u;     // +inf
+  while (lo < hi) {
+    const uint32_t mid = (lo + hi) >> 1;
+    const float v = DT == SUBSPEC_BF16 ? bf16_bits_to_float(mid) : f16_bits_to_float(mid);
+    if (Elem<DT>::round(v * q) >= tau_key) hi = mid; else lo = mid + 1;
+  }
+  return lo;
+}
 
 template <int DT, int VEC> struct PTile;
 template <> struct PTile<SUBSPEC_F32, 4> {
@@ -117,8 +139,8 @@ __global__ __launch_bounds__(kTopkThreads) void topk_slice_kernel(
     const void* __restrict__ probs, const void* __restrict__ parent_probs, int64_t vocab, int leaves, int splits,
     int64_t chunk, int k, uint64_t* __restrict__ cand, int32_t* __restrict__ cand_count) {
   __shared__ uint64_t list[kTopkCap];
-  __shared__ uint64_t sample[kTopkThreads];
   __shared__ uint64_t kth_slot;
+  __shared__ uint32_t wave_prefix[kTopkThreads / kWave];
   __shared__ int count, overflow;
 
   const int64_t row = blockIdx.y;                      // b * leaves + l
@@ -132,9 +154,11 @@ __global__ __launch_bounds__(kTopkThreads) void topk_slice_kernel(
   const float q = Elem<DT>::load(parent_probs, row);
   const uint32_t flat0 = (uint32_t)((int64_t)leaf * vocab + c0);
 
-  // ---- threshold from a sample: k-th largest of the per-thread maxima over the first 4 tiles
+  // ---- threshold from a sample: the per-thread maxima over the first 4 tiles.  Each wavefront
+  // finds, by a 16-step bit search with ballots (no memory traffic), the largest 16-bit key prefix
+  // that at least m = ceil(k/4) of its lanes reach; the ceil(k/m)-th largest of those prefixes is
+  // reached by at least k elements of the slice, hence a valid lower bound for its k-th best.
   float smax = -INFINITY;
-  uint32_t sflat = 0;
   bool sany = false;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
@@ -145,14 +169,34 @@ __global__ __launch_bounds__(kTopkThreads) void topk_slice_kernel(
 #pragma unroll
       for (int e = 0; e < VEC; ++e) {
         const float key = Elem<DT>::round(t.get(e) * q);
-        if (!sany || key > smax) { smax = key; sflat = flat0 + (uint32_t)(j * VEC + e); sany = true; }
+        if (!sany || key > smax) { smax = key; sany = true; }
       }
     }
   }
-  sample[tid] = sany ? pack_candidate(smax, sflat) : 0;
   if (tid == 0) { count = 0; overflow = 0; }
+  {
+    const int m = (k + 3) / 4;
+    const uint32_t prefix = sany ? (uint32_t)(pack_candidate(smax, 0) >> 48) : 0u;
+    uint32_t best = 0;
+    for (int bit = 15; bit >= 0; --bit) {
+      const uint32_t trial = best | (1u << bit);
+      if (__popcll(__ballot(prefix >= trial)) >= m) best = trial;
+    }
+    if ((tid & (kWave - 1)) == 0) wave_prefix[tid / kWave] = best;
+  }
   __syncthreads();
-  uint64_t tau = kth_best<kTopkThreads>(sample, kTopkThreads, k, &kth_slot);
+  uint64_t tau;
+  {
+    const int m = (k + 3) / 4, need = (k + m - 1) / m;            // need <= 4 wavefronts
+    uint32_t chosen = 0;                               // the prefix of rank need-1 among the 8
+    for (int w = 0; w < kTopkThreads / kWave; ++w) {
+      int r = 0;
+      const uint32_t o = wave_prefix[w];
+      for (int w2 = 0; w2 < kTopkThreads / kWave; ++w2) r += (wave_prefix[w2] > o) || (wave_prefix[w2] == o && w2 < w);
+      if (r == need - 1) chosen = o;
+    }
+    tau = (uint64_t)chosen << 48;
+  }
   float tau_key = tau ? candidate_key(tau) : -INFINITY;
 
   // ---- stream the slice; survivors go to the LDS list
@@ -170,19 +214,50 @@ __global__ __launch_bounds__(kTopkThreads) void topk_slice_kernel(
       }
     }
   };
-  // fast path: four tiles per thread in flight, no bookkeeping between groups
+  // fast path: four tiles per thread in flight, no bookkeeping between groups.  For 16-bit rows a
+  // tile is first screened with packed unsigned maxima against the bit pattern of the threshold
+  // (five instructions for eight elements); only tiles that may hold a survivor are unpacked.
   constexpr int U = 4;
+  uint32_t screen = 0;                                 // (pattern - 1) in both halves; 0: screen nothing out
+  if constexpr (VEC == 8) {
+    const uint32_t thr = min_pattern_reaching<DT>(q, tau_key);
+    screen = thr ? (thr - 1) * 0x10001u : 0;
+  }
   for (int64_t g0 = 0; g0 < ngroups; g0 += U) {
     PTile<DT, VEC> t[U];
 #pragma unroll
-    for (int i = 0; i < U; ++i) {
-      const int64_t j = (g0 + i) * kTopkThreads + tid;
-      if (j < ntiles) t[i].load(probs, base + j * VEC);
+    for (int i = 0; i < U; ++i) {                      // unconditional loads (clamped index): back to back
+      const int64_t j = min((g0 + i) * kTopkThreads + tid, ntiles - 1);
+      t[i].load(probs, base + j * VEC);
     }
 #pragma unroll
     for (int i = 0; i < U; ++i) {
       const int64_t j = (g0 + i) * kTopkThreads + tid;
-      if (j < ntiles) scan_tile(t[i], j);
+      if (j < ntiles) {
+        if constexpr (VEC == 8) {
+          const uint32_t mm = pk_max_u16(pk_max_u16(t[i].r.x, t[i].r.y), pk_max_u16(t[i].r.z, t[i].r.w));
+          if (screen == 0 || pk_max_u16(mm, screen) != screen) scan_tile(t[i], j);
+        } else {
+          scan_tile(t[i], j);
+        }
+      }
+    }
+    // two checkpoints tighten the threshold to the exact k-th best of what has been seen, so that
+    // few later elements survive and the final selection stays small
+    if ((g0 == U || g0 == 4 * U) && g0 + U < ngroups) {
+      __syncthreads();
+      const int cnt = count;
+      const int lost = overflow;
+      __syncthreads();
+      if (!lost && cnt > k) {
+        tau = kth_best<kTopkThreads>(list, cnt, k, &kth_slot);
+        tau_key = candidate_key(tau);
+        prune_list<kTopkThreads>(list, cnt, tau, &count);
+        if constexpr (VEC == 8) {
+          const uint32_t thr = min_pattern_reaching<DT>(q, tau_key);
+          screen = thr ? (thr - 1) * 0x10001u : 0;
+        }
+      }
     }
   }
   __syncthreads();
@@ -195,18 +270,27 @@ __global__ __launch_bounds__(kTopkThreads) void topk_slice_kernel(
     __syncthreads();
     for (int64_t g = 0; g < ngroups; ++g) {
       const int64_t j = g * kTopkThreads + tid;
-      if (j < ntiles) {
-        PTile<DT, VEC> t;
-        t.load(probs, base + j * VEC);
-        scan_tile(t, j);
-      }
-      __syncthreads();
-      const int cnt = count;
-      __syncthreads();                                 // nobody appends before everyone has read it
-      if (cnt > kTopkPruneAt) {
-        tau = kth_best<kTopkThreads>(list, cnt, k, &kth_slot);
-        tau_key = candidate_key(tau);
-        prune_list<kTopkThreads>(list, cnt, tau, &count);
+      PTile<DT, VEC> t;
+      if (j < ntiles) t.load(probs, base + j * VEC);
+      for (int e = 0; e < VEC; ++e) {                  // one element per thread and step: <= 512 appends
+        if (j < ntiles) {
+          float v = t.get(0);
+#pragma unroll
+          for (int e2 = 1; e2 < VEC; ++e2) v = (e == e2) ? t.get(e2) : v;
+          const float key = Elem<DT>::round(v * q);
+          if (key >= tau_key) {
+            const uint64_t pc = pack_candidate(key, flat0 + (uint32_t)(j * VEC + e));
+            if (pc >= tau) list[atomicAdd(&count, 1)] = pc;
+          }
+        }
+        __syncthreads();
+        const int cnt = count;
+        __syncthreads();                               // nobody appends before everyone has read it
+        if (cnt > kTopkPruneAt) {
+          tau = kth_best<kTopkThreads>(list, cnt, k, &kth_slot);
+          tau_key = candidate_key(tau);
+          prune_list<kTopkThreads>(list, cnt, tau, &count);
+        }
       }
     }
     __syncthreads();

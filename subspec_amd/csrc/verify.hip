@@ -242,10 +242,13 @@ __global__ __launch_bounds__(kRowThreads) void row_partial_kernel(
     for (int64_t j0 = tid; j0 < ntiles; j0 += (int64_t)kRowThreads * U) {
       Tile<DT, VEC> t[U];
 #pragma unroll
-      for (int i = 0; i < U; ++i) {
+      for (int i = 0; i < U; ++i) {                    // unconditional loads (clamped index): back to back
         const int64_t j = j0 + (int64_t)i * kRowThreads;
-        if (j < ntiles) t[i].load(logits, base + j * VEC); else t[i].fill_neg_inf();
+        t[i].load(logits, base + min(j, ntiles - 1) * VEC);
       }
+#pragma unroll
+      for (int i = 0; i < U; ++i)
+        if (j0 + (int64_t)i * kRowThreads >= ntiles) t[i].fill_neg_inf();
 #pragma unroll
       for (int i = 0; i < U; ++i) {
         const float tmax = tile_accumulate<DT, VEC>(t[i], mb, s, u);
