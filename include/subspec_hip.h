@@ -133,6 +133,33 @@ int subspec_topk_expand(const void* probs, const void* parent_probs, int dtype, 
                         int64_t vocab, int32_t k, void* workspace, size_t workspace_bytes,
                         int64_t* token_ids, void* topk_probs, int64_t* parent_indices, void* stream);
 
+/* ------------------------------------------------------------------------------------------
+ * Tree-masked GQA attention of the draft tree against the static KV cache:
+ * out = softmax(q k^T * scale + mask) v, where tree row i attends to cache rows [0, prefix_len) and
+ * to tree slot prefix_len + j iff bit j of anc_bits[i] is set (node j is node i or an ancestor).
+ *
+ * Replaces  HF sdpa_attention_forward under SDPBackend.MATH with the additive finfo.min mask and
+ *           repeat_kv, as reached from _tree_decoding   specdecodes/models/generators/classic_sd.py:57-109
+ *           (run/pipelines/run_test.py:64); mask construction Tree.create_attention_mask
+ *           specdecodes/models/utils/cpu_tree.py:263-286, _get_tree_mask / invert_mask
+ *           generators/classic_sd.py:33-55, utils/utils.py:4-6.  The FlashInfer form is
+ *           flashinfer/attention_wrapper.py:116-151,288-316.
+ *
+ * q          device [batch, n_q_heads, n_rows, head_dim]      bf16 / fp16, head_dim = 128, n_rows <= 64
+ * k_cache    device [batch, n_kv_heads, kv_seq_stride, head_dim]  (HF static-cache layout); the K/V of
+ * v_cache    the tree nodes must already sit in rows prefix_len .. prefix_len + n_rows - 1
+ * out        device [batch, n_rows, n_q_heads, head_dim]       (= [batch, n_rows, hidden])
+ * anc_bits   device uint64 [*, n_rows]; batch element b uses row b * anc_batch_stride (0: shared tree)
+ * workspace  partial results when the keys are split over workgroups (may be NULL if the size is 256)
+ */
+size_t subspec_tree_attention_workspace(int64_t batch, int64_t n_q_heads, int64_t prefix_len, int64_t n_rows);
+
+int subspec_tree_attention(const void* q, const void* k_cache, const void* v_cache, void* out, int dtype,
+                           int64_t batch, int64_t n_q_heads, int64_t n_kv_heads, int64_t n_rows, int64_t head_dim,
+                           int64_t kv_seq_stride, int64_t prefix_len, const uint64_t* anc_bits,
+                           int64_t anc_batch_stride, float scale, void* workspace, size_t workspace_bytes,
+                           void* stream);
+
 #ifdef __cplusplus
 }
 #endif

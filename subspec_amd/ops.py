@@ -163,3 +163,49 @@ def topk_expand(sampled_probs: torch.Tensor, parent_probs: torch.Tensor, k: int,
         token_ids.data_ptr(), vals.data_ptr(), parents.data_ptr(), _stream(dev))
     L.check(code, "subspec_topk_expand")
     return token_ids, vals, parents
+
+
+def ancestor_bits_tensor(parents, device=None) -> torch.Tensor:
+    """uint64 ancestor-or-self bitsets (as an int64 tensor) from a parent array with parent < child."""
+    bits = []
+    for i, p in enumerate(parents):
+        v = (1 << i) | (bits[int(p)] if int(p) >= 0 else 0)
+        bits.append(v)
+    signed = [b - (1 << 64) if b >= (1 << 63) else b for b in bits]
+    return torch.tensor(signed, dtype=torch.int64, device=device)
+
+
+def tree_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, anc_bits: torch.Tensor,
+                   prefix_len: int, scale: Optional[float] = None, workspace: Optional[torch.Tensor] = None):
+    """``q`` [B, Hq, n, D], caches [B, Hkv, S, D] (tree K/V already written at rows prefix_len..),
+    ``anc_bits`` int64 [n] (shared tree) or [B, n].  Returns [B, n, Hq * D]."""
+    dev = _require_gpu(q, k_cache, v_cache, anc_bits)
+    if q.dim() != 4 or k_cache.dim() != 4 or v_cache.shape != k_cache.shape:
+        raise ValueError("expected q [B, Hq, n, D] and k/v caches [B, Hkv, S, D]")
+    if q.dtype != k_cache.dtype or q.dtype != v_cache.dtype:
+        raise ValueError("q, k_cache and v_cache must share a dtype")
+    B, Hq, n, D = q.shape
+    Hkv, S = k_cache.shape[1], k_cache.shape[2]
+    if k_cache.shape[0] != B or k_cache.shape[3] != D:
+        raise ValueError("cache shape does not match q")
+    if not (k_cache.is_contiguous() and v_cache.is_contiguous()):
+        raise ValueError("tree_attention: the KV caches must be contiguous [B, Hkv, S, D]")
+    if anc_bits.dtype != torch.int64 or anc_bits.shape[-1] != n:
+        raise ValueError("anc_bits must be int64 with one word per tree row")
+    q = q.contiguous()
+    anc_bits = anc_bits.contiguous()
+    if anc_bits.dim() == 2 and anc_bits.shape[0] not in (1, B):
+        raise ValueError("anc_bits batch dimension must be 1 or B")
+    stride = n if (anc_bits.dim() == 2 and anc_bits.shape[0] == B and B > 1) else 0
+    lib = L.lib()
+    need = lib.subspec_tree_attention_workspace(B, Hq, int(prefix_len), n)
+    if workspace is None and need > 256:
+        workspace = torch.empty(need, dtype=torch.uint8, device=dev)
+    out = torch.empty((B, n, Hq * D), dtype=q.dtype, device=dev)
+    code = lib.subspec_tree_attention(
+        q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), _dtype_code(q), B, Hq, Hkv, n, D, S,
+        int(prefix_len), anc_bits.data_ptr(), stride, float(D ** -0.5 if scale is None else scale),
+        None if workspace is None else workspace.data_ptr(),
+        0 if workspace is None else workspace.numel() * workspace.element_size(), _stream(dev))
+    L.check(code, "subspec_tree_attention")
+    return out

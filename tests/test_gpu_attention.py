@@ -1,0 +1,78 @@
+"""GPU parity: tree-masked GQA attention through the C ABI against the fp32 oracle on the same
+bf16 / fp16 inputs.  Tolerance (stated by the benchmark definition): 1e-2 relative; checked as
+max |diff| <= 1e-2 * max |ref| per batch element plus an element-wise allclose."""
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+from oracle import attention as oa
+from subspec_amd import ops, workloads as W
+
+DEV = "cuda:0"
+
+
+def _case(seed, B, Hq, Hkv, n, P, S, dtype, depth=8):
+    g = torch.Generator().manual_seed(seed)
+    parents, _, _ = W.random_tree(g, n=n, max_depth=depth, max_children=4, vocab=1000, chain_depth=min(depth, n - 1))
+    q = torch.randn(B, Hq, n, 128, generator=g).to(dtype)
+    k = torch.randn(B, Hkv, S, 128, generator=g).to(dtype)
+    v = torch.randn(B, Hkv, S, 128, generator=g).to(dtype)
+    return parents, q, k, v
+
+
+def _check(parents, q, k, v, P, tag):
+    print("attention", tag, tuple(q.shape), tuple(k.shape), P, flush=True)
+    anc = ops.ancestor_bits_tensor(parents, device=DEV)
+    out = ops.tree_attention(q.to(DEV), k.to(DEV), v.to(DEV), anc, P)
+    torch.cuda.synchronize()
+    ref = oa.tree_attention(q, k, v, parents, P)
+    got = out.float().cpu()
+    assert got.shape == ref.shape
+    err = (got - ref).abs().amax().item()
+    assert err <= 1e-2 * ref.abs().amax().item(), (tag, err, ref.abs().amax().item())
+    assert torch.allclose(got, ref, rtol=1e-2, atol=2e-2), tag
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_small_shapes(dtype):
+    for seed, (B, Hq, Hkv, n, P, S) in enumerate([(1, 4, 2, 9, 0, 16), (2, 7, 1, 17, 5, 64), (1, 28, 4, 64, 100, 200),
+                                                  (3, 8, 8, 33, 63, 128), (1, 14, 2, 1, 300, 301), (2, 4, 4, 64, 64, 128)]):
+        parents, q, k, v = _case(seed, B, Hq, Hkv, n, P, S, dtype, depth=6)
+        _check(parents, q, k, v, P, f"small{seed}")
+
+
+@pytest.mark.parametrize("B", [1, 8])
+def test_config3_qwen_geometry(B):
+    parents, q, k, v = _case(100 + B, B, 28, 4, 64, 4096, 4160, torch.bfloat16)
+    _check(parents, q, k, v, 4096, f"cfg3-B{B}")
+
+
+def test_stale_cache_tail_and_per_batch_trees():
+    # the static cache is longer than prefix + n and holds garbage beyond: it must not be read into the result
+    parents, q, k, v = _case(7, 2, 28, 4, 40, 1000, 2113, torch.bfloat16)
+    k[:, :, 1040:] = 1e3
+    v[:, :, 1040:] = -1e3
+    _check(parents, q, k, v, 1000, "stale-tail")
+    # different tree per batch element
+    g = torch.Generator().manual_seed(5)
+    p2, _, _ = W.random_tree(g, n=40, max_depth=5, max_children=4, vocab=1000)
+    anc = torch.stack([ops.ancestor_bits_tensor(parents), ops.ancestor_bits_tensor(p2)]).to(DEV)
+    out = ops.tree_attention(q.to(DEV), k.to(DEV), v.to(DEV), anc, 1000).float().cpu()
+    ref = torch.cat([oa.tree_attention(q[:1], k[:1], v[:1], parents, 1000), oa.tree_attention(q[1:], k[1:], v[1:], p2, 1000)])
+    assert torch.allclose(out, ref, rtol=1e-2, atol=2e-2)
+
+
+def test_argument_errors():
+    q = torch.zeros(1, 4, 8, 128, dtype=torch.bfloat16, device=DEV)
+    k = torch.zeros(1, 2, 64, 128, dtype=torch.bfloat16, device=DEV)
+    anc = torch.zeros(8, dtype=torch.int64, device=DEV)
+    with pytest.raises(ValueError):
+        ops.tree_attention(q, k, k, anc, 60)                       # prefix + n beyond the cache
+    with pytest.raises(ValueError):
+        ops.tree_attention(q.float(), k.float(), k.float(), anc, 8)   # fp32 not supported
+    with pytest.raises(ValueError):
+        ops.tree_attention(torch.zeros(1, 4, 65, 128, dtype=torch.bfloat16, device=DEV), k, k,
+                           torch.zeros(65, dtype=torch.int64, device=DEV), 0)
+    with pytest.raises(ValueError):
+        ops.tree_attention(q[..., :64].contiguous(), k[..., :64].contiguous(), k[..., :64].contiguous(), anc, 8)

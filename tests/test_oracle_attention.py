@@ -1,0 +1,39 @@
+"""Pins the attention oracle: explicit softmax(QK^T)V == F.scaled_dot_product_attention with the
+additive mask; mask == the host tree's create_attention_mask; single-key special case.  No GPU."""
+import torch
+
+from oracle import attention as oa
+from subspec_amd import ops, workloads as W
+from subspec_amd.cpu_tree import Tree
+
+
+def test_explicit_equals_sdpa_and_mask_properties():
+    g = torch.Generator().manual_seed(0)
+    parents, _, _ = W.random_tree(g, n=12, max_depth=4, max_children=3, vocab=100)
+    B, Hq, Hkv, n, D, P, S = 2, 4, 2, 12, 16, 20, 40
+    q = torch.randn(B, Hq, n, D, generator=g).to(torch.bfloat16)
+    k = torch.randn(B, Hkv, S, D, generator=g).to(torch.bfloat16)
+    v = torch.randn(B, Hkv, S, D, generator=g).to(torch.bfloat16)
+    a = oa.tree_attention(q, k, v, parents, P)
+    b = oa.tree_attention_sdpa(q, k, v, parents, P)
+    assert torch.allclose(a, b, rtol=1e-5, atol=1e-5)
+    # rows beyond prefix+n never matter: poison them
+    k2, v2 = k.clone(), v.clone()
+    k2[:, :, P + n:] = 1e4
+    v2[:, :, P + n:] = -1e4
+    assert torch.allclose(oa.tree_attention(q, k2, v2, parents, P), a)
+    # node 0 (root) with an empty prefix attends to itself only -> output is its own V row
+    o0 = oa.tree_attention(q, k, v, parents, 0)
+    assert torch.allclose(o0[:, 0].view(B, Hq, D), v[:, :, 0].float().repeat_interleave(2, dim=1), atol=1e-6)
+
+
+def test_mask_matches_host_tree_and_bitsets():
+    t = Tree(torch.tensor(1))
+    t.add_nodes(torch.tensor([[[5, 6, 7], [8, 9, 10]]]), torch.rand(1, 2, 3), torch.tensor([[[0, 0, 0], [0, 0, 2]]]))
+    parents = t.get_tree_data()["parent_indices"].tolist()
+    m = oa.allowed_mask(parents, 3, 3 + t.size())
+    assert torch.equal(m, t.create_attention_mask(3)[0, 0])
+    bits = ops.ancestor_bits_tensor(parents).tolist()
+    assert bits == t.ancestor_bits()
+    for i, w in enumerate(bits):
+        assert [bool((w >> j) & 1) for j in range(t.size())] == m[i, 3:].tolist()
