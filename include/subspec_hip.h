@@ -160,6 +160,30 @@ int subspec_tree_attention(const void* q, const void* k_cache, const void* v_cac
                            int64_t anc_batch_stride, float scale, void* workspace, size_t workspace_bytes,
                            void* stream);
 
+/* ------------------------------------------------------------------------------------------
+ * int4 group-wise (group 64 along the input dimension, fp16 scale and zero per row and group)
+ * linear layer of the substitute draft:  y[M, N] = x[M, K] * ((Wq - zero) * scale)^T (+ bias).
+ *
+ * Replaces  hqq HQQLinear -> gemlite A16W4 GEMV/GEMM as installed by HqqQuantizer.quantize_model
+ *           specdecodes/helpers/quantizers/hqq/__init__.py:17-120 (AutoHQQHFModel.quantize_model
+ *           quantizers/hqq/hf/base.py:94-230) for BaseQuantizeConfig(nbits=4, group_size=64, axis=1)
+ *           specdecodes/helpers/recipes/subspec/hqq_4bit_postspec.py:17-58.
+ *
+ * x     device [M, K]  bf16 / fp16, 1 <= M <= 64 (tree width), K % 64 == 0
+ * wq    device uint32, tiled codes: [N/16][K/64][4][16] entries of 8 bytes; entry (c, r) holds the 16
+ *       codes of row 16*nt + r for k = 64*g + 16*c .. +15, word j the codes of k = .. + 8j .. +7
+ *       with code(8j + 2i) in bits 4i..4i+3 and code(8j + 2i + 1) in bits 16+4i..16+4i+3
+ * sz    device uint32 [N/16][K/64][16]: fp16 scale (low half) and fp16 zero (high half) of
+ *       row 16*nt + r, group g
+ * bias  device [N] (same dtype as x) or NULL
+ * y     device [M, N], same dtype as x;  N % 16 == 0
+ */
+size_t subspec_int4_linear_workspace(int64_t M, int64_t N, int64_t K);
+
+int subspec_int4_linear(const void* x, const uint32_t* wq, const uint32_t* sz, const void* bias, void* y, int dtype,
+                        int64_t M, int64_t N, int64_t K, int64_t group_size, void* workspace, size_t workspace_bytes,
+                        void* stream);
+
 #ifdef __cplusplus
 }
 #endif

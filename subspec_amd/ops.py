@@ -209,3 +209,33 @@ def tree_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
         0 if workspace is None else workspace.numel() * workspace.element_size(), _stream(dev))
     L.check(code, "subspec_tree_attention")
     return out
+
+
+def int4_linear(x: torch.Tensor, wq: torch.Tensor, sz: torch.Tensor, out_features: int,
+                bias: Optional[torch.Tensor] = None, workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``x`` [..., K] (bf16 / fp16, at most 64 rows in total) times the tiled int4 weight
+    (``wq`` int32, ``sz`` int32 as produced by ``subspec_amd.quant.pack_tiled``) -> [..., N]."""
+    dev = _require_gpu(x, wq, sz)
+    K = x.shape[-1]
+    M = x.numel() // K
+    N = int(out_features)
+    if wq.dtype != torch.int32 or sz.dtype != torch.int32:
+        raise ValueError("int4_linear: wq and sz must be int32 tensors in the tiled layout")
+    if wq.numel() * 8 != N * K or sz.numel() * 64 != N * K:
+        raise ValueError(f"int4_linear: packed weight does not describe a [{N}, {K}] matrix")
+    x2 = x.reshape(M, K).contiguous()
+    if bias is not None:
+        if bias.dtype != x.dtype or bias.numel() != N:
+            raise ValueError("int4_linear: bias must be [N] in the activation dtype")
+        bias = bias.contiguous()
+    lib = L.lib()
+    need = lib.subspec_int4_linear_workspace(M, N, K)
+    if workspace is None and M > 1:
+        workspace = torch.empty(need, dtype=torch.uint8, device=dev)
+    y = torch.empty((M, N), dtype=x.dtype, device=dev)
+    code = lib.subspec_int4_linear(
+        x2.data_ptr(), wq.data_ptr(), sz.data_ptr(), None if bias is None else bias.data_ptr(), y.data_ptr(),
+        _dtype_code(x2), M, N, K, 64, None if workspace is None else workspace.data_ptr(),
+        0 if workspace is None else workspace.numel() * workspace.element_size(), _stream(dev))
+    L.check(code, "subspec_int4_linear")
+    return y.reshape(*x.shape[:-1], N)

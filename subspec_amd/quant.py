@@ -1,0 +1,120 @@
+"""int4 group-wise quantization of the substitute draft's linear layers and the module / quantizer
+classes that plug it into a model.
+
+Mirrors the reference's quantizer seam: ``HqqQuantizer.quantize_model(model, quant_config,
+compute_dtype, device)`` (specdecodes/helpers/quantizers/hqq/__init__.py:17-120) replaces every
+``nn.Linear`` named in ``quant_config`` by a quantized module; the per-layer config is the
+``BaseQuantizeConfig(nbits=4, group_size=64, axis=1)`` of
+specdecodes/helpers/recipes/subspec/hqq_4bit_postspec.py:17-58 (here a plain dict
+``{"nbits": 4, "group_size": 64, "axis": 1}``).
+
+The quantizer is the plain affine min/max rule of the benchmark definition: per (output row,
+64-wide input group) ``s = (max - min) / 15``, ``z = -min / s`` (both stored as fp16),
+``Wq = clamp(round(W / s + z), 0, 15)``.  hqq's proximal refinement of the zero point is a
+separate, un-vendored algorithm and is not reproduced; the kernels only rely on the affine
+dequantization ``(Wq - z) * s``.
+"""
+from __future__ import annotations
+
+from typing import Dict, Optional, Tuple
+
+import torch
+import torch.nn as nn
+
+from . import ops
+
+GROUP = 64
+
+
+def quantize_int4_g64(weight: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """``weight`` [N, K] -> (codes uint8 [N, K] in 0..15, scale fp16 [N, K/64], zero fp16 [N, K/64])."""
+    N, K = weight.shape
+    if K % GROUP:
+        raise ValueError(f"in_features={K} must be a multiple of {GROUP}")
+    w = weight.detach().float().reshape(N, K // GROUP, GROUP)
+    lo, hi = w.amin(-1), w.amax(-1)
+    scale = ((hi - lo) / 15.0).clamp_min(1e-8).to(torch.float16)
+    s = scale.float()
+    zero = (-lo / s).to(torch.float16)
+    codes = torch.clamp(torch.round(w / s.unsqueeze(-1) + zero.float().unsqueeze(-1)), 0, 15).to(torch.uint8)
+    return codes.reshape(N, K), scale, zero
+
+
+def dequantize(codes: torch.Tensor, scale: torch.Tensor, zero: torch.Tensor) -> torch.Tensor:
+    N, K = codes.shape
+    c = codes.float().reshape(N, K // GROUP, GROUP)
+    return ((c - zero.float().unsqueeze(-1)) * scale.float().unsqueeze(-1)).reshape(N, K)
+
+
+def pack_tiled(codes: torch.Tensor, scale: torch.Tensor, zero: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Tiled device layout consumed by the kernels (see include/subspec_hip.h): returns
+    (wq int32 [N/16, K/64, 4, 16, 2], sz int32 [N/16, K/64, 16])."""
+    N, K = codes.shape
+    if N % 16 or K % GROUP:
+        raise ValueError(f"[{N}, {K}]: out_features must be a multiple of 16 and in_features of {GROUP}")
+    G = K // GROUP
+    # [nt, r, g, c, j, i, parity] : k = 64 g + 16 c + 8 j + 2 i + parity
+    q = codes.to(torch.int64).reshape(N // 16, 16, G, 4, 2, 4, 2)
+    shifts = torch.tensor([0, 4, 8, 12], dtype=torch.int64, device=codes.device).view(1, 1, 1, 1, 1, 4)
+    word = (q[..., 0] << shifts).sum(-1) | ((q[..., 1] << (shifts + 16)).sum(-1))        # [nt, r, g, c, j]
+    word = word.permute(0, 2, 3, 1, 4).contiguous()                                        # [nt, g, c, r, j]
+    wq = torch.where(word >= 2 ** 31, word - 2 ** 32, word).to(torch.int32)
+    s_bits = scale.contiguous().view(torch.int16).to(torch.int64) & 0xFFFF
+    z_bits = zero.contiguous().view(torch.int16).to(torch.int64) & 0xFFFF
+    both = (s_bits | (z_bits << 16)).reshape(N // 16, 16, G).permute(0, 2, 1).contiguous()
+    sz = torch.where(both >= 2 ** 31, both - 2 ** 32, both).to(torch.int32)
+    return wq, sz
+
+
+class HqqInt4Linear(nn.Module):
+    """Drop-in for ``nn.Linear`` holding tiled int4 weights; forward runs the HIP GEMV / GEMM."""
+
+    def __init__(self, in_features: int, out_features: int, wq: torch.Tensor, sz: torch.Tensor,
+                 bias: Optional[torch.Tensor] = None):
+        super().__init__()
+        self.in_features, self.out_features = in_features, out_features
+        self.register_buffer("wq", wq)
+        self.register_buffer("sz", sz)
+        self.register_buffer("bias", bias)
+
+    @classmethod
+    def from_linear(cls, linear: nn.Linear, compute_dtype: torch.dtype = torch.bfloat16, device=None):
+        device = device or linear.weight.device
+        codes, scale, zero = quantize_int4_g64(linear.weight.data.to(device))
+        wq, sz = pack_tiled(codes, scale, zero)
+        bias = None if linear.bias is None else linear.bias.data.to(device=device, dtype=compute_dtype)
+        return cls(linear.in_features, linear.out_features, wq.to(device), sz.to(device), bias)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        rows = x.numel() // x.shape[-1]
+        if rows <= 64:
+            return ops.int4_linear(x, self.wq, self.sz, self.out_features, self.bias)
+        # wider inputs (prefill) are processed in slabs of 64 rows
+        flat = x.reshape(rows, x.shape[-1])
+        out = [ops.int4_linear(flat[i:i + 64], self.wq, self.sz, self.out_features, self.bias)
+               for i in range(0, rows, 64)]
+        return torch.cat(out).reshape(*x.shape[:-1], self.out_features)
+
+    def extra_repr(self) -> str:
+        return f"in_features={self.in_features}, out_features={self.out_features}, nbits=4, group_size={GROUP}"
+
+
+class HqqQuantizer:
+    """``quantize_model(model, quant_config, compute_dtype, device)`` as the reference recipe calls it
+    (specdecodes/helpers/recipes/base_recipe.py:43-52): ``quant_config`` maps module names to a
+    per-layer config; every named ``nn.Linear`` is replaced in place."""
+
+    @classmethod
+    def quantize_model(cls, model: nn.Module, quant_config: Dict[str, dict], compute_dtype: torch.dtype, device):
+        for name, cfg in quant_config.items():
+            nbits = int(cfg.get("nbits", 4)) if isinstance(cfg, dict) else int(getattr(cfg, "nbits", 4))
+            gsize = int(cfg.get("group_size", GROUP)) if isinstance(cfg, dict) else int(getattr(cfg, "group_size", GROUP))
+            if nbits != 4 or gsize != GROUP:
+                raise ValueError(f"{name}: only nbits=4, group_size={GROUP} is supported (got {nbits}, {gsize})")
+            parent_name, _, child = name.rpartition(".")
+            parent = model.get_submodule(parent_name) if parent_name else model
+            linear = getattr(parent, child)
+            if not isinstance(linear, nn.Linear):
+                raise TypeError(f"{name} is {type(linear).__name__}, expected nn.Linear")
+            setattr(parent, child, HqqInt4Linear.from_linear(linear, compute_dtype, device))
+        return model

@@ -1,0 +1,75 @@
+"""GPU parity: int4 g64 linear (GEMV for M = 1, MFMA GEMM for M = 2..64) through the C ABI against
+x.float() @ ((Wq - z) * s).T on identical (Wq, scale, zero).  Tolerance 1e-2 relative
+(max |diff| <= 1e-2 * max |ref|, outputs rounded to the activation dtype)."""
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+from oracle import int4 as oi
+from subspec_amd import ops, quant
+
+DEV = "cuda:0"
+
+
+def _check(N, K, M, dtype, seed, bias=False):
+    print("int4", N, K, M, dtype, flush=True)
+    g = torch.Generator().manual_seed(seed)
+    W = torch.randn(N, K, generator=g) * 0.02
+    codes, scale, zero = quant.quantize_int4_g64(W)
+    wq, sz = quant.pack_tiled(codes, scale, zero)
+    x = torch.randn(M, K, generator=g).to(dtype)
+    b = (torch.randn(N, generator=g) * 0.1).to(dtype) if bias else None
+    y = ops.int4_linear(x.to(DEV), wq.to(DEV), sz.to(DEV), N, None if b is None else b.to(DEV))
+    torch.cuda.synchronize()
+    ref = oi.linear(x, codes, scale, zero, b)
+    got = y.float().cpu()
+    assert got.shape == ref.shape
+    err = (got - ref).abs().amax().item()
+    assert err <= 1e-2 * ref.abs().amax().item(), (N, K, M, err, ref.abs().amax().item())
+    return got, ref
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_small_shapes(dtype):
+    for seed, (N, K, M) in enumerate([(16, 64, 1), (48, 192, 1), (64, 256, 2), (80, 512, 16), (128, 1024, 17),
+                                      (256, 2048, 33), (64, 3584, 64), (512, 128, 5)]):
+        _check(N, K, M, dtype, seed, bias=seed % 2 == 0)
+
+
+@pytest.mark.parametrize("N,K", [(4608, 3584), (3584, 3584), (37888, 3584), (3584, 18944)])
+@pytest.mark.parametrize("M", [1, 16, 64])
+def test_config4_qwen_shapes(N, K, M):
+    _check(N, K, M, torch.bfloat16, 100 + M)
+
+
+def test_exact_integer_case_and_module():
+    # scale = 1, zero = 0, small integer activations: every product is exact -> bit-exact result
+    g = torch.Generator().manual_seed(3)
+    N, K = 64, 256
+    codes = torch.randint(0, 16, (N, K), generator=g, dtype=torch.uint8)
+    scale = torch.ones(N, K // 64, dtype=torch.float16)
+    zero = torch.zeros(N, K // 64, dtype=torch.float16)
+    wq, sz = quant.pack_tiled(codes, scale, zero)
+    for M in (1, 7, 64):
+        x = torch.randint(-2, 3, (M, K), generator=g).to(torch.bfloat16)
+        y = ops.int4_linear(x.to(DEV), wq.to(DEV), sz.to(DEV), N).float().cpu()
+        assert torch.equal(y, (x.float() @ codes.float().T).to(torch.bfloat16).float())
+    lin = torch.nn.Linear(256, 64, bias=True)
+    q = quant.HqqInt4Linear.from_linear(lin, torch.bfloat16, DEV)
+    x = torch.randn(2, 5, 256).to(torch.bfloat16)
+    y = q(x.to(DEV))
+    assert y.shape == (2, 5, 64) and y.dtype == torch.bfloat16
+    ref = oi.linear(x.reshape(10, 256), *quant.quantize_int4_g64(lin.weight.data), lin.bias.data.to(torch.bfloat16))
+    assert (y.float().cpu().reshape(10, 64) - ref).abs().amax() <= 1e-2 * ref.abs().amax()
+
+
+def test_argument_errors():
+    wq = torch.zeros(1, 1, 4, 16, 2, dtype=torch.int32, device=DEV)
+    sz = torch.zeros(1, 1, 16, dtype=torch.int32, device=DEV)
+    with pytest.raises(ValueError):
+        ops.int4_linear(torch.zeros(1, 64, device=DEV), wq, sz, 16)                       # fp32 activations
+    with pytest.raises(ValueError):
+        ops.int4_linear(torch.zeros(65, 64, dtype=torch.bfloat16, device=DEV), wq, sz, 16)  # more than 64 rows
+    with pytest.raises(ValueError):
+        ops.int4_linear(torch.zeros(1, 128, dtype=torch.bfloat16, device=DEV), wq, sz, 16)  # shape mismatch
