@@ -28,7 +28,127 @@ def parse():
     ap.add_argument("--cpu-trees", type=int, default=4, help="trees in the bounded CPU-baseline sample")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="lower bound of CPU-baseline work")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--new-tokens", type=int, default=256, help="e2e workload: tokens to generate")
+    ap.add_argument("--workload", default="verify-cycle", choices=["verify-cycle", "attention", "int4", "greedy", "e2e"],
+                    help="verify-cycle (default, BASELINE config 2) is the benchmark line; the others time one "
+                         "kernel family of configs 1, 3 and 4 and print one JSON line per shape")
     return ap.parse_args()
+
+
+def _time_us(fn, steps, warmup):
+    """Average duration of fn() in microseconds, events on the launch stream."""
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(steps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return 1e3 * e0.elapsed_time(e1) / steps
+
+
+def _kernel_line(name, workload, us, nbytes, flops=None, extra=None):
+    gbs = nbytes / (us * 1e-6) / 1e9
+    line = {"metric": name, "value": round(us, 2), "unit": "us", "n_gpus": 1, "higher_is_better": False,
+            "data": "synthetic", "config": dict({"workload": workload}, **(extra or {})),
+            "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None, "bytes_per_launch": nbytes}}
+    if flops:
+        line["tflops"] = round(flops / (us * 1e-6) / 1e12, 2)
+    print(json.dumps(line), flush=True)
+
+
+def bench_attention(args):
+    import torch
+    from subspec_amd import ops, workloads as W
+    dev = torch.device("cuda:0")
+    g = torch.Generator().manual_seed(0)
+    parents, _, _ = W.random_tree(g, n=64, max_depth=8, max_children=4, vocab=1000, chain_depth=8)
+    anc = ops.ancestor_bits_tensor(parents, device=dev)
+    for B in (1, 8):
+        q = torch.randn(B, 28, 64, 128, device=dev).to(torch.bfloat16)
+        k = torch.randn(B, 4, 4160, 128, device=dev).to(torch.bfloat16)
+        v = torch.randn(B, 4, 4160, 128, device=dev).to(torch.bfloat16)
+        need = ops.L.lib().subspec_tree_attention_workspace(B, 28, 4096, 64)
+        ws = torch.empty(max(need, 256), dtype=torch.uint8, device=dev)
+        us = _time_us(lambda: ops.tree_attention(q, k, v, anc, 4096, workspace=ws), args.steps, args.warmup)
+        nbytes = B * (2 * 4 * 4160 * 128 * 2 + 2 * 28 * 64 * 128 * 2)
+        _kernel_line("tree-masked GQA attention latency", f"BASELINE config 3, B={B}: q [B,28,64,128], KV [B,4,4160,128] bf16",
+                     us, nbytes, flops=B * 4 * 64 * 28 * 4160 * 128, extra={"batch": B})
+
+
+def bench_int4(args):
+    import torch
+    from subspec_amd import ops, quant
+    dev = torch.device("cuda:0")
+    for N, K in ((4608, 3584), (3584, 3584), (37888, 3584), (3584, 18944)):
+        W_ = torch.randn(N, K, device=dev) * 0.02
+        wq, sz = quant.pack_tiled(*quant.quantize_int4_g64(W_))
+        del W_
+        for M in (1, 16, 64):
+            x = torch.randn(M, K, device=dev).to(torch.bfloat16)
+            ws = torch.empty(max(ops.L.lib().subspec_int4_linear_workspace(M, N, K), 256), dtype=torch.uint8, device=dev)
+            us = _time_us(lambda: ops.int4_linear(x, wq, sz, N, workspace=ws), args.steps, args.warmup)
+            nbytes = N * K // 2 + N * (K // 64) * 4 + M * (K + N) * 2
+            _kernel_line("int4 g64 linear latency", f"BASELINE config 4: {K}->{N}, M={M}, bf16 activations", us, nbytes,
+                         flops=2 * M * N * K, extra={"N": N, "K": K, "M": M})
+
+
+def bench_e2e(args):
+    """BASELINE config 5: random-init Qwen2.5-7B-shaped decoder, target bf16 with layers 14-27 streamed
+    from pinned host memory every forward, substitute draft int4 g64 resident, depth-8 / k-8 tree
+    capped at 64 nodes, prompt 2048 random ids, 256 new tokens; exact and lossy verification."""
+    import torch
+    from subspec_amd.cache import create_kv_cache
+    from subspec_amd.draft import SubSpecSDDraftModel
+    from subspec_amd.generator import SubSpecSDGenerator
+    from subspec_amd.model import DecoderConfig, build_models
+    from subspec_amd.utils import DraftParams
+    from subspec_amd.wandb_logger import wandb_logger
+    dev = "cuda:0"
+    cfg = DecoderConfig()
+    t0 = time.perf_counter()
+    kv = create_kv_cache("static", max_cache_len=2048 + 256 + 64 + 8, config=cfg, device=dev, dtype=torch.bfloat16)
+    target, draft, _ = build_models(cfg, kv, seed=0, device=dev, first_streamed=14)
+    print(f"# models built in {time.perf_counter() - t0:.1f} s", file=sys.stderr, flush=True)
+    prompt = torch.randint(0, cfg.vocab_size, (1, 2048), generator=torch.Generator().manual_seed(0)).to(dev)
+    for method, vk in (("exact", None), ("lossy", dict(threshold=0.3, window_size=6, threshold_method="entropy"))):
+        gen = SubSpecSDGenerator(target, None, SubSpecSDDraftModel(draft),
+                                 DraftParams(temperature=0.2, max_depth=8, topk_len=8, max_verify_tokens=64),
+                                 generator_kwargs=dict(verify_method=method, verify_kwargs=vk))
+        kv.reset()
+        wandb_logger.clear_log_data()
+        target.streamer.bytes_streamed = 0
+        out = gen.generate(prompt, max_new_tokens=args.new_tokens, do_sample=False, past_key_values=kv)
+        log = dict(wandb_logger.log_data)
+        line = {"metric": "accepted tokens/sec, end-to-end speculative cycle", "value": round(log["tput"], 2),
+                "unit": "tokens/s", "n_gpus": 1, "higher_is_better": True, "dtype": "bf16", "data": "synthetic",
+                "config": {"workload": "BASELINE config 5: Qwen2.5-7B shape, layers 14-27 streamed, int4 draft, depth 8, k 8, "
+                                       f"<=64 nodes, prompt 2048, {args.new_tokens} new tokens, verify {method}",
+                           "verify_method": method, "n_iter": log["n_iter"], "n_tokens": log["n_tokens"],
+                           "tokens_per_cycle": round(log["avg_sampled"], 3),
+                           "avg_draft_s": round(log.get("avg_draft_time", 0), 5),
+                           "avg_target_s": round(log.get("avg_target_time", 0), 5),
+                           "avg_verify_s": round(log.get("avg_verify_time", 0), 6),
+                           "elapsed_s": round(log["elapsed_time"], 3),
+                           "host_to_device_GB": round(target.streamer.bytes_streamed / 1e9, 2)}}
+        print(json.dumps(line), flush=True)
+
+
+def bench_greedy(args):
+    import torch
+    from subspec_amd import ops, workloads as W
+    dev = torch.device("cuda:0")
+    cfg = W.greedy_config(0, device=dev)
+    tok = torch.tensor(cfg["tokens"], dtype=torch.int32, device=dev)
+    par = torch.tensor(cfg["parents"], dtype=torch.int32, device=dev)
+    ws = torch.empty(ops.L.lib().subspec_tree_verify_workspace(1, 64, 152064, 0), dtype=torch.uint8, device=dev)
+    us = _time_us(lambda: ops.tree_verify(cfg["logits"], tok, par, workspace=ws), args.steps, args.warmup)
+    _kernel_line("greedy tree verify latency", "BASELINE config 1: fp32 logits [64,152064], 64-node tree", us,
+                 64 * 152064 * 4)
 
 
 def cpu_baseline(cfg, probs_rows, parent_rows, n_trees, min_seconds):
@@ -87,6 +207,9 @@ def main():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(1)
     L.lib()                                            # fail loudly when the HIP library is missing
+    if args.workload != "verify-cycle":
+        {"attention": bench_attention, "int4": bench_int4, "greedy": bench_greedy, "e2e": bench_e2e}[args.workload](args)
+        return
     dev = torch.device("cuda:0")
     B, V, n, k = args.batch, args.vocab, 64, 16
 

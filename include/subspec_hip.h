@@ -135,8 +135,10 @@ int subspec_topk_expand(const void* probs, const void* parent_probs, int dtype, 
 
 /* ------------------------------------------------------------------------------------------
  * Tree-masked GQA attention of the draft tree against the static KV cache:
- * out = softmax(q k^T * scale + mask) v, where tree row i attends to cache rows [0, prefix_len) and
- * to tree slot prefix_len + j iff bit j of anc_bits[i] is set (node j is node i or an ancestor).
+ * out = softmax(q k^T * scale + mask) v, where query row i attends to cache rows [0, prefix_len) and
+ * to tree slot prefix_len + j (j < n_tree_slots <= 64) iff bit j of anc_bits[i] is set (the node in
+ * slot j is row i's node or one of its ancestors).  The verify forward has one query row per slot;
+ * a draft step queries only the newest level (n_rows < n_tree_slots).
  *
  * Replaces  HF sdpa_attention_forward under SDPBackend.MATH with the additive finfo.min mask and
  *           repeat_kv, as reached from _tree_decoding   specdecodes/models/generators/classic_sd.py:57-109
@@ -147,15 +149,16 @@ int subspec_topk_expand(const void* probs, const void* parent_probs, int dtype, 
  *
  * q          device [batch, n_q_heads, n_rows, head_dim]      bf16 / fp16, head_dim = 128, n_rows <= 64
  * k_cache    device [batch, n_kv_heads, kv_seq_stride, head_dim]  (HF static-cache layout); the K/V of
- * v_cache    the tree nodes must already sit in rows prefix_len .. prefix_len + n_rows - 1
+ * v_cache    the tree nodes must already sit in rows prefix_len .. prefix_len + n_tree_slots - 1
  * out        device [batch, n_rows, n_q_heads, head_dim]       (= [batch, n_rows, hidden])
  * anc_bits   device uint64 [*, n_rows]; batch element b uses row b * anc_batch_stride (0: shared tree)
  * workspace  partial results when the keys are split over workgroups (may be NULL if the size is 256)
  */
-size_t subspec_tree_attention_workspace(int64_t batch, int64_t n_q_heads, int64_t prefix_len, int64_t n_rows);
+size_t subspec_tree_attention_workspace(int64_t batch, int64_t n_q_heads, int64_t prefix_len, int64_t n_tree_slots);
 
 int subspec_tree_attention(const void* q, const void* k_cache, const void* v_cache, void* out, int dtype,
-                           int64_t batch, int64_t n_q_heads, int64_t n_kv_heads, int64_t n_rows, int64_t head_dim,
+                           int64_t batch, int64_t n_q_heads, int64_t n_kv_heads, int64_t n_rows,
+                           int64_t n_tree_slots, int64_t head_dim,
                            int64_t kv_seq_stride, int64_t prefix_len, const uint64_t* anc_bits,
                            int64_t anc_batch_stride, float scale, void* workspace, size_t workspace_bytes,
                            void* stream);
@@ -183,6 +186,17 @@ size_t subspec_int4_linear_workspace(int64_t M, int64_t N, int64_t K);
 int subspec_int4_linear(const void* x, const uint32_t* wq, const uint32_t* sz, const void* bias, void* y, int dtype,
                         int64_t M, int64_t N, int64_t K, int64_t group_size, void* workspace, size_t workspace_bytes,
                         void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Layer streaming: asynchronous copy of one weight slab from pinned host memory to its device
+ * slab on the caller's copy stream (hipMemcpyAsync).  Ordering against the compute stream
+ * (copy-done before use, last-reader-done before overwrite) is the caller's, with events.
+ *
+ * Replaces  ChunkedPinMemory / PrefetchOffloader's Tensor.copy_(pinned, non_blocking=True) on a side stream
+ *           specdecodes/helpers/offloaders/prefetch_offloader_postspec.py:6-48,174-221 and the
+ *           keep_first_n_layers_on_gpu placement of recipes/offload/layer_offload.py:9-56.
+ */
+int subspec_stream_copy_h2d(void* dst_device, const void* src_pinned_host, size_t bytes, void* stream);
 
 #ifdef __cplusplus
 }

@@ -32,10 +32,11 @@ _SIGNATURES = {
     "subspec_topk_expand_workspace": (_sz, [_i64, _i64, _i64, _i32]),
     "subspec_topk_expand": (C.c_int, [_p, _p, C.c_int, _i64, _i64, _i64, _i32, _p, _sz, _p, _p, _p, _p]),
     "subspec_tree_attention_workspace": (_sz, [_i64, _i64, _i64, _i64]),
-    "subspec_tree_attention": (C.c_int, [_p, _p, _p, _p, C.c_int, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _p, _i64,
+    "subspec_tree_attention": (C.c_int, [_p, _p, _p, _p, C.c_int, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _p, _i64,
                                          C.c_float, _p, _sz, _p]),
     "subspec_int4_linear_workspace": (_sz, [_i64, _i64, _i64]),
     "subspec_int4_linear": (C.c_int, [_p, _p, _p, _p, _p, C.c_int, _i64, _i64, _i64, _i64, _p, _sz, _p]),
+    "subspec_stream_copy_h2d": (C.c_int, [_p, _p, _sz, _p]),
     "subspec_kv_compact": (C.c_int, [_p, _p, _i64, _i64, _i64, _i64, _i64, _p, _p, _i32, _i32, _p]),
 }
 

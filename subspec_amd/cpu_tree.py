@@ -172,6 +172,14 @@ class Tree:
         self._rebuild(keep)
         return torch.tensor(keep, dtype=torch.long)
 
+    def truncate(self, n: int) -> torch.Tensor:
+        """Keep the first ``n`` nodes (level order, so every kept node keeps its parent).  Used to cap
+        the tree at ``max_verify_tokens``; the dropped nodes are the least probable of the last level."""
+        if n >= self.current_size:
+            return torch.arange(self.current_size)
+        self._rebuild(list(range(max(1, int(n)))))
+        return torch.arange(self.current_size)
+
     # ------------------------------------------------------------------ export
     def get_tree_data(self, skip_nodes: int = 0) -> Dict[str, torch.Tensor]:
         s = int(skip_nodes)

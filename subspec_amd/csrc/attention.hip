@@ -7,10 +7,11 @@
 // among the tree slots, only node i and its ancestors.
 //
 // Layout and mapping
-//   q        [B, Hq, n, D]            (n <= 64 tree rows, D = 128)
+//   q        [B, Hq, n, D]            (n <= 64 query rows, D = 128)
 //   k, v     [B, Hkv, S, D]           static cache; rows [0, prefix) are the prompt, rows
-//                                     [prefix, prefix + n) hold the tree nodes
-//   anc      [B or 1, n] u64          bit j of word i: node j is node i or one of its ancestors
+//                                     [prefix, prefix + slots) hold the tree nodes (slots <= 64)
+//   anc      [B or 1, n] u64          bit j of word i: query row i may attend to tree slot j
+//                                     (the node in slot j is the row's node or one of its ancestors)
 //   out      [B, n, Hq, D]
 // One workgroup (4 wavefronts) owns one query head's 64 rows and one chunk of the keys; wavefront
 // w owns rows 16w..16w+15.  Scores are produced TRANSPOSED, S^T = K Q^T, with
@@ -61,7 +62,7 @@ __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
 }
 
 struct AttnParams {
-  int64_t batch, hq, hkv, n_rows, seq_stride, prefix, anc_batch_stride;
+  int64_t batch, hq, hkv, n_rows, n_slots, seq_stride, prefix, anc_batch_stride;
   int chunks;
   int64_t chunk_keys;          // multiple of kKeyBlock
   float scale_log2;            // softmax scale * log2(e)
@@ -82,7 +83,7 @@ __global__ __launch_bounds__(kAttnThreads) void tree_attention_kernel(
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int lq = lane & 15, lg = lane >> 4;            // query column of the lane, lane group
   const int n = (int)ap.n_rows;
-  const int64_t kv_len = ap.prefix + n;
+  const int64_t kv_len = ap.prefix + ap.n_slots;
   const int row = wave * 16 + lq;                      // query row of this lane
   const bool row_ok = row < n;
 
@@ -236,9 +237,9 @@ static int attn_chunks(int64_t batch, int64_t hq, int64_t kv_len) {
 
 using namespace subspec;
 
-extern "C" size_t subspec_tree_attention_workspace(int64_t batch, int64_t n_q_heads, int64_t prefix_len, int64_t n_rows) {
+extern "C" size_t subspec_tree_attention_workspace(int64_t batch, int64_t n_q_heads, int64_t prefix_len, int64_t n_tree_slots) {
   if (batch <= 0 || n_q_heads <= 0) return 256;
-  const int chunks = attn_chunks(batch, n_q_heads, prefix_len + n_rows);
+  const int chunks = attn_chunks(batch, n_q_heads, prefix_len + n_tree_slots);
   if (chunks == 1) return 256;
   const size_t slots = (size_t)batch * n_q_heads * chunks * kAttnRows;
   return align_up(slots * kAttnD * sizeof(float), 256) + align_up(slots * 2 * sizeof(float), 256);
@@ -246,7 +247,7 @@ extern "C" size_t subspec_tree_attention_workspace(int64_t batch, int64_t n_q_he
 
 extern "C" int subspec_tree_attention(const void* q, const void* k_cache, const void* v_cache, void* out, int dtype,
                                       int64_t batch, int64_t n_q_heads, int64_t n_kv_heads, int64_t n_rows,
-                                      int64_t head_dim, int64_t kv_seq_stride, int64_t prefix_len,
+                                      int64_t n_tree_slots, int64_t head_dim, int64_t kv_seq_stride, int64_t prefix_len,
                                       const uint64_t* anc_bits, int64_t anc_batch_stride, float scale,
                                       void* workspace, size_t workspace_bytes, void* stream) {
   if (dtype != SUBSPEC_BF16 && dtype != SUBSPEC_F16)
@@ -258,16 +259,20 @@ extern "C" int subspec_tree_attention(const void* q, const void* k_cache, const 
                  (long long)n_kv_heads);
   if (n_rows <= 0 || n_rows > kAttnRows)
     SUBSPEC_FAIL(SUBSPEC_ERR_LIMIT, "tree_attention: n_rows=%lld outside [1, %d]", (long long)n_rows, kAttnRows);
-  if (prefix_len < 0 || prefix_len + n_rows > kv_seq_stride)
-    SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "tree_attention: prefix_len=%lld + n_rows=%lld exceeds the cache length %lld",
-                 (long long)prefix_len, (long long)n_rows, (long long)kv_seq_stride);
+  if (n_tree_slots < 1 || n_tree_slots > 64)
+    SUBSPEC_FAIL(SUBSPEC_ERR_LIMIT, "tree_attention: n_tree_slots=%lld outside [1, 64] (one 64-bit mask word per row)",
+                 (long long)n_tree_slots);
+  if (prefix_len < 0 || prefix_len + n_tree_slots > kv_seq_stride)
+    SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "tree_attention: prefix_len=%lld + n_tree_slots=%lld exceeds the cache length %lld",
+                 (long long)prefix_len, (long long)n_tree_slots, (long long)kv_seq_stride);
   if (batch * n_q_heads > 65535) SUBSPEC_FAIL(SUBSPEC_ERR_LIMIT, "tree_attention: batch*heads=%lld too large", (long long)(batch * n_q_heads));
   if ((uintptr_t)q % 8 || (uintptr_t)k_cache % 16 || (uintptr_t)v_cache % 16 || (uintptr_t)out % 8)
     SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "tree_attention: q/out must be 8-byte and k/v 16-byte aligned");
   AttnParams ap;
-  ap.batch = batch; ap.hq = n_q_heads; ap.hkv = n_kv_heads; ap.n_rows = n_rows; ap.seq_stride = kv_seq_stride;
+  ap.batch = batch; ap.hq = n_q_heads; ap.hkv = n_kv_heads; ap.n_rows = n_rows; ap.n_slots = n_tree_slots;
+  ap.seq_stride = kv_seq_stride;
   ap.prefix = prefix_len; ap.anc_batch_stride = anc_batch_stride;
-  const int64_t kv_len = prefix_len + n_rows;
+  const int64_t kv_len = prefix_len + n_tree_slots;
   ap.chunks = attn_chunks(batch, n_q_heads, kv_len);
   const int64_t blocks = (kv_len + kKeyBlock - 1) / kKeyBlock;
   ap.chunk_keys = (blocks + ap.chunks - 1) / ap.chunks * kKeyBlock;

@@ -1,0 +1,220 @@
+"""Minimal Qwen2-shaped decoder used by the cycle driver: RMSNorm, rotary embeddings, GQA attention
+against the shared static KV cache, SwiGLU MLP.  Random-init weights of the real shapes; nothing is
+downloaded.
+
+Plain library work (bf16 GEMMs, norms, rotary, the causal prefill attention) goes through torch;
+the hot-path pieces are the HIP kernels: tree-masked attention for every tree forward, int4
+GEMV / GEMM for the draft's projections, layer streaming for the target's offloaded layers.
+q/k/v and gate/up are stored fused (rows concatenated), which leaves every output row and its
+quantization groups unchanged.
+"""
+from __future__ import annotations
+
+import math
+from dataclasses import dataclass
+from typing import Callable, Dict, List, Optional
+
+import torch
+import torch.nn.functional as F
+
+from . import ops, quant
+from .cache import KVManager
+from .offload import LayerSlabLayout, LayerStreamer
+
+
+@dataclass
+class DecoderConfig:
+    num_hidden_layers: int = 28
+    hidden_size: int = 3584
+    num_attention_heads: int = 28
+    num_key_value_heads: int = 4
+    head_dim: int = 128
+    intermediate_size: int = 18944
+    vocab_size: int = 152064
+    rms_norm_eps: float = 1e-6
+    rope_theta: float = 1e6
+    max_position_embeddings: int = 32768
+
+    @property
+    def q_size(self) -> int:
+        return self.num_attention_heads * self.head_dim
+
+    @property
+    def kv_size(self) -> int:
+        return self.num_key_value_heads * self.head_dim
+
+
+def layer_shapes(cfg: DecoderConfig) -> Dict[str, tuple]:
+    H, F_ = cfg.hidden_size, cfg.intermediate_size
+    return {
+        "input_layernorm.weight": (H,),
+        "qkv_proj.weight": (cfg.q_size + 2 * cfg.kv_size, H),
+        "qkv_proj.bias": (cfg.q_size + 2 * cfg.kv_size,),
+        "o_proj.weight": (H, cfg.q_size),
+        "post_attention_layernorm.weight": (H,),
+        "gate_up_proj.weight": (2 * F_, H),
+        "down_proj.weight": (H, F_),
+    }
+
+
+QUANTIZED = ("qkv_proj", "o_proj", "gate_up_proj", "down_proj")
+
+
+def init_weights(cfg: DecoderConfig, seed: int, device, dtype=torch.bfloat16) -> dict:
+    g = torch.Generator(device=device).manual_seed(seed)
+
+    def rnd(*shape, std=0.02):
+        return (torch.randn(*shape, generator=g, device=device, dtype=torch.float32) * std).to(dtype)
+
+    layers = []
+    for _ in range(cfg.num_hidden_layers):
+        w = {}
+        for name, shape in layer_shapes(cfg).items():
+            if name.endswith("layernorm.weight"):
+                w[name] = torch.ones(shape, device=device, dtype=dtype)
+            elif name.endswith(".bias"):
+                w[name] = rnd(*shape, std=0.02)
+            else:
+                w[name] = rnd(*shape)
+        layers.append(w)
+    return {"embed": rnd(cfg.vocab_size, cfg.hidden_size), "layers": layers,
+            "norm": torch.ones(cfg.hidden_size, device=device, dtype=dtype),
+            "lm_head": rnd(cfg.vocab_size, cfg.hidden_size)}
+
+
+def quantize_layers(layers: List[Dict[str, torch.Tensor]]) -> List[Dict[str, torch.Tensor]]:
+    """int4 g64 copies of the four projections of every layer (norms and biases are shared)."""
+    out = []
+    for w in layers:
+        q = {k: v for k, v in w.items() if not any(k == n + ".weight" for n in QUANTIZED)}
+        for n in QUANTIZED:
+            wq, sz = quant.pack_tiled(*quant.quantize_int4_g64(w[n + ".weight"]))
+            q[n + ".wq"], q[n + ".sz"] = wq, sz
+            q[n + ".out_features"] = w[n + ".weight"].shape[0]
+        out.append(q)
+    return out
+
+
+def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+    xf = x.float()
+    xf = xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps)
+    return weight * xf.to(x.dtype)
+
+
+def _linear(w: Dict[str, torch.Tensor], name: str, x: torch.Tensor) -> torch.Tensor:
+    bias = w.get(name + ".bias")
+    if name + ".wq" in w:
+        return ops.int4_linear(x, w[name + ".wq"], w[name + ".sz"], w[name + ".out_features"], bias)
+    return F.linear(x, w[name + ".weight"], bias)
+
+
+class Decoder:
+    """One decoder stack over a shared KV cache.  ``layers[i]`` holds either bf16 weights or int4
+    packed weights; layers from ``first_streamed`` on are fetched through ``streamer``."""
+
+    def __init__(self, cfg: DecoderConfig, embed, layers, norm, lm_head, kv: KVManager,
+                 streamer: Optional[LayerStreamer] = None, first_streamed: Optional[int] = None):
+        self.cfg, self.embed, self.layers, self.norm, self.lm_head, self.kv = cfg, embed, layers, norm, lm_head, kv
+        self.streamer = streamer
+        self.first_streamed = cfg.num_hidden_layers if first_streamed is None else first_streamed
+        self.device, self.dtype = embed.device, embed.dtype
+        inv = 1.0 / (cfg.rope_theta ** (torch.arange(0, cfg.head_dim, 2, device=self.device, dtype=torch.float32) / cfg.head_dim))
+        pos = torch.arange(kv.cache.max_cache_len + 8, device=self.device, dtype=torch.float32)
+        freqs = torch.outer(pos, inv)
+        self.cos = torch.cat([freqs, freqs], -1).cos()
+        self.sin = torch.cat([freqs, freqs], -1).sin()
+
+    # ------------------------------------------------------------------ pieces
+    def _rope(self, t: torch.Tensor, positions: torch.Tensor) -> torch.Tensor:
+        """t: [n, heads, D]"""
+        cos = self.cos[positions].unsqueeze(1).to(t.dtype)
+        sin = self.sin[positions].unsqueeze(1).to(t.dtype)
+        half = t.shape[-1] // 2
+        rot = torch.cat([-t[..., half:], t[..., :half]], -1)
+        return t * cos + rot * sin
+
+    def _layer(self, i: int, w: Dict[str, torch.Tensor], x: torch.Tensor, positions: torch.Tensor,
+               rows: torch.Tensor, attn: Callable[[int, torch.Tensor], torch.Tensor]) -> torch.Tensor:
+        cfg = self.cfg
+        n = x.shape[0]
+        h = rms_norm(x, w["input_layernorm.weight"], cfg.rms_norm_eps)
+        qkv = _linear(w, "qkv_proj", h)
+        q, k, v = qkv.split([cfg.q_size, cfg.kv_size, cfg.kv_size], dim=-1)
+        q = self._rope(q.reshape(n, cfg.num_attention_heads, cfg.head_dim), positions)
+        k = self._rope(k.reshape(n, cfg.num_key_value_heads, cfg.head_dim), positions)
+        v = v.reshape(n, cfg.num_key_value_heads, cfg.head_dim)
+        self.kv.cache.write(i, rows, k.transpose(0, 1).unsqueeze(0), v.transpose(0, 1).unsqueeze(0))
+        a = attn(i, q.transpose(0, 1).unsqueeze(0).contiguous())          # [1, Hq, n, D] -> [n, Hq*D]
+        x = x + _linear(w, "o_proj", a)
+        h = rms_norm(x, w["post_attention_layernorm.weight"], cfg.rms_norm_eps)
+        gate, up = _linear(w, "gate_up_proj", h).chunk(2, dim=-1)
+        return x + _linear(w, "down_proj", F.silu(gate) * up)
+
+    def _run_layers(self, x, positions, rows, attn) -> torch.Tensor:
+        state = {"x": x}
+        for i in range(min(self.first_streamed, len(self.layers))):
+            state["x"] = self._layer(i, self.layers[i], state["x"], positions, rows, attn)
+        if self.streamer is not None and self.streamer.n:
+            base = self.first_streamed
+
+            def step(j, w):
+                state["x"] = self._layer(base + j, w, state["x"], positions, rows, attn)
+
+            self.streamer.run(step)
+        return state["x"]
+
+    def logits(self, x: torch.Tensor) -> torch.Tensor:
+        return F.linear(rms_norm(x, self.norm, self.cfg.rms_norm_eps), self.lm_head)
+
+    # ------------------------------------------------------------------ forwards
+    def prefill(self, token_ids: torch.Tensor, start: int) -> torch.Tensor:
+        """Causal forward of ``token_ids`` [n] at cache rows start..start+n-1; returns the last logits [1, V]."""
+        n = token_ids.numel()
+        positions = torch.arange(start, start + n, device=self.device)
+        cfg = self.cfg
+        rep = cfg.num_attention_heads // cfg.num_key_value_heads
+
+        def attn(i, q):
+            k = self.kv.cache.k(i)[:, :, :start + n].repeat_interleave(rep, dim=1)
+            v = self.kv.cache.v(i)[:, :, :start + n].repeat_interleave(rep, dim=1)
+            mask = torch.ones(n, start + n, dtype=torch.bool, device=self.device).tril(diagonal=start)
+            o = F.scaled_dot_product_attention(q, k, v, attn_mask=mask)
+            return o.transpose(1, 2).reshape(n, cfg.q_size)
+
+        x = self._run_layers(self.embed[token_ids], positions, positions, attn)
+        return self.logits(x[-1:])
+
+    def tree_forward(self, token_ids: torch.Tensor, depths: torch.Tensor, anc_bits: torch.Tensor, prefix_len: int,
+                     first_slot: int = 0, n_tree_slots: Optional[int] = None) -> torch.Tensor:
+        """Forward of tree nodes occupying cache rows prefix_len+first_slot.. ; ``depths`` are the node
+        depths (rotary position = prefix_len + depth), ``anc_bits`` int64 [n] bitsets over tree
+        slots.  Returns logits [n, V]."""
+        n = token_ids.numel()
+        slots = first_slot + n if n_tree_slots is None else n_tree_slots
+        positions = depths.to(self.device) + prefix_len
+        rows = torch.arange(prefix_len + first_slot, prefix_len + first_slot + n, device=self.device)
+        cfg = self.cfg
+
+        def attn(i, q):
+            return ops.tree_attention(q, self.kv.cache.k(i), self.kv.cache.v(i), anc_bits, prefix_len,
+                                      n_tree_slots=slots).reshape(n, cfg.q_size)
+
+        return self.logits(self._run_layers(self.embed[token_ids], positions, rows, attn))
+
+
+def build_models(cfg: DecoderConfig, kv: KVManager, seed: int = 0, device="cuda:0", dtype=torch.bfloat16,
+                 first_streamed: Optional[int] = None):
+    """Target (bf16, layers >= first_streamed in pinned host memory) and substitute draft (same
+    weights, int4 g64, resident) over one shared KV cache."""
+    w = init_weights(cfg, seed, device, dtype)
+    draft_layers = quantize_layers(w["layers"])
+    streamer = None
+    layers = w["layers"]
+    if first_streamed is not None and first_streamed < cfg.num_hidden_layers:
+        layout = LayerSlabLayout(layer_shapes(cfg), dtype)
+        host = [{k: v.cpu() for k, v in layers[i].items()} for i in range(first_streamed, cfg.num_hidden_layers)]
+        streamer = LayerStreamer(layout, host, device)
+        layers = layers[:first_streamed]
+    target = Decoder(cfg, w["embed"], layers, w["norm"], w["lm_head"], kv, streamer, first_streamed)
+    draft = Decoder(cfg, w["embed"], draft_layers, w["norm"], w["lm_head"], kv)
+    return target, draft, w

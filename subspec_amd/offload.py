@@ -1,0 +1,93 @@
+"""Layer streaming: target decoder layers kept in pinned host memory and copied into two device
+slabs, one layer ahead of the compute stream.
+
+Replaces the reference's hook-chain offloaders (``PrefetchOffloader``,
+specdecodes/helpers/offloaders/prefetch_offloader_postspec.py:54-241; placement by
+``LayerOffloadRecipe(keep_first_n_layers_on_gpu)``, recipes/offload/layer_offload.py:9-56) with an
+explicit schedule:
+
+* every offloaded layer is ONE contiguous pinned slab (all seven projections + norms), so a layer
+  is one ``hipMemcpyAsync`` instead of seven hooked ``copy_`` calls;
+* two device slabs alternate; the copy of layer i+2 into a slab waits on an event recorded after
+  layer i's last kernel (the write-after-read edge the reference leaves to timing), and layer
+  i's compute waits on its copy event;
+* the copy stream runs at default priority.
+"""
+from __future__ import annotations
+
+from typing import Callable, Dict, List, Sequence, Tuple
+
+import torch
+
+from . import _lib as L
+
+
+class LayerSlabLayout:
+    """Names, shapes and byte offsets of one layer's tensors inside a slab (256-byte aligned)."""
+
+    def __init__(self, shapes: Dict[str, Tuple[int, ...]], dtype: torch.dtype):
+        self.dtype = dtype
+        self.entries: List[Tuple[str, Tuple[int, ...], int, int]] = []
+        off = 0
+        esize = torch.empty((), dtype=dtype).element_size()
+        for name, shape in shapes.items():
+            numel = 1
+            for s in shape:
+                numel *= int(s)
+            self.entries.append((name, tuple(shape), off, numel))
+            off += (numel * esize + 255) // 256 * 256
+        self.nbytes = off
+        self.esize = esize
+
+    def views(self, slab: torch.Tensor) -> Dict[str, torch.Tensor]:
+        """Typed views into a uint8 slab."""
+        out = {}
+        for name, shape, off, numel in self.entries:
+            out[name] = slab[off:off + numel * self.esize].view(self.dtype).view(shape)
+        return out
+
+
+class LayerStreamer:
+    def __init__(self, layout: LayerSlabLayout, host_layers: Sequence[Dict[str, torch.Tensor]], device):
+        self.layout = layout
+        self.device = torch.device(device)
+        self.n = len(host_layers)
+        # pinned host arena: one slab per offloaded layer (allocated pinned, never registered afterwards)
+        self.host = torch.empty((self.n, layout.nbytes), dtype=torch.uint8, pin_memory=True)
+        for i, tensors in enumerate(host_layers):
+            views = layout.views(self.host[i])
+            for name, t in tensors.items():
+                views[name].copy_(t)
+        self.slabs = [torch.empty(layout.nbytes, dtype=torch.uint8, device=self.device) for _ in range(2)]
+        self.slab_views = [layout.views(s) for s in self.slabs]
+        self.copy_stream = torch.cuda.Stream(device=self.device)          # default priority
+        self.copied = [torch.cuda.Event() for _ in range(2)]
+        self.released = [torch.cuda.Event() for _ in range(2)]
+        self._released_valid = [False, False]
+        self.bytes_streamed = 0
+
+    def _issue(self, layer: int) -> None:
+        slot = layer % 2
+        if self._released_valid[slot]:
+            self.copy_stream.wait_event(self.released[slot])              # last reader of this slab is done
+        code = L.lib().subspec_stream_copy_h2d(self.slabs[slot].data_ptr(), self.host[layer].data_ptr(),
+                                               self.layout.nbytes, self.copy_stream.cuda_stream)
+        L.check(code, "subspec_stream_copy_h2d")
+        self.copied[slot].record(self.copy_stream)
+        self.bytes_streamed += self.layout.nbytes
+
+    def run(self, fn: Callable[[int, Dict[str, torch.Tensor]], None]) -> None:
+        """Calls ``fn(i, weights_of_layer_i)`` for every offloaded layer in order on the current
+        stream, with layer i+1's copy in flight while layer i computes."""
+        compute = torch.cuda.current_stream(self.device)
+        if self.n == 0:
+            return
+        self._issue(0)
+        for i in range(self.n):
+            slot = i % 2
+            if i + 1 < self.n:
+                self._issue(i + 1)
+            compute.wait_event(self.copied[slot])
+            fn(i, self.slab_views[slot])
+            self.released[slot].record(compute)
+            self._released_valid[slot] = True

@@ -176,9 +176,11 @@ def ancestor_bits_tensor(parents, device=None) -> torch.Tensor:
 
 
 def tree_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, anc_bits: torch.Tensor,
-                   prefix_len: int, scale: Optional[float] = None, workspace: Optional[torch.Tensor] = None):
+                   prefix_len: int, scale: Optional[float] = None, workspace: Optional[torch.Tensor] = None,
+                   n_tree_slots: Optional[int] = None):
     """``q`` [B, Hq, n, D], caches [B, Hkv, S, D] (tree K/V already written at rows prefix_len..),
-    ``anc_bits`` int64 [n] (shared tree) or [B, n].  Returns [B, n, Hq * D]."""
+    ``anc_bits`` int64 [n] (shared tree) or [B, n]: bit j = row may attend to tree slot j.
+    ``n_tree_slots`` (default n) is the number of occupied tree slots.  Returns [B, n, Hq * D]."""
     dev = _require_gpu(q, k_cache, v_cache, anc_bits)
     if q.dim() != 4 or k_cache.dim() != 4 or v_cache.shape != k_cache.shape:
         raise ValueError("expected q [B, Hq, n, D] and k/v caches [B, Hkv, S, D]")
@@ -198,12 +200,13 @@ def tree_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
         raise ValueError("anc_bits batch dimension must be 1 or B")
     stride = n if (anc_bits.dim() == 2 and anc_bits.shape[0] == B and B > 1) else 0
     lib = L.lib()
-    need = lib.subspec_tree_attention_workspace(B, Hq, int(prefix_len), n)
+    slots = n if n_tree_slots is None else int(n_tree_slots)
+    need = lib.subspec_tree_attention_workspace(B, Hq, int(prefix_len), slots)
     if workspace is None and need > 256:
         workspace = torch.empty(need, dtype=torch.uint8, device=dev)
     out = torch.empty((B, n, Hq * D), dtype=q.dtype, device=dev)
     code = lib.subspec_tree_attention(
-        q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), _dtype_code(q), B, Hq, Hkv, n, D, S,
+        q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), _dtype_code(q), B, Hq, Hkv, n, slots, D, S,
         int(prefix_len), anc_bits.data_ptr(), stride, float(D ** -0.5 if scale is None else scale),
         None if workspace is None else workspace.data_ptr(),
         0 if workspace is None else workspace.numel() * workspace.element_size(), _stream(dev))

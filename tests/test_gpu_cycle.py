@@ -1,0 +1,137 @@
+"""GPU: layer streaming, the substitute draft and the whole speculative cycle on a small
+Qwen2-shaped decoder (same code path as the 7B shape).
+
+What the reference fixes for these rows are invariants rather than vectors:
+  * a streamed forward equals the all-resident forward bit for bit (only data placement differs);
+  * every token the cycle emits is the target's greedy choice at its context, the kept KV rows are
+    the accepted contexts' rows, and the final sequence length honours max_length;
+  * draft tree levels are the canonical top-k of (leaf x vocab) cumulative probabilities.
+"""
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+from oracle import kv as okv
+from oracle import topk as ot
+from oracle import verify as ov
+from subspec_amd import ops
+from subspec_amd.cache import KVManager, StaticKVCache, create_kv_cache
+from subspec_amd.draft import SubSpecSDDraftModel
+from subspec_amd.generator import SubSpecSDGenerator
+from subspec_amd.model import DecoderConfig, build_models
+from subspec_amd.utils import DraftParams
+from subspec_amd.wandb_logger import wandb_logger
+
+DEV = "cuda:0"
+CFG = DecoderConfig(num_hidden_layers=4, hidden_size=256, num_attention_heads=2, num_key_value_heads=1,
+                    head_dim=128, intermediate_size=512, vocab_size=2048)
+
+
+def _models(first_streamed=None, max_len=256, seed=3):
+    kv = create_kv_cache("static", max_cache_len=max_len, config=CFG, device=DEV, dtype=torch.bfloat16)
+    target, draft, w = build_models(CFG, kv, seed=seed, device=DEV, first_streamed=first_streamed)
+    return kv, target, draft, w
+
+
+def test_streamed_forward_is_bit_identical_to_resident():
+    prompt = torch.randint(0, CFG.vocab_size, (40,), generator=torch.Generator().manual_seed(1)).to(DEV)
+    kv_a, tgt_a, _, _ = _models(first_streamed=None)
+    kv_b, tgt_b, _, _ = _models(first_streamed=2)
+    la = tgt_a.prefill(prompt, 0)
+    lb = tgt_b.prefill(prompt, 0)
+    assert tgt_b.streamer is not None and tgt_b.streamer.n == 2
+    assert torch.equal(la, lb)
+    assert torch.equal(kv_a.cache.data, kv_b.cache.data)
+    # several forwards in a row reuse the two slabs; still identical
+    for _ in range(3):
+        assert torch.equal(tgt_a.prefill(prompt[:7], 40), tgt_b.prefill(prompt[:7], 40))
+    assert tgt_b.streamer.bytes_streamed == 4 * 2 * tgt_b.streamer.layout.nbytes
+
+
+def test_draft_tree_levels_are_canonical_topk():
+    kv, target, draft, _ = _models()
+    prompt = torch.randint(0, CFG.vocab_size, (1, 24), generator=torch.Generator().manual_seed(2)).to(DEV)
+    target.prefill(prompt[0], 0)
+    kv.seq_len = 24
+    dm = SubSpecSDDraftModel(draft)
+    dm.draft_params = DraftParams(temperature=0.5, max_depth=4, topk_len=4)
+    dm.set_past_key_values(kv)
+    tree = dm.speculate(torch.tensor([[5]], device=DEV))
+    assert tree.size() == 1 + 4 * 4
+    d = tree.get_tree_data()
+    par = d["parent_indices"].tolist()
+    assert all(p < i for i, p in enumerate(par)) and d["depths"].tolist()[1:] == sorted(d["depths"].tolist()[1:])
+    # first level == canonical top-k of softmax(root logits / T) computed independently
+    logits = draft.tree_forward(torch.tensor([5], device=DEV), torch.zeros(1, dtype=torch.long, device=DEV),
+                                torch.ones(1, dtype=torch.int64, device=DEV), 24)
+    probs = torch.softmax(logits / 0.5, -1).unsqueeze(0)
+    tok, val, _ = ot.topk_expand(probs.cpu(), torch.ones(1, 1, dtype=probs.dtype), 4)
+    assert d["token_ids"].tolist()[1:5] == tok[0].tolist()
+    assert d["cumulative_probabilities"].tolist()[1:5] == val[0].float().tolist()
+    # cumulative probabilities never increase along an edge
+    cp = d["cumulative_probabilities"].tolist()
+    assert all(cp[i] <= cp[par[i]] + 1e-6 for i in range(1, len(par)))
+
+
+@pytest.mark.parametrize("method,kwargs", [("exact", None),
+                                           ("lossy", dict(threshold=0.9, window_size=1, threshold_method="entropy"))])
+def test_cycle_emits_target_greedy_tokens_and_compacts_kv(method, kwargs):
+    kv, target, draft, _ = _models(first_streamed=2)
+    gen = SubSpecSDGenerator(target, None, SubSpecSDDraftModel(draft), DraftParams(temperature=0.2, max_depth=4, topk_len=4),
+                             generator_kwargs=dict(verify_method=method, verify_kwargs=kwargs))
+    prompt = torch.randint(0, CFG.vocab_size, (1, 32), generator=torch.Generator().manual_seed(4))
+    wandb_logger.clear_log_data()
+    out = gen.generate(prompt.to(DEV), max_new_tokens=24, do_sample=False, past_key_values=kv)
+    assert out.shape[1] == 32 + 24 and torch.equal(out[0, :32].cpu(), prompt[0])
+    log = wandb_logger.log_data
+    assert log["n_tokens"] == 24 and log["n_iter"] >= 1 and log["avg_sampled"] >= 1.0 and log["tput"] > 0
+    assert kv.get_seq_length() == out.shape[1] - 1            # everything but the last sampled token is cached
+    # the compacted cache equals what a fresh prefill of the produced sequence writes (same weights)
+    kv2, target2, _, _ = _models(first_streamed=None)
+    target2.prefill(out[0, :-1], 0)
+    L = out.shape[1] - 1
+    a, b = kv.cache.data[..., :L, :].float(), kv2.cache.data[..., :L, :].float()
+    assert (a - b).abs().amax() <= 5e-2 * b.abs().amax()
+
+
+def test_one_cycle_against_the_oracle():
+    kv, target, draft, _ = _models()
+    prompt = torch.randint(0, CFG.vocab_size, (48,), generator=torch.Generator().manual_seed(6)).to(DEV)
+    lg = target.prefill(prompt, 0)
+    kv.seq_len = 48
+    dm = SubSpecSDDraftModel(draft)
+    gen = SubSpecSDGenerator(target, None, dm, DraftParams(temperature=0.2, max_depth=5, topk_len=4))
+    dm.set_past_key_values(kv)
+    root = lg.argmax(-1).view(1, 1)
+    tree = dm.speculate(root)
+    before = None
+    logits = gen._tree_decoding(tree, kv, position_offset=48)
+    before = kv.cache.data.clone()
+    out = gen._verify(tree, 0, logits)
+    kv.reorder_cache_with_offset(out["contexts"][0], offset=48, dim=2, count_dev=out["counts"][0, 0:1])
+    torch.cuda.synchronize()
+    d = tree.get_tree_data()
+    exp_t, exp_c, (_, exp_a) = ov.verify_logits(logits.cpu(), d["token_ids"].tolist(), d["parent_indices"].tolist())
+    emitted, accept = int(out["counts"][0, 0]), int(out["counts"][0, 1])
+    assert out["tokens"][0, :emitted].tolist() == exp_t and out["contexts"][0, :emitted].tolist() == exp_c
+    assert accept == exp_a
+    assert torch.equal(kv.cache.data.cpu(), okv.compact_static(before.cpu(), exp_c, 48))
+
+
+def test_generator_argument_errors():
+    kv, target, draft, _ = _models()
+    gen = SubSpecSDGenerator(target, None, SubSpecSDDraftModel(draft), DraftParams(max_depth=2, topk_len=2))
+    ids = torch.zeros(1, 4, dtype=torch.long, device=DEV)
+    with pytest.raises(ValueError):
+        gen.generate(ids, do_sample=False, past_key_values=kv)                  # no max_length
+    with pytest.raises(ValueError):
+        gen.generate(ids, max_new_tokens=4, do_sample=False)                    # no cache
+    with pytest.raises(NotImplementedError):
+        gen.generate(ids, max_new_tokens=4, do_sample=True, past_key_values=kv)
+    with pytest.raises(ValueError):
+        create_kv_cache("dynamic", max_cache_len=8, config=CFG)
+    bad = SubSpecSDGenerator(target, None, SubSpecSDDraftModel(draft), DraftParams(max_depth=2, topk_len=2),
+                             generator_kwargs=dict(verify_method="bogus"))
+    with pytest.raises(ValueError):
+        bad.generate(ids, max_new_tokens=4, do_sample=False, past_key_values=kv)
