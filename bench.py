@@ -16,6 +16,12 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per launch at the default workload, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs scaled
+# by a copy of known size (profiles/verify_cycle_config2_hbm_counters.md); None for other sizes.
+MEASURED_TRAFFIC = {
+    ("verify", 32, 152064): int(307331.9 * 1024 * 2.0 + 64.0 * 1024),
+    ("topk", 32, 152064): int(325291.2 * 1024 * 2.0 + 331.5 * 1024),
+}
 
 
 def parse():
@@ -28,6 +34,9 @@ def parse():
     ap.add_argument("--cpu-trees", type=int, default=4, help="trees in the bounded CPU-baseline sample")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="lower bound of CPU-baseline work")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--pmc-calibration", action="store_true",
+                    help="also run three plain copies of the logits tensor (known size) so that hardware byte counters "
+                         "collected by rocprofv3 --pmc can be scaled")
     ap.add_argument("--new-tokens", type=int, default=256, help="e2e workload: tokens to generate")
     ap.add_argument("--workload", default="verify-cycle", choices=["verify-cycle", "attention", "int4", "greedy", "e2e"],
                     help="verify-cycle (default, BASELINE config 2) is the benchmark line; the others time one "
@@ -236,6 +245,11 @@ def main():
     for _ in range(args.warmup):
         out, top = step()
     torch.cuda.synchronize()
+    if args.pmc_calibration:
+        for _ in range(3):
+            calib = cfg["logits"].clone()                # copy kernel: reads and writes B*n*V*2 bytes
+        torch.cuda.synchronize()
+        del calib
 
     # per-call durations with events on the stream the kernels are launched on (torch's current stream)
     ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
@@ -260,10 +274,10 @@ def main():
     bytes_verify = B * n * V * 2
     bytes_topk = B * n * V * 2
 
-    def roof(nbytes, ms):
+    def roof(nbytes, ms, which):
         gbs = nbytes / (ms * 1e-3) / 1e9
         return {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None}
+                "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC.get((which, B, V))}
 
     result = {
         "metric": "accepted tokens/sec + verify-cycle latency (Qwen2.5-7B shape); % HBM roofline",
@@ -278,9 +292,9 @@ def main():
                    "trees": B, "nodes": n, "vocab": V, "topk": k,
                    "tokens_per_step": tokens_per_step, "accepted_draft_tokens_per_step": accepted_per_step,
                    "verify_ms": round(verify_ms, 4), "topk_ms": round(topk_ms, 4)},
-        "roofline": dict(roof(bytes_verify, verify_ms), kernel="row_partial_kernel (+2 tail kernels of tree_verify)",
+        "roofline": dict(roof(bytes_verify, verify_ms, "verify"), kernel="row_partial_kernel (+2 tail kernels of tree_verify)",
                          bytes_per_launch=bytes_verify),
-        "roofline_topk": dict(roof(bytes_topk, topk_ms), kernel="topk_slice_kernel (+ merge)",
+        "roofline_topk": dict(roof(bytes_topk, topk_ms, "topk"), kernel="topk_slice_kernel (+ merge)",
                               bytes_per_launch=bytes_topk),
     }
     if not args.no_cpu_baseline:
