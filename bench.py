@@ -253,6 +253,7 @@ def main():
 
     # per-call durations with events on the stream the kernels are launched on (torch's current stream)
     ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
+    lib.subspec_profile_enable(1)                      # event pair around the dominant kernel of every call
     t0 = time.perf_counter()
     for i in range(args.steps):
         ev[i][0].record()
@@ -263,6 +264,11 @@ def main():
         ev[i][2].record()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
+    lib.subspec_profile_enable(0)
+    n_prof = lib.subspec_profile_count()
+    kern = [lib.subspec_profile_read_ms(i) for i in range(n_prof)]
+    row_kernel_ms = sum(kern[0::2]) / max(1, len(kern[0::2]))     # calls alternate: verify, top-k
+    topk_kernel_ms = sum(kern[1::2]) / max(1, len(kern[1::2]))
 
     verify_ms = sum(e[0].elapsed_time(e[1]) for e in ev) / args.steps
     topk_ms = sum(e[1].elapsed_time(e[2]) for e in ev) / args.steps
@@ -292,10 +298,12 @@ def main():
                    "trees": B, "nodes": n, "vocab": V, "topk": k,
                    "tokens_per_step": tokens_per_step, "accepted_draft_tokens_per_step": accepted_per_step,
                    "verify_ms": round(verify_ms, 4), "topk_ms": round(topk_ms, 4)},
-        "roofline": dict(roof(bytes_verify, verify_ms, "verify"), kernel="row_partial_kernel (+2 tail kernels of tree_verify)",
-                         bytes_per_launch=bytes_verify),
-        "roofline_topk": dict(roof(bytes_topk, topk_ms, "topk"), kernel="topk_slice_kernel (+ merge)",
-                              bytes_per_launch=bytes_topk),
+        "roofline": dict(roof(bytes_verify, row_kernel_ms, "verify"), kernel="subspec::row_partial_kernel",
+                         bytes_per_launch=bytes_verify, kernel_ms=round(row_kernel_ms, 4),
+                         sequence_frac=round(bytes_verify / (verify_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)),
+        "roofline_topk": dict(roof(bytes_topk, topk_kernel_ms, "topk"), kernel="subspec::topk_slice_kernel",
+                              bytes_per_launch=bytes_topk, kernel_ms=round(topk_kernel_ms, 4),
+                              sequence_frac=round(bytes_topk / (topk_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)),
     }
     if not args.no_cpu_baseline:
         cfg_cpu = dict(cfg)

@@ -52,6 +52,16 @@ extern "C" {
 int subspec_abi_version(void);
 const char* subspec_last_error(void);
 
+/* Measurement aid (no counterpart in the reference, whose phase timing is CUDA events around Python
+ * calls, specdecodes/models/utils/mixin.py:101-224): while enabled, each entry-point call records a pair
+ * of events on its launch stream around its dominant kernel (the one pass over the logits /
+ * probabilities / KV / weights).  Up to 512 calls are kept since the last enable;
+ * subspec_profile_read_ms(i) waits for call i's pair and returns that kernel's duration in
+ * milliseconds (-1 if out of range).  Process-wide, not thread-safe. */
+int subspec_profile_enable(int on);
+int subspec_profile_count(void);
+float subspec_profile_read_ms(int index);
+
 /* ------------------------------------------------------------------------------------------
  * Tree verification, fused: softmax statistics, first-index argmax of the rounded probabilities,
  * normalized entropy, p[parent(i), token(i)] for every node, then the greedy walk or the lossy

@@ -25,6 +25,9 @@ _p, _i32, _i64, _f64, _sz = C.c_void_p, C.c_int32, C.c_int64, C.c_double, C.c_si
 _SIGNATURES = {
     "subspec_abi_version": (C.c_int, []),
     "subspec_last_error": (C.c_char_p, []),
+    "subspec_profile_enable": (C.c_int, [C.c_int]),
+    "subspec_profile_count": (C.c_int, []),
+    "subspec_profile_read_ms": (C.c_float, [C.c_int]),
     "subspec_tree_verify_workspace": (_sz, [_i64, _i64, _i64, C.c_int]),
     "subspec_tree_verify": (C.c_int, [_p, C.c_int, _i64, _i64, _i64, _p, _p, _i64, _i32, _i32, _i64,
                                       C.c_int, C.c_int, _f64, _i32, C.c_int, _p, _sz,

@@ -293,14 +293,20 @@ extern "C" int subspec_tree_attention(const void* q, const void* k_cache, const 
   hipStream_t st = (hipStream_t)stream;
   const dim3 grid(ap.chunks, (unsigned)(batch * n_q_heads));
   if (dtype == SUBSPEC_BF16) {
-    hipLaunchKernelGGL((tree_attention_kernel<SUBSPEC_BF16>), grid, dim3(kAttnThreads), 0, st, (const uint16_t*)q,
-                       (const uint16_t*)k_cache, (const uint16_t*)v_cache, anc_bits, ap, (uint16_t*)out, part_o, part_ml);
+    {
+      DominantKernelTimer timer(st);
+      hipLaunchKernelGGL((tree_attention_kernel<SUBSPEC_BF16>), grid, dim3(kAttnThreads), 0, st, (const uint16_t*)q,
+                         (const uint16_t*)k_cache, (const uint16_t*)v_cache, anc_bits, ap, (uint16_t*)out, part_o, part_ml);
+    }
     if (ap.chunks > 1)
       hipLaunchKernelGGL((tree_attention_merge_kernel<SUBSPEC_BF16>), dim3((unsigned)n_rows, (unsigned)(batch * n_q_heads)),
                          dim3(kAttnD), 0, st, part_o, part_ml, ap, (uint16_t*)out);
   } else {
-    hipLaunchKernelGGL((tree_attention_kernel<SUBSPEC_F16>), grid, dim3(kAttnThreads), 0, st, (const uint16_t*)q,
-                       (const uint16_t*)k_cache, (const uint16_t*)v_cache, anc_bits, ap, (uint16_t*)out, part_o, part_ml);
+    {
+      DominantKernelTimer timer(st);
+      hipLaunchKernelGGL((tree_attention_kernel<SUBSPEC_F16>), grid, dim3(kAttnThreads), 0, st, (const uint16_t*)q,
+                         (const uint16_t*)k_cache, (const uint16_t*)v_cache, anc_bits, ap, (uint16_t*)out, part_o, part_ml);
+    }
     if (ap.chunks > 1)
       hipLaunchKernelGGL((tree_attention_merge_kernel<SUBSPEC_F16>), dim3((unsigned)n_rows, (unsigned)(batch * n_q_heads)),
                          dim3(kAttnD), 0, st, part_o, part_ml, ap, (uint16_t*)out);

@@ -26,6 +26,16 @@ void set_error(const char* fmt, ...);
     if (e_ != hipSuccess) SUBSPEC_FAIL(SUBSPEC_ERR_HIP, "%s failed: %s", #expr, hipGetErrorString(e_)); \
   } while (0)
 
+// ---------------------------------------------------------------- optional timing of the dominant kernel
+// When enabled (subspec_profile_enable), every entry point brackets its dominant kernel with a
+// pair of events on the launch stream; subspec_profile_last_ms() returns that kernel's duration.
+struct DominantKernelTimer {
+  explicit DominantKernelTimer(hipStream_t st);
+  ~DominantKernelTimer();
+  hipStream_t st_;
+  bool on_;
+};
+
 inline size_t dtype_size(int dtype) { return dtype == SUBSPEC_F32 ? 4 : 2; }
 inline bool dtype_ok(int dtype) { return dtype == SUBSPEC_F32 || dtype == SUBSPEC_F16 || dtype == SUBSPEC_BF16; }
 inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }

@@ -266,6 +266,7 @@ static int run_int4(const void* x, const uint32_t* wq, const uint32_t* sz, const
                     int64_t N, int64_t K, void* workspace, hipStream_t st) {
   if (M == 1) {
     const size_t smem = (size_t)K * 2 + (size_t)(K / 16) * 4 + 64 * 4;
+    DominantKernelTimer timer(st);
     hipLaunchKernelGGL((int4_gemv_kernel<DT>), dim3((unsigned)(N / 16)), dim3(kI4Threads), smem, st, (const uint16_t*)x,
                        (const uint2*)wq, sz, (const uint16_t*)bias, (uint16_t*)y, N, K);
   } else {
@@ -278,9 +279,12 @@ static int run_int4(const void* x, const uint32_t* wq, const uint32_t* sz, const
   hipLaunchKernelGGL((int4_gemm_kernel<DT, MT>), grid, dim3(kI4Threads), 0, st, (const uint16_t*)x, xsum,           \
                      (const uint2*)wq, sz, (const uint16_t*)bias, (uint16_t*)y, partial, M, N, K, pl.splits,        \
                      pl.groups_per_split)
-    if (M <= 16) SUBSPEC_I4_LAUNCH(1);
-    else if (M <= 32) SUBSPEC_I4_LAUNCH(2);
-    else SUBSPEC_I4_LAUNCH(4);
+    {
+      DominantKernelTimer timer(st);
+      if (M <= 16) SUBSPEC_I4_LAUNCH(1);
+      else if (M <= 32) SUBSPEC_I4_LAUNCH(2);
+      else SUBSPEC_I4_LAUNCH(4);
+    }
 #undef SUBSPEC_I4_LAUNCH
     if (pl.splits > 1)
       hipLaunchKernelGGL((int4_reduce_kernel<DT>), dim3((unsigned)((M * N + 255) / 256)), dim3(256), 0, st, partial,

@@ -359,12 +359,15 @@ static int run_topk(const void* probs, const void* parent_probs, int64_t batch, 
                     const TopkPlan& pl, uint64_t* cand, int32_t* cand_count, int64_t* token_ids, void* topk_probs,
                     int64_t* parent_indices, hipStream_t st) {
   const dim3 grid(pl.splits, (unsigned)(batch * leaves));
-  if (pl.vec == 1)
-    hipLaunchKernelGGL((topk_slice_kernel<DT, 1>), grid, dim3(kTopkThreads), 0, st, probs, parent_probs, vocab, leaves,
-                       pl.splits, pl.chunk, k, cand, cand_count);
-  else
-    hipLaunchKernelGGL((topk_slice_kernel<DT, (DT == SUBSPEC_F32 ? 4 : 8)>), grid, dim3(kTopkThreads), 0, st, probs,
-                       parent_probs, vocab, leaves, pl.splits, pl.chunk, k, cand, cand_count);
+  {
+    DominantKernelTimer timer(st);
+    if (pl.vec == 1)
+      hipLaunchKernelGGL((topk_slice_kernel<DT, 1>), grid, dim3(kTopkThreads), 0, st, probs, parent_probs, vocab, leaves,
+                         pl.splits, pl.chunk, k, cand, cand_count);
+    else
+      hipLaunchKernelGGL((topk_slice_kernel<DT, (DT == SUBSPEC_F32 ? 4 : 8)>), grid, dim3(kTopkThreads), 0, st, probs,
+                         parent_probs, vocab, leaves, pl.splits, pl.chunk, k, cand, cand_count);
+  }
   hipLaunchKernelGGL((topk_merge_kernel<DT>), dim3((unsigned)batch), dim3(kMergeThreads), 0, st, cand, cand_count,
                      vocab, leaves, pl.splits, k, token_ids, topk_probs, parent_indices);
   SUBSPEC_CHECK_HIP(hipGetLastError());

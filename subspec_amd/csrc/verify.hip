@@ -559,8 +559,11 @@ static int run_verify(const void* logits, int64_t batch, int64_t rows, int64_t v
                       int32_t* out_counts, int64_t* node_target, float* node_entropy, float* node_child_prob,
                       hipStream_t st) {
   const dim3 grid(pl.splits, (unsigned)(batch * rows));
-  if (pl.vec == 1) launch_partial<DT, 1>(grid, st, logits, vp, p1, p2);
-  else launch_partial<DT, (DT == SUBSPEC_F32 ? 4 : 8)>(grid, st, logits, vp, p1, p2);
+  {
+    DominantKernelTimer timer(st);
+    if (pl.vec == 1) launch_partial<DT, 1>(grid, st, logits, vp, p1, p2);
+    else launch_partial<DT, (DT == SUBSPEC_F32 ? 4 : 8)>(grid, st, logits, vp, p1, p2);
+  }
   if (pl.splits > 1) hipLaunchKernelGGL((row_exact_kernel<DT>), grid, dim3(kRowThreads), 0, st, logits, vp, p1, p2);
   const int64_t widest = std::max<int64_t>(rows, tp.n_nodes);
   const int slots = widest <= kWave ? 1 : widest <= 2 * kWave ? 2 : 4;
