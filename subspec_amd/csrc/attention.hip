@@ -13,13 +13,17 @@
 //   anc      [B or 1, n] u64          bit j of word i: query row i may attend to tree slot j
 //                                     (the node in slot j is the row's node or one of its ancestors)
 //   out      [B, n, Hq, D]
-// One workgroup (4 wavefronts) owns one query head's 64 rows and one chunk of the keys; wavefront
-// w owns rows 16w..16w+15.  Scores are produced TRANSPOSED, S^T = K Q^T, with
-// v_mfma_f32_16x16x16: the accumulator then holds, per lane, four consecutive keys of one query,
-// which is exactly the B-operand layout of the second product O^T = V^T P^T, so probabilities go
-// from one MFMA to the next without leaving registers, and the row maximum / sum need only two
-// cross-lane steps.  The ancestor bitset of the lane's query sits in a register pair; prefix keys
-// need no mask at all.  K is staged row-major in LDS, V transposed, both with 16-byte global loads.
+// One workgroup (8 wavefronts) owns FOUR query heads of one KV head (256 rows) and one chunk of
+// the keys, so a staged K/V tile feeds four heads' worth of matrix work; wavefront w owns 32 rows
+// (two 16-row tiles) of head w/2.  Scores are produced TRANSPOSED, S^T = K Q^T, with v_mfma_f32_16x16x32: the
+// accumulator then holds, per lane, four consecutive keys of one query, and two such tiles are
+// exactly the eight-key B operand of the second product O^T = V^T P^T (with the matching key
+// permutation applied to the V^T operand), so probabilities go from one MFMA to the next without
+// leaving registers and the row maximum / sum need only two cross-lane steps.  The ancestor bitset
+// of a lane's query sits in a register pair; prefix keys need no mask at all.  K is staged
+// row-major in LDS, V transposed; the global loads of the next 64-key block are issued before the
+// current block is multiplied.  Workgroups that share a KV chunk get consecutive slots on the same
+// XCD (linear id modulo 8), so the chunk is fetched from HBM once and served from that XCD's L2.
 // When the keys are split over several workgroups the partial (O, max, sum) triples are merged by
 // tree_attention_merge_kernel.
 // HBM-bound at the benchmark sizes provided QK^T / PV run on the matrix cores:
@@ -29,35 +33,40 @@
 
 namespace subspec {
 
-constexpr int kAttnThreads = 256;
-constexpr int kAttnRows = 64;          // query rows per workgroup (one q head)
+constexpr int kAttnThreads = 512;
+constexpr int kAttnRows = 64;          // query rows per head
+constexpr int kHeadsPerWG = 4;
 constexpr int kAttnD = 128;
 constexpr int kKeyBlock = 64;
 constexpr int kKStride = kAttnD + 8;   // LDS row stride (elements) of the K tile
 constexpr int kVStride = kKeyBlock + 8;  // LDS row stride (elements) of the transposed V tile
+constexpr int kXcds = 8;
 
-typedef short v4s __attribute__((ext_vector_type(4)));
-typedef _Float16 v4h __attribute__((ext_vector_type(4)));
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 typedef float v4f __attribute__((ext_vector_type(4)));
 
 template <int DT>
-__device__ __forceinline__ v4f mfma16(uint2 a, uint2 b, v4f c) {
+__device__ __forceinline__ v4f mfma32(uint4 a, uint4 b, v4f c) {
   if constexpr (DT == SUBSPEC_BF16) {
-    return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(v4s, a), __builtin_bit_cast(v4s, b), c, 0, 0, 0);
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, a), __builtin_bit_cast(v8bf, b), c, 0, 0, 0);
   } else {
-    return __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(v4h, a), __builtin_bit_cast(v4h, b), c, 0, 0, 0);
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, a), __builtin_bit_cast(v8h, b), c, 0, 0, 0);
   }
 }
 
+typedef __bf16 v2bf_t __attribute__((ext_vector_type(2)));
+typedef _Float16 v2h_t __attribute__((ext_vector_type(2)));
+typedef float v2f_t __attribute__((ext_vector_type(2)));
+
+// two floats -> one packed pair of 16-bit floats (round to nearest even), one conversion instruction
 template <int DT>
 __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+  const v2f_t v = {lo, hi};
   if constexpr (DT == SUBSPEC_BF16) {
-    return (__float_as_uint(round_bf16(lo)) >> 16) | (__float_as_uint(round_bf16(hi)) & 0xffff0000u);
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, v2bf_t));
   } else {
-    union { _Float16 h[2]; uint32_t u; } c;
-    c.h[0] = (_Float16)lo;
-    c.h[1] = (_Float16)hi;
-    return c.u;
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, v2h_t));
   }
 }
 
@@ -65,143 +74,243 @@ struct AttnParams {
   int64_t batch, hq, hkv, n_rows, n_slots, seq_stride, prefix, anc_batch_stride;
   int chunks;
   int64_t chunk_keys;          // multiple of kKeyBlock
+  int pairs_per_kv;            // workgroups (head pairs) per KV head
+  int64_t units;               // batch * hkv * chunks
   float scale_log2;            // softmax scale * log2(e)
 };
 
 template <int DT>
-__global__ __launch_bounds__(kAttnThreads) void tree_attention_kernel(
+__global__ __launch_bounds__(kAttnThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void tree_attention_kernel(
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ kc, const uint16_t* __restrict__ vc,
     const uint64_t* __restrict__ anc, AttnParams ap, uint16_t* __restrict__ out, float* __restrict__ part_o,
     float* __restrict__ part_ml) {
-  __shared__ __attribute__((aligned(16))) uint16_t Ks[kKeyBlock * kKStride];
-  __shared__ __attribute__((aligned(16))) uint16_t Vt[kAttnD * kVStride];
+  // two stages of (K row-major, V transposed): block i+1 is written while block i is multiplied
+  __shared__ __attribute__((aligned(16))) uint16_t Ks2[2][kKeyBlock * kKStride];
+  __shared__ __attribute__((aligned(16))) uint16_t Vt2[2][kAttnD * kVStride];
 
-  const int chunk = blockIdx.x;
-  const int bh = blockIdx.y;                           // b * hq + qh
-  const int b = bh / (int)ap.hq, qh = bh % (int)ap.hq;
-  const int kvh = qh / (int)(ap.hq / ap.hkv);
+  // workgroups of one (batch, kv head, chunk) unit sit in consecutive slots of one XCD
+  const int64_t lin = blockIdx.x;
+  const int xcd = (int)(lin % kXcds);
+  const int64_t slot = lin / kXcds;
+  const int pair = (int)(slot % ap.pairs_per_kv);
+  const int64_t unit = (slot / ap.pairs_per_kv) * kXcds + xcd;
+  if (unit >= ap.units) return;
+  const int chunk = (int)(unit % ap.chunks);
+  const int64_t bkv = unit / ap.chunks;
+  const int kvh = (int)(bkv % ap.hkv), b = (int)(bkv / ap.hkv);
+  const int group = (int)(ap.hq / ap.hkv);
+
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int lq = lane & 15, lg = lane >> 4;            // query column of the lane, lane group
+  const int head_in_group = pair * kHeadsPerWG + (wave >> 1);
+  const bool head_ok = head_in_group < group;
+  const int qh = kvh * group + (head_ok ? head_in_group : 0);
+  const int bh = b * (int)ap.hq + qh;
   const int n = (int)ap.n_rows;
   const int64_t kv_len = ap.prefix + ap.n_slots;
-  const int row = wave * 16 + lq;                      // query row of this lane
-  const bool row_ok = row < n;
 
-  // ---- Q^T operands: Q[row][16*ks + 4*lg .. +3]
-  uint2 qreg[kAttnD / 16];
-  {
-    const uint16_t* qp = q + ((int64_t)bh * n + (row_ok ? row : 0)) * kAttnD;
+  // ---- Q^T operands of the wave's two 16-row tiles: Q[row][32*ks + 8*lg .. +7]
+  int row[2];
+  bool row_ok[2];
+  uint4 qreg[2][kAttnD / 32];
+  uint64_t bits[2];
 #pragma unroll
-    for (int ks = 0; ks < kAttnD / 16; ++ks) {
-      qreg[ks] = row_ok ? *(const uint2*)(qp + ks * 16 + lg * 4) : make_uint2(0, 0);
-    }
+  for (int nt = 0; nt < 2; ++nt) {
+    row[nt] = (wave & 1) * 32 + nt * 16 + lq;
+    row_ok[nt] = head_ok && row[nt] < n;
+    const uint16_t* qp = q + ((int64_t)bh * n + (row_ok[nt] ? row[nt] : 0)) * kAttnD;
+#pragma unroll
+    for (int ks = 0; ks < kAttnD / 32; ++ks)
+      qreg[nt][ks] = row_ok[nt] ? *(const uint4*)(qp + ks * 32 + lg * 8) : make_uint4(0, 0, 0, 0);
+    bits[nt] = row_ok[nt] ? anc[(int64_t)b * ap.anc_batch_stride + row[nt]] : 0ull;
   }
-  const uint64_t bits = row_ok ? anc[(int64_t)b * ap.anc_batch_stride + row] : 0ull;
 
-  v4f oacc[kAttnD / 16];
+  v4f oacc[2][kAttnD / 16];
+  float m_run[2], l_run[2];
 #pragma unroll
-  for (int mt = 0; mt < kAttnD / 16; ++mt) oacc[mt] = v4f{0.f, 0.f, 0.f, 0.f};
-  float m_run = -INFINITY, l_run = 0.f;
+  for (int nt = 0; nt < 2; ++nt) {
+    m_run[nt] = -INFINITY;
+    l_run[nt] = 0.f;
+#pragma unroll
+    for (int mt = 0; mt < kAttnD / 16; ++mt) oacc[nt][mt] = v4f{0.f, 0.f, 0.f, 0.f};
+  }
 
   const uint16_t* kbase = kc + ((int64_t)b * ap.hkv + kvh) * ap.seq_stride * kAttnD;
   const uint16_t* vbase = vc + ((int64_t)b * ap.hkv + kvh) * ap.seq_stride * kAttnD;
   const int64_t key0 = (int64_t)chunk * ap.chunk_keys;
   const int64_t key1 = min(key0 + ap.chunk_keys, kv_len);
 
-  for (int64_t kb = key0; kb < key1; kb += kKeyBlock) {
-    // ---- stage K (row-major) and V (transposed) of this 64-key block
-    __syncthreads();
-#pragma unroll
-    for (int it = 0; it < 4; ++it) {
-      const int key = it * 16 + (tid >> 4), dc = tid & 15;
-      const int64_t pos = min(kb + key, kv_len - 1);
-      const uint4 kv = *(const uint4*)(kbase + pos * kAttnD + dc * 8);
-      *(uint4*)(Ks + key * kKStride + dc * 8) = kv;
-    }
-#pragma unroll
-    for (int it = 0; it < 4; ++it) {
-      const int key = tid & 63, dg = it * 4 + (tid >> 6);
-      const int64_t pos = min(kb + key, kv_len - 1);
-      const uint4 vv = *(const uint4*)(vbase + pos * kAttnD + dg * 8);
-      const uint32_t w[4] = {vv.x, vv.y, vv.z, vv.w};
-#pragma unroll
-      for (int e = 0; e < 8; ++e)
-        Vt[(dg * 8 + e) * kVStride + key] = (uint16_t)((e & 1) ? (w[e >> 1] >> 16) : (w[e >> 1] & 0xffffu));
-    }
-    __syncthreads();
+  // staging registers: this thread's share (2 x 16 bytes of K, 2 x 16 bytes of V) of one 64-key
+  // block; the next block is requested as soon as the current one sits in LDS, so the request
+  // travels while the current block is multiplied.  Plain scalars on purpose: arrays captured by
+  // a lambda end up in memory and every prefetch would be waited for at once.
+  uint4 k0, k1, v0, v1;
+  const int skey = tid >> 4, sdc = tid & 15;           // this thread stages keys skey, skey + 32, d-chunk sdc
+#define SUBSPEC_ATTN_FETCH(KB)                                                                   \
+  do {                                                                                           \
+    const int64_t p0_ = min((KB) + skey, kv_len - 1), p1_ = min((KB) + 32 + skey, kv_len - 1);   \
+    k0 = *(const uint4*)(kbase + p0_ * kAttnD + sdc * 8);                                        \
+    k1 = *(const uint4*)(kbase + p1_ * kAttnD + sdc * 8);                                        \
+    v0 = *(const uint4*)(vbase + p0_ * kAttnD + sdc * 8);                                        \
+    v1 = *(const uint4*)(vbase + p1_ * kAttnD + sdc * 8);                                        \
+  } while (0)
+  // V^T[d][column]: the eight keys one lane needs for a 32-key MFMA step (keys 32j + 4g + r and
+  // 32j + 16 + 4g + r) are stored contiguously (column 32j + 8g + 4h + r for key 32j + 16h + 4g + r),
+  // and the 16-byte column groups are XOR-swizzled with d/8 to spread the banks of the
+  // transposing writes
+  auto vt_column = [&](int key) {
+    const int grp = ((key >> 5) << 2) | ((key >> 2) & 3);                    // 4j + g
+    return ((grp ^ (sdc & 7)) << 3) | (((key >> 4) & 1) << 2) | (key & 3);
+  };
+  const int col0 = vt_column(skey), col1 = vt_column(skey + 32);
+#define SUBSPEC_ATTN_VT(VTW, V, COL)                                                             \
+  do {                                                                                           \
+    uint16_t* p_ = (VTW) + (sdc * 8) * kVStride + (COL);                                         \
+    p_[0 * kVStride] = (uint16_t)((V).x & 0xffffu); p_[1 * kVStride] = (uint16_t)((V).x >> 16);  \
+    p_[2 * kVStride] = (uint16_t)((V).y & 0xffffu); p_[3 * kVStride] = (uint16_t)((V).y >> 16);  \
+    p_[4 * kVStride] = (uint16_t)((V).z & 0xffffu); p_[5 * kVStride] = (uint16_t)((V).z >> 16);  \
+    p_[6 * kVStride] = (uint16_t)((V).w & 0xffffu); p_[7 * kVStride] = (uint16_t)((V).w >> 16);  \
+  } while (0)
+#define SUBSPEC_ATTN_STAGE(BUF)                                                                  \
+  do {                                                                                           \
+    uint16_t* ksw_ = Ks2[BUF];                                                                   \
+    uint16_t* vtw_ = Vt2[BUF];                                                                   \
+    *(uint4*)(ksw_ + skey * kKStride + sdc * 8) = k0;                                            \
+    *(uint4*)(ksw_ + (skey + 32) * kKStride + sdc * 8) = k1;                                     \
+    SUBSPEC_ATTN_VT(vtw_, v0, col0);                                                             \
+    SUBSPEC_ATTN_VT(vtw_, v1, col1);                                                             \
+  } while (0)
 
-    // ---- S^T tiles: 4 x (16 keys x 16 queries); lane holds keys 16*kt + 4*lg + r of query lq
-    float s[4][4];
-    float mloc = -INFINITY;
+  SUBSPEC_ATTN_FETCH(key0);
+  SUBSPEC_ATTN_STAGE(0);
+  if (key0 + kKeyBlock < key1) SUBSPEC_ATTN_FETCH(key0 + kKeyBlock);
+
+  int buf = 0;
+  for (int64_t kb = key0; kb < key1; kb += kKeyBlock, buf ^= 1) {
+    // one barrier per block: stage `buf` is complete, and everyone has left the other stage
+    __syncthreads();
+    if (kb + kKeyBlock < key1) {
+      SUBSPEC_ATTN_STAGE(buf ^ 1);                     // next block -> the stage nobody reads now
+      if (kb + 2 * kKeyBlock < key1) SUBSPEC_ATTN_FETCH(kb + 2 * kKeyBlock);
+    }
+    const uint16_t* Ks = Ks2[buf];
+    const uint16_t* Vt = Vt2[buf];
+
+    // ---- S^T tiles: 4 x (16 keys x 16 queries) per row tile; lane holds keys 16*kt + 4*lg + r of query lq.
+    //      Scores stay unscaled; the softmax scale is folded into the exp2 argument.
+    float s[2][4][4];
+    float mloc[2] = {-INFINITY, -INFINITY};
+    const bool plain = kb + kKeyBlock <= ap.prefix;    // block lies entirely in the prefix: no mask (uniform)
+    v4f acc[4][2];
+#pragma unroll
+    for (int kt = 0; kt < 4; ++kt) acc[kt][0] = acc[kt][1] = v4f{0.f, 0.f, 0.f, 0.f};
+    // eight independent accumulator chains (4 key tiles x 2 row tiles) keep the matrix pipe busy
+#pragma unroll
+    for (int ks = 0; ks < kAttnD / 32; ++ks) {
+#pragma unroll
+      for (int kt = 0; kt < 4; ++kt) {
+        const uint4 a = *(const uint4*)(Ks + (kt * 16 + lq) * kKStride + ks * 32 + lg * 8);
+        acc[kt][0] = mfma32<DT>(a, qreg[0][ks], acc[kt][0]);
+        acc[kt][1] = mfma32<DT>(a, qreg[1][ks], acc[kt][1]);
+      }
+    }
 #pragma unroll
     for (int kt = 0; kt < 4; ++kt) {
-      v4f acc = v4f{0.f, 0.f, 0.f, 0.f};
+      if (plain) {
 #pragma unroll
-      for (int ks = 0; ks < kAttnD / 16; ++ks) {
-        const uint2 a = *(const uint2*)(Ks + (kt * 16 + lq) * kKStride + ks * 16 + lg * 4);
-        acc = mfma16<DT>(a, qreg[ks], acc);
-      }
+        for (int r = 0; r < 4; ++r) {
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int64_t pos = kb + kt * 16 + lg * 4 + r;
-        bool ok = pos < kv_len;
-        if (pos >= ap.prefix) ok = ok && ((bits >> (int)(pos - ap.prefix)) & 1ull);
-        const float t = ok ? acc[r] * ap.scale_log2 : -INFINITY;
-        s[kt][r] = t;
-        mloc = fmaxf(mloc, t);
+          for (int nt = 0; nt < 2; ++nt) {
+            s[nt][kt][r] = acc[kt][nt][r];
+            mloc[nt] = fmaxf(mloc[nt], acc[kt][nt][r]);
+          }
+        }
+      } else {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int64_t pos = kb + kt * 16 + lg * 4 + r;
+          const bool in_range = pos < kv_len;
+          const bool tree = pos >= ap.prefix;
+          const int sh = tree ? (int)(pos - ap.prefix) & 63 : 0;
+#pragma unroll
+          for (int nt = 0; nt < 2; ++nt) {
+            const bool ok = in_range && (!tree || ((bits[nt] >> sh) & 1ull));
+            const float t = ok ? acc[kt][nt][r] : -INFINITY;
+            s[nt][kt][r] = t;
+            mloc[nt] = fmaxf(mloc[nt], t);
+          }
+        }
       }
     }
-    mloc = fmaxf(mloc, __shfl_xor(mloc, 16, kWave));
-    mloc = fmaxf(mloc, __shfl_xor(mloc, 32, kWave));
-    const float m_new = fmaxf(m_run, mloc);
-    const float m_use = m_new == -INFINITY ? 0.f : m_new;
-    const float alpha = __builtin_amdgcn_exp2f(m_run - m_use);      // m_run = -inf -> 0
-    m_run = m_new;
-    l_run *= alpha;
+    // running maximum in units of raw scores (the scale is positive, so the order is the same)
+    float mneg[2];                                     // -max * scale_log2, the additive term of the exp2 argument
 #pragma unroll
-    for (int mt = 0; mt < kAttnD / 16; ++mt) oacc[mt] *= alpha;
-
-    // ---- P^T as B operands, straight from the accumulator layout
-    uint2 pb[4];
+    for (int nt = 0; nt < 2; ++nt) {
+      float mx = mloc[nt];
+      mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+      const float m_new = fmaxf(m_run[nt], mx);
+      const float m_use = m_new == -INFINITY ? 0.f : m_new;
+      const float alpha = __builtin_amdgcn_exp2f((m_run[nt] - m_use) * ap.scale_log2);   // m_run = -inf -> 0
+      m_run[nt] = m_new;
+      mneg[nt] = -m_use * ap.scale_log2;
+      if (__any(alpha != 1.0f)) {                      // the maximum settles after a few blocks
+        l_run[nt] *= alpha;
 #pragma unroll
-    for (int kt = 0; kt < 4; ++kt) {
-      float p[4];
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        p[r] = __builtin_amdgcn_exp2f(s[kt][r] - m_use);
-        l_run += p[r];
+        for (int mt = 0; mt < kAttnD / 16; ++mt) oacc[nt][mt] *= alpha;
       }
-      pb[kt] = make_uint2(pack2<DT>(p[0], p[1]), pack2<DT>(p[2], p[3]));
     }
-    // ---- O^T += V^T P^T : 8 tiles of 16 head-dims
+    // ---- P^T as B operands straight from the accumulators: k index 8*lg + e of step j is key
+    //      32*j + 16*(e/4) + 4*lg + e%4, i.e. registers of score tiles 2j and 2j+1
+    uint4 pb[2][2];
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt) {
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        float p[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          p[e] = __builtin_amdgcn_exp2f(fmaf(s[nt][2 * j + (e >> 2)][e & 3], ap.scale_log2, mneg[nt]));
+          l_run[nt] += p[e];
+        }
+        pb[nt][j] = make_uint4(pack2<DT>(p[0], p[1]), pack2<DT>(p[2], p[3]), pack2<DT>(p[4], p[5]), pack2<DT>(p[6], p[7]));
+      }
+    }
+    // ---- O^T += V^T P^T : 8 tiles of 16 head-dims, two 32-key steps, the same V^T operand for both row tiles
 #pragma unroll
     for (int mt = 0; mt < kAttnD / 16; ++mt) {
 #pragma unroll
-      for (int kt = 0; kt < 4; ++kt) {
-        const uint2 a = *(const uint2*)(Vt + (mt * 16 + lq) * kVStride + kt * 16 + lg * 4);
-        oacc[mt] = mfma16<DT>(a, pb[kt], oacc[mt]);
+      for (int j = 0; j < 2; ++j) {
+        const int d = mt * 16 + lq;
+        const uint4 a = *(const uint4*)(Vt + d * kVStride + (((j * 4 + lg) ^ ((d >> 3) & 7)) << 3));
+        oacc[0][mt] = mfma32<DT>(a, pb[0][j], oacc[0][mt]);
+        oacc[1][mt] = mfma32<DT>(a, pb[1][j], oacc[1][mt]);
       }
     }
   }
-  // the four lane groups hold disjoint keys of the same query
-  l_run += __shfl_xor(l_run, 16, kWave);
-  l_run += __shfl_xor(l_run, 32, kWave);
 
-  if (!row_ok) return;
-  if (ap.chunks == 1) {
-    const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
-    uint16_t* op = out + (((int64_t)b * n + row) * ap.hq + qh) * kAttnD;
 #pragma unroll
-    for (int mt = 0; mt < kAttnD / 16; ++mt) {
-      const uint2 v = make_uint2(pack2<DT>(oacc[mt][0] * inv, oacc[mt][1] * inv), pack2<DT>(oacc[mt][2] * inv, oacc[mt][3] * inv));
-      *(uint2*)(op + mt * 16 + lg * 4) = v;
+  for (int nt = 0; nt < 2; ++nt) {
+    // the four lane groups hold disjoint keys of the same query
+    float l = l_run[nt];
+    l += __shfl_xor(l, 16, kWave);
+    l += __shfl_xor(l, 32, kWave);
+    if (!row_ok[nt]) continue;
+    if (ap.chunks == 1) {
+      const float inv = l > 0.f ? 1.0f / l : 0.f;
+      uint16_t* op = out + (((int64_t)b * n + row[nt]) * ap.hq + qh) * kAttnD;
+#pragma unroll
+      for (int mt = 0; mt < kAttnD / 16; ++mt) {
+        const v4f o = oacc[nt][mt];
+        *(uint2*)(op + mt * 16 + lg * 4) = make_uint2(pack2<DT>(o[0] * inv, o[1] * inv), pack2<DT>(o[2] * inv, o[3] * inv));
+      }
+    } else {
+      const int64_t pslot = ((int64_t)bh * ap.chunks + chunk) * kAttnRows + row[nt];
+      float* po = part_o + pslot * kAttnD;
+#pragma unroll
+      for (int mt = 0; mt < kAttnD / 16; ++mt) *(v4f*)(po + mt * 16 + lg * 4) = oacc[nt][mt];
+      if (lg == 0) { part_ml[pslot * 2] = m_run[nt] * ap.scale_log2; part_ml[pslot * 2 + 1] = l; }
     }
-  } else {
-    const int64_t slot = ((int64_t)bh * ap.chunks + chunk) * kAttnRows + row;
-    float* po = part_o + slot * kAttnD;
-#pragma unroll
-    for (int mt = 0; mt < kAttnD / 16; ++mt) *(v4f*)(po + mt * 16 + lg * 4) = oacc[mt];
-    if (lg == 0) { part_ml[slot * 2] = m_run; part_ml[slot * 2 + 1] = l_run; }
   }
 }
 
@@ -211,16 +320,18 @@ __global__ __launch_bounds__(kAttnD) void tree_attention_merge_kernel(
   const int row = blockIdx.x, bh = blockIdx.y;
   const int b = bh / (int)ap.hq, qh = bh % (int)ap.hq;
   const int d = threadIdx.x;
+  const int64_t slot0 = (int64_t)bh * ap.chunks * kAttnRows + row;     // chunk c: slot0 + c * kAttnRows
   float m = -INFINITY;
-  for (int c = 0; c < ap.chunks; ++c) m = fmaxf(m, part_ml[(((int64_t)bh * ap.chunks + c) * kAttnRows + row) * 2]);
+#pragma unroll 8
+  for (int c = 0; c < ap.chunks; ++c) m = fmaxf(m, part_ml[(slot0 + (int64_t)c * kAttnRows) * 2]);
   float num = 0.f, den = 0.f;
+#pragma unroll 8
   for (int c = 0; c < ap.chunks; ++c) {
-    const int64_t slot = ((int64_t)bh * ap.chunks + c) * kAttnRows + row;
-    const float mc = part_ml[slot * 2];
-    if (mc == -INFINITY) continue;
-    const float w = __builtin_amdgcn_exp2f(mc - m);
-    num = fmaf(w, part_o[slot * kAttnD + d], num);
-    den = fmaf(w, part_ml[slot * 2 + 1], den);
+    const int64_t slot = slot0 + (int64_t)c * kAttnRows;
+    const float mc = part_ml[slot * 2], lc = part_ml[slot * 2 + 1], oc = part_o[slot * kAttnD + d];
+    const float w = mc == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mc - m);
+    num = fmaf(w, oc, num);
+    den = fmaf(w, lc, den);
   }
   const float o = den > 0.f ? num / den : 0.f;
   Elem<DT>::store(out, (((int64_t)b * ap.n_rows + row) * ap.hq + qh) * kAttnD + d, o);
@@ -228,7 +339,8 @@ __global__ __launch_bounds__(kAttnD) void tree_attention_merge_kernel(
 
 static int attn_chunks(int64_t batch, int64_t hq, int64_t kv_len) {
   const int64_t blocks = (kv_len + kKeyBlock - 1) / kKeyBlock;
-  int64_t chunks = std::max<int64_t>(1, 512 / std::max<int64_t>(1, batch * hq));
+  // one workgroup per two query heads; aim at roughly one workgroup per compute unit
+  int64_t chunks = std::max<int64_t>(1, 1024 / std::max<int64_t>(1, batch * hq));
   chunks = std::min<int64_t>(chunks, std::max<int64_t>(1, blocks / 2));   // at least 128 keys per chunk
   return (int)std::min<int64_t>(chunks, 64);
 }
@@ -278,6 +390,9 @@ extern "C" int subspec_tree_attention(const void* q, const void* k_cache, const 
   ap.chunk_keys = (blocks + ap.chunks - 1) / ap.chunks * kKeyBlock;
   ap.chunks = (int)((kv_len + ap.chunk_keys - 1) / ap.chunk_keys);
   ap.scale_log2 = scale * kLog2e;
+  const int group = (int)(n_q_heads / n_kv_heads);
+  ap.pairs_per_kv = (group + kHeadsPerWG - 1) / kHeadsPerWG;
+  ap.units = batch * n_kv_heads * ap.chunks;
   float* part_o = nullptr;
   float* part_ml = nullptr;
   if (ap.chunks > 1) {
@@ -291,7 +406,7 @@ extern "C" int subspec_tree_attention(const void* q, const void* k_cache, const 
     part_ml = (float*)((char*)workspace + align_up(slots * kAttnD * sizeof(float), 256));
   }
   hipStream_t st = (hipStream_t)stream;
-  const dim3 grid(ap.chunks, (unsigned)(batch * n_q_heads));
+  const dim3 grid((unsigned)((ap.units + kXcds - 1) / kXcds * kXcds * ap.pairs_per_kv));
   if (dtype == SUBSPEC_BF16) {
     {
       DominantKernelTimer timer(st);
