@@ -14,6 +14,8 @@ LIB_PATH = os.path.join(LIB_DIR, "libsubspec_hip.so")
 HIPCC_FLAGS = [
     "-O3", "-std=c++17", "-fPIC", "--offload-arch=gfx950", "-ffp-contract=off",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # MFMA results that feed vector ALU work stay in VGPRs instead of bouncing through AGPRs
+    "-mllvm", "-amdgpu-mfma-vgpr-form=1",
     "-Wno-unused-result",
 ]
 

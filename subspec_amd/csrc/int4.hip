@@ -21,9 +21,10 @@
 //   sum_k (q_k - z) s x_k = s * (sum_k (off + q_k) x_k - (z + off) * sum_k x_k)    per group.
 // M = 1   : int4_gemv_kernel, v_dot2_f32 on (weight pair, activation pair); HBM-bound,
 //           algorithmic bytes = N*K/2 + N*(K/64)*4 (+ activations).
-// M = 2-64: int4_gemm_kernel, v_mfma_f32_16x16x16 with the weight tile as A operand; the 16 k of
-//           one MFMA step all come from one quantization group, so the raw accumulator of a
-//           group is scaled once.  Split-K partials are reduced in a fixed order.
+// M = 2-64: int4_gemm_kernel, v_mfma_f32_16x16x32 with the activations as A and the weight tile as
+//           B operand; the 32 k of one MFMA step all come from one quantization group, so the raw
+//           accumulator of a group is scaled once.  The wavefronts of a workgroup split K, their
+//           partial sums and the split-K partials across workgroups are reduced in a fixed order.
 #include "common.h"
 #include <algorithm>
 
@@ -57,8 +58,8 @@ template <int DT> struct I4 {
     return DT == SUBSPEC_BF16 ? bf16_bits_to_float(bits16) : f16_bits_to_float(bits16);
   }
 };
-__device__ __forceinline__ uint32_t code_pair(uint32_t w, int shift, uint32_t magic) {
-  return ((w >> shift) & 0x000f000fu) | magic;
+__device__ __forceinline__ uint32_t code_pair(uint32_t w, int shift, uint32_t magic, uint32_t mask = 0x000f000fu) {
+  return ((w >> shift) & mask) | magic;
 }
 
 // ------------------------------------------------------------------ M = 1
@@ -130,106 +131,172 @@ __global__ __launch_bounds__(kI4Threads) void int4_gemv_kernel(
   }
 }
 
-// ------------------------------------------------------------------ per-group activation sums
+// ------------------------------------------------------------------ 2 <= M <= 64
+// y^T is not formed: the activations are the MFMA A operand (rows m) and the weight tile the B
+// operand (columns n), so a lane's accumulators all belong to ONE weight row n = lane % 16 and its
+// scale / zero is a single word per (tile, group).  v_mfma_f32_16x16x32: one step covers 32 k, the
+// k permutation "step s, lane group c, element e -> k = 16c + 8s + e" is applied to both operands.
+//
+// A workgroup owns up to RT consecutive 16-row weight tiles; its 4 wavefronts split K by GROUP
+// (wavefront w takes groups w, w + 4, ... of the workgroup's K range) and never synchronise until
+// the end: each one loads its activation operands straight from global memory (they stay in L2)
+// and its weight words from HBM, both two groups ahead into two register sets, so every wavefront
+// is an independent software pipeline.  One activation operand feeds RT + 1 MFMAs: one per tile and
+// one against a B operand of ones, which yields the group's activation sums in exactly the
+// accumulator layout the zero-point term needs.  The four partial accumulators are summed through
+// LDS in wavefront order at the end.
+typedef uint32_t i4_u4 __attribute__((ext_vector_type(4)));
+typedef uint32_t i4_u2 __attribute__((ext_vector_type(2)));
+typedef __bf16 i4_v8bf __attribute__((ext_vector_type(8)));
+typedef _Float16 i4_v8h __attribute__((ext_vector_type(8)));
 template <int DT>
-__global__ __launch_bounds__(256) void group_sum_kernel(const uint16_t* __restrict__ x, float* __restrict__ xsum,
-                                                        int64_t K) {
-  const int64_t m = blockIdx.x;
-  const int G = (int)(K / kGroup);
-  for (int g = threadIdx.x; g < G; g += 256) {
-    const uint16_t* p = x + m * K + (int64_t)g * kGroup;
-    float a = 0.f;
-    for (int e = 0; e < kGroup; ++e) a += I4<DT>::to_float(p[e]);
-    xsum[m * G + g] = a;
-  }
+__device__ __forceinline__ i4_v4f i4_mfma32(i4_u4 a, i4_u4 b, i4_v4f c) {
+  if constexpr (DT == SUBSPEC_BF16)
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(i4_v8bf, a), __builtin_bit_cast(i4_v8bf, b), c, 0, 0, 0);
+  else
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(i4_v8h, a), __builtin_bit_cast(i4_v8h, b), c, 0, 0, 0);
 }
 
-// ------------------------------------------------------------------ 2 <= M <= 64
-constexpr int kXStride = kGroup + 8;        // LDS row stride (elements) of one group's activations
-
-template <int DT, int MT>
+template <int DT, int MT, int RT>
 __global__ __launch_bounds__(kI4Threads) void int4_gemm_kernel(
-    const uint16_t* __restrict__ x, const float* __restrict__ xsum, const uint2* __restrict__ wq,
-    const uint32_t* __restrict__ sz, const uint16_t* __restrict__ bias, uint16_t* __restrict__ y,
-    float* __restrict__ partial, int64_t M, int64_t N, int64_t K, int splits, int groups_per_split) {
-  constexpr int GB = 4;                                         // groups staged per barrier
-  __shared__ __attribute__((aligned(16))) uint16_t xt[GB][MT * 16 * kXStride];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int lm = lane & 15, c = lane >> 4;
-  const int G = (int)(K / kGroup);
-  const int64_t nt = (int64_t)blockIdx.x * 4 + wave;
-  const bool tile_ok = nt * 16 < N;
+    const uint16_t* __restrict__ x, const uint2* __restrict__ wq, const uint32_t* __restrict__ sz,
+    const uint16_t* __restrict__ bias, uint16_t* __restrict__ y, float* __restrict__ partial, int M, int64_t N,
+    int K, int splits, int groups_per_split) {
+  __shared__ __attribute__((aligned(16))) float red[4 * MT * 256];   // one accumulator tile set per wavefront
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int ln = lane & 15, c = lane >> 4;
+  const int G = K / kGroup;
+  const int n_tiles = (int)(N / 16);
   const int ks = blockIdx.y;
   const int g_begin = ks * groups_per_split, g_end = min(G, g_begin + groups_per_split);
+  const int g_first = g_begin + wave;                            // this wavefront's groups: g_first + 4j
+  const int nj = g_first < g_end ? (g_end - g_first + 3) / 4 : 0;
 
-  i4_v4f acc[MT];
-#pragma unroll
-  for (int mt = 0; mt < MT; ++mt) acc[mt] = i4_v4f{0.f, 0.f, 0.f, 0.f};
-  const uint2* wrow = wq + (tile_ok ? nt : 0) * G * 64 + lane;
-  const uint32_t* szrow = sz + (tile_ok ? nt : 0) * G * 16 + c * 4;
+  // tiles [tile0, tile0 + ntl) of this workgroup: an even split of all tiles over the grid
+  const int tile0 = (int)((int64_t)blockIdx.x * n_tiles / gridDim.x);
+  const int ntl = (int)((int64_t)(blockIdx.x + 1) * n_tiles / gridDim.x) - tile0;     // 1 .. RT
 
-  for (int g0 = g_begin; g0 < g_end; g0 += GB) {
-    __syncthreads();
-    // stage the activations of GB groups: rows m < M (zero beyond), 64 k each
-    for (int i = tid; i < GB * MT * 16 * 8; i += kI4Threads) {
-      const int gi = i / (MT * 16 * 8), rem = i % (MT * 16 * 8);
-      const int m = rem / 8, part = rem % 8;
-      uint4 v = make_uint4(0, 0, 0, 0);
-      if (m < M && g0 + gi < g_end) v = *(const uint4*)(x + (int64_t)m * K + (int64_t)(g0 + gi) * kGroup + part * 8);
-      *(uint4*)(&xt[gi][m * kXStride + part * 8]) = v;
-    }
-    uint2 wv[GB];
-    uint4 szv[GB];
+  i4_v4f acc[RT][MT];
 #pragma unroll
-    for (int gi = 0; gi < GB; ++gi) {
-      const int g = min(g0 + gi, g_end - 1);
-      wv[gi] = wrow[(int64_t)g * 64];
-      szv[gi] = *(const uint4*)(szrow + (int64_t)g * 16);
-    }
-    __syncthreads();
+  for (int t = 0; t < RT; ++t)
 #pragma unroll
-    for (int gi = 0; gi < GB; ++gi) {
-      const int g = g0 + gi;
-      if (g >= g_end) break;
-      uint2 a[4];
-      a[0] = make_uint2(code_pair(wv[gi].x, 0, I4<DT>::kMagic), code_pair(wv[gi].x, 4, I4<DT>::kMagic));
-      a[1] = make_uint2(code_pair(wv[gi].x, 8, I4<DT>::kMagic), code_pair(wv[gi].x, 12, I4<DT>::kMagic));
-      a[2] = make_uint2(code_pair(wv[gi].y, 0, I4<DT>::kMagic), code_pair(wv[gi].y, 4, I4<DT>::kMagic));
-      a[3] = make_uint2(code_pair(wv[gi].y, 8, I4<DT>::kMagic), code_pair(wv[gi].y, 12, I4<DT>::kMagic));
-      const uint32_t szw[4] = {szv[gi].x, szv[gi].y, szv[gi].z, szv[gi].w};
+    for (int mt = 0; mt < MT; ++mt) acc[t][mt] = i4_v4f{0.f, 0.f, 0.f, 0.f};
+
+  // Loads go through buffer descriptors: the builtin calls keep their place in the program (plain
+  // loads feeding a loop-carried value get merged into one load at the loop head, which would undo
+  // the prefetch distance), uniform address parts ride in the scalar offset, and a request outside
+  // the tensor returns zeros instead of faulting.
+  // A operand of (mt, s): x[m = 16mt + ln][64 g + 16c + 8s .. +7]; rows past M read zeros and only
+  // feed accumulator rows that are never stored.  Requests past the last group re-read it.
+  const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)x, 0, M * K * 2, 0x00027000);
+  const __amdgpu_buffer_rsrc_t w_rsrc =
+      __builtin_amdgcn_make_buffer_rsrc((void*)wq, 0, (int)(n_tiles * (int64_t)G * 512), 0x00027000);
+  const __amdgpu_buffer_rsrc_t sz_rsrc =
+      __builtin_amdgcn_make_buffer_rsrc((void*)sz, 0, (int)(n_tiles * (int64_t)G * 64), 0x00027000);
+  int xoff[MT];                                                  // byte offsets
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) xoff[mt] = ((mt * 16 + ln) * K + c * 16) * 2;
+  int wofs[RT];                                                  // (tile, group 0) in units of groups
+#pragma unroll
+  for (int t = 0; t < RT; ++t) wofs[t] = (tile0 + min(t, ntl - 1)) * G;
+
+  i4_u4 xa[2][MT][2];
+  i4_u2 wbuf[2][RT];
+  uint32_t szbuf[2][RT];
+  // Both constants of ((w >> s) & mask) | magic as run-time values (M >> 30 is zero): with two
+  // literals the compiler emits v_and + v_or, with a scalar and a vector register operand one v_and_or_b32.
+  // (xoff[0] >> 31 is zero too and lives in a vector register.)
+  const uint32_t kmask = 0x000f000fu | (uint32_t)(M >> 30), kmagic = I4<DT>::kMagic | ((uint32_t)xoff[0] >> 31);
+  const uint32_t one2 = DT == SUBSPEC_BF16 ? 0x3f803f80u : 0x3c003c00u;
+  const i4_u4 ones = i4_u4{one2, one2, one2, one2};
+
+#define SUBSPEC_I4_FETCH_X(SLOT, J)                                                                     \
+  {                                                                                                     \
+    const int kc = min(g_first + 4 * (J), G - 1) * (kGroup * 2);                                        \
+    _Pragma("unroll") for (int mt = 0; mt < MT; ++mt) {                                                 \
+      xa[SLOT][mt][0] = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, xoff[mt], kc, 0);                 \
+      xa[SLOT][mt][1] = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, xoff[mt] + 16, kc, 0);            \
+    }                                                                                                   \
+  }
+#define SUBSPEC_I4_FETCH_W(SLOT, J, T)                                                                  \
+  {                                                                                                     \
+    const int g = wofs[T] + min(g_first + 4 * (J), G - 1);                                              \
+    wbuf[SLOT][T] = __builtin_amdgcn_raw_buffer_load_b64(w_rsrc, lane * 8, g * 512, 0);                 \
+    szbuf[SLOT][T] = __builtin_amdgcn_raw_buffer_load_b32(sz_rsrc, ln * 4, g * 64, 0);                  \
+  }
+#define SUBSPEC_I4_STEP(SLOT, J)                                                                        \
+  {                                                                                                     \
+    const bool step_live = (J) < nj;                /* a dead step multiplies by a zero scale: no branch */ \
+    i4_v4f xs[MT];                                  /* sum of the group's activations, rows 16mt + 4c + rr */ \
+    _Pragma("unroll") for (int mt = 0; mt < MT; ++mt) {                                                 \
+      xs[mt] = i4_mfma32<DT>(xa[SLOT][mt][0], ones, i4_v4f{0.f, 0.f, 0.f, 0.f});                        \
+      xs[mt] = i4_mfma32<DT>(xa[SLOT][mt][1], ones, xs[mt]);                                            \
+    }                                                                                                   \
+    _Pragma("unroll") for (int t = 0; t < RT; ++t) {                                                    \
+      const uint32_t w0 = wbuf[SLOT][t].x, w1 = wbuf[SLOT][t].y, szw = szbuf[SLOT][t];                  \
+      const i4_u4 b0 = i4_u4{code_pair(w0, 0, kmagic, kmask), code_pair(w0, 4, kmagic, kmask),        \
+                             code_pair(w0, 8, kmagic, kmask), code_pair(w0, 12, kmagic, kmask)};      \
+      const i4_u4 b1 = i4_u4{code_pair(w1, 0, kmagic, kmask), code_pair(w1, 4, kmagic, kmask),        \
+                             code_pair(w1, 8, kmagic, kmask), code_pair(w1, 12, kmagic, kmask)};      \
+      const float sc = (step_live && t < ntl) ? f16_bits_to_float(szw & 0xffffu) : 0.f;                 \
+      const float szo = -sc * (f16_bits_to_float(szw >> 16) + I4<DT>::kOffset);                         \
+      SUBSPEC_I4_FETCH_W(SLOT, (J) + 2, t);                                                             \
+      _Pragma("unroll") for (int mt = 0; mt < MT; ++mt) {                                               \
+        i4_v4f raw = i4_mfma32<DT>(xa[SLOT][mt][0], b0, i4_v4f{0.f, 0.f, 0.f, 0.f});                    \
+        raw = i4_mfma32<DT>(xa[SLOT][mt][1], b1, raw);                                                  \
+        _Pragma("unroll") for (int rr = 0; rr < 4; ++rr)                                                \
+          acc[t][mt][rr] = fmaf(sc, raw[rr], fmaf(szo, xs[mt][rr], acc[t][mt][rr]));                    \
+      }                                                                                                 \
+    }                                                                                                   \
+    __builtin_amdgcn_sched_barrier(0);              /* keep the refill here: one full step ahead of its use */ \
+    SUBSPEC_I4_FETCH_X(SLOT, (J) + 2);                                                                  \
+    __builtin_amdgcn_sched_barrier(0);                                                                  \
+  }
+
+  SUBSPEC_I4_FETCH_X(0, 0);
+#pragma unroll
+  for (int t = 0; t < RT; ++t) SUBSPEC_I4_FETCH_W(0, 0, t);
+  SUBSPEC_I4_FETCH_X(1, 1);
+#pragma unroll
+  for (int t = 0; t < RT; ++t) SUBSPEC_I4_FETCH_W(1, 1, t);
+  for (int j = 0; j < nj; j += 2) {
+    SUBSPEC_I4_STEP(0, j);
+    SUBSPEC_I4_STEP(1, j + 1);
+  }
+#undef SUBSPEC_I4_FETCH_X
+#undef SUBSPEC_I4_FETCH_W
+#undef SUBSPEC_I4_STEP
+
+  // ---- sum the four wavefronts' partial accumulators in wavefront order; wavefront t % 4 finishes tile t.
+  // accumulator layout: rows m = 16*mt + 4*c + rr, column n = 16*tile + ln
+#pragma unroll
+  for (int t = 0; t < RT; ++t) {
+    if (t >= ntl) break;                                         // uniform
+    if (t > 0) __syncthreads();                                  // the previous round has been read
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) *(i4_v4f*)(&red[((wave * MT + mt) * 64 + lane) * 4]) = acc[t][mt];
+    __syncthreads();
+    if (wave == (t & 3)) {
+      const int64_t n = (int64_t)(tile0 + t) * 16 + ln;
+      const float bv = (splits == 1 && bias) ? I4<DT>::to_float(bias[n]) : 0.f;
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) {
-        i4_v4f raw = i4_v4f{0.f, 0.f, 0.f, 0.f};
+        i4_v4f v = *(const i4_v4f*)(&red[((0 * MT + mt) * 64 + lane) * 4]);
 #pragma unroll
-        for (int s = 0; s < 4; ++s) {
-          const uint2 b = *(const uint2*)(&xt[gi][(mt * 16 + lm) * kXStride + c * 16 + s * 4]);
-          raw = I4<DT>::mfma(a[s], b, raw);
+        for (int w = 1; w < 4; ++w) {
+          const i4_v4f o = *(const i4_v4f*)(&red[((w * MT + mt) * 64 + lane) * 4]);
+#pragma unroll
+          for (int rr = 0; rr < 4; ++rr) v[rr] += o[rr];
         }
-        const int m = mt * 16 + lm;
-        const float xs = m < M ? xsum[(int64_t)m * G + g] : 0.f;
 #pragma unroll
         for (int rr = 0; rr < 4; ++rr) {
-          const float s = f16_bits_to_float(szw[rr] & 0xffffu), z = f16_bits_to_float(szw[rr] >> 16);
-          acc[mt][rr] = fmaf(s, raw[rr] - (z + I4<DT>::kOffset) * xs, acc[mt][rr]);
+          const int m = mt * 16 + c * 4 + rr;
+          if (m >= M) continue;
+          if (splits == 1) Elem<DT>::store(y, (int64_t)m * N + n, v[rr] + bv);
+          else partial[((int64_t)ks * M + m) * N + n] = v[rr];
         }
       }
-    }
-  }
-  if (!tile_ok) return;
-  // accumulator layout: rows n = 16*nt + 4*c + rr, column m = 16*mt + lm
-#pragma unroll
-  for (int mt = 0; mt < MT; ++mt) {
-    const int m = mt * 16 + lm;
-    if (m >= M) continue;
-    const int64_t n0 = nt * 16 + c * 4;
-    if (splits == 1) {
-      float v[4];
-#pragma unroll
-      for (int rr = 0; rr < 4; ++rr) v[rr] = acc[mt][rr] + (bias ? I4<DT>::to_float(bias[n0 + rr]) : 0.f);
-#pragma unroll
-      for (int rr = 0; rr < 4; ++rr) Elem<DT>::store(y, (int64_t)m * N + n0 + rr, v[rr]);
-    } else {
-      *(i4_v4f*)(partial + ((int64_t)ks * M + m) * N + n0) = acc[mt];
     }
   }
 }
@@ -246,19 +313,25 @@ __global__ __launch_bounds__(256) void int4_reduce_kernel(const float* __restric
   Elem<DT>::store(y, i, v);
 }
 
-struct I4Plan { int splits, groups_per_split; };
-
+struct I4Plan { int wgs, row_tiles, splits, groups_per_split; };
+constexpr int kI4MaxRowTiles = 5;
+static int i4_row_tile_variant(int64_t need) { return need <= 1 ? 1 : need <= 2 ? 2 : need <= 3 ? 3 : kI4MaxRowTiles; }
+// Resident workgroups the launch is balanced for (register use allows 2 per SIMD row for M > 32).
+static int i4_slots(int64_t M) { return M > 32 ? 512 : 1024; }
 static I4Plan i4_plan(int64_t M, int64_t N, int64_t K) {
-  (void)M;
   const int G = (int)(K / kGroup);
-  const int64_t wgs = (N + 63) / 64;
-  int splits = (int)std::max<int64_t>(1, (384 + wgs - 1) / wgs);
-  splits = std::min(splits, std::max(1, G / 8));              // at least 8 groups (512 k) per split
+  const int64_t tiles = N / 16, slots = i4_slots(M);
+  // row tiles per workgroup: the smallest compiled variant that covers all tiles in one resident wave of
+  // workgroups; the grid then splits the tiles evenly, so every workgroup has row_tiles or row_tiles - 1
+  const int row_tiles = i4_row_tile_variant((tiles + slots - 1) / slots);
+  const int64_t wgs = (tiles + row_tiles - 1) / row_tiles;
+  int splits = (int)std::max<int64_t>(1, slots / wgs);
+  splits = std::min(splits, std::max(1, G / 16));             // at least 16 groups (4 per wavefront) per split
   splits = std::min(splits, 32);
   int gps = (G + splits - 1) / splits;
   gps = (gps + 3) / 4 * 4;
   splits = (G + gps - 1) / gps;
-  return I4Plan{splits, gps};
+  return I4Plan{(int)wgs, row_tiles, splits, gps};
 }
 
 template <int DT>
@@ -271,20 +344,26 @@ static int run_int4(const void* x, const uint32_t* wq, const uint32_t* sz, const
                        (const uint2*)wq, sz, (const uint16_t*)bias, (uint16_t*)y, N, K);
   } else {
     const I4Plan pl = i4_plan(M, N, K);
-    float* xsum = (float*)workspace;
-    float* partial = (float*)((char*)workspace + align_up((size_t)M * (K / kGroup) * sizeof(float), 256));
-    hipLaunchKernelGGL((group_sum_kernel<DT>), dim3((unsigned)M), dim3(256), 0, st, (const uint16_t*)x, xsum, K);
-    const dim3 grid((unsigned)((N + 63) / 64), (unsigned)pl.splits);
-#define SUBSPEC_I4_LAUNCH(MT)                                                                                      \
-  hipLaunchKernelGGL((int4_gemm_kernel<DT, MT>), grid, dim3(kI4Threads), 0, st, (const uint16_t*)x, xsum,           \
-                     (const uint2*)wq, sz, (const uint16_t*)bias, (uint16_t*)y, partial, M, N, K, pl.splits,        \
-                     pl.groups_per_split)
+    float* partial = (float*)workspace;
+    const dim3 grid((unsigned)pl.wgs, (unsigned)pl.splits);
+#define SUBSPEC_I4_LAUNCH(MT, RT)                                                                                  \
+  hipLaunchKernelGGL((int4_gemm_kernel<DT, MT, RT>), grid, dim3(kI4Threads), 0, st, (const uint16_t*)x,            \
+                     (const uint2*)wq, sz, (const uint16_t*)bias, (uint16_t*)y, partial, (int)M, N, (int)K,        \
+                     pl.splits, pl.groups_per_split)
+#define SUBSPEC_I4_LAUNCH_MT(MT)                                                                                   \
+  do {                                                                                                             \
+    if (pl.row_tiles == 1) SUBSPEC_I4_LAUNCH(MT, 1);                                                               \
+    else if (pl.row_tiles == 2) SUBSPEC_I4_LAUNCH(MT, 2);                                                          \
+    else if (pl.row_tiles == 3) SUBSPEC_I4_LAUNCH(MT, 3);                                                          \
+    else SUBSPEC_I4_LAUNCH(MT, kI4MaxRowTiles);                                                                    \
+  } while (0)
     {
       DominantKernelTimer timer(st);
-      if (M <= 16) SUBSPEC_I4_LAUNCH(1);
-      else if (M <= 32) SUBSPEC_I4_LAUNCH(2);
-      else SUBSPEC_I4_LAUNCH(4);
+      if (M <= 16) SUBSPEC_I4_LAUNCH_MT(1);
+      else if (M <= 32) SUBSPEC_I4_LAUNCH_MT(2);
+      else SUBSPEC_I4_LAUNCH_MT(4);
     }
+#undef SUBSPEC_I4_LAUNCH_MT
 #undef SUBSPEC_I4_LAUNCH
     if (pl.splits > 1)
       hipLaunchKernelGGL((int4_reduce_kernel<DT>), dim3((unsigned)((M * N + 255) / 256)), dim3(256), 0, st, partial,
@@ -301,8 +380,7 @@ using namespace subspec;
 extern "C" size_t subspec_int4_linear_workspace(int64_t M, int64_t N, int64_t K) {
   if (M <= 1 || N <= 0 || K <= 0) return 256;
   const I4Plan pl = i4_plan(M, N, K);
-  return align_up((size_t)M * (K / kGroup) * sizeof(float), 256) +
-         (pl.splits > 1 ? align_up((size_t)pl.splits * M * N * sizeof(float), 256) : 0) + 256;
+  return (pl.splits > 1 ? align_up((size_t)pl.splits * M * N * sizeof(float), 256) : 0) + 256;
 }
 
 extern "C" int subspec_int4_linear(const void* x, const uint32_t* wq, const uint32_t* sz, const void* bias, void* y,
@@ -317,6 +395,8 @@ extern "C" int subspec_int4_linear(const void* x, const uint32_t* wq, const uint
                  (long long)M, (long long)N, (long long)K);
   if (M > 64) SUBSPEC_FAIL(SUBSPEC_ERR_LIMIT, "int4_linear: M=%lld exceeds the 64-row limit (tree width)", (long long)M);
   if (K > 65536) SUBSPEC_FAIL(SUBSPEC_ERR_LIMIT, "int4_linear: K=%lld too large", (long long)K);
+  if (N * K / 2 >= ((int64_t)1 << 31))
+    SUBSPEC_FAIL(SUBSPEC_ERR_LIMIT, "int4_linear: N*K/2=%lld bytes of codes exceed the 2 GiB descriptor range", (long long)(N * K / 2));
   if ((uintptr_t)x % 16 || (uintptr_t)wq % 16 || (uintptr_t)sz % 16 || (uintptr_t)y % 8)
     SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "int4_linear: x / wq / sz must be 16-byte aligned, y 8-byte aligned");
   if (M > 1) {
