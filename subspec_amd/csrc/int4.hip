@@ -139,12 +139,13 @@ __global__ __launch_bounds__(kI4Threads) void int4_gemv_kernel(
 //
 // A workgroup owns up to RT consecutive 16-row weight tiles; its 4 wavefronts split K by GROUP
 // (wavefront w takes groups w, w + 4, ... of the workgroup's K range) and never synchronise until
-// the end: each one loads its activation operands straight from global memory (they stay in L2)
-// and its weight words from HBM, both two groups ahead into two register sets, so every wavefront
-// is an independent software pipeline.  One activation operand feeds RT + 1 MFMAs: one per tile and
+// the end: each one fetches its activation block (L2-resident) through a private LDS stage and its
+// weight words from HBM two groups ahead into two register sets, so every wavefront is an
+// independent software pipeline.  One activation operand feeds RT + 1 MFMAs: one per tile and
 // one against a B operand of ones, which yields the group's activation sums in exactly the
 // accumulator layout the zero-point term needs.  The four partial accumulators are summed through
 // LDS in wavefront order at the end.
+constexpr int kXlStride = kGroup + 8;                          // LDS row stride (elements) of a parked activation block
 typedef uint32_t i4_u4 __attribute__((ext_vector_type(4)));
 typedef uint32_t i4_u2 __attribute__((ext_vector_type(2)));
 typedef __bf16 i4_v8bf __attribute__((ext_vector_type(8)));
@@ -162,7 +163,12 @@ __global__ __launch_bounds__(kI4Threads) void int4_gemm_kernel(
     const uint16_t* __restrict__ x, const uint2* __restrict__ wq, const uint32_t* __restrict__ sz,
     const uint16_t* __restrict__ bias, uint16_t* __restrict__ y, float* __restrict__ partial, int M, int64_t N,
     int K, int splits, int groups_per_split) {
-  __shared__ __attribute__((aligned(16))) float red[4 * MT * 256];   // one accumulator tile set per wavefront
+  // 4 wavefronts x 2 stages of a [16*MT][64] activation block; reused for the final reduction
+  // (two rounds of one accumulator tile set per wavefront)
+  constexpr int kStageBytes = 4 * 2 * MT * 16 * kXlStride * 2, kRedBytes = 2 * 4 * MT * 256 * 4;
+  __shared__ __attribute__((aligned(16))) unsigned char lds_raw[kStageBytes > kRedBytes ? kStageBytes : kRedBytes];
+  uint16_t* const xstage = (uint16_t*)lds_raw;
+  float* const red = (float*)lds_raw;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int ln = lane & 15, c = lane >> 4;
@@ -187,115 +193,139 @@ __global__ __launch_bounds__(kI4Threads) void int4_gemm_kernel(
   // loads feeding a loop-carried value get merged into one load at the loop head, which would undo
   // the prefetch distance), uniform address parts ride in the scalar offset, and a request outside
   // the tensor returns zeros instead of faulting.
-  // A operand of (mt, s): x[m = 16mt + ln][64 g + 16c + 8s .. +7]; rows past M read zeros and only
-  // feed accumulator rows that are never stored.  Requests past the last group re-read it.
+  //
+  // Activations: an MFMA operand wants lane (ln, c) to hold row ln, which no coalesced load can
+  // deliver (adjacent lanes would sit a whole row apart).  Each wavefront therefore fetches its
+  // group's [16*MT rows][64 k] block with 8 lanes per 128-byte row segment, parks it in a
+  // wavefront-private LDS stage (row stride 144 bytes: conflict-free 16-byte reads) and reads the
+  // operands back from there.  No other wavefront touches the stage, so no barrier is involved.
+  // Rows past M read zeros and only feed accumulator rows that are never stored; requests past
+  // the last group re-read it and meet a zero scale.
   const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)x, 0, M * K * 2, 0x00027000);
   const __amdgpu_buffer_rsrc_t w_rsrc =
       __builtin_amdgcn_make_buffer_rsrc((void*)wq, 0, (int)(n_tiles * (int64_t)G * 512), 0x00027000);
   const __amdgpu_buffer_rsrc_t sz_rsrc =
       __builtin_amdgcn_make_buffer_rsrc((void*)sz, 0, (int)(n_tiles * (int64_t)G * 64), 0x00027000);
-  int xoff[MT];                                                  // byte offsets
-#pragma unroll
-  for (int mt = 0; mt < MT; ++mt) xoff[mt] = ((mt * 16 + ln) * K + c * 16) * 2;
+  constexpr int kXg = MT * 2;                                    // 16-byte pieces per lane of one group block
+  const int xg_off = ((lane >> 3) * K + (lane & 7) * 8) * 2;     // byte offset of piece 0; piece i is 8 rows further
+  uint16_t* const xl = xstage + wave * (2 * MT * 16 * kXlStride);  // this wavefront's two stages
+  const int xl_write = (lane >> 3) * kXlStride + (lane & 7) * 8;
+  const int xl_read = ln * kXlStride + c * 16;
   int wofs[RT];                                                  // (tile, group 0) in units of groups
 #pragma unroll
   for (int t = 0; t < RT; ++t) wofs[t] = (tile0 + min(t, ntl - 1)) * G;
 
-  i4_u4 xa[2][MT][2];
+  i4_u4 xg[kXg];                                                 // block on its way from global memory to LDS
   i4_u2 wbuf[2][RT];
   uint32_t szbuf[2][RT];
   // Both constants of ((w >> s) & mask) | magic as run-time values (M >> 30 is zero): with two
   // literals the compiler emits v_and + v_or, with a scalar and a vector register operand one v_and_or_b32.
-  // (xoff[0] >> 31 is zero too and lives in a vector register.)
-  const uint32_t kmask = 0x000f000fu | (uint32_t)(M >> 30), kmagic = I4<DT>::kMagic | ((uint32_t)xoff[0] >> 31);
+  // (xg_off >> 31 is zero too and lives in a vector register.)
+  const uint32_t kmask = 0x000f000fu | (uint32_t)(M >> 30), kmagic = I4<DT>::kMagic | ((uint32_t)xg_off >> 31);
   const uint32_t one2 = DT == SUBSPEC_BF16 ? 0x3f803f80u : 0x3c003c00u;
   const i4_u4 ones = i4_u4{one2, one2, one2, one2};
 
-#define SUBSPEC_I4_FETCH_X(SLOT, J)                                                                     \
+#define SUBSPEC_I4_FETCH_X(J)                                                                           \
   {                                                                                                     \
     const int kc = min(g_first + 4 * (J), G - 1) * (kGroup * 2);                                        \
-    _Pragma("unroll") for (int mt = 0; mt < MT; ++mt) {                                                 \
-      xa[SLOT][mt][0] = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, xoff[mt], kc, 0);                 \
-      xa[SLOT][mt][1] = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, xoff[mt] + 16, kc, 0);            \
-    }                                                                                                   \
+    _Pragma("unroll") for (int i = 0; i < kXg; ++i)                                                     \
+      xg[i] = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, xg_off + i * 16 * K, kc, 0);                \
   }
+#define SUBSPEC_I4_PARK_X(SLOT)                                                                         \
+  _Pragma("unroll") for (int i = 0; i < kXg; ++i)                                                       \
+    *(i4_u4*)(&xl[(SLOT) * (MT * 16 * kXlStride) + i * 8 * kXlStride + xl_write]) = xg[i];
 #define SUBSPEC_I4_FETCH_W(SLOT, J, T)                                                                  \
   {                                                                                                     \
     const int g = wofs[T] + min(g_first + 4 * (J), G - 1);                                              \
     wbuf[SLOT][T] = __builtin_amdgcn_raw_buffer_load_b64(w_rsrc, lane * 8, g * 512, 0);                 \
     szbuf[SLOT][T] = __builtin_amdgcn_raw_buffer_load_b32(sz_rsrc, ln * 4, g * 64, 0);                  \
   }
+  // Step J works on LDS stage SLOT = J & 1.  Once its operands are in registers the stage is free:
+  // the block of group J + 2 (requested one step ago) is parked there and group J + 3 requested.
 #define SUBSPEC_I4_STEP(SLOT, J)                                                                        \
   {                                                                                                     \
     const bool step_live = (J) < nj;                /* a dead step multiplies by a zero scale: no branch */ \
+    i4_u4 xa[MT][2];                                                                                    \
+    _Pragma("unroll") for (int mt = 0; mt < MT; ++mt) {                                                 \
+      const uint16_t* xr = &xl[(SLOT) * (MT * 16 * kXlStride) + mt * 16 * kXlStride + xl_read];         \
+      xa[mt][0] = *(const i4_u4*)xr;                                                                    \
+      xa[mt][1] = *(const i4_u4*)(xr + 8);                                                              \
+    }                                                                                                   \
+    SUBSPEC_I4_PARK_X(SLOT);                                                                            \
+    SUBSPEC_I4_FETCH_X((J) + 3);                                                                        \
+    __builtin_amdgcn_sched_barrier(0);              /* keep the requests here: a full step ahead of their use */ \
     i4_v4f xs[MT];                                  /* sum of the group's activations, rows 16mt + 4c + rr */ \
     _Pragma("unroll") for (int mt = 0; mt < MT; ++mt) {                                                 \
-      xs[mt] = i4_mfma32<DT>(xa[SLOT][mt][0], ones, i4_v4f{0.f, 0.f, 0.f, 0.f});                        \
-      xs[mt] = i4_mfma32<DT>(xa[SLOT][mt][1], ones, xs[mt]);                                            \
+      xs[mt] = i4_mfma32<DT>(xa[mt][0], ones, i4_v4f{0.f, 0.f, 0.f, 0.f});                              \
+      xs[mt] = i4_mfma32<DT>(xa[mt][1], ones, xs[mt]);                                                  \
     }                                                                                                   \
     _Pragma("unroll") for (int t = 0; t < RT; ++t) {                                                    \
       const uint32_t w0 = wbuf[SLOT][t].x, w1 = wbuf[SLOT][t].y, szw = szbuf[SLOT][t];                  \
-      const i4_u4 b0 = i4_u4{code_pair(w0, 0, kmagic, kmask), code_pair(w0, 4, kmagic, kmask),        \
-                             code_pair(w0, 8, kmagic, kmask), code_pair(w0, 12, kmagic, kmask)};      \
-      const i4_u4 b1 = i4_u4{code_pair(w1, 0, kmagic, kmask), code_pair(w1, 4, kmagic, kmask),        \
-                             code_pair(w1, 8, kmagic, kmask), code_pair(w1, 12, kmagic, kmask)};      \
+      const i4_u4 b0 = i4_u4{code_pair(w0, 0, kmagic, kmask), code_pair(w0, 4, kmagic, kmask),          \
+                             code_pair(w0, 8, kmagic, kmask), code_pair(w0, 12, kmagic, kmask)};        \
+      const i4_u4 b1 = i4_u4{code_pair(w1, 0, kmagic, kmask), code_pair(w1, 4, kmagic, kmask),          \
+                             code_pair(w1, 8, kmagic, kmask), code_pair(w1, 12, kmagic, kmask)};        \
       const float sc = (step_live && t < ntl) ? f16_bits_to_float(szw & 0xffffu) : 0.f;                 \
       const float szo = -sc * (f16_bits_to_float(szw >> 16) + I4<DT>::kOffset);                         \
       SUBSPEC_I4_FETCH_W(SLOT, (J) + 2, t);                                                             \
       _Pragma("unroll") for (int mt = 0; mt < MT; ++mt) {                                               \
-        i4_v4f raw = i4_mfma32<DT>(xa[SLOT][mt][0], b0, i4_v4f{0.f, 0.f, 0.f, 0.f});                    \
-        raw = i4_mfma32<DT>(xa[SLOT][mt][1], b1, raw);                                                  \
+        i4_v4f raw = i4_mfma32<DT>(xa[mt][0], b0, i4_v4f{0.f, 0.f, 0.f, 0.f});                          \
+        raw = i4_mfma32<DT>(xa[mt][1], b1, raw);                                                        \
         _Pragma("unroll") for (int rr = 0; rr < 4; ++rr)                                                \
           acc[t][mt][rr] = fmaf(sc, raw[rr], fmaf(szo, xs[mt][rr], acc[t][mt][rr]));                    \
       }                                                                                                 \
     }                                                                                                   \
-    __builtin_amdgcn_sched_barrier(0);              /* keep the refill here: one full step ahead of its use */ \
-    SUBSPEC_I4_FETCH_X(SLOT, (J) + 2);                                                                  \
     __builtin_amdgcn_sched_barrier(0);                                                                  \
   }
 
-  SUBSPEC_I4_FETCH_X(0, 0);
+  SUBSPEC_I4_FETCH_X(0);
 #pragma unroll
   for (int t = 0; t < RT; ++t) SUBSPEC_I4_FETCH_W(0, 0, t);
-  SUBSPEC_I4_FETCH_X(1, 1);
+  SUBSPEC_I4_PARK_X(0);
+  SUBSPEC_I4_FETCH_X(1);
 #pragma unroll
   for (int t = 0; t < RT; ++t) SUBSPEC_I4_FETCH_W(1, 1, t);
+  SUBSPEC_I4_PARK_X(1);
+  SUBSPEC_I4_FETCH_X(2);
   for (int j = 0; j < nj; j += 2) {
     SUBSPEC_I4_STEP(0, j);
     SUBSPEC_I4_STEP(1, j + 1);
   }
+  __syncthreads();                                               // the stages are reused for the reduction below
+#undef SUBSPEC_I4_PARK_X
 #undef SUBSPEC_I4_FETCH_X
 #undef SUBSPEC_I4_FETCH_W
 #undef SUBSPEC_I4_STEP
 
-  // ---- sum the four wavefronts' partial accumulators in wavefront order; wavefront t % 4 finishes tile t.
+  // ---- sum the four wavefronts' partial accumulators in wavefront order (0, 1, 2, 3), one tile per
+  // round.  LDS holds two rounds, so a round needs one barrier; wavefront w finishes the activation
+  // row blocks mt = w, w + 4, ... of the tile, so the sums and stores are spread over the workgroup.
   // accumulator layout: rows m = 16*mt + 4*c + rr, column n = 16*tile + ln
 #pragma unroll
   for (int t = 0; t < RT; ++t) {
     if (t >= ntl) break;                                         // uniform
-    if (t > 0) __syncthreads();                                  // the previous round has been read
+    float* stage = red + (t & 1) * (4 * MT * 256);
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) *(i4_v4f*)(&red[((wave * MT + mt) * 64 + lane) * 4]) = acc[t][mt];
-    __syncthreads();
-    if (wave == (t & 3)) {
-      const int64_t n = (int64_t)(tile0 + t) * 16 + ln;
-      const float bv = (splits == 1 && bias) ? I4<DT>::to_float(bias[n]) : 0.f;
+    for (int mt = 0; mt < MT; ++mt) *(i4_v4f*)(&stage[((wave * MT + mt) * 64 + lane) * 4]) = acc[t][mt];
+    __syncthreads();                                             // round t written; round t - 1 fully read
+    const int64_t n = (int64_t)(tile0 + t) * 16 + ln;
+    const float bv = (splits == 1 && bias) ? I4<DT>::to_float(bias[n]) : 0.f;
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) {
-        i4_v4f v = *(const i4_v4f*)(&red[((0 * MT + mt) * 64 + lane) * 4]);
+    for (int mt = 0; mt < MT; ++mt) {
+      if ((mt & 3) != wave) continue;                            // uniform
+      i4_v4f v = *(const i4_v4f*)(&stage[((0 * MT + mt) * 64 + lane) * 4]);
 #pragma unroll
-        for (int w = 1; w < 4; ++w) {
-          const i4_v4f o = *(const i4_v4f*)(&red[((w * MT + mt) * 64 + lane) * 4]);
+      for (int w = 1; w < 4; ++w) {
+        const i4_v4f o = *(const i4_v4f*)(&stage[((w * MT + mt) * 64 + lane) * 4]);
 #pragma unroll
-          for (int rr = 0; rr < 4; ++rr) v[rr] += o[rr];
-        }
+        for (int rr = 0; rr < 4; ++rr) v[rr] += o[rr];
+      }
 #pragma unroll
-        for (int rr = 0; rr < 4; ++rr) {
-          const int m = mt * 16 + c * 4 + rr;
-          if (m >= M) continue;
-          if (splits == 1) Elem<DT>::store(y, (int64_t)m * N + n, v[rr] + bv);
-          else partial[((int64_t)ks * M + m) * N + n] = v[rr];
-        }
+      for (int rr = 0; rr < 4; ++rr) {
+        const int m = mt * 16 + c * 4 + rr;
+        if (m >= M) continue;
+        if (splits == 1) Elem<DT>::store(y, (int64_t)m * N + n, v[rr] + bv);
+        else partial[((int64_t)ks * M + m) * N + n] = v[rr];
       }
     }
   }
@@ -325,7 +355,7 @@ static I4Plan i4_plan(int64_t M, int64_t N, int64_t K) {
   // workgroups; the grid then splits the tiles evenly, so every workgroup has row_tiles or row_tiles - 1
   const int row_tiles = i4_row_tile_variant((tiles + slots - 1) / slots);
   const int64_t wgs = (tiles + row_tiles - 1) / row_tiles;
-  int splits = (int)std::max<int64_t>(1, slots / wgs);
+  int splits = (int)std::max<int64_t>(1, (slots + wgs / 2) / wgs);
   splits = std::min(splits, std::max(1, G / 16));             // at least 16 groups (4 per wavefront) per split
   splits = std::min(splits, 32);
   int gps = (G + splits - 1) / splits;
