@@ -16,6 +16,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+MFMA_BF16_PEAK_TFLOPS = 2500.0
 # HBM bytes per launch at the default workload, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs scaled
 # by a copy of known size (profiles/verify_cycle_config2_hbm_counters.md); None for other sizes.
 MEASURED_TRAFFIC = {
@@ -45,8 +46,11 @@ def parse():
 
 
 def _time_us(fn, steps, warmup):
-    """Average duration of fn() in microseconds, events on the launch stream."""
+    """(entry-point latency, dominant-kernel duration) of fn() in microseconds; events on the launch
+    stream, the kernel duration from the library's event pair around its dominant kernel."""
     import torch
+    from subspec_amd import _lib as L
+    lib = L.lib()
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
@@ -56,17 +60,32 @@ def _time_us(fn, steps, warmup):
         fn()
     e1.record()
     torch.cuda.synchronize()
-    return 1e3 * e0.elapsed_time(e1) / steps
+    call_us = 1e3 * e0.elapsed_time(e1) / steps
+    lib.subspec_profile_enable(1)
+    for _ in range(min(steps, 64)):
+        fn()
+    torch.cuda.synchronize()
+    lib.subspec_profile_enable(0)
+    kern = sorted(lib.subspec_profile_read_ms(i) for i in range(lib.subspec_profile_count()))
+    kernel_us = 1e3 * kern[len(kern) // 2] if kern else call_us
+    return call_us, kernel_us
 
 
-def _kernel_line(name, workload, us, nbytes, flops=None, extra=None):
-    gbs = nbytes / (us * 1e-6) / 1e9
-    line = {"metric": name, "value": round(us, 2), "unit": "us", "n_gpus": 1, "higher_is_better": False,
-            "data": "synthetic", "config": dict({"workload": workload}, **(extra or {})),
-            "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                         "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None, "bytes_per_launch": nbytes}}
-    if flops:
-        line["tflops"] = round(flops / (us * 1e-6) / 1e12, 2)
+def _kernel_line(name, workload, call_us, kernel_us, nbytes, flops, kernel, bound="hbm", extra=None):
+    """One JSON line for a kernel family; `roofline` prices the dominant kernel against the bound named."""
+    gbs = nbytes / (kernel_us * 1e-6) / 1e9
+    tfl = flops / (kernel_us * 1e-6) / 1e12
+    if bound == "hbm":
+        roof = {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None}
+    else:
+        roof = {"bound": "mfma", "achieved": round(tfl, 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                "frac": round(tfl / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None}
+    roof.update(kernel=kernel, kernel_us=round(kernel_us, 2), bytes_per_launch=nbytes, flops_per_launch=flops,
+                hbm_frac=round(gbs / HBM_PEAK_GBS, 4), mfma_frac=round(tfl / MFMA_BF16_PEAK_TFLOPS, 4))
+    line = {"metric": name, "value": round(call_us, 2), "unit": "us", "n_gpus": 1, "higher_is_better": False,
+            "data": "synthetic", "dtype": "bf16", "config": dict({"workload": workload}, **(extra or {})),
+            "roofline": roof}
     print(json.dumps(line), flush=True)
 
 
@@ -83,10 +102,12 @@ def bench_attention(args):
         v = torch.randn(B, 4, 4160, 128, device=dev).to(torch.bfloat16)
         need = ops.L.lib().subspec_tree_attention_workspace(B, 28, 4096, 64)
         ws = torch.empty(max(need, 256), dtype=torch.uint8, device=dev)
-        us = _time_us(lambda: ops.tree_attention(q, k, v, anc, 4096, workspace=ws), args.steps, args.warmup)
+        call_us, kernel_us = _time_us(lambda: ops.tree_attention(q, k, v, anc, 4096, workspace=ws), args.steps, args.warmup)
         nbytes = B * (2 * 4 * 4160 * 128 * 2 + 2 * 28 * 64 * 128 * 2)
-        _kernel_line("tree-masked GQA attention latency", f"BASELINE config 3, B={B}: q [B,28,64,128], KV [B,4,4160,128] bf16",
-                     us, nbytes, flops=B * 4 * 64 * 28 * 4160 * 128, extra={"batch": B})
+        # 3.82 GFLOP per sequence over 9.44 MB: at 405 FLOP/B the shape sits above the ridge (310 FLOP/B)
+        _kernel_line("tree-masked GQA attention latency",
+                     f"BASELINE config 3, B={B}: q [B,28,64,128], KV [B,4,4160,128] bf16", call_us, kernel_us, nbytes,
+                     B * 4 * 64 * 28 * 4160 * 128, "subspec::tree_attention_kernel", bound="mfma", extra={"batch": B})
 
 
 def bench_int4(args):
@@ -100,10 +121,12 @@ def bench_int4(args):
         for M in (1, 16, 64):
             x = torch.randn(M, K, device=dev).to(torch.bfloat16)
             ws = torch.empty(max(ops.L.lib().subspec_int4_linear_workspace(M, N, K), 256), dtype=torch.uint8, device=dev)
-            us = _time_us(lambda: ops.int4_linear(x, wq, sz, N, workspace=ws), args.steps, args.warmup)
+            call_us, kernel_us = _time_us(lambda: ops.int4_linear(x, wq, sz, N, workspace=ws), args.steps, args.warmup)
             nbytes = N * K // 2 + N * (K // 64) * 4 + M * (K + N) * 2
-            _kernel_line("int4 g64 linear latency", f"BASELINE config 4: {K}->{N}, M={M}, bf16 activations", us, nbytes,
-                         flops=2 * M * N * K, extra={"N": N, "K": K, "M": M})
+            _kernel_line("int4 g64 linear latency", f"BASELINE config 4: {K}->{N}, M={M}, bf16 activations", call_us,
+                         kernel_us, nbytes, 2 * M * N * K,
+                         "subspec::int4_gemv_kernel" if M == 1 else "subspec::int4_gemm_kernel",
+                         extra={"N": N, "K": K, "M": M})
 
 
 def bench_e2e(args):
@@ -155,9 +178,9 @@ def bench_greedy(args):
     tok = torch.tensor(cfg["tokens"], dtype=torch.int32, device=dev)
     par = torch.tensor(cfg["parents"], dtype=torch.int32, device=dev)
     ws = torch.empty(ops.L.lib().subspec_tree_verify_workspace(1, 64, 152064, 0), dtype=torch.uint8, device=dev)
-    us = _time_us(lambda: ops.tree_verify(cfg["logits"], tok, par, workspace=ws), args.steps, args.warmup)
-    _kernel_line("greedy tree verify latency", "BASELINE config 1: fp32 logits [64,152064], 64-node tree", us,
-                 64 * 152064 * 4)
+    call_us, kernel_us = _time_us(lambda: ops.tree_verify(cfg["logits"], tok, par, workspace=ws), args.steps, args.warmup)
+    _kernel_line("greedy tree verify latency", "BASELINE config 1: fp32 logits [64,152064], 64-node tree", call_us,
+                 kernel_us, 64 * 152064 * 4, 0, "subspec::row_partial_kernel")
 
 
 def cpu_baseline(cfg, probs_rows, parent_rows, n_trees, min_seconds):

@@ -314,27 +314,38 @@ __global__ __launch_bounds__(kAttnThreads) __attribute__((amdgpu_waves_per_eu(2,
   }
 }
 
+// Merge of the per-chunk (O, max, sum) triples: 32 lanes x float4 cover the 128 dims of one
+// (head, row); a workgroup takes blockDim.x / 32 rows (8, or 2 when the launch would otherwise be
+// too small to fill the chip).  Slot of (bh, chunk c, row) = (bh * chunks + c) * 64 + row; maxima
+// are stored already multiplied by scale * log2(e).
 template <int DT>
-__global__ __launch_bounds__(kAttnD) void tree_attention_merge_kernel(
+__global__ __launch_bounds__(256) void tree_attention_merge_kernel(
     const float* __restrict__ part_o, const float* __restrict__ part_ml, AttnParams ap, uint16_t* __restrict__ out) {
-  const int row = blockIdx.x, bh = blockIdx.y;
+  const int row = blockIdx.x * (blockDim.x >> 5) + (threadIdx.x >> 5), bh = blockIdx.y;
+  if (row >= ap.n_rows) return;
   const int b = bh / (int)ap.hq, qh = bh % (int)ap.hq;
-  const int d = threadIdx.x;
+  const int d4 = threadIdx.x & 31;
   const int64_t slot0 = (int64_t)bh * ap.chunks * kAttnRows + row;     // chunk c: slot0 + c * kAttnRows
   float m = -INFINITY;
 #pragma unroll 8
   for (int c = 0; c < ap.chunks; ++c) m = fmaxf(m, part_ml[(slot0 + (int64_t)c * kAttnRows) * 2]);
-  float num = 0.f, den = 0.f;
+  v4f num = {0.f, 0.f, 0.f, 0.f};
+  float den = 0.f;
 #pragma unroll 8
   for (int c = 0; c < ap.chunks; ++c) {
     const int64_t slot = slot0 + (int64_t)c * kAttnRows;
-    const float mc = part_ml[slot * 2], lc = part_ml[slot * 2 + 1], oc = part_o[slot * kAttnD + d];
-    const float w = mc == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mc - m);
-    num = fmaf(w, oc, num);
-    den = fmaf(w, lc, den);
+    const v2f_t ml = *(const v2f_t*)(&part_ml[slot * 2]);
+    const v4f oc = *(const v4f*)(&part_o[slot * kAttnD + d4 * 4]);
+    const float w = ml[0] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(ml[0] - m);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) num[i] = fmaf(w, oc[i], num[i]);
+    den = fmaf(w, ml[1], den);
   }
-  const float o = den > 0.f ? num / den : 0.f;
-  Elem<DT>::store(out, (((int64_t)b * ap.n_rows + row) * ap.hq + qh) * kAttnD + d, o);
+  const float inv = den > 0.f ? 1.f / den : 0.f;
+  uint2 packed;
+  packed.x = pack2<DT>(num[0] * inv, num[1] * inv);
+  packed.y = pack2<DT>(num[2] * inv, num[3] * inv);
+  *(uint2*)(out + (((int64_t)b * ap.n_rows + row) * ap.hq + qh) * kAttnD + d4 * 4) = packed;
 }
 
 static int attn_chunks(int64_t batch, int64_t hq, int64_t kv_len) {
@@ -407,6 +418,7 @@ extern "C" int subspec_tree_attention(const void* q, const void* k_cache, const 
   }
   hipStream_t st = (hipStream_t)stream;
   const dim3 grid((unsigned)((ap.units + kXcds - 1) / kXcds * kXcds * ap.pairs_per_kv));
+  const int64_t merge_rows = batch * n_q_heads * n_rows / 8 >= 1024 ? 8 : 2;   // rows per merge workgroup
   if (dtype == SUBSPEC_BF16) {
     {
       DominantKernelTimer timer(st);
@@ -414,8 +426,8 @@ extern "C" int subspec_tree_attention(const void* q, const void* k_cache, const 
                          (const uint16_t*)k_cache, (const uint16_t*)v_cache, anc_bits, ap, (uint16_t*)out, part_o, part_ml);
     }
     if (ap.chunks > 1)
-      hipLaunchKernelGGL((tree_attention_merge_kernel<SUBSPEC_BF16>), dim3((unsigned)n_rows, (unsigned)(batch * n_q_heads)),
-                         dim3(kAttnD), 0, st, part_o, part_ml, ap, (uint16_t*)out);
+      hipLaunchKernelGGL((tree_attention_merge_kernel<SUBSPEC_BF16>), dim3((unsigned)((n_rows + merge_rows - 1) / merge_rows), (unsigned)(batch * n_q_heads)),
+                         dim3(merge_rows * 32), 0, st, part_o, part_ml, ap, (uint16_t*)out);
   } else {
     {
       DominantKernelTimer timer(st);
@@ -423,8 +435,8 @@ extern "C" int subspec_tree_attention(const void* q, const void* k_cache, const 
                          (const uint16_t*)k_cache, (const uint16_t*)v_cache, anc_bits, ap, (uint16_t*)out, part_o, part_ml);
     }
     if (ap.chunks > 1)
-      hipLaunchKernelGGL((tree_attention_merge_kernel<SUBSPEC_F16>), dim3((unsigned)n_rows, (unsigned)(batch * n_q_heads)),
-                         dim3(kAttnD), 0, st, part_o, part_ml, ap, (uint16_t*)out);
+      hipLaunchKernelGGL((tree_attention_merge_kernel<SUBSPEC_F16>), dim3((unsigned)((n_rows + merge_rows - 1) / merge_rows), (unsigned)(batch * n_q_heads)),
+                         dim3(merge_rows * 32), 0, st, part_o, part_ml, ap, (uint16_t*)out);
   }
   SUBSPEC_CHECK_HIP(hipGetLastError());
   return SUBSPEC_OK;
