@@ -198,6 +198,61 @@ int subspec_int4_linear(const void* x, const uint32_t* wq, const uint32_t* sz, c
                         void* stream);
 
 /* ------------------------------------------------------------------------------------------
+ * One int4 decoder layer of the substitute draft over the rows of a tree level, issued as a fixed
+ * sequence of launches from one host call (no per-module Python dispatch):
+ *   x += o_proj(attn(rope(qkv_proj(rmsnorm(x)))));  x += down_proj(silu(gate) * up),
+ *   gate|up = gate_up_proj(rmsnorm(x)).  K and V of the rows are written into the static cache
+ *   at cache_rows before attention; attention is subspec_tree_attention with batch 1.
+ *
+ * Replaces  one HuggingFace Qwen2 / Llama decoder layer of the draft whose q,k,v,o,gate,up,down
+ *           projections are the HQQ int4 linears of
+ *           specdecodes/helpers/recipes/subspec/hqq_4bit_postspec.py:17-58, as run per tree level by
+ *           specdecodes/models/draft_models/classic_sd.py:85-118 (speculate_once); the reference
+ *           removes the per-module launch cost with torch.compile / captured graphs
+ *           (specdecodes/models/draft_models/subspec_sd_fi.py:65-179).
+ *
+ * Projections are fused as in BASELINE config 4: qkv = q|k|v rows, gate_up = gate|up rows, all in
+ * the tiled int4 layout of subspec_int4_linear.  Rotary embedding is the rotate-half form with
+ * angle = position * rope_theta^(-2i / head_dim).
+ *
+ * x           device [n_rows, hidden], updated in place (the residual stream)
+ * positions   device int32 [n_rows]   rotary position of each row (prefix_len + node depth)
+ * cache_rows  device int32 [n_rows]   cache row each row's K / V is written to (prefix_len + slot)
+ * anc_bits    device uint64 [n_rows]  as for subspec_tree_attention
+ * k_cache, v_cache  device [n_kv_heads, kv_seq_stride, head_dim] of THIS layer (batch 1)
+ * Limits: n_rows <= 64, n_tree_slots <= 64, head_dim 128, hidden % 64 == 0 and <= 16384,
+ *         intermediate % 64 == 0.
+ */
+typedef struct subspec_decoder_layer_dims {
+  int32_t dtype;            /* SUBSPEC_BF16 or SUBSPEC_F16 */
+  int32_t reserved;
+  int64_t n_rows, hidden, intermediate, n_q_heads, n_kv_heads, head_dim;
+  int64_t kv_seq_stride, prefix_len, n_tree_slots;
+  float rms_eps, rope_theta;
+} subspec_decoder_layer_dims;
+
+typedef struct subspec_decoder_layer_weights {
+  const void* input_norm;   /* [hidden] */
+  const void* post_norm;    /* [hidden] */
+  const uint32_t* qkv_wq;   /* N = (n_q_heads + 2 n_kv_heads) * head_dim, K = hidden */
+  const uint32_t* qkv_sz;
+  const void* qkv_bias;     /* [N] or NULL */
+  const uint32_t* o_wq;     /* N = hidden, K = n_q_heads * head_dim */
+  const uint32_t* o_sz;
+  const uint32_t* gate_up_wq; /* N = 2 * intermediate, K = hidden */
+  const uint32_t* gate_up_sz;
+  const uint32_t* down_wq;  /* N = hidden, K = intermediate */
+  const uint32_t* down_sz;
+} subspec_decoder_layer_weights;
+
+/* 0 when the dimensions are rejected (subspec_last_error says why) */
+size_t subspec_int4_decoder_layer_workspace(const subspec_decoder_layer_dims* dims);
+
+int subspec_int4_decoder_layer(const subspec_decoder_layer_dims* dims, const subspec_decoder_layer_weights* weights,
+                               void* x, const int32_t* positions, const int32_t* cache_rows, const uint64_t* anc_bits,
+                               void* k_cache, void* v_cache, void* workspace, size_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------------------------------
  * Layer streaming: asynchronous copy of one weight slab from pinned host memory to its device
  * slab on the caller's copy stream (hipMemcpyAsync).  Ordering against the compute stream
  * (copy-done before use, last-reader-done before overwrite) is the caller's, with events.

@@ -22,6 +22,22 @@ MAX_TREE_NODES = 256
 _lib = None
 
 _p, _i32, _i64, _f64, _sz = C.c_void_p, C.c_int32, C.c_int64, C.c_double, C.c_size_t
+
+
+class DecoderLayerDims(C.Structure):
+    """subspec_decoder_layer_dims"""
+    _fields_ = [("dtype", C.c_int32), ("reserved", C.c_int32),
+                ("n_rows", _i64), ("hidden", _i64), ("intermediate", _i64), ("n_q_heads", _i64), ("n_kv_heads", _i64),
+                ("head_dim", _i64), ("kv_seq_stride", _i64), ("prefix_len", _i64), ("n_tree_slots", _i64),
+                ("rms_eps", C.c_float), ("rope_theta", C.c_float)]
+
+
+class DecoderLayerWeights(C.Structure):
+    """subspec_decoder_layer_weights"""
+    _fields_ = [(n, _p) for n in ("input_norm", "post_norm", "qkv_wq", "qkv_sz", "qkv_bias", "o_wq", "o_sz",
+                                  "gate_up_wq", "gate_up_sz", "down_wq", "down_sz")]
+
+
 _SIGNATURES = {
     "subspec_abi_version": (C.c_int, []),
     "subspec_last_error": (C.c_char_p, []),
@@ -39,6 +55,9 @@ _SIGNATURES = {
                                          C.c_float, _p, _sz, _p]),
     "subspec_int4_linear_workspace": (_sz, [_i64, _i64, _i64]),
     "subspec_int4_linear": (C.c_int, [_p, _p, _p, _p, _p, C.c_int, _i64, _i64, _i64, _i64, _p, _sz, _p]),
+    "subspec_int4_decoder_layer_workspace": (_sz, [C.POINTER(DecoderLayerDims)]),
+    "subspec_int4_decoder_layer": (C.c_int, [C.POINTER(DecoderLayerDims), C.POINTER(DecoderLayerWeights), _p, _p, _p, _p,
+                                             _p, _p, _p, _sz, _p]),
     "subspec_stream_copy_h2d": (C.c_int, [_p, _p, _sz, _p]),
     "subspec_kv_compact": (C.c_int, [_p, _p, _i64, _i64, _i64, _i64, _i64, _p, _p, _i32, _i32, _p]),
 }

@@ -1,0 +1,281 @@
+// One int4 decoder layer of the substitute draft over the tree rows, launched from one host call.
+//
+// The reference runs the draft as a HuggingFace Qwen2 / Llama decoder layer whose seven projections
+// were replaced by HQQ int4 linears (specdecodes/helpers/recipes/subspec/hqq_4bit_postspec.py:17-58)
+// and hides the per-module launch cost behind torch.compile / captured graphs
+// (specdecodes/models/draft_models/classic_sd.py:85-118 for the step it repeats per tree level).
+// Here the layer is a fixed sequence of launches issued by native code on the caller's stream:
+//   h      = rmsnorm(x) * w_in
+//   qkv    = int4(h) + bias                     [M, (Hq + 2 Hkv) D]
+//   q, K/V = rope(qkv), K and V rows written into the static cache at cache_rows
+//   a      = tree attention(q, cache)           [M, Hq D]
+//   x     += int4(a)                            (o_proj; the add is fused into the next rmsnorm)
+//   h      = rmsnorm(x) * w_post
+//   act    = silu(gate) * up,  gate|up = int4(h)
+//   x     += int4(act)                          (down_proj)
+// Rounding follows the eager torch layer: every intermediate tensor is rounded to the activation
+// dtype where torch would materialise it (normalised activations before the weight product, the
+// two rotary products and their sum, silu before the product with `up`, both residual sums).
+#include "common.h"
+#include <algorithm>
+
+namespace subspec {
+
+typedef uint32_t dec_u4 __attribute__((ext_vector_type(4)));
+
+template <int DT>
+__device__ __forceinline__ void unpack8(dec_u4 v, float* f) {
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    if constexpr (DT == SUBSPEC_BF16) {
+      f[2 * j] = bf16_bits_to_float(v[j] & 0xffffu);
+      f[2 * j + 1] = bf16_bits_to_float(v[j] >> 16);
+    } else {
+      f[2 * j] = f16_bits_to_float(v[j] & 0xffffu);
+      f[2 * j + 1] = f16_bits_to_float(v[j] >> 16);
+    }
+  }
+}
+template <int DT>
+__device__ __forceinline__ uint32_t to_bits(float v) {
+  if constexpr (DT == SUBSPEC_BF16) {
+    return __float_as_uint(round_bf16(v)) >> 16;
+  } else {
+    union { uint16_t u; _Float16 h; } c;
+    c.h = (_Float16)v;
+    return c.u;
+  }
+}
+template <int DT>
+__device__ __forceinline__ dec_u4 pack8(const float* f) {
+  dec_u4 v;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) v[j] = to_bits<DT>(f[2 * j]) | (to_bits<DT>(f[2 * j + 1]) << 16);
+  return v;
+}
+
+// x[m] (+= delta[m], rounded, written back) ; y[m] = w * round(x * rsqrt(mean(x^2) + eps))
+// One workgroup per row; H % 8 == 0.  kMaxPieces 16-byte pieces per thread cover H <= 256 * 8 * kMaxPieces.
+constexpr int kNormThreads = 256;
+constexpr int kNormMaxPieces = 8;
+template <int DT, bool kAdd>
+__global__ __launch_bounds__(kNormThreads) void add_rmsnorm_kernel(uint16_t* __restrict__ x, const uint16_t* __restrict__ delta,
+                                                                   const uint16_t* __restrict__ w, uint16_t* __restrict__ y,
+                                                                   int H, float eps) {
+  __shared__ float scratch[kNormThreads / kWave];
+  const int m = blockIdx.x, tid = threadIdx.x, pieces = H / 8;
+  dec_u4* xr = (dec_u4*)(x + (int64_t)m * H);
+  const dec_u4* dr = (const dec_u4*)(delta + (int64_t)m * H);
+  float v[kNormMaxPieces][8];
+  float ss = 0.f;
+#pragma unroll
+  for (int p = 0; p < kNormMaxPieces; ++p) {
+    const int i = p * kNormThreads + tid;
+    if (i < pieces) {
+      unpack8<DT>(xr[i], v[p]);
+      if constexpr (kAdd) {
+        float d[8];
+        unpack8<DT>(dr[i], d);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[p][j] = Elem<DT>::round(v[p][j] + d[j]);
+        xr[i] = pack8<DT>(v[p]);
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j) ss = fmaf(v[p][j], v[p][j], ss);
+    }
+  }
+  const float tot = block_sum<kNormThreads>(ss, scratch);
+  const float r = rsqrtf(tot / (float)H + eps);
+#pragma unroll
+  for (int p = 0; p < kNormMaxPieces; ++p) {
+    const int i = p * kNormThreads + tid;
+    if (i < pieces) {
+      float wv[8], o[8];
+      unpack8<DT>(((const dec_u4*)w)[i], wv);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) o[j] = wv[j] * Elem<DT>::round(v[p][j] * r);
+      ((dec_u4*)(y + (int64_t)m * H))[i] = pack8<DT>(o);
+    }
+  }
+}
+
+// x += delta (rounded), 8 elements per thread
+template <int DT>
+__global__ __launch_bounds__(256) void add_kernel(uint16_t* __restrict__ x, const uint16_t* __restrict__ delta, int64_t pieces) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= pieces) return;
+  float a[8], d[8];
+  unpack8<DT>(((const dec_u4*)x)[i], a);
+  unpack8<DT>(((const dec_u4*)delta)[i], d);
+#pragma unroll
+  for (int j = 0; j < 8; ++j) a[j] = Elem<DT>::round(a[j] + d[j]);
+  ((dec_u4*)x)[i] = pack8<DT>(a);
+}
+
+// act[m, f] = round(silu(gate)) * up with gate = gu[m, f], up = gu[m, F + f]
+template <int DT>
+__global__ __launch_bounds__(256) void silu_mul_kernel(const uint16_t* __restrict__ gu, uint16_t* __restrict__ act, int F,
+                                                       int64_t pieces) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= pieces) return;
+  const int per_row = F / 8;
+  const int64_t m = i / per_row;
+  const int p = (int)(i % per_row);
+  float g[8], u[8];
+  unpack8<DT>(((const dec_u4*)(gu + m * 2 * F))[p], g);
+  unpack8<DT>(((const dec_u4*)(gu + m * 2 * F + F))[p], u);
+#pragma unroll
+  for (int j = 0; j < 8; ++j) g[j] = Elem<DT>::round(g[j] / (1.f + __expf(-g[j]))) * u[j];
+  ((dec_u4*)(act + m * F))[p] = pack8<DT>(g);
+}
+
+// Rotary embedding (rotate-half form, angle = position * theta^(-2i/D)) of the q and k heads of
+// qkv [M, (Hq + 2 Hkv) * D]; q goes to q_out [Hq, M, D], k and v to rows cache_rows[m] of the
+// layer's [Hkv, S, D] caches.  One wavefront per (row, head); lane i handles dims i and i + D/2.
+template <int DT>
+__global__ __launch_bounds__(64) void rope_write_kernel(const uint16_t* __restrict__ qkv, const int32_t* __restrict__ positions,
+                                                        const int32_t* __restrict__ cache_rows, uint16_t* __restrict__ q_out,
+                                                        uint16_t* __restrict__ k_cache, uint16_t* __restrict__ v_cache,
+                                                        int M, int Hq, int Hkv, int D, int64_t seq_stride, float log2_theta) {
+  const int m = blockIdx.x, hh = blockIdx.y, i = threadIdx.x;
+  const int half = D / 2;
+  if (i >= half) return;
+  const uint16_t* src = qkv + ((int64_t)m * (Hq + 2 * Hkv) + hh) * D;
+  const float lo = Elem<DT>::load(src, i), hi = Elem<DT>::load(src, i + half);
+  uint16_t* dst;
+  if (hh < Hq) dst = q_out + ((int64_t)hh * M + m) * D;
+  else if (hh < Hq + Hkv) dst = k_cache + ((int64_t)(hh - Hq) * seq_stride + cache_rows[m]) * D;
+  else dst = v_cache + ((int64_t)(hh - Hq - Hkv) * seq_stride + cache_rows[m]) * D;
+  if (hh >= Hq + Hkv) {                                 // value heads are copied
+    Elem<DT>::store(dst, i, lo);
+    Elem<DT>::store(dst, i + half, hi);
+    return;
+  }
+  const float inv_freq = exp2f(-(float)(2 * i) / (float)D * log2_theta);
+  float s, c;
+  sincosf((float)positions[m] * inv_freq, &s, &c);
+  c = Elem<DT>::round(c);
+  s = Elem<DT>::round(s);
+  // t * cos + rotate_half(t) * sin, each product and the sum rounded like the eager tensor ops
+  const float o_lo = Elem<DT>::round(lo * c) + Elem<DT>::round(-hi * s);
+  const float o_hi = Elem<DT>::round(hi * c) + Elem<DT>::round(lo * s);
+  Elem<DT>::store(dst, i, o_lo);
+  Elem<DT>::store(dst, i + half, o_hi);
+}
+
+struct LayerPlan {
+  size_t h, qkv, q, a, o, gu, act, d, sub, sub_bytes, total;
+};
+static LayerPlan layer_plan(const subspec_decoder_layer_dims& s) {
+  LayerPlan p;
+  const size_t es = 2, M = (size_t)s.n_rows, H = (size_t)s.hidden, Q = (size_t)s.n_q_heads * s.head_dim,
+               KV = (size_t)s.n_kv_heads * s.head_dim, F = (size_t)s.intermediate;
+  size_t off = 0;
+  auto take = [&](size_t bytes) { size_t o = off; off += align_up(bytes, 256); return o; };
+  p.h = take(M * H * es);
+  p.qkv = take(M * (Q + 2 * KV) * es);
+  p.q = take(M * Q * es);
+  p.a = take(M * Q * es);
+  p.o = take(M * H * es);
+  p.gu = take(M * 2 * F * es);
+  p.act = take(M * F * es);
+  p.d = take(M * H * es);
+  size_t sub = subspec_int4_linear_workspace(s.n_rows, Q + 2 * KV, H);
+  sub = std::max(sub, subspec_int4_linear_workspace(s.n_rows, H, Q));
+  sub = std::max(sub, subspec_int4_linear_workspace(s.n_rows, 2 * F, H));
+  sub = std::max(sub, subspec_int4_linear_workspace(s.n_rows, H, F));
+  sub = std::max(sub, subspec_tree_attention_workspace(1, s.n_q_heads, s.prefix_len, s.n_tree_slots));
+  p.sub_bytes = align_up(sub, 256);
+  p.sub = take(p.sub_bytes);
+  p.total = off;
+  return p;
+}
+
+static int check_dims(const subspec_decoder_layer_dims* s) {
+  if (!s) SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "decoder_layer: null dims");
+  if (s->dtype != SUBSPEC_BF16 && s->dtype != SUBSPEC_F16)
+    SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "decoder_layer: dtype %d not supported (bf16 / fp16 only)", s->dtype);
+  if (s->n_rows < 1 || s->n_rows > 64) SUBSPEC_FAIL(SUBSPEC_ERR_LIMIT, "decoder_layer: n_rows=%lld outside 1..64", (long long)s->n_rows);
+  if (s->head_dim != 128) SUBSPEC_FAIL(SUBSPEC_ERR_LIMIT, "decoder_layer: head_dim=%lld (built for 128)", (long long)s->head_dim);
+  if (s->hidden <= 0 || s->hidden % 64 != 0 || s->hidden > 8 * kNormThreads * kNormMaxPieces)
+    SUBSPEC_FAIL(SUBSPEC_ERR_LIMIT, "decoder_layer: hidden=%lld must be a multiple of 64 and at most %d", (long long)s->hidden,
+                 8 * kNormThreads * kNormMaxPieces);
+  if (s->intermediate <= 0 || s->intermediate % 64 != 0)
+    SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "decoder_layer: intermediate=%lld must be a multiple of 64", (long long)s->intermediate);
+  if (s->n_q_heads <= 0 || s->n_kv_heads <= 0 || s->n_q_heads % s->n_kv_heads != 0)
+    SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "decoder_layer: %lld query heads over %lld kv heads", (long long)s->n_q_heads, (long long)s->n_kv_heads);
+  if (s->n_tree_slots < 1 || s->n_tree_slots > 64 || s->prefix_len < 0 || s->prefix_len + s->n_tree_slots > s->kv_seq_stride)
+    SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "decoder_layer: prefix_len=%lld, n_tree_slots=%lld do not fit a cache of %lld rows",
+                 (long long)s->prefix_len, (long long)s->n_tree_slots, (long long)s->kv_seq_stride);
+  if (!(s->rope_theta > 1.f) || !(s->rms_eps > 0.f)) SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "decoder_layer: rope_theta / rms_eps out of range");
+  return SUBSPEC_OK;
+}
+
+template <int DT>
+static int run_layer(const subspec_decoder_layer_dims& s, const subspec_decoder_layer_weights& w, uint16_t* x,
+                     const int32_t* positions, const int32_t* cache_rows, const uint64_t* anc_bits, uint16_t* k_cache,
+                     uint16_t* v_cache, char* ws, hipStream_t st) {
+  const LayerPlan p = layer_plan(s);
+  const int M = (int)s.n_rows, H = (int)s.hidden, Hq = (int)s.n_q_heads, Hkv = (int)s.n_kv_heads, D = (int)s.head_dim,
+            F = (int)s.intermediate;
+  const int64_t Q = (int64_t)Hq * D, KV = (int64_t)Hkv * D;
+  uint16_t *h = (uint16_t*)(ws + p.h), *qkv = (uint16_t*)(ws + p.qkv), *q = (uint16_t*)(ws + p.q), *a = (uint16_t*)(ws + p.a),
+           *o = (uint16_t*)(ws + p.o), *gu = (uint16_t*)(ws + p.gu), *act = (uint16_t*)(ws + p.act), *d = (uint16_t*)(ws + p.d);
+  void* sub = ws + p.sub;
+  int rc;
+  hipLaunchKernelGGL((add_rmsnorm_kernel<DT, false>), dim3(M), dim3(kNormThreads), 0, st, x, (const uint16_t*)nullptr,
+                     (const uint16_t*)w.input_norm, h, H, s.rms_eps);
+  if ((rc = subspec_int4_linear(h, w.qkv_wq, w.qkv_sz, w.qkv_bias, qkv, DT, M, Q + 2 * KV, H, 64, sub, p.sub_bytes, st))) return rc;
+  hipLaunchKernelGGL((rope_write_kernel<DT>), dim3(M, Hq + 2 * Hkv), dim3(64), 0, st, qkv, positions, cache_rows, q, k_cache,
+                     v_cache, M, Hq, Hkv, D, s.kv_seq_stride, log2f(s.rope_theta));
+  if ((rc = subspec_tree_attention(q, k_cache, v_cache, a, DT, 1, Hq, Hkv, M, s.n_tree_slots, D, s.kv_seq_stride, s.prefix_len,
+                                   anc_bits, 0, 1.f / sqrtf((float)D), sub, p.sub_bytes, st)))
+    return rc;
+  if ((rc = subspec_int4_linear(a, w.o_wq, w.o_sz, nullptr, o, DT, M, H, Q, 64, sub, p.sub_bytes, st))) return rc;
+  hipLaunchKernelGGL((add_rmsnorm_kernel<DT, true>), dim3(M), dim3(kNormThreads), 0, st, x, o, (const uint16_t*)w.post_norm, h, H,
+                     s.rms_eps);
+  if ((rc = subspec_int4_linear(h, w.gate_up_wq, w.gate_up_sz, nullptr, gu, DT, M, 2 * (int64_t)F, H, 64, sub, p.sub_bytes, st)))
+    return rc;
+  const int64_t act_pieces = (int64_t)M * F / 8;
+  hipLaunchKernelGGL((silu_mul_kernel<DT>), dim3((unsigned)((act_pieces + 255) / 256)), dim3(256), 0, st, gu, act, F, act_pieces);
+  if ((rc = subspec_int4_linear(act, w.down_wq, w.down_sz, nullptr, d, DT, M, H, F, 64, sub, p.sub_bytes, st))) return rc;
+  const int64_t x_pieces = (int64_t)M * H / 8;
+  hipLaunchKernelGGL((add_kernel<DT>), dim3((unsigned)((x_pieces + 255) / 256)), dim3(256), 0, st, x, d, x_pieces);
+  SUBSPEC_CHECK_HIP(hipGetLastError());
+  return SUBSPEC_OK;
+}
+
+}  // namespace subspec
+
+using namespace subspec;
+
+extern "C" size_t subspec_int4_decoder_layer_workspace(const subspec_decoder_layer_dims* dims) {
+  if (!dims || check_dims(dims) != SUBSPEC_OK) return 0;
+  return layer_plan(*dims).total;
+}
+
+extern "C" int subspec_int4_decoder_layer(const subspec_decoder_layer_dims* dims, const subspec_decoder_layer_weights* weights,
+                                          void* x, const int32_t* positions, const int32_t* cache_rows,
+                                          const uint64_t* anc_bits, void* k_cache, void* v_cache, void* workspace,
+                                          size_t workspace_bytes, void* stream) {
+  const int rc = check_dims(dims);
+  if (rc != SUBSPEC_OK) return rc;
+  if (!weights || !x || !positions || !cache_rows || !anc_bits || !k_cache || !v_cache)
+    SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "decoder_layer: null pointer argument");
+  const subspec_decoder_layer_weights& w = *weights;
+  if (!w.input_norm || !w.post_norm || !w.qkv_wq || !w.qkv_sz || !w.o_wq || !w.o_sz || !w.gate_up_wq || !w.gate_up_sz ||
+      !w.down_wq || !w.down_sz)
+    SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "decoder_layer: null weight pointer");
+  if ((uintptr_t)x % 16 || (uintptr_t)w.input_norm % 16 || (uintptr_t)w.post_norm % 16 || (uintptr_t)k_cache % 16 ||
+      (uintptr_t)v_cache % 16)
+    SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "decoder_layer: x, norm weights and caches must be 16-byte aligned");
+  const size_t need = layer_plan(*dims).total;
+  if (!workspace || workspace_bytes < need)
+    SUBSPEC_FAIL(SUBSPEC_ERR_WORKSPACE, "decoder_layer: workspace of %zu bytes is smaller than the %zu required", workspace_bytes, need);
+  if ((uintptr_t)workspace % 256) SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "decoder_layer: workspace must be 256-byte aligned");
+  if (dims->dtype == SUBSPEC_BF16)
+    return run_layer<SUBSPEC_BF16>(*dims, w, (uint16_t*)x, positions, cache_rows, anc_bits, (uint16_t*)k_cache, (uint16_t*)v_cache,
+                                   (char*)workspace, (hipStream_t)stream);
+  return run_layer<SUBSPEC_F16>(*dims, w, (uint16_t*)x, positions, cache_rows, anc_bits, (uint16_t*)k_cache, (uint16_t*)v_cache,
+                                (char*)workspace, (hipStream_t)stream);
+}

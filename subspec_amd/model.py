@@ -118,11 +118,42 @@ class Decoder:
         self.streamer = streamer
         self.first_streamed = cfg.num_hidden_layers if first_streamed is None else first_streamed
         self.device, self.dtype = embed.device, embed.dtype
+        self._native = None
+        self.use_native_layers = True            # False: run every module through its own torch / library call
         inv = 1.0 / (cfg.rope_theta ** (torch.arange(0, cfg.head_dim, 2, device=self.device, dtype=torch.float32) / cfg.head_dim))
         pos = torch.arange(kv.cache.max_cache_len + 8, device=self.device, dtype=torch.float32)
         freqs = torch.outer(pos, inv)
         self.cos = torch.cat([freqs, freqs], -1).cos()
         self.sin = torch.cat([freqs, freqs], -1).sin()
+
+    # ------------------------------------------------------------------ native int4 layers
+    @property
+    def native_layers(self) -> bool:
+        """True when every layer is int4-packed, i.e. the stack can run through the library's decoder-layer
+        entry point (one host call per layer instead of one per module)."""
+        if self._native is None:
+            self._native = bool(self.layers) and all("qkv_proj.wq" in w for w in self.layers)
+            if self._native:
+                self._native_weights = [ops.decoder_layer_weights(w) for w in self.layers]
+                self._native_ws = {}
+        return self._native
+
+    def _run_native_layers(self, x, positions, rows, anc_bits, prefix_len: int, slots: int) -> torch.Tensor:
+        cfg, cache = self.cfg, self.kv.cache
+        n = x.shape[0]
+        dims = ops.decoder_layer_dims(self.dtype, n, cfg.hidden_size, cfg.intermediate_size, cfg.num_attention_heads,
+                                      cfg.num_key_value_heads, cfg.head_dim, cache.max_cache_len, int(prefix_len),
+                                      int(slots), cfg.rms_norm_eps, cfg.rope_theta)
+        need = ops.decoder_layer_workspace(dims)
+        ws = self._native_ws.get("ws")
+        if ws is None or ws.numel() < need:
+            ws = self._native_ws["ws"] = torch.empty(need, dtype=torch.uint8, device=self.device)
+        x = x.contiguous().clone()
+        pos32, rows32 = positions.to(torch.int32), rows.to(torch.int32)
+        bits = anc_bits.to(torch.int64).contiguous()
+        for i, w in enumerate(self._native_weights):
+            ops.int4_decoder_layer_(x, dims, w, pos32, rows32, bits, cache.k(i), cache.v(i), ws)
+        return x
 
     # ------------------------------------------------------------------ pieces
     def _rope(self, t: torch.Tensor, positions: torch.Tensor) -> torch.Tensor:
@@ -194,6 +225,8 @@ class Decoder:
         positions = depths.to(self.device) + prefix_len
         rows = torch.arange(prefix_len + first_slot, prefix_len + first_slot + n, device=self.device)
         cfg = self.cfg
+        if self.use_native_layers and self.native_layers and self.streamer is None and n <= 64 and slots <= 64:
+            return self.logits(self._run_native_layers(self.embed[token_ids], positions, rows, anc_bits, prefix_len, slots))
 
         def attn(i, q):
             return ops.tree_attention(q, self.kv.cache.k(i), self.kv.cache.v(i), anc_bits, prefix_len,

@@ -5,6 +5,7 @@ libsubspec_hip.so.
 """
 from __future__ import annotations
 
+import ctypes
 from typing import Dict, Optional
 
 import torch
@@ -242,3 +243,58 @@ def int4_linear(x: torch.Tensor, wq: torch.Tensor, sz: torch.Tensor, out_feature
         0 if workspace is None else workspace.numel() * workspace.element_size(), _stream(dev))
     L.check(code, "subspec_int4_linear")
     return y.reshape(*x.shape[:-1], N)
+
+
+# ---------------------------------------------------------------------------------------------- decoder layer
+def decoder_layer_dims(dtype: torch.dtype, n_rows: int, hidden: int, intermediate: int, n_q_heads: int, n_kv_heads: int,
+                       head_dim: int, kv_seq_stride: int, prefix_len: int, n_tree_slots: int, rms_eps: float,
+                       rope_theta: float) -> "L.DecoderLayerDims":
+    code = {torch.bfloat16: L.BF16, torch.float16: L.F16}.get(dtype)
+    if code is None:
+        raise ValueError(f"decoder layer: dtype {dtype} not supported (bf16 / fp16 only)")
+    return L.DecoderLayerDims(code, 0, n_rows, hidden, intermediate, n_q_heads, n_kv_heads, head_dim, kv_seq_stride,
+                              prefix_len, n_tree_slots, rms_eps, rope_theta)
+
+
+def decoder_layer_weights(w: dict) -> "L.DecoderLayerWeights":
+    """Pointer table of one layer's tensors (``input_layernorm.weight``, ``qkv_proj.wq`` ... as produced by
+    ``subspec_amd.model.quantize_layers``).  The caller keeps the tensors alive."""
+    def ptr(name):
+        t = w.get(name)
+        return None if t is None else t.data_ptr()
+    for name in ("qkv_proj.wq", "o_proj.wq", "gate_up_proj.wq", "down_proj.wq"):
+        if name not in w:
+            raise ValueError(f"decoder layer: {name} missing (the layer must be int4-packed)")
+    return L.DecoderLayerWeights(ptr("input_layernorm.weight"), ptr("post_attention_layernorm.weight"),
+                                 ptr("qkv_proj.wq"), ptr("qkv_proj.sz"), ptr("qkv_proj.bias"),
+                                 ptr("o_proj.wq"), ptr("o_proj.sz"), ptr("gate_up_proj.wq"), ptr("gate_up_proj.sz"),
+                                 ptr("down_proj.wq"), ptr("down_proj.sz"))
+
+
+def decoder_layer_workspace(dims: "L.DecoderLayerDims") -> int:
+    need = L.lib().subspec_int4_decoder_layer_workspace(ctypes.byref(dims))
+    if need == 0:
+        raise ValueError("decoder layer: " + L.lib().subspec_last_error().decode("utf-8", "replace"))
+    return int(need)
+
+
+def int4_decoder_layer_(x: torch.Tensor, dims: "L.DecoderLayerDims", weights: "L.DecoderLayerWeights",
+                        positions: torch.Tensor, cache_rows: torch.Tensor, anc_bits: torch.Tensor,
+                        k_cache: torch.Tensor, v_cache: torch.Tensor, workspace: torch.Tensor) -> torch.Tensor:
+    """In-place update of the residual stream ``x`` [n_rows, hidden] by one int4 decoder layer;
+    ``positions`` / ``cache_rows`` int32 [n_rows], ``anc_bits`` int64 [n_rows], ``k_cache`` /
+    ``v_cache`` [1, Hkv, S, D] views of this layer's cache."""
+    dev = _require_gpu(x, positions, cache_rows, anc_bits, k_cache, v_cache, workspace)
+    if positions.dtype != torch.int32 or cache_rows.dtype != torch.int32 or anc_bits.dtype != torch.int64:
+        raise ValueError("decoder layer: positions / cache_rows must be int32 and anc_bits int64")
+    if not (x.is_contiguous() and k_cache.is_contiguous() and v_cache.is_contiguous()):
+        raise ValueError("decoder layer: x and the layer's cache views must be contiguous")
+    if x.shape != (dims.n_rows, dims.hidden) or positions.numel() != dims.n_rows or cache_rows.numel() != dims.n_rows \
+            or anc_bits.numel() != dims.n_rows:
+        raise ValueError("decoder layer: tensor shapes do not match the dimensions given")
+    code = L.lib().subspec_int4_decoder_layer(
+        ctypes.byref(dims), ctypes.byref(weights), x.data_ptr(), positions.data_ptr(), cache_rows.data_ptr(),
+        anc_bits.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), workspace.data_ptr(),
+        workspace.numel() * workspace.element_size(), _stream(dev))
+    L.check(code, "subspec_int4_decoder_layer")
+    return x
