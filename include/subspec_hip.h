@@ -211,7 +211,7 @@ int subspec_int4_linear(const void* x, const uint32_t* wq, const uint32_t* sz, c
  *           removes the per-module launch cost with torch.compile / captured graphs
  *           (specdecodes/models/draft_models/subspec_sd_fi.py:65-179).
  *
- * Projections are fused as in BASELINE config 4: qkv = q|k|v rows, gate_up = gate|up rows, all in
+ * Projections are fused: qkv = q|k|v rows (N = 4608 at the Qwen2.5-7B shape), gate_up = gate|up rows, all in
  * the tiled int4 layout of subspec_int4_linear.  Rotary embedding is the rotate-half form with
  * angle = position * rope_theta^(-2i / head_dim).
  *

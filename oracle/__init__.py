@@ -31,4 +31,8 @@ How each function is pinned (so a wrong sign / index / dropped term fails a test
 * ``int4.linear``                          – closed form x @ ((Wq - z) * s).T; the special case
   s=1, z=0 reduces to an integer matmul.  The HQQ *quantizer* itself (hqq==0.2.6, absent) is
   **parity unpinned**: parity is defined on the linear given identical (Wq, scale, zero).
+* ``decoder.decoder_layer``                – float32 restatement of the published Qwen2 decoder layer
+  (transformers 4.52.3, not in the reference tree) with the affine int4 linears; **parity
+  unpinned** beyond closed forms: rotary is a rotation, identity at position 0 and relative; zero
+  output projections leave the residual stream; its attention block equals ``attention.tree_attention``.
 """

@@ -66,6 +66,43 @@ def pack_tiled(codes: torch.Tensor, scale: torch.Tensor, zero: torch.Tensor) -> 
     return wq, sz
 
 
+def from_hqq_tensors(W_q: torch.Tensor, scale: torch.Tensor, zero: torch.Tensor, shape: Tuple[int, int]
+                     ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """Convert the tensors an ``hqq.core.quantize.HQQLinear`` holds for ``nbits=4, group_size=64, axis=1``
+    (the configuration of specdecodes/helpers/recipes/subspec/hqq_4bit_postspec.py:17-58) into
+    ``(codes [N, K], scale [N, K/64], zero [N, K/64])`` for ``pack_tiled``.
+
+    hqq (pinned at 0.2.6 by the reference's requirements.txt:7; not installed here, so this follows its
+    published layout and is not checked against the package) quantizes ``W.reshape(-1, 64)``: row r of that
+    matrix is group ``r % (K/64)`` of output row ``r // (K/64)``, with one ``scale`` / ``zero`` per row
+    (``meta['scale']``, ``meta['zero']`` of shape ``[N*K/64, 1]``), and stores the codes with
+    ``BitPack.pack_4bit_u8``: the first half of the rows in the high nibble, the second half in the low
+    nibble of a uint8 matrix ``[N*K/128, 64]``."""
+    N, K = int(shape[0]), int(shape[1])
+    if K % GROUP:
+        raise ValueError(f"in_features={K} must be a multiple of {GROUP}")
+    rows = N * K // GROUP
+    if rows % 2:
+        raise ValueError("hqq 4-bit packing needs an even number of groups")
+    if W_q.dtype != torch.uint8 or W_q.numel() != rows // 2 * GROUP:
+        raise ValueError(f"W_q must be the uint8 [{rows // 2}, {GROUP}] matrix of pack_4bit_u8")
+    if scale.numel() != rows or zero.numel() != rows:
+        raise ValueError(f"scale and zero must hold {rows} entries (one per 64-wide group)")
+    packed = W_q.reshape(rows // 2, GROUP)
+    codes = torch.cat([packed >> 4, packed & 0x0F], dim=0).reshape(N, K)
+    return codes, scale.reshape(N, K // GROUP).to(torch.float16), zero.reshape(N, K // GROUP).to(torch.float16)
+
+
+def to_hqq_tensors(codes: torch.Tensor, scale: torch.Tensor, zero: torch.Tensor
+                   ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """Inverse of ``from_hqq_tensors``: (W_q uint8 [N*K/128, 64], scale [N*K/64, 1], zero [N*K/64, 1])."""
+    N, K = codes.shape
+    rows = N * K // GROUP
+    flat = codes.reshape(rows, GROUP).to(torch.uint8)
+    W_q = (flat[:rows // 2] << 4) | flat[rows // 2:]
+    return W_q, scale.reshape(rows, 1), zero.reshape(rows, 1)
+
+
 class HqqInt4Linear(nn.Module):
     """Drop-in for ``nn.Linear`` holding tiled int4 weights; forward runs the HIP GEMV / GEMM."""
 

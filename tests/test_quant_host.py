@@ -49,3 +49,29 @@ def test_quantizer_replaces_named_linears_and_rejects_other_configs():
     from subspec_amd._lib import SubspecHipError
     with pytest.raises(SubspecHipError):                   # no CPU fallback
         model.a(torch.zeros(1, 128, dtype=torch.bfloat16))
+
+
+def test_hqq_tensor_layout_round_trip():
+    """``from_hqq_tensors`` reads hqq's published 4-bit layout (first half of the 64-wide groups in the
+    high nibble, second half in the low nibble).  hqq itself is absent, so the layout is restated here
+    independently, element by element, and checked in both directions."""
+    g = torch.Generator().manual_seed(7)
+    N, K = 48, 256
+    codes = torch.randint(0, 16, (N, K), generator=g, dtype=torch.uint8)
+    scale = (torch.rand(N, K // 64, generator=g) * 0.01 + 1e-3).to(torch.float16)
+    zero = (torch.rand(N, K // 64, generator=g) * 15).to(torch.float16)
+    rows = N * K // 64
+    flat = codes.reshape(rows, 64)
+    packed = torch.empty(rows // 2, 64, dtype=torch.uint8)
+    for r in range(rows // 2):                                   # element-wise restatement of pack_4bit_u8
+        for c in range(64):
+            packed[r, c] = (int(flat[r, c]) << 4) | int(flat[r + rows // 2, c])
+    c2, s2, z2 = quant.from_hqq_tensors(packed, scale.reshape(rows, 1), zero.reshape(rows, 1), (N, K))
+    assert torch.equal(c2, codes) and torch.equal(s2, scale) and torch.equal(z2, zero)
+    W_q, s3, z3 = quant.to_hqq_tensors(codes, scale, zero)
+    assert torch.equal(W_q, packed) and s3.shape == (rows, 1) and z3.shape == (rows, 1)
+    # dequantization in hqq's own arrangement equals the [N, K] form
+    deq_rows = (torch.cat([packed >> 4, packed & 15], 0).float() - zero.reshape(rows, 1).float()) * scale.reshape(rows, 1).float()
+    assert torch.equal(deq_rows.reshape(N, K), quant.dequantize(codes, scale, zero))
+    with pytest.raises(ValueError):
+        quant.from_hqq_tensors(packed[:-1], scale, zero, (N, K))
