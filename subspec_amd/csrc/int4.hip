@@ -33,8 +33,6 @@ namespace subspec {
 constexpr int kI4Threads = 256;
 constexpr int kGroup = 64;
 
-typedef short i4_v4s __attribute__((ext_vector_type(4)));
-typedef _Float16 i4_v4h __attribute__((ext_vector_type(4)));
 typedef float i4_v4f __attribute__((ext_vector_type(4)));
 typedef __bf16 i4_v2bf __attribute__((ext_vector_type(2)));
 typedef _Float16 i4_v2h __attribute__((ext_vector_type(2)));
@@ -47,12 +45,6 @@ template <int DT> struct I4 {
       return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(i4_v2bf, a), __builtin_bit_cast(i4_v2bf, b), c, false);
     else
       return __builtin_amdgcn_fdot2(__builtin_bit_cast(i4_v2h, a), __builtin_bit_cast(i4_v2h, b), c, false);
-  }
-  static __device__ __forceinline__ i4_v4f mfma(uint2 a, uint2 b, i4_v4f c) {
-    if constexpr (DT == SUBSPEC_BF16)
-      return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(i4_v4s, a), __builtin_bit_cast(i4_v4s, b), c, 0, 0, 0);
-    else
-      return __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(i4_v4h, a), __builtin_bit_cast(i4_v4h, b), c, 0, 0, 0);
   }
   static __device__ __forceinline__ float to_float(uint32_t bits16) {
     return DT == SUBSPEC_BF16 ? bf16_bits_to_float(bits16) : f16_bits_to_float(bits16);
