@@ -1,5 +1,5 @@
-"""Layer streaming: target decoder layers kept in pinned host memory and copied into two device
-slabs, one layer ahead of the compute stream.
+"""Layer streaming: target decoder layers kept in pinned host memory and copied into a small ring of
+device slabs ahead of the compute stream.
 
 Replaces the reference's hook-chain offloaders (``PrefetchOffloader``,
 specdecodes/helpers/offloaders/prefetch_offloader_postspec.py:54-241; placement by
@@ -8,9 +8,11 @@ explicit schedule:
 
 * every offloaded layer is ONE contiguous pinned slab (all seven projections + norms), so a layer
   is one ``hipMemcpyAsync`` instead of seven hooked ``copy_`` calls;
-* two device slabs alternate; the copy of layer i+2 into a slab waits on an event recorded after
-  layer i's last kernel (the write-after-read edge the reference leaves to timing), and layer
-  i's compute waits on its copy event;
+* a ring of device slabs; a copy into a slab waits on an event recorded after the last kernel that
+  read the slab (the write-after-read edge the reference leaves to timing), and a layer's compute
+  waits on its copy event;
+* the ring does not stop at the end of a forward: the next forward's first layers are prefetched
+  while the cycle verifies and speculates;
 * the copy stream runs at default priority.
 """
 from __future__ import annotations
@@ -48,46 +50,60 @@ class LayerSlabLayout:
 
 
 class LayerStreamer:
-    def __init__(self, layout: LayerSlabLayout, host_layers: Sequence[Dict[str, torch.Tensor]], device):
+    """``n_slabs`` device slabs form a ring indexed by the running count of layer visits (not by the
+    layer number), so the ring keeps turning across forwards: when a forward ends, the copies of the
+    NEXT forward's first ``n_slabs - 1`` layers are already on their way and overlap whatever runs in
+    between (verification, the draft's speculation)."""
+
+    def __init__(self, layout: LayerSlabLayout, host_layers: Sequence[Dict[str, torch.Tensor]], device,
+                 n_slabs: int = 4):
         self.layout = layout
         self.device = torch.device(device)
         self.n = len(host_layers)
+        self.n_slabs = max(2, min(int(n_slabs), max(2, self.n)))
         # pinned host arena: one slab per offloaded layer (allocated pinned, never registered afterwards)
         self.host = torch.empty((self.n, layout.nbytes), dtype=torch.uint8, pin_memory=True)
         for i, tensors in enumerate(host_layers):
             views = layout.views(self.host[i])
             for name, t in tensors.items():
                 views[name].copy_(t)
-        self.slabs = [torch.empty(layout.nbytes, dtype=torch.uint8, device=self.device) for _ in range(2)]
+        self.slabs = [torch.empty(layout.nbytes, dtype=torch.uint8, device=self.device) for _ in range(self.n_slabs)]
         self.slab_views = [layout.views(s) for s in self.slabs]
         self.copy_stream = torch.cuda.Stream(device=self.device)          # default priority
-        self.copied = [torch.cuda.Event() for _ in range(2)]
-        self.released = [torch.cuda.Event() for _ in range(2)]
-        self._released_valid = [False, False]
+        self.copied = [torch.cuda.Event() for _ in range(self.n_slabs)]
+        self.released = [torch.cuda.Event() for _ in range(self.n_slabs)]
+        self._released_valid = [False] * self.n_slabs
+        self._visit = 0                 # visits computed so far (visit v = layer v % n, slab v % n_slabs)
+        self._issued = 0                # visits whose copy has been issued
         self.bytes_streamed = 0
 
-    def _issue(self, layer: int) -> None:
-        slot = layer % 2
-        if self._released_valid[slot]:
-            self.copy_stream.wait_event(self.released[slot])              # last reader of this slab is done
-        code = L.lib().subspec_stream_copy_h2d(self.slabs[slot].data_ptr(), self.host[layer].data_ptr(),
-                                               self.layout.nbytes, self.copy_stream.cuda_stream)
-        L.check(code, "subspec_stream_copy_h2d")
-        self.copied[slot].record(self.copy_stream)
-        self.bytes_streamed += self.layout.nbytes
+    def _issue_until(self, visit: int) -> None:
+        """Issue the copies of all visits up to and including ``visit``."""
+        while self._issued <= visit:
+            v = self._issued
+            slot, layer = v % self.n_slabs, v % self.n
+            if self._released_valid[slot]:
+                self.copy_stream.wait_event(self.released[slot])          # last reader of this slab is done
+            code = L.lib().subspec_stream_copy_h2d(self.slabs[slot].data_ptr(), self.host[layer].data_ptr(),
+                                                   self.layout.nbytes, self.copy_stream.cuda_stream)
+            L.check(code, "subspec_stream_copy_h2d")
+            self.copied[slot].record(self.copy_stream)
+            self.bytes_streamed += self.layout.nbytes
+            self._issued += 1
 
     def run(self, fn: Callable[[int, Dict[str, torch.Tensor]], None]) -> None:
         """Calls ``fn(i, weights_of_layer_i)`` for every offloaded layer in order on the current
-        stream, with layer i+1's copy in flight while layer i computes."""
+        stream, with the copies of the following ``n_slabs - 1`` visits in flight while layer i computes."""
         compute = torch.cuda.current_stream(self.device)
         if self.n == 0:
             return
-        self._issue(0)
+        assert self._visit % self.n == 0, "a previous forward stopped half way"
         for i in range(self.n):
-            slot = i % 2
-            if i + 1 < self.n:
-                self._issue(i + 1)
+            v = self._visit
+            slot = v % self.n_slabs
+            self._issue_until(v + self.n_slabs - 1)
             compute.wait_event(self.copied[slot])
             fn(i, self.slab_views[slot])
             self.released[slot].record(compute)
             self._released_valid[slot] = True
+            self._visit += 1

@@ -46,7 +46,9 @@ def test_streamed_forward_is_bit_identical_to_resident():
     # several forwards in a row reuse the two slabs; still identical
     for _ in range(3):
         assert torch.equal(tgt_a.prefill(prompt[:7], 40), tgt_b.prefill(prompt[:7], 40))
-    assert tgt_b.streamer.bytes_streamed == 4 * 2 * tgt_b.streamer.layout.nbytes
+    # 4 forwards x 2 streamed layers, plus the prefetch of the next forward's first layers that the ring keeps in flight
+    st = tgt_b.streamer
+    assert 4 * 2 * st.layout.nbytes <= st.bytes_streamed <= (4 * 2 + st.n_slabs - 1) * st.layout.nbytes
 
 
 def test_draft_tree_levels_are_canonical_topk():
