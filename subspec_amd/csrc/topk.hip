@@ -158,17 +158,24 @@ __global__ __launch_bounds__(kTopkThreads) void topk_slice_kernel(
   // finds, by a 16-step bit search with ballots (no memory traffic), the largest 16-bit key prefix
   // that at least m = ceil(k/4) of its lanes reach; the ceil(k/m)-th largest of those prefixes is
   // reached by at least k elements of the slice, hence a valid lower bound for its k-th best.
+  // The sample IS the first group of the streaming loop below: its four tiles stay in registers
+  // and are scanned once the threshold is known, so nothing is read twice.
+  constexpr int U = 4;
+  PTile<DT, VEC> t[U];
+#pragma unroll
+  for (int i = 0; i < U; ++i) {                        // unconditional loads (clamped index): back to back
+    const int64_t j = min((int64_t)i * kTopkThreads + tid, ntiles - 1);
+    t[i].load(probs, base + j * VEC);
+  }
   float smax = -INFINITY;
   bool sany = false;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
+  for (int i = 0; i < U; ++i) {
     const int64_t j = tid + (int64_t)i * kTopkThreads;
     if (j < ntiles) {
-      PTile<DT, VEC> t;
-      t.load(probs, base + j * VEC);
 #pragma unroll
       for (int e = 0; e < VEC; ++e) {
-        const float key = Elem<DT>::round(t.get(e) * q);
+        const float key = Elem<DT>::round(t[i].get(e) * q);
         if (!sany || key > smax) { smax = key; sany = true; }
       }
     }
@@ -217,18 +224,18 @@ __global__ __launch_bounds__(kTopkThreads) void topk_slice_kernel(
   // fast path: four tiles per thread in flight, no bookkeeping between groups.  For 16-bit rows a
   // tile is first screened with packed unsigned maxima against the bit pattern of the threshold
   // (five instructions for eight elements); only tiles that may hold a survivor are unpacked.
-  constexpr int U = 4;
   uint32_t screen = 0;                                 // (pattern - 1) in both halves; 0: screen nothing out
   if constexpr (VEC == 8) {
     const uint32_t thr = min_pattern_reaching<DT>(q, tau_key);
     screen = thr ? (thr - 1) * 0x10001u : 0;
   }
   for (int64_t g0 = 0; g0 < ngroups; g0 += U) {
-    PTile<DT, VEC> t[U];
+    if (g0 > 0) {                                      // group 0 is already in registers (the sample)
 #pragma unroll
-    for (int i = 0; i < U; ++i) {                      // unconditional loads (clamped index): back to back
-      const int64_t j = min((g0 + i) * kTopkThreads + tid, ntiles - 1);
-      t[i].load(probs, base + j * VEC);
+      for (int i = 0; i < U; ++i) {                    // unconditional loads (clamped index): back to back
+        const int64_t j = min((g0 + i) * kTopkThreads + tid, ntiles - 1);
+        t[i].load(probs, base + j * VEC);
+      }
     }
 #pragma unroll
     for (int i = 0; i < U; ++i) {
