@@ -137,7 +137,8 @@ __device__ int prune_list(uint64_t* list, int count, uint64_t cut, int* counter)
 template <int DT, int VEC>
 __global__ __launch_bounds__(kTopkThreads) void topk_slice_kernel(
     const void* __restrict__ probs, const void* __restrict__ parent_probs, int64_t vocab, int leaves, int splits,
-    int64_t chunk, int k, uint64_t* __restrict__ cand, int32_t* __restrict__ cand_count) {
+    int64_t chunk, int k, uint64_t* __restrict__ cand, int32_t* __restrict__ cand_count,
+    int64_t* __restrict__ token_ids, void* __restrict__ topk_probs, int64_t* __restrict__ parent_indices) {
   __shared__ uint64_t list[kTopkCap];
   __shared__ uint64_t kth_slot;
   __shared__ uint32_t wave_prefix[kTopkThreads / kWave];
@@ -307,6 +308,23 @@ __global__ __launch_bounds__(kTopkThreads) void topk_slice_kernel(
   int cnt = min(count, kTopkCap);
   tau = kth_best<kTopkThreads>(list, cnt, k, &kth_slot);
   cnt = prune_list<kTopkThreads>(list, cnt, tau, &count);
+  if (leaves * splits == 1) {
+    // this workgroup has seen the whole output row: rank the (distinct) candidates and write the
+    // result directly, no merge launch
+    __syncthreads();
+    for (int i = tid; i < cnt; i += kTopkThreads) {
+      const uint64_t mine = list[i];
+      int rank = 0;
+      for (int j = 0; j < cnt; ++j) rank += list[j] > mine;
+      if (rank < k) {
+        const uint32_t flat = candidate_flat(mine);
+        token_ids[row * k + rank] = flat % vocab;
+        parent_indices[row * k + rank] = flat / vocab;
+        Elem<DT>::store(topk_probs, row * k + rank, candidate_key(mine));
+      }
+    }
+    return;
+  }
   const int64_t slot0 = (row * splits + c) * kTopkMaxK;
   for (int i = tid; i < cnt; i += kTopkThreads) cand[slot0 + i] = list[i];
   if (tid == 0) cand_count[row * splits + c] = cnt;
@@ -370,12 +388,14 @@ static int run_topk(const void* probs, const void* parent_probs, int64_t batch, 
     DominantKernelTimer timer(st);
     if (pl.vec == 1)
       hipLaunchKernelGGL((topk_slice_kernel<DT, 1>), grid, dim3(kTopkThreads), 0, st, probs, parent_probs, vocab, leaves,
-                         pl.splits, pl.chunk, k, cand, cand_count);
+                         pl.splits, pl.chunk, k, cand, cand_count, token_ids, topk_probs, parent_indices);
     else
       hipLaunchKernelGGL((topk_slice_kernel<DT, (DT == SUBSPEC_F32 ? 4 : 8)>), grid, dim3(kTopkThreads), 0, st, probs,
-                         parent_probs, vocab, leaves, pl.splits, pl.chunk, k, cand, cand_count);
+                         parent_probs, vocab, leaves, pl.splits, pl.chunk, k, cand, cand_count, token_ids, topk_probs,
+                         parent_indices);
   }
-  hipLaunchKernelGGL((topk_merge_kernel<DT>), dim3((unsigned)batch), dim3(kMergeThreads), 0, st, cand, cand_count,
+  if (leaves * pl.splits > 1)
+    hipLaunchKernelGGL((topk_merge_kernel<DT>), dim3((unsigned)batch), dim3(kMergeThreads), 0, st, cand, cand_count,
                      vocab, leaves, pl.splits, k, token_ids, topk_probs, parent_indices);
   SUBSPEC_CHECK_HIP(hipGetLastError());
   return SUBSPEC_OK;
