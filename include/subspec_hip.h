@@ -174,6 +174,19 @@ int subspec_tree_attention(const void* q, const void* k_cache, const void* v_cac
                            void* stream);
 
 /* ------------------------------------------------------------------------------------------
+ * Draft probabilities: out = softmax(round(logits / temperature)) over the last axis, in the logits
+ * dtype (the quotient is rounded to the dtype first, the softmax is evaluated in fp32 and each
+ * probability rounded once).
+ *
+ * Replaces  ClassicSDDraftModel.forward(with_softmax=True): torch.softmax(logits / temperature, -1)
+ *           specdecodes/models/draft_models/classic_sd.py:10-16
+ *
+ * logits, out  device [rows, vocab], same dtype (fp32 / fp16 / bf16); out may alias logits.
+ */
+int subspec_softmax_temperature(const void* logits, void* out, int dtype, int64_t rows, int64_t vocab,
+                                float temperature, void* stream);
+
+/* ------------------------------------------------------------------------------------------
  * int4 group-wise (group 64 along the input dimension, fp16 scale and zero per row and group)
  * linear layer of the substitute draft:  y[M, N] = x[M, K] * ((Wq - zero) * scale)^T (+ bias).
  *

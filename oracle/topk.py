@@ -42,3 +42,10 @@ def topk_brute_force(sampled_probs: torch.Tensor, parent_probs: torch.Tensor, k:
         out.append([(-i) for _, i in items[:k]])
     idx = torch.tensor(out)
     return (idx % V).long(), torch.gather(buf, 1, idx), (idx // V).long()
+
+
+def draft_probs(logits: torch.Tensor, temperature: float) -> torch.Tensor:
+    """The draft's probability rows: ``torch.softmax(logits / temperature, dim=-1)`` in the logits dtype
+    (specdecodes/models/draft_models/classic_sd.py:10-16).  Pinned by the library routine itself; the
+    quotient is a tensor op and therefore rounded to the dtype before the softmax."""
+    return torch.softmax(logits / temperature, dim=-1)

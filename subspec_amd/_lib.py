@@ -53,6 +53,7 @@ _SIGNATURES = {
     "subspec_tree_attention_workspace": (_sz, [_i64, _i64, _i64, _i64]),
     "subspec_tree_attention": (C.c_int, [_p, _p, _p, _p, C.c_int, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _p, _i64,
                                          C.c_float, _p, _sz, _p]),
+    "subspec_softmax_temperature": (C.c_int, [_p, _p, C.c_int, _i64, _i64, C.c_float, _p]),
     "subspec_int4_linear_workspace": (_sz, [_i64, _i64, _i64]),
     "subspec_int4_linear": (C.c_int, [_p, _p, _p, _p, _p, C.c_int, _i64, _i64, _i64, _i64, _p, _sz, _p]),
     "subspec_int4_decoder_layer_workspace": (_sz, [C.POINTER(DecoderLayerDims)]),

@@ -48,7 +48,7 @@ class SubSpecSDDraftModel:
         return ops.topk_expand(sampled_probs.contiguous(), parent_probs.contiguous(), sample_k)
 
     def _probs(self, logits: torch.Tensor) -> torch.Tensor:
-        return torch.softmax(logits / self.draft_params.temperature, dim=-1)      # classic_sd.py:10-16
+        return ops.softmax_temperature(logits, self.draft_params.temperature)       # classic_sd.py:10-16
 
     # ------------------------------------------------------------------ tree growth
     @torch.no_grad()

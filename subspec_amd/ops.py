@@ -245,6 +245,21 @@ def int4_linear(x: torch.Tensor, wq: torch.Tensor, sz: torch.Tensor, out_feature
     return y.reshape(*x.shape[:-1], N)
 
 
+# ---------------------------------------------------------------------------------------------- draft probabilities
+def softmax_temperature(logits: torch.Tensor, temperature: float) -> torch.Tensor:
+    """``torch.softmax(logits / temperature, -1)`` in the logits dtype (draft_models/classic_sd.py:10-16)."""
+    dev = _require_gpu(logits)
+    if not temperature > 0:
+        raise ValueError("softmax_temperature: temperature must be positive")
+    x = logits.contiguous()
+    out = torch.empty_like(x)
+    vocab = x.shape[-1]
+    code = L.lib().subspec_softmax_temperature(x.data_ptr(), out.data_ptr(), _dtype_code(x), x.numel() // vocab, vocab,
+                                               float(temperature), _stream(dev))
+    L.check(code, "subspec_softmax_temperature")
+    return out
+
+
 # ---------------------------------------------------------------------------------------------- decoder layer
 def decoder_layer_dims(dtype: torch.dtype, n_rows: int, hidden: int, intermediate: int, n_q_heads: int, n_kv_heads: int,
                        head_dim: int, kv_seq_stride: int, prefix_len: int, n_tree_slots: int, rms_eps: float,

@@ -86,3 +86,31 @@ def test_argument_errors():
         ops.topk_expand(p, torch.ones(1, 1, device=DEV), 100)       # k beyond the kernel's limit
     tok, val, par = ops.topk_expand(torch.rand(1, 1, 5, device=DEV), torch.ones(1, 1, device=DEV), 50)
     assert tok.shape == (1, 5)                                     # k clamps to the vocabulary
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_draft_probabilities_softmax_with_temperature(dtype):
+    """softmax(logits / T) of a draft step against torch on the CPU.  Floating point: the two differ in
+    the last place of exp and of the row sum, so values agree to one unit in the last place of the
+    dtype (tolerance 2^-7 relative for bf16, 2^-10 for fp16, 1e-5 for fp32) and nearly all are equal."""
+    g = torch.Generator().manual_seed(11)
+    for rows, V, T in ((8, 152064, 0.2), (1, 152064, 1.0), (5, 1000, 0.7), (3, 77, 0.2)):
+        print("softmax_temperature", dtype, rows, V, T, flush=True)
+        logits = (torch.randn(rows, V, generator=g) * 3).to(dtype)
+        logits[0, 3] = float("-inf")                                  # masked entry
+        ref = ot.draft_probs(logits, T)
+        got = ops.softmax_temperature(logits.to(DEV), T).cpu()
+        assert got.dtype == dtype and got.shape == ref.shape
+        rtol = {torch.bfloat16: 2.0 ** -7, torch.float16: 2.0 ** -10, torch.float32: 1e-5}[dtype]
+        atol = {torch.bfloat16: 2.0 ** -133, torch.float16: 2.0 ** -24, torch.float32: 1e-38}[dtype]   # one subnormal step
+        assert torch.allclose(got.float(), ref.float(), rtol=rtol, atol=atol)
+        assert (got == ref).float().mean().item() >= (0.98 if dtype != torch.float32 else 0.0)
+        assert got[0, 3] == 0
+        assert torch.allclose(got.float().sum(-1), torch.ones(rows), atol=2e-2)
+        # the expansion on top of the device probabilities equals the oracle's on the same rows
+        parent = torch.rand(1, rows, generator=g).to(dtype)
+        tok, val, par = ops.topk_expand(got.reshape(1, rows, V).to(DEV), parent.to(DEV), 8)
+        e_tok, e_val, e_par = ot.topk_expand(got.reshape(1, rows, V), parent, 8)
+        assert torch.equal(tok.cpu(), e_tok) and torch.equal(val.cpu(), e_val) and torch.equal(par.cpu(), e_par)
+    with pytest.raises(ValueError):
+        ops.softmax_temperature(torch.zeros(2, 8, device=DEV), 0.0)
