@@ -73,3 +73,17 @@ def test_argument_errors():
         ops.int4_linear(torch.zeros(65, 64, dtype=torch.bfloat16, device=DEV), wq, sz, 16)  # more than 64 rows
     with pytest.raises(ValueError):
         ops.int4_linear(torch.zeros(1, 128, dtype=torch.bfloat16, device=DEV), wq, sz, 16)  # shape mismatch
+
+
+def test_random_shape_sweep():
+    """Ragged everything: tile counts that do not divide the grid, group counts that are not multiples of
+    four (dead pipeline steps), every activation-row tile count, with and without bias."""
+    g = torch.Generator().manual_seed(2024)
+    for i in range(24):
+        N = 16 * int(torch.randint(1, 700, (1,), generator=g))
+        K = 64 * int(torch.randint(1, 40, (1,), generator=g))
+        M = int(torch.randint(1, 65, (1,), generator=g))
+        _check(N, K, M, torch.bfloat16 if i % 3 else torch.float16, 500 + i, bias=bool(i % 2))
+    # a very wide layer: more tiles than one resident wave of workgroups covers with five tiles each
+    _check(16 * 6000, 256, 64, torch.bfloat16, 900)
+    _check(16 * 6000, 256, 7, torch.bfloat16, 901)
