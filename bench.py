@@ -39,6 +39,10 @@ def parse():
                     help="also run three plain copies of the logits tensor (known size) so that hardware byte counters "
                          "collected by rocprofv3 --pmc can be scaled")
     ap.add_argument("--new-tokens", type=int, default=256, help="e2e workload: tokens to generate")
+    ap.add_argument("--checkpoint", default=None,
+                    help="e2e workload: local HuggingFace checkpoint directory (config.json + *.safetensors, Qwen2 / "
+                         "Llama naming) to use instead of random-init weights of the Qwen2.5-7B shape")
+    ap.add_argument("--keep-layers", type=int, default=14, help="e2e workload: target layers kept resident; the rest stream")
     ap.add_argument("--workload", default="verify-cycle", choices=["verify-cycle", "attention", "int4", "greedy", "e2e"],
                     help="verify-cycle (default, BASELINE config 2) is the benchmark line; the others time one "
                          "kernel family of configs 1, 3 and 4 and print one JSON line per shape")
@@ -137,14 +141,19 @@ def bench_e2e(args):
     from subspec_amd.cache import create_kv_cache
     from subspec_amd.draft import SubSpecSDDraftModel
     from subspec_amd.generator import SubSpecSDGenerator
-    from subspec_amd.model import DecoderConfig, build_models
+    from subspec_amd.model import DecoderConfig, build_models, load_hf_checkpoint
     from subspec_amd.utils import DraftParams
     from subspec_amd.wandb_logger import wandb_logger
     dev = "cuda:0"
-    cfg = DecoderConfig()
     t0 = time.perf_counter()
-    kv = create_kv_cache("static", max_cache_len=2048 + 256 + 64 + 8, config=cfg, device=dev, dtype=torch.bfloat16)
-    target, draft, _ = build_models(cfg, kv, seed=0, device=dev, first_streamed=14)
+    weights = None
+    if args.checkpoint:
+        cfg, weights = load_hf_checkpoint(args.checkpoint, device=dev)
+    else:
+        cfg = DecoderConfig()
+    kv = create_kv_cache("static", max_cache_len=2048 + args.new_tokens + 64 + 8, config=cfg, device=dev, dtype=torch.bfloat16)
+    target, draft, _ = build_models(cfg, kv, seed=0, device=dev, first_streamed=min(args.keep_layers, cfg.num_hidden_layers),
+                                    weights=weights)
     print(f"# models built in {time.perf_counter() - t0:.1f} s", file=sys.stderr, flush=True)
     prompt = torch.randint(0, cfg.vocab_size, (1, 2048), generator=torch.Generator().manual_seed(0)).to(dev)
     for method, vk in (("exact", None), ("lossy", dict(threshold=0.3, window_size=6, threshold_method="entropy"))):
@@ -153,12 +162,15 @@ def bench_e2e(args):
                                  generator_kwargs=dict(verify_method=method, verify_kwargs=vk))
         kv.reset()
         wandb_logger.clear_log_data()
-        target.streamer.bytes_streamed = 0
+        if target.streamer is not None:
+            target.streamer.bytes_streamed = 0
         out = gen.generate(prompt, max_new_tokens=args.new_tokens, do_sample=False, past_key_values=kv)
         log = dict(wandb_logger.log_data)
         line = {"metric": "accepted tokens/sec, end-to-end speculative cycle", "value": round(log["tput"], 2),
-                "unit": "tokens/s", "n_gpus": 1, "higher_is_better": True, "dtype": "bf16", "data": "synthetic",
-                "config": {"workload": "BASELINE config 5: Qwen2.5-7B shape, layers 14-27 streamed, int4 draft, depth 8, k 8, "
+                "unit": "tokens/s", "n_gpus": 1, "higher_is_better": True, "dtype": "bf16",
+                "data": "synthetic prompt, weights from " + args.checkpoint if args.checkpoint else "synthetic",
+                "config": {"workload": f"BASELINE config 5: {'checkpoint' if args.checkpoint else 'Qwen2.5-7B shape'}, layers "
+                                       f"{min(args.keep_layers, cfg.num_hidden_layers)}-{cfg.num_hidden_layers - 1} streamed, int4 draft, depth 8, k 8, "
                                        f"<=64 nodes, prompt 2048, {args.new_tokens} new tokens, verify {method}",
                            "verify_method": method, "n_iter": log["n_iter"], "n_tokens": log["n_tokens"],
                            "tokens_per_cycle": round(log["avg_sampled"], 3),
@@ -166,7 +178,7 @@ def bench_e2e(args):
                            "avg_target_s": round(log.get("avg_target_time", 0), 5),
                            "avg_verify_s": round(log.get("avg_verify_time", 0), 6),
                            "elapsed_s": round(log["elapsed_time"], 3),
-                           "host_to_device_GB": round(target.streamer.bytes_streamed / 1e9, 2)}}
+                           "host_to_device_GB": round((target.streamer.bytes_streamed if target.streamer else 0) / 1e9, 2)}}
         print(json.dumps(line), flush=True)
 
 

@@ -235,11 +235,81 @@ class Decoder:
         return self.logits(self._run_layers(self.embed[token_ids], positions, rows, attn))
 
 
+def config_from_hf(config: dict) -> DecoderConfig:
+    """``DecoderConfig`` from the fields of a HuggingFace ``config.json`` (Qwen2 / Llama family)."""
+    heads = int(config["num_attention_heads"])
+    return DecoderConfig(
+        num_hidden_layers=int(config["num_hidden_layers"]), hidden_size=int(config["hidden_size"]),
+        num_attention_heads=heads, num_key_value_heads=int(config.get("num_key_value_heads", heads)),
+        head_dim=int(config.get("head_dim") or int(config["hidden_size"]) // heads),
+        intermediate_size=int(config["intermediate_size"]), vocab_size=int(config["vocab_size"]),
+        rms_norm_eps=float(config.get("rms_norm_eps", 1e-6)), rope_theta=float(config.get("rope_theta", 1e4)),
+        max_position_embeddings=int(config.get("max_position_embeddings", 32768)))
+
+
+def load_hf_checkpoint(path: str, device="cpu", dtype=torch.bfloat16):
+    """Weights of a LOCAL HuggingFace checkpoint directory (``config.json`` + ``*.safetensors``, Qwen2 or
+    Llama naming) in this package's fused layout: ``qkv_proj = q|k|v`` rows, ``gate_up_proj = gate|up`` rows.
+    Returns ``(DecoderConfig, weights)`` with ``weights`` as produced by ``init_weights``.
+
+    The reference loads the same checkpoints by model name through ``AutoModelForCausalLM.from_pretrained``
+    (run/core/builder.py:94-103); nothing is downloaded here and only safetensors files are read."""
+    import glob
+    import json
+    import os
+
+    from safetensors import safe_open
+
+    with open(os.path.join(path, "config.json")) as f:
+        hf = json.load(f)
+    cfg = config_from_hf(hf)
+    tensors: Dict[str, torch.Tensor] = {}
+    files = sorted(glob.glob(os.path.join(path, "*.safetensors")))
+    if not files:
+        raise FileNotFoundError(f"no .safetensors file in {path}")
+    for fn in files:
+        with safe_open(fn, framework="pt", device="cpu") as sf:
+            for key in sf.keys():
+                tensors[key] = sf.get_tensor(key)
+
+    def take(name: str, required: bool = True) -> Optional[torch.Tensor]:
+        t = tensors.get(name)
+        if t is None:
+            if required:
+                raise KeyError(f"{name} missing from the checkpoint in {path}")
+            return None
+        return t.to(device=device, dtype=dtype)
+
+    layers = []
+    for i in range(cfg.num_hidden_layers):
+        pre = f"model.layers.{i}."
+        w = {"input_layernorm.weight": take(pre + "input_layernorm.weight"),
+             "post_attention_layernorm.weight": take(pre + "post_attention_layernorm.weight"),
+             "qkv_proj.weight": torch.cat([take(pre + f"self_attn.{n}_proj.weight") for n in "qkv"], 0),
+             "o_proj.weight": take(pre + "self_attn.o_proj.weight"),
+             "gate_up_proj.weight": torch.cat([take(pre + "mlp.gate_proj.weight"), take(pre + "mlp.up_proj.weight")], 0),
+             "down_proj.weight": take(pre + "mlp.down_proj.weight")}
+        biases = [take(pre + f"self_attn.{n}_proj.bias", required=False) for n in "qkv"]
+        # Qwen2 has q/k/v biases, Llama has none: a zero bias keeps one layer layout for both
+        sizes = (cfg.q_size, cfg.kv_size, cfg.kv_size)
+        w["qkv_proj.bias"] = torch.cat([b if b is not None else torch.zeros(n, device=device, dtype=dtype)
+                                        for b, n in zip(biases, sizes)], 0)
+        for name, shape in layer_shapes(cfg).items():
+            if name in w and tuple(w[name].shape) != tuple(shape):
+                raise ValueError(f"layer {i}: {name} has shape {tuple(w[name].shape)}, expected {tuple(shape)}")
+        layers.append(w)
+    embed = take("model.embed_tokens.weight")
+    head = take("lm_head.weight", required=False)
+    if head is None:                                              # tie_word_embeddings
+        head = embed
+    return cfg, {"embed": embed, "layers": layers, "norm": take("model.norm.weight"), "lm_head": head}
+
+
 def build_models(cfg: DecoderConfig, kv: KVManager, seed: int = 0, device="cuda:0", dtype=torch.bfloat16,
-                 first_streamed: Optional[int] = None):
+                 first_streamed: Optional[int] = None, weights: Optional[dict] = None):
     """Target (bf16, layers >= first_streamed in pinned host memory) and substitute draft (same
     weights, int4 g64, resident) over one shared KV cache."""
-    w = init_weights(cfg, seed, device, dtype)
+    w = init_weights(cfg, seed, device, dtype) if weights is None else weights     # e.g. from load_hf_checkpoint
     draft_layers = quantize_layers(w["layers"])
     streamer = None
     layers = w["layers"]
