@@ -146,9 +146,10 @@ int subspec_topk_expand(const void* probs, const void* parent_probs, int dtype, 
 /* ------------------------------------------------------------------------------------------
  * Tree-masked GQA attention of the draft tree against the static KV cache:
  * out = softmax(q k^T * scale + mask) v, where query row i attends to cache rows [0, prefix_len) and
- * to tree slot prefix_len + j (j < n_tree_slots <= 64) iff bit j of anc_bits[i] is set (the node in
- * slot j is row i's node or one of its ancestors).  The verify forward has one query row per slot;
- * a draft step queries only the newest level (n_rows < n_tree_slots).
+ * to tree slot prefix_len + j (j < n_tree_slots <= 128) iff bit j of row i's ancestor bitset is set (the
+ * node in slot j is row i's node or one of its ancestors).  The verify forward has one query row per
+ * slot; a draft step queries only the newest level (n_rows < n_tree_slots); a tree extended during
+ * the target forward (post-speculation) may occupy up to 128 slots.
  *
  * Replaces  HF sdpa_attention_forward under SDPBackend.MATH with the additive finfo.min mask and
  *           repeat_kv, as reached from _tree_decoding   specdecodes/models/generators/classic_sd.py:57-109
@@ -161,7 +162,8 @@ int subspec_topk_expand(const void* probs, const void* parent_probs, int dtype, 
  * k_cache    device [batch, n_kv_heads, kv_seq_stride, head_dim]  (HF static-cache layout); the K/V of
  * v_cache    the tree nodes must already sit in rows prefix_len .. prefix_len + n_tree_slots - 1
  * out        device [batch, n_rows, n_q_heads, head_dim]       (= [batch, n_rows, hidden])
- * anc_bits   device uint64 [*, n_rows]; batch element b uses row b * anc_batch_stride (0: shared tree)
+ * anc_bits   device uint64 [*, n_rows, words], words = 1 for n_tree_slots <= 64, else 2 (bit j of a row is bit
+ *            j % 64 of word j / 64); batch element b uses rows from b * anc_batch_stride (0: shared tree)
  * workspace  partial results when the keys are split over workgroups (may be NULL if the size is 256)
  */
 size_t subspec_tree_attention_workspace(int64_t batch, int64_t n_q_heads, int64_t prefix_len, int64_t n_tree_slots);
@@ -231,9 +233,9 @@ int subspec_int4_linear(const void* x, const uint32_t* wq, const uint32_t* sz, c
  * x           device [n_rows, hidden], updated in place (the residual stream)
  * positions   device int32 [n_rows]   rotary position of each row (prefix_len + node depth)
  * cache_rows  device int32 [n_rows]   cache row each row's K / V is written to (prefix_len + slot)
- * anc_bits    device uint64 [n_rows]  as for subspec_tree_attention
+ * anc_bits    device uint64 [n_rows, words]  as for subspec_tree_attention (words = 2 above 64 tree slots)
  * k_cache, v_cache  device [n_kv_heads, kv_seq_stride, head_dim] of THIS layer (batch 1)
- * Limits: n_rows <= 64, n_tree_slots <= 64, head_dim 128, hidden % 64 == 0 and <= 16384,
+ * Limits: n_rows <= 64, n_tree_slots <= 128, head_dim 128, hidden % 64 == 0 and <= 16384,
  *         intermediate % 64 == 0.
  */
 typedef struct subspec_decoder_layer_dims {

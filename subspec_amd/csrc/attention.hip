@@ -9,9 +9,10 @@
 // Layout and mapping
 //   q        [B, Hq, n, D]            (n <= 64 query rows, D = 128)
 //   k, v     [B, Hkv, S, D]           static cache; rows [0, prefix) are the prompt, rows
-//                                     [prefix, prefix + slots) hold the tree nodes (slots <= 64)
-//   anc      [B or 1, n] u64          bit j of word i: query row i may attend to tree slot j
-//                                     (the node in slot j is the row's node or one of its ancestors)
+//                                     [prefix, prefix + slots) hold the tree nodes (slots <= 128)
+//   anc      [B or 1, n, words] u64   bit j of row i (word j / 64): query row i may attend to tree slot j
+//                                     (the node in slot j is the row's node or one of its ancestors);
+//                                     words = 1 for up to 64 tree slots, 2 for up to 128
 //   out      [B, n, Hq, D]
 // One workgroup (8 wavefronts) owns FOUR query heads of one KV head (256 rows) and one chunk of
 // the keys, so a staged K/V tile feeds four heads' worth of matrix work; wavefront w owns 32 rows
@@ -72,6 +73,7 @@ __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
 
 struct AttnParams {
   int64_t batch, hq, hkv, n_rows, n_slots, seq_stride, prefix, anc_batch_stride;
+  int mask_words;              // 64-bit words per ancestor bitset: 1 (<= 64 tree slots) or 2 (<= 128)
   int chunks;
   int64_t chunk_keys;          // multiple of kKeyBlock
   int pairs_per_kv;            // workgroups (head pairs) per KV head
@@ -113,7 +115,7 @@ __global__ __launch_bounds__(kAttnThreads) __attribute__((amdgpu_waves_per_eu(2,
   int row[2];
   bool row_ok[2];
   uint4 qreg[2][kAttnD / 32];
-  uint64_t bits[2];
+  uint64_t bits[2][2];                                  // [row tile][mask word]
 #pragma unroll
   for (int nt = 0; nt < 2; ++nt) {
     row[nt] = (wave & 1) * 32 + nt * 16 + lq;
@@ -122,7 +124,9 @@ __global__ __launch_bounds__(kAttnThreads) __attribute__((amdgpu_waves_per_eu(2,
 #pragma unroll
     for (int ks = 0; ks < kAttnD / 32; ++ks)
       qreg[nt][ks] = row_ok[nt] ? *(const uint4*)(qp + ks * 32 + lg * 8) : make_uint4(0, 0, 0, 0);
-    bits[nt] = row_ok[nt] ? anc[(int64_t)b * ap.anc_batch_stride + row[nt]] : 0ull;
+    const uint64_t* ap_bits = anc + ((int64_t)b * ap.anc_batch_stride + row[nt]) * ap.mask_words;
+    bits[nt][0] = row_ok[nt] ? ap_bits[0] : 0ull;
+    bits[nt][1] = (row_ok[nt] && ap.mask_words > 1) ? ap_bits[1] : 0ull;
   }
 
   v4f oacc[2][kAttnD / 16];
@@ -231,10 +235,12 @@ __global__ __launch_bounds__(kAttnThreads) __attribute__((amdgpu_waves_per_eu(2,
           const int64_t pos = kb + kt * 16 + lg * 4 + r;
           const bool in_range = pos < kv_len;
           const bool tree = pos >= ap.prefix;
-          const int sh = tree ? (int)(pos - ap.prefix) & 63 : 0;
+          const int rel = tree ? (int)(pos - ap.prefix) : 0;   // tree slot, < 64 * mask_words
+          const int sh = rel & 63;
 #pragma unroll
           for (int nt = 0; nt < 2; ++nt) {
-            const bool ok = in_range && (!tree || ((bits[nt] >> sh) & 1ull));
+            const uint64_t word = rel < 64 ? bits[nt][0] : bits[nt][1];
+            const bool ok = in_range && (!tree || ((word >> sh) & 1ull));
             const float t = ok ? acc[kt][nt][r] : -INFINITY;
             s[nt][kt][r] = t;
             mloc[nt] = fmaxf(mloc[nt], t);
@@ -382,8 +388,8 @@ extern "C" int subspec_tree_attention(const void* q, const void* k_cache, const 
                  (long long)n_kv_heads);
   if (n_rows <= 0 || n_rows > kAttnRows)
     SUBSPEC_FAIL(SUBSPEC_ERR_LIMIT, "tree_attention: n_rows=%lld outside [1, %d]", (long long)n_rows, kAttnRows);
-  if (n_tree_slots < 1 || n_tree_slots > 64)
-    SUBSPEC_FAIL(SUBSPEC_ERR_LIMIT, "tree_attention: n_tree_slots=%lld outside [1, 64] (one 64-bit mask word per row)",
+  if (n_tree_slots < 1 || n_tree_slots > 128)
+    SUBSPEC_FAIL(SUBSPEC_ERR_LIMIT, "tree_attention: n_tree_slots=%lld outside [1, 128] (at most two 64-bit mask words per row)",
                  (long long)n_tree_slots);
   if (prefix_len < 0 || prefix_len + n_tree_slots > kv_seq_stride)
     SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "tree_attention: prefix_len=%lld + n_tree_slots=%lld exceeds the cache length %lld",
@@ -395,6 +401,7 @@ extern "C" int subspec_tree_attention(const void* q, const void* k_cache, const 
   ap.batch = batch; ap.hq = n_q_heads; ap.hkv = n_kv_heads; ap.n_rows = n_rows; ap.n_slots = n_tree_slots;
   ap.seq_stride = kv_seq_stride;
   ap.prefix = prefix_len; ap.anc_batch_stride = anc_batch_stride;
+  ap.mask_words = n_tree_slots > 64 ? 2 : 1;
   const int64_t kv_len = prefix_len + n_tree_slots;
   ap.chunks = attn_chunks(batch, n_q_heads, kv_len);
   const int64_t blocks = (kv_len + kKeyBlock - 1) / kKeyBlock;

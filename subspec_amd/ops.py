@@ -166,22 +166,37 @@ def topk_expand(sampled_probs: torch.Tensor, parent_probs: torch.Tensor, k: int,
     return token_ids, vals, parents
 
 
+def bits_to_words(bits, n_slots: int, device=None) -> torch.Tensor:
+    """Python-int bitsets -> int64 tensor [n] (up to 64 slots) or [n, 2] (up to 128 slots): bit j of a row is
+    bit j % 64 of word j // 64."""
+    def signed(w):
+        return w - (1 << 64) if w >= (1 << 63) else w
+    mask = (1 << 64) - 1
+    if n_slots <= 64:
+        return torch.tensor([signed(int(b) & mask) for b in bits], dtype=torch.int64, device=device)
+    if n_slots > 128:
+        raise ValueError(f"{n_slots} tree slots exceed the 128 the attention kernel masks")
+    return torch.tensor([[signed(int(b) & mask), signed((int(b) >> 64) & mask)] for b in bits], dtype=torch.int64,
+                        device=device)
+
+
 def ancestor_bits_tensor(parents, device=None) -> torch.Tensor:
-    """uint64 ancestor-or-self bitsets (as an int64 tensor) from a parent array with parent < child."""
+    """uint64 ancestor-or-self bitsets (as an int64 tensor, [n] or [n, 2] above 64 nodes) from a parent
+    array with parent < child."""
     bits = []
     for i, p in enumerate(parents):
         v = (1 << i) | (bits[int(p)] if int(p) >= 0 else 0)
         bits.append(v)
-    signed = [b - (1 << 64) if b >= (1 << 63) else b for b in bits]
-    return torch.tensor(signed, dtype=torch.int64, device=device)
+    return bits_to_words(bits, len(bits), device)
 
 
 def tree_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, anc_bits: torch.Tensor,
                    prefix_len: int, scale: Optional[float] = None, workspace: Optional[torch.Tensor] = None,
                    n_tree_slots: Optional[int] = None):
     """``q`` [B, Hq, n, D], caches [B, Hkv, S, D] (tree K/V already written at rows prefix_len..),
-    ``anc_bits`` int64 [n] (shared tree) or [B, n]: bit j = row may attend to tree slot j.
-    ``n_tree_slots`` (default n) is the number of occupied tree slots.  Returns [B, n, Hq * D]."""
+    ``anc_bits`` int64 [n] (shared tree) or [B, n], with a trailing dimension of 2 words when more than 64
+    tree slots are occupied: bit j = row may attend to tree slot j.  ``n_tree_slots`` (default n) is the
+    number of occupied tree slots (<= 128).  Returns [B, n, Hq * D]."""
     dev = _require_gpu(q, k_cache, v_cache, anc_bits)
     if q.dim() != 4 or k_cache.dim() != 4 or v_cache.shape != k_cache.shape:
         raise ValueError("expected q [B, Hq, n, D] and k/v caches [B, Hkv, S, D]")
@@ -193,15 +208,18 @@ def tree_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
         raise ValueError("cache shape does not match q")
     if not (k_cache.is_contiguous() and v_cache.is_contiguous()):
         raise ValueError("tree_attention: the KV caches must be contiguous [B, Hkv, S, D]")
-    if anc_bits.dtype != torch.int64 or anc_bits.shape[-1] != n:
-        raise ValueError("anc_bits must be int64 with one word per tree row")
+    slots = n if n_tree_slots is None else int(n_tree_slots)
+    words = 2 if slots > 64 else 1
+    rows_shape = anc_bits.shape[:-1] if words == 2 else anc_bits.shape       # [n] or [B, n]
+    if anc_bits.dtype != torch.int64 or (words == 2 and anc_bits.shape[-1] != 2) or len(rows_shape) not in (1, 2) \
+            or rows_shape[-1] != n:
+        raise ValueError("anc_bits must be int64 [n] / [B, n] (two words per row, [..., n, 2], above 64 tree slots)")
     q = q.contiguous()
     anc_bits = anc_bits.contiguous()
-    if anc_bits.dim() == 2 and anc_bits.shape[0] not in (1, B):
+    if len(rows_shape) == 2 and rows_shape[0] not in (1, B):
         raise ValueError("anc_bits batch dimension must be 1 or B")
-    stride = n if (anc_bits.dim() == 2 and anc_bits.shape[0] == B and B > 1) else 0
+    stride = n if (len(rows_shape) == 2 and rows_shape[0] == B and B > 1) else 0
     lib = L.lib()
-    slots = n if n_tree_slots is None else int(n_tree_slots)
     need = lib.subspec_tree_attention_workspace(B, Hq, int(prefix_len), slots)
     if workspace is None and need > 256:
         workspace = torch.empty(need, dtype=torch.uint8, device=dev)
@@ -305,7 +323,7 @@ def int4_decoder_layer_(x: torch.Tensor, dims: "L.DecoderLayerDims", weights: "L
     if not (x.is_contiguous() and k_cache.is_contiguous() and v_cache.is_contiguous()):
         raise ValueError("decoder layer: x and the layer's cache views must be contiguous")
     if x.shape != (dims.n_rows, dims.hidden) or positions.numel() != dims.n_rows or cache_rows.numel() != dims.n_rows \
-            or anc_bits.numel() != dims.n_rows:
+            or anc_bits.numel() != dims.n_rows * (2 if dims.n_tree_slots > 64 else 1):
         raise ValueError("decoder layer: tensor shapes do not match the dimensions given")
     code = L.lib().subspec_int4_decoder_layer(
         ctypes.byref(dims), ctypes.byref(weights), x.data_ptr(), positions.data_ptr(), cache_rows.data_ptr(),

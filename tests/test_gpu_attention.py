@@ -63,6 +63,31 @@ def test_stale_cache_tail_and_per_batch_trees():
     assert torch.allclose(out, ref, rtol=1e-2, atol=2e-2)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_extended_tree_up_to_128_slots(dtype):
+    """A tree grown during the target forward occupies up to 128 slots (two mask words per row); the
+    query rows are a window of at most 64 of its nodes."""
+    for seed, (B, n_slots, P, S) in enumerate([(1, 128, 70, 256), (2, 100, 1000, 1200), (1, 65, 0, 80)]):
+        g = torch.Generator().manual_seed(40 + seed)
+        parents, _, _ = W.random_tree(g, n=n_slots, max_depth=16, max_children=4, vocab=1000, chain_depth=16)
+        q = torch.randn(B, 8, n_slots, 128, generator=g).to(dtype)
+        k = torch.randn(B, 2, S, 128, generator=g).to(dtype)
+        v = torch.randn(B, 2, S, 128, generator=g).to(dtype)
+        k[:, :, P + n_slots:] = 1e3                                   # stale rows beyond the tree
+        ref = oa.tree_attention(q, k, v, parents, P)                   # all n_slots rows
+        anc = ops.ancestor_bits_tensor(parents, device=DEV)
+        assert anc.shape == (n_slots, 2)
+        for lo, hi in ((0, 64), (n_slots - 40, n_slots), (60, 70)):
+            print("attention 128-slot", dtype, B, n_slots, P, lo, hi, flush=True)
+            out = ops.tree_attention(q[:, :, lo:hi].contiguous().to(DEV), k.to(DEV), v.to(DEV), anc[lo:hi].contiguous(), P,
+                                     n_tree_slots=n_slots).float().cpu()
+            want = ref[:, lo:hi]
+            assert (out - want).abs().amax().item() <= 1e-2 * want.abs().amax().item()
+            assert torch.allclose(out, want, rtol=1e-2, atol=2e-2)
+    with pytest.raises(ValueError):
+        ops.ancestor_bits_tensor([-1] + list(range(128)))              # 129 nodes
+
+
 def test_argument_errors():
     q = torch.zeros(1, 4, 8, 128, dtype=torch.bfloat16, device=DEV)
     k = torch.zeros(1, 2, 64, 128, dtype=torch.bfloat16, device=DEV)
