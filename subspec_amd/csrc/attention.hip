@@ -40,7 +40,7 @@ constexpr int kHeadsPerWG = 4;
 constexpr int kAttnD = 128;
 constexpr int kKeyBlock = 64;
 constexpr int kKStride = kAttnD + 8;   // LDS row stride (elements) of the K tile
-constexpr int kVStride = kKeyBlock + 8;  // LDS row stride (elements) of the transposed V tile
+constexpr int kVStride = kAttnD + 16;  // LDS row stride (elements) of the V tile: 8-dword rows of the transposing reads tile the banks
 constexpr int kXcds = 8;
 
 typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
@@ -71,6 +71,15 @@ __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
   }
 }
 
+// Transposing LDS read of 16-bit elements (ds_read_b64_tr_b16): within each group of 16 lanes,
+// lane i receives element i%4 of the four 8-byte rows addressed by lanes i/4, i/4 + 4, i/4 + 8,
+// i/4 + 12 of the group.
+typedef short v4s_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ uint2 lds_read_tr16(const uint16_t* p) {
+  const v4s_t v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s_t*)p);
+  return __builtin_bit_cast(uint2, v);
+}
+
 struct AttnParams {
   int64_t batch, hq, hkv, n_rows, n_slots, seq_stride, prefix, anc_batch_stride;
   int mask_words;              // 64-bit words per ancestor bitset: 1 (<= 64 tree slots) or 2 (<= 128)
@@ -86,9 +95,9 @@ __global__ __launch_bounds__(kAttnThreads) __attribute__((amdgpu_waves_per_eu(2,
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ kc, const uint16_t* __restrict__ vc,
     const uint64_t* __restrict__ anc, AttnParams ap, uint16_t* __restrict__ out, float* __restrict__ part_o,
     float* __restrict__ part_ml) {
-  // two stages of (K row-major, V transposed): block i+1 is written while block i is multiplied
+  // two stages of (K, V), both row-major [key][d]: block i+1 is written while block i is multiplied
   __shared__ __attribute__((aligned(16))) uint16_t Ks2[2][kKeyBlock * kKStride];
-  __shared__ __attribute__((aligned(16))) uint16_t Vt2[2][kAttnD * kVStride];
+  __shared__ __attribute__((aligned(16))) uint16_t Vs2[2][kKeyBlock * kVStride];
 
   // workgroups of one (batch, kv head, chunk) unit sit in consecutive slots of one XCD
   const int64_t lin = blockIdx.x;
@@ -158,31 +167,14 @@ __global__ __launch_bounds__(kAttnThreads) __attribute__((amdgpu_waves_per_eu(2,
     v0 = *(const uint4*)(vbase + p0_ * kAttnD + sdc * 8);                                        \
     v1 = *(const uint4*)(vbase + p1_ * kAttnD + sdc * 8);                                        \
   } while (0)
-  // V^T[d][column]: the eight keys one lane needs for a 32-key MFMA step (keys 32j + 4g + r and
-  // 32j + 16 + 4g + r) are stored contiguously (column 32j + 8g + 4h + r for key 32j + 16h + 4g + r),
-  // and the 16-byte column groups are XOR-swizzled with d/8 to spread the banks of the
-  // transposing writes
-  auto vt_column = [&](int key) {
-    const int grp = ((key >> 5) << 2) | ((key >> 2) & 3);                    // 4j + g
-    return ((grp ^ (sdc & 7)) << 3) | (((key >> 4) & 1) << 2) | (key & 3);
-  };
-  const int col0 = vt_column(skey), col1 = vt_column(skey + 32);
-#define SUBSPEC_ATTN_VT(VTW, V, COL)                                                             \
-  do {                                                                                           \
-    uint16_t* p_ = (VTW) + (sdc * 8) * kVStride + (COL);                                         \
-    p_[0 * kVStride] = (uint16_t)((V).x & 0xffffu); p_[1 * kVStride] = (uint16_t)((V).x >> 16);  \
-    p_[2 * kVStride] = (uint16_t)((V).y & 0xffffu); p_[3 * kVStride] = (uint16_t)((V).y >> 16);  \
-    p_[4 * kVStride] = (uint16_t)((V).z & 0xffffu); p_[5 * kVStride] = (uint16_t)((V).z >> 16);  \
-    p_[6 * kVStride] = (uint16_t)((V).w & 0xffffu); p_[7 * kVStride] = (uint16_t)((V).w >> 16);  \
-  } while (0)
 #define SUBSPEC_ATTN_STAGE(BUF)                                                                  \
   do {                                                                                           \
     uint16_t* ksw_ = Ks2[BUF];                                                                   \
-    uint16_t* vtw_ = Vt2[BUF];                                                                   \
+    uint16_t* vsw_ = Vs2[BUF];                                                                   \
     *(uint4*)(ksw_ + skey * kKStride + sdc * 8) = k0;                                            \
     *(uint4*)(ksw_ + (skey + 32) * kKStride + sdc * 8) = k1;                                     \
-    SUBSPEC_ATTN_VT(vtw_, v0, col0);                                                             \
-    SUBSPEC_ATTN_VT(vtw_, v1, col1);                                                             \
+    *(uint4*)(vsw_ + skey * kVStride + sdc * 8) = v0;                                            \
+    *(uint4*)(vsw_ + (skey + 32) * kVStride + sdc * 8) = v1;                                     \
   } while (0)
 
   SUBSPEC_ATTN_FETCH(key0);
@@ -198,7 +190,7 @@ __global__ __launch_bounds__(kAttnThreads) __attribute__((amdgpu_waves_per_eu(2,
       if (kb + 2 * kKeyBlock < key1) SUBSPEC_ATTN_FETCH(kb + 2 * kKeyBlock);
     }
     const uint16_t* Ks = Ks2[buf];
-    const uint16_t* Vt = Vt2[buf];
+    const uint16_t* Vs = Vs2[buf];
 
     // ---- S^T tiles: 4 x (16 keys x 16 queries) per row tile; lane holds keys 16*kt + 4*lg + r of query lq.
     //      Scores stay unscaled; the softmax scale is folded into the exp2 argument.
@@ -282,13 +274,19 @@ __global__ __launch_bounds__(kAttnThreads) __attribute__((amdgpu_waves_per_eu(2,
         pb[nt][j] = make_uint4(pack2<DT>(p[0], p[1]), pack2<DT>(p[2], p[3]), pack2<DT>(p[4], p[5]), pack2<DT>(p[6], p[7]));
       }
     }
-    // ---- O^T += V^T P^T : 8 tiles of 16 head-dims, two 32-key steps, the same V^T operand for both row tiles
+    // ---- O^T += V^T P^T : 8 tiles of 16 head-dims, two 32-key steps, the same V^T operand for both row tiles.
+    //      V sits row-major in LDS; the transposing LDS read hands lane (lq, lg) the values
+    //      V[key_e][16*mt + lq], e = 0..3, when lane r of the 16-lane group supplies the address of
+    //      V[key_{r/4}][16*mt + 4*(r%4)].  Two such reads (keys 32j + 4lg + e and 32j + 16 + 4lg + e)
+    //      give the eight keys of the lane's k indices, in the order the P^T operand uses.
+    const uint16_t* vlane = Vs + (lg * 4 + (lq >> 2)) * kVStride + (lq & 3) * 4;
 #pragma unroll
     for (int mt = 0; mt < kAttnD / 16; ++mt) {
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
-        const int d = mt * 16 + lq;
-        const uint4 a = *(const uint4*)(Vt + d * kVStride + (((j * 4 + lg) ^ ((d >> 3) & 7)) << 3));
+        const uint16_t* vp = vlane + (j * 32) * kVStride + mt * 16;
+        const uint2 lo = lds_read_tr16(vp), hi = lds_read_tr16(vp + 16 * kVStride);
+        const uint4 a = make_uint4(lo.x, lo.y, hi.x, hi.y);
         oacc[0][mt] = mfma32<DT>(a, pb[0][j], oacc[0][mt]);
         oacc[1][mt] = mfma32<DT>(a, pb[1][j], oacc[1][mt]);
       }
