@@ -43,7 +43,7 @@ def parse():
                     help="e2e workload: local HuggingFace checkpoint directory (config.json + *.safetensors, Qwen2 / "
                          "Llama naming) to use instead of random-init weights of the Qwen2.5-7B shape")
     ap.add_argument("--keep-layers", type=int, default=14, help="e2e workload: target layers kept resident; the rest stream")
-    ap.add_argument("--workload", default="verify-cycle", choices=["verify-cycle", "attention", "int4", "greedy", "e2e"],
+    ap.add_argument("--workload", default="verify-cycle", choices=["verify-cycle", "attention", "int4", "greedy", "sampling", "e2e"],
                     help="verify-cycle (default, BASELINE config 2) is the benchmark line; the others time one "
                          "kernel family of configs 1, 3 and 4 and print one JSON line per shape")
     return ap.parse_args()
@@ -195,6 +195,28 @@ def bench_greedy(args):
                  kernel_us, 64 * 152064 * 4, 0, "subspec::row_partial_kernel")
 
 
+def bench_sampling(args):
+    """Config 2's logits verified against a SAMPLED target (temperature 0.8): statistics pass + one
+    Philox draw per row + walk.  The draw re-reads the rows, so its algorithmic bytes are the rows again."""
+    import torch
+    from subspec_amd import ops, workloads as W
+    dev = torch.device("cuda:0")
+    cfg = W.lossy_config(0, batch=32, device=dev)
+    tok = torch.tensor(cfg["tokens"], dtype=torch.int32, device=dev)
+    par = torch.tensor(cfg["parents"], dtype=torch.int32, device=dev)
+    ws = torch.empty(ops.L.lib().subspec_tree_verify_workspace(32, 64, 152064, 2), dtype=torch.uint8, device=dev)
+    step = [0]
+
+    def fn():
+        step[0] += 1
+        ops.tree_verify(cfg["logits"], tok, par, workspace=ws, verify_method="exact", do_sample=True, temperature=0.8,
+                        seed=1, offset=step[0])
+
+    call_us, kernel_us = _time_us(fn, args.steps, args.warmup)
+    _kernel_line("sampling tree verify latency", "config 2 logits [32,64,152064] bf16, sampled target (T = 0.8), exact walk",
+                 call_us, kernel_us, 32 * 64 * 152064 * 2, 0, "subspec::row_sample_kernel")
+
+
 def cpu_baseline(cfg, probs_rows, parent_rows, n_trees, min_seconds):
     """The oracle (torch-on-CPU restatement of the reference path) on a bounded sample of the same
     workload: `n_trees` trees of the batch + their 64 top-k rows each, repeated until at least
@@ -252,7 +274,8 @@ def main():
         sys.exit(1)
     L.lib()                                            # fail loudly when the HIP library is missing
     if args.workload != "verify-cycle":
-        {"attention": bench_attention, "int4": bench_int4, "greedy": bench_greedy, "e2e": bench_e2e}[args.workload](args)
+        {"attention": bench_attention, "int4": bench_int4, "greedy": bench_greedy, "sampling": bench_sampling,
+         "e2e": bench_e2e}[args.workload](args)
         return
     dev = torch.device("cuda:0")
     B, V, n, k = args.batch, args.vocab, 64, 16

@@ -102,6 +102,38 @@ int subspec_tree_verify(const void* logits, int dtype, int64_t batch, int64_t ro
                         int64_t* node_target, float* node_entropy, float* node_child_prob,
                         void* stream);
 
+/* Tree verification with a SAMPLED target token (do_sample=True).
+ *
+ * Replaces the same call sites as subspec_tree_verify when the generator samples:
+ *   GeneratorBase._sample_token(do_sample=True)   specdecodes/models/generators/base.py:116-132
+ *     (TemperatureLogitsWarper, softmax in the logits dtype, torch.multinomial(probs, 1))
+ *   ClassicSDGeneratorBase._verify_step            specdecodes/models/generators/classic_sd.py:111-116
+ *   lossy_bottom_up_verify target_tokens           specdecodes/models/utils/lossy_tree_verify.py:75-77
+ *
+ * Every logits row is divided by `temperature` and rounded to its dtype, its probabilities
+ * p_i = softmax rounded to the dtype are formed as in subspec_tree_verify, and ONE token per row is
+ * drawn by the exponential race  argmax_i p_i / E_i  (first index on equal keys),
+ *   E_i = -log(u_i),  u_i = ((w >> 9) + 0.5) * 2^-23,
+ *   w   = word (i mod 4) of Philox4x32-10(counter = {i / 4, batch_index * rows + row,
+ *                                                    offset low word, offset high word},
+ *                                         key = {seed low word, seed high word}).
+ * The draw of a row is used wherever the greedy verifier uses the row's argmax: at most one draw
+ * per context, as in the reference's walk.  The probability gate, the entropy gate and
+ * node_child_prob / node_entropy refer to the warped rows; node_target holds the draws.  Callers
+ * advance `offset` between calls to get fresh noise from one seed.  Other arguments, outputs and
+ * the workspace are those of subspec_tree_verify.  A one-node tree (n_nodes = 1, rows = 1) returns
+ * the draw of a single row in out_tokens[0]: the first token after the prefill.
+ */
+int subspec_tree_verify_sample(const void* logits, int dtype, int64_t batch, int64_t rows, int64_t vocab,
+                               const int32_t* token_ids, const int32_t* parents, int64_t n_nodes,
+                               int32_t root, int32_t skip_nodes, int64_t eos_token_id,
+                               int verify_method, int threshold_method, double threshold,
+                               int32_t window_size, int entropy_policy, float temperature, uint64_t seed,
+                               uint64_t offset, void* workspace, size_t workspace_bytes,
+                               int64_t* out_tokens, int64_t* out_ctx, int32_t* out_counts,
+                               int64_t* node_target, float* node_entropy, float* node_child_prob,
+                               void* stream);
+
 /* ------------------------------------------------------------------------------------------
  * KV-cache compaction after verification: for every slab (one [seq, row_bytes] matrix: one
  * layer x {K,V} x batch x kv-head), row offset+j <- row offset+ctx[j] for j < count, with
@@ -187,6 +219,17 @@ int subspec_tree_attention(const void* q, const void* k_cache, const void* v_cac
  */
 int subspec_softmax_temperature(const void* logits, void* out, int dtype, int64_t rows, int64_t vocab,
                                 float temperature, void* stream);
+
+/* TemperatureLogitsWarper alone: out[i] = logits[i] / temperature, the IEEE quotient rounded once to
+ * the logits dtype (what ``scores / temperature`` gives for a tensor in that dtype).
+ *
+ * Replaces  logits_processor(None, logits) with a TemperatureLogitsWarper in
+ *           GeneratorBase._sample_token   specdecodes/models/generators/base.py:57-58,121-123
+ * for callers that want the warped scores themselves; the sampling verifier and
+ * subspec_softmax_temperature apply the same quotient internally.  n = number of elements.
+ */
+int subspec_temperature_warp(const void* logits, void* out, int dtype, int64_t n, float temperature,
+                             void* stream);
 
 /* ------------------------------------------------------------------------------------------
  * int4 group-wise (group 64 along the input dimension, fp16 scale and zero per row and group)

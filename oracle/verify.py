@@ -46,14 +46,20 @@ def exact_verify(
     root: int = 0,
     eos_token_id: Optional[int] = None,
     skip_nodes: int = 0,
+    target_tokens: Optional[Sequence[int]] = None,
 ) -> Tuple[List[int], List[int], Tuple[int, int]]:
-    """Greedy walk (tree_verify.py:49-106).
+    """Walk from the root (tree_verify.py:49-106).  The target token of a context is the argmax of
+    its row, or, for a sampling target, ``target_tokens[row]``: the reference draws
+    ``p.multinomial(1)`` once per visited context (classic_sd.py:112; the bonus draw of :99-100 is
+    taken only for a context that has not been drawn yet), so one pre-drawn token per row
+    restates it.
 
     ``token_ids``/``children`` use ORIGINAL node indexing for the whole tree;
     ``probs[r]`` is the distribution at original node ``r + skip_nodes``.
     Returns (sampled_tokens, hidden_indices (original indexing), (total_len, accept_len)).
     """
     rows = int(probs.shape[0])
+    target = (lambda r: int(probs[r].argmax())) if target_tokens is None else (lambda r: int(target_tokens[r]))
     cur = int(root)
     out_tok: List[int] = []
     out_ctx: List[int] = []
@@ -62,7 +68,7 @@ def exact_verify(
     kids = list(children[cur])
     while kids:
         total += 1
-        t = int(probs[cur - skip_nodes].argmax())          # classic_sd.py:112
+        t = target(cur - skip_nodes)                        # classic_sd.py:112
         match = [c for c in kids if int(token_ids[c]) == t]
         if not match:                                       # classic_sd.py:115-116
             bonus = t
@@ -81,7 +87,7 @@ def exact_verify(
             break
     if (not out_tok) or eos_token_id is None or out_tok[-1] != int(eos_token_id):  # :97
         if bonus is None:
-            bonus = int(probs[cur - skip_nodes].argmax())
+            bonus = target(cur - skip_nodes)
         out_tok.append(bonus)
         out_ctx.append(cur)
     return out_tok, out_ctx, (total, accept)
@@ -113,8 +119,10 @@ def lossy_verify(
     threshold_method: str = "prob",
     internal: Optional[dict] = None,
     log: Optional[dict] = None,
+    target_tokens: Optional[Sequence[int]] = None,
 ) -> Tuple[List[int], List[int], int]:
-    """Bottom-up DP verifier in LOCAL indexing (lossy_tree_verify.py:9-343), greedy target.
+    """Bottom-up DP verifier in LOCAL indexing (lossy_tree_verify.py:9-343).  ``target_tokens`` (one per
+    row) stands for the ``torch.multinomial`` draw of a sampling target (:75-77); None = argmax.
 
     ``internal``/``log`` play the role of ``wandb_logger.internal_data`` / ``.log_data``
     (running accumulators and exported metrics); pass the same dicts across calls to accumulate.
@@ -127,7 +135,7 @@ def lossy_verify(
     need = max(0, int(window_size))
     n = int(probs.shape[0])
     tok = [int(t) for t in token_ids]
-    tgt = probs.argmax(dim=-1).tolist()                                  # :75-77
+    tgt = probs.argmax(dim=-1).tolist() if target_tokens is None else [int(t) for t in target_tokens]   # :75-77
     h = normalized_entropy(probs) if use_entropy else None               # :103-105
 
     mismatch = [bool(children[u]) and all(tok[c] != tgt[u] for c in children[u]) for u in range(n)]
@@ -249,8 +257,12 @@ def verify_logits(
     verify_kwargs: Optional[dict] = None,
     internal: Optional[dict] = None,
     log: Optional[dict] = None,
+    temperature: Optional[float] = None,
+    target_tokens: Optional[Sequence[int]] = None,
 ):
-    """``verify_tree`` restated on plain arrays (tree_verify.py:8-163), greedy target only.
+    """``verify_tree`` restated on plain arrays (tree_verify.py:8-163).  Greedy target by default; for a
+    sampling target pass the warper's ``temperature`` and one pre-drawn token per row
+    (``oracle.sampling.draw_tokens`` on ``oracle.sampling.warp_probs``).
 
     ``token_ids``/``parents`` describe the WHOLE tree in original indexing, ``logits`` is
     ``[rows, V]`` for original nodes ``skip_nodes .. skip_nodes+rows-1``.
@@ -258,10 +270,12 @@ def verify_logits(
     """
     method = str(verify_method or "exact").strip().lower()
     vk = dict(verify_kwargs or {})
+    if temperature is not None and float(temperature) != 1.0:
+        logits = logits.cpu() / float(temperature)                        # generators/base.py:57-58
     probs = target_probs(logits)
     kids_all = children_from_parents(parents)
     if method == "exact":
-        return exact_verify(probs, token_ids, kids_all, root, eos_token_id, skip_nodes)
+        return exact_verify(probs, token_ids, kids_all, root, eos_token_id, skip_nodes, target_tokens)
     if method != "lossy":
         raise ValueError(f"Unsupported verify_method: {verify_method!r} (supported: 'exact', 'lossy')")
     rows = int(probs.shape[0])
@@ -281,12 +295,13 @@ def verify_logits(
         threshold=float(vk.get("threshold", 0.0)),
         window_size=int(vk.get("window_size", 1)),
         threshold_method=str(vk.get("threshold_method", "prob") or "prob").strip().lower(),
-        internal=internal, log=log,
+        internal=internal, log=log, target_tokens=target_tokens,
     )
     return toks, [c + skip_nodes for c in ctx_local], (len(toks), acc)
 
 
-def brute_force_lossy_len(probs, token_ids, children, root, threshold, window_size, threshold_method):
+def brute_force_lossy_len(probs, token_ids, children, root, threshold, window_size, threshold_method,
+                          target_tokens=None):
     """Independent check: longest admissible root path by exhaustive recursion (tiny trees only).
 
     Admissibility of an edge u->c (lossy_tree_verify.py:135-146): exact if tok[c]==argmax p[u];
@@ -294,7 +309,7 @@ def brute_force_lossy_len(probs, token_ids, children, root, threshold, window_si
     run of exact edges below c.
     """
     tok = [int(t) for t in token_ids]
-    tgt = probs.argmax(dim=-1).tolist()
+    tgt = probs.argmax(dim=-1).tolist() if target_tokens is None else [int(t) for t in target_tokens]
     h = normalized_entropy(probs)
     use_entropy = threshold_method == "entropy"
 

@@ -48,12 +48,16 @@ _SIGNATURES = {
     "subspec_tree_verify": (C.c_int, [_p, C.c_int, _i64, _i64, _i64, _p, _p, _i64, _i32, _i32, _i64,
                                       C.c_int, C.c_int, _f64, _i32, C.c_int, _p, _sz,
                                       _p, _p, _p, _p, _p, _p, _p]),
+    "subspec_tree_verify_sample": (C.c_int, [_p, C.c_int, _i64, _i64, _i64, _p, _p, _i64, _i32, _i32, _i64,
+                                             C.c_int, C.c_int, _f64, _i32, C.c_int, C.c_float, C.c_uint64, C.c_uint64,
+                                             _p, _sz, _p, _p, _p, _p, _p, _p, _p]),
     "subspec_topk_expand_workspace": (_sz, [_i64, _i64, _i64, _i32]),
     "subspec_topk_expand": (C.c_int, [_p, _p, C.c_int, _i64, _i64, _i64, _i32, _p, _sz, _p, _p, _p, _p]),
     "subspec_tree_attention_workspace": (_sz, [_i64, _i64, _i64, _i64]),
     "subspec_tree_attention": (C.c_int, [_p, _p, _p, _p, C.c_int, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _p, _i64,
                                          C.c_float, _p, _sz, _p]),
     "subspec_softmax_temperature": (C.c_int, [_p, _p, C.c_int, _i64, _i64, C.c_float, _p]),
+    "subspec_temperature_warp": (C.c_int, [_p, _p, C.c_int, _i64, C.c_float, _p]),
     "subspec_int4_linear_workspace": (_sz, [_i64, _i64, _i64]),
     "subspec_int4_linear": (C.c_int, [_p, _p, _p, _p, _p, C.c_int, _i64, _i64, _i64, _i64, _p, _sz, _p]),
     "subspec_int4_decoder_layer_workspace": (_sz, [C.POINTER(DecoderLayerDims)]),

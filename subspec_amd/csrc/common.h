@@ -86,6 +86,22 @@ template <> struct Elem<SUBSPEC_BF16> {
   static __device__ __forceinline__ float min_normal() { return 1.17549435e-38f; }
 };
 
+// x / t correctly rounded (round to nearest even) from inv_t = RN(1 / t): q = RN(x * inv_t) lies within one
+// ulp of the quotient, the residual r = x - t * q is exact in one fma, and RN(q + r * inv_t) is the
+// correctly rounded quotient (P. Markstein, "Computation of elementary functions on the IBM RISC
+// System/6000 processor", IBM J. Res. Dev. 34, 1990, theorem on division by a correctly rounded
+// reciprocal).  Three instructions instead of the generic division sequence.  Infinite quotients
+// are returned as they are (their residual is not a number).  The residual must be a normal
+// number for the step to be exact: guaranteed for |x| >= 2^-100, i.e. for anything a logit can be.
+struct Divisor { float t, inv_t; };
+inline Divisor make_divisor(float t) { return Divisor{t, (float)(1.0 / (double)t)}; }
+__device__ __forceinline__ float div_rn(float x, const Divisor& d) {
+  const float q = x * d.inv_t;
+  const float r = fmaf(-d.t, q, x);
+  const float q1 = fmaf(r, d.inv_t, q);
+  return fabsf(q) == INFINITY ? q : q1;
+}
+
 // ---------------------------------------------------------------- wave / block reductions
 __device__ __forceinline__ float wave_max(float v) {
 #pragma unroll

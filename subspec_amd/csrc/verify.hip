@@ -14,6 +14,14 @@
 //      p[parent(i), token(i)], runs the greedy walk or the bottom-up DP on the <= 256 nodes in LDS
 //      and writes the accepted path, contexts and bonus token.
 //
+// Sampling target (do_sample=True): the rows are first warped as TemperatureLogitsWarper does
+// (x / T rounded to the row dtype), steps 1-2 run on the warped values, and row_sample_kernel
+// draws one token per row from the rounded probabilities by an exponential race,
+// argmax_i p_i / E_i with E_i = -log(u_i) and u_i from Philox4x32-10 keyed by the caller's seed
+// (the formulation torch.multinomial uses for one sample); the walk / DP of step 3 then uses the
+// drawn token where the greedy target uses the argmax (classic_sd.py:111-116,
+// lossy_tree_verify.py:75-77).
+//
 // Semantics follow the reference's verify_tree / lossy_bottom_up_verify
 // (specdecodes/models/utils/tree_verify.py:49-163, lossy_tree_verify.py:66-168,247-291):
 // argmax is the FIRST index whose probability, rounded to the logits dtype, equals the rounded
@@ -32,6 +40,7 @@ constexpr int kTailThreads = 64;
 // t = (x - ref) * log2(e), true maximum of the slice and the first index holding it
 struct Part1 { float ref; float s; float u; float m; int32_t idx; int32_t pad[3]; };
 struct Part2 { float esum; int32_t tie_idx; };
+struct Part3 { float key; int32_t idx; };             // best race key of a slice and its first index
 
 // ------------------------------------------------------------------ packed register tiles
 template <int DT, int VEC> struct Tile;
@@ -96,7 +105,23 @@ struct VerifyParams {
   int entropy_policy;
   float theta;
   float ln_vocab;       // float(ln V), or 1 when V == 1 (lossy_tree_verify.py:68)
+  int sample;           // 1: the target token of a row is drawn from its distribution
+  Divisor temperature;  // rows are divided by .t (and rounded to their dtype) when .t != 1
+  uint32_t key[2];      // Philox key: the caller's 64-bit seed
+  uint32_t offset[2];   // Philox counter words 2, 3: the caller's 64-bit stream offset
 };
+
+// TemperatureLogitsWarper on one element: IEEE quotient, one rounding to the row dtype
+template <int DT, bool WARP>
+__device__ __forceinline__ float warped(float x, const Divisor& temperature) {
+  if constexpr (WARP) return Elem<DT>::round(div_rn(x, temperature));
+  return x;
+}
+template <int DT>
+__device__ __forceinline__ float load_warped(const void* logits, int64_t i, const VerifyParams& vp) {
+  const float x = Elem<DT>::load(logits, i);
+  return vp.temperature.t != 1.0f ? Elem<DT>::round(div_rn(x, vp.temperature)) : x;
+}
 
 template <int DT>
 __device__ __forceinline__ float finish_entropy(float H, float ln_vocab) {
@@ -159,7 +184,7 @@ __device__ __forceinline__ void row_exact_body(const void* __restrict__ logits, 
   float acc = 0.f;
   int tie = 0x7fffffff;
   for (int64_t i = threadIdx.x; i < n; i += kRowThreads) {
-    const float x = Elem<DT>::load(logits, base + i);
+    const float x = load_warped<DT>(logits, base + i, vp);
     const float p = rounded_prob<DT>(x, rs.m, rs.S);
     if (rs.need_emu && p > 0.f) acc += Elem<DT>::round(-p * Elem<DT>::round(logf(p)));
     if (p == rs.pmax && tie == 0x7fffffff) tie = (int)(c0 + i);
@@ -186,11 +211,12 @@ __global__ __launch_bounds__(kRowThreads) void row_exact_kernel(
 // ------------------------------------------------------------------ kernel 1: one pass over HBM
 // sum exp and sum t*exp of one tile relative to the reference `mb = -ref * log2(e)`;
 // t is clamped so that exp2(t) == 0 implies t * exp2(t) == 0 (x may be -inf).
-template <int DT, int VEC>
-__device__ __forceinline__ float tile_accumulate(const Tile<DT, VEC>& t, float mb, float (&s)[2], float (&u)[2]) {
+template <int DT, int VEC, bool WARP>
+__device__ __forceinline__ float tile_accumulate(const Tile<DT, VEC>& t, float mb, const Divisor& temperature,
+                                                 float (&s)[2], float (&u)[2]) {
   float x[VEC];
 #pragma unroll
-  for (int k = 0; k < VEC; ++k) x[k] = t.get(k);
+  for (int k = 0; k < VEC; ++k) x[k] = warped<DT, WARP>(t.get(k), temperature);
   float tmax = x[0];
 #pragma unroll
   for (int k = 1; k < VEC; ++k) tmax = fmaxf(tmax, x[k]);
@@ -204,7 +230,7 @@ __device__ __forceinline__ float tile_accumulate(const Tile<DT, VEC>& t, float m
   return tmax;
 }
 
-template <int DT, int VEC, int U>
+template <int DT, int VEC, int U, bool WARP>
 __global__ __launch_bounds__(kRowThreads) void row_partial_kernel(
     const void* __restrict__ logits, VerifyParams vp, Part1* __restrict__ part, Part2* __restrict__ part2) {
   const int64_t vocab = vp.vocab, chunk = vp.chunk;
@@ -226,9 +252,9 @@ __global__ __launch_bounds__(kRowThreads) void row_partial_kernel(
   {
     Tile<DT, VEC> t0;
     if (tid < ntiles) t0.load(logits, base + (int64_t)tid * VEC); else t0.fill_neg_inf();
-    float r = t0.get(0);
+    float r = warped<DT, WARP>(t0.get(0), vp.temperature);
 #pragma unroll
-    for (int k = 1; k < VEC; ++k) r = fmaxf(r, t0.get(k));
+    for (int k = 1; k < VEC; ++k) r = fmaxf(r, warped<DT, WARP>(t0.get(k), vp.temperature));
     ref = block_max<kRowThreads>(r, red_f);
     if (ref == -INFINITY) ref = -1e30f;
   }
@@ -251,7 +277,7 @@ __global__ __launch_bounds__(kRowThreads) void row_partial_kernel(
         if (j0 + (int64_t)i * kRowThreads >= ntiles) t[i].fill_neg_inf();
 #pragma unroll
       for (int i = 0; i < U; ++i) {
-        const float tmax = tile_accumulate<DT, VEC>(t[i], mb, s, u);
+        const float tmax = tile_accumulate<DT, VEC, WARP>(t[i], mb, vp.temperature, s, u);
         if (tmax > vmax) { vmax = tmax; best_tile = j0 + (int64_t)i * kRowThreads; }
       }
     }
@@ -268,7 +294,7 @@ __global__ __launch_bounds__(kRowThreads) void row_partial_kernel(
     tb.load(logits, base + best_tile * VEC);
 #pragma unroll
     for (int k = VEC - 1; k >= 0; --k)
-      if (tb.get(k) == m) idx = (int)(c0 + best_tile * VEC + k);
+      if (warped<DT, WARP>(tb.get(k), vp.temperature) == m) idx = (int)(c0 + best_tile * VEC + k);
   }
   const float ssum = block_sum<kRowThreads>(s[0] + s[1], red_f);
   const float usum = block_sum<kRowThreads>(u[0] + u[1], red_f);
@@ -281,6 +307,94 @@ __global__ __launch_bounds__(kRowThreads) void row_partial_kernel(
     const RowStat rs = combine_row<DT>(&mine, vp);
     if (rs.need_emu || rs.need_tie) row_exact_body<DT>(logits, vp, rs, row, 0, red_f, red_i, part2);
   }
+}
+
+// ------------------------------------------------------------------ kernel 2b: one draw per row
+// Philox4x32-10 (Salmon et al., "Parallel random numbers: as easy as 1, 2, 3", SC'11).
+__device__ __forceinline__ void philox4x32_10(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3, uint32_t k0,
+                                              uint32_t k1, uint32_t (&out)[4]) {
+#pragma unroll
+  for (int r = 0; r < 10; ++r) {
+    const uint64_t p0 = (uint64_t)0xD2511F53u * c0;    // one 32 x 32 -> 64 bit multiply each
+    const uint64_t p1 = (uint64_t)0xCD9E8D57u * c2;
+    c0 = (uint32_t)(p1 >> 32) ^ c1 ^ k0;
+    c1 = (uint32_t)p1;
+    c2 = (uint32_t)(p0 >> 32) ^ c3 ^ k1;
+    c3 = (uint32_t)p0;
+    k0 += 0x9E3779B9u;
+    k1 += 0xBB67AE85u;
+  }
+  out[0] = c0; out[1] = c1; out[2] = c2; out[3] = c3;
+}
+
+// Relative and absolute rounding bounds of one value stored in the row dtype (generous).
+template <int DT> struct RoundBound;
+template <> struct RoundBound<SUBSPEC_F32> { static constexpr float rel = 0x1p-21f, abs = 0.f; };
+template <> struct RoundBound<SUBSPEC_F16> { static constexpr float rel = 0x1p-10f, abs = 0x1p-24f; };
+template <> struct RoundBound<SUBSPEC_BF16> { static constexpr float rel = 0x1p-8f, abs = 0.f; };
+
+// Element i of global row `row` uses word i % 4 of Philox(counter = {i / 4, row, offset}, key = seed);
+// u = ((word >> 9) + 0.5) * 2^-23 lies strictly inside (0, 1) and is exact in fp32.
+// A slice starts at a multiple of 4, so a 4-element group never straddles two workgroups.
+//
+// The race key of an element is p / -log(u), evaluated exactly as defined (rounded probability,
+// accurate logarithm, IEEE quotient) only for the few elements that can still win: -log(u) >= 1 - u
+// and p <= an upper bound from the hardware exponential give key <= bound / (1 - u), and an
+// element whose bound stays below the best key any lane of the wavefront has seen is skipped.
+// What is left per element is the Philox block, one exponential and a compare.
+template <int DT>
+__global__ __launch_bounds__(kRowThreads) void row_sample_kernel(
+    const void* __restrict__ logits, VerifyParams vp, const Part1* __restrict__ part1, Part3* __restrict__ part3) {
+  __shared__ float red_f[kRowThreads / kWave];
+  __shared__ int red_i[kRowThreads / kWave];
+  const int64_t row = blockIdx.y;
+  const int c = blockIdx.x;
+  const RowStat rs = combine_row<DT>(part1 + row * vp.splits, vp);
+  const int64_t c0 = (int64_t)c * vp.chunk;
+  const int64_t n = min(vp.chunk, vp.vocab - c0);
+  const int64_t base = row * vp.vocab + c0;
+  const bool warp = vp.temperature.t != 1.0f;
+  const float inv_t = warp ? vp.temperature.inv_t : 1.0f;
+  const float round_up = warp ? RoundBound<DT>::rel : 0.f;          // x / T rounded to the dtype, relative
+  const float round_abs = warp ? RoundBound<DT>::abs + 1e-30f : 0.f;
+  const float mb = -rs.m * kLog2e;
+  // p <= exp2((x' - m) log2 e) / S * (1 + rounding of p, of the hardware exp2 and of this arithmetic)
+  const float p_scale = (1.0f / rs.S) * (1.0f + 4.0f * RoundBound<DT>::rel + 1e-4f);
+  float best = -1.f;
+  int idx = 0x7fffffff;
+  float thr = 0.f;                                     // 0.9999 * 2^-23 * best key of the wavefront
+  for (int64_t g0 = 0; g0 * 4 < n; g0 += kRowThreads) {   // same trip count for every lane: the votes below see whole wavefronts
+    const int64_t g = g0 + threadIdx.x;
+    float xs[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e)                        // unconditional loads (clamped index), in flight during the Philox rounds
+      xs[e] = Elem<DT>::load(logits, base + min(g * 4 + e, n - 1));
+    uint32_t w[4];
+    philox4x32_10((uint32_t)(c0 / 4 + g), (uint32_t)row, vp.offset[0], vp.offset[1], vp.key[0], vp.key[1], w);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int64_t i = g * 4 + e;
+      const float x = xs[e];
+      const float xa = fmaxf(x * inv_t, -1e30f);                     // masked (-inf) logits stay finite below
+      const float xu = fmaf(fabsf(xa), round_up, xa) + round_abs;
+      const float bound = fmaf(__builtin_amdgcn_exp2f(fmaf(xu, kLog2e, mb)), p_scale, RoundBound<DT>::abs);
+      const float one_minus_u = (float)((~w[e]) >> 9) + 0.5f;        // (1 - u) * 2^23, exact
+      const bool cand = i < n && !(bound < thr * one_minus_u);
+      if (__any(cand)) {                               // wavefront-uniform
+        if (cand) {
+          const float xw = warp ? Elem<DT>::round(div_rn(x, vp.temperature)) : x;
+          const float p = rounded_prob<DT>(xw, rs.m, rs.S);
+          const float u = ((float)(w[e] >> 9) + 0.5f) * 0x1p-23f;
+          const float key = p / -logf(u);
+          if (key > best) { best = key; idx = (int)(c0 + i); }   // indices ascend: the first maximum stays
+        }
+        thr = fmaxf(wave_max(best), 0.f) * (0.9999f * 0x1p-23f);
+      }
+    }
+  }
+  const float top = block_max<kRowThreads>(best, red_f);
+  idx = block_min_i<kRowThreads>(best == top ? idx : 0x7fffffff, red_i);
+  if (threadIdx.x == 0) part3[row * vp.splits + c] = Part3{top, idx};
 }
 
 // ------------------------------------------------------------------ kernel 3: per-tree tail
@@ -320,7 +434,7 @@ __device__ __forceinline__ T pick_slot(const T (&a)[kSlots], int slot) {
 template <int DT, int kSlots, bool LOSSY>
 __global__ __launch_bounds__(kTailThreads) void tree_accept_kernel(
     const void* __restrict__ logits, VerifyParams vp, TreeParams tp,
-    const Part1* __restrict__ part1, const Part2* __restrict__ part2,
+    const Part1* __restrict__ part1, const Part2* __restrict__ part2, const Part3* __restrict__ part3,
     const int32_t* __restrict__ token_ids, const int32_t* __restrict__ parents,
     int64_t* __restrict__ out_tokens, int64_t* __restrict__ out_ctx, int32_t* __restrict__ out_counts,
     int64_t* __restrict__ node_target, float* __restrict__ node_entropy, float* __restrict__ node_child_prob) {
@@ -358,6 +472,15 @@ __global__ __launch_bounds__(kTailThreads) void tree_accept_kernel(
         if (rs.need_tie && tie != 0x7fffffff) tgt = tie;
         if (rs.need_emu) h = finish_entropy<DT>(H, vp.ln_vocab);
       }
+      if (vp.sample) {                                 // the drawn token replaces the argmax
+        float top = -1.f;
+        int drawn = 0x7fffffff;
+        for (int c = 0; c < vp.splits; ++c) {
+          const Part3 q = part3[grow * vp.splits + c];
+          if (q.key > top || (q.key == top && q.idx < drawn)) { top = q.key; drawn = q.idx; }
+        }
+        if (drawn != 0x7fffffff) tgt = drawn;
+      }
       sm_m[r] = rs.m;
       sm_S[r] = rs.S;
       sm_tgt[r] = tgt;
@@ -385,7 +508,7 @@ __global__ __launch_bounds__(kTailThreads) void tree_accept_kernel(
         int rp = par[s] - skip;
         if (rp < 0 && !lossy) rp += rows;              // the exact walk indexes rows like a python list
         if (rp >= 0 && rp < rows && tok[s] >= 0 && tok[s] < vp.vocab) {
-          const float x = Elem<DT>::load(logits, ((int64_t)b * rows + rp) * vp.vocab + tok[s]);
+          const float x = load_warped<DT>(logits, ((int64_t)b * rows + rp) * vp.vocab + tok[s], vp);
           cp[s] = rounded_prob<DT>(x, sm_m[rp], sm_S[rp]);
         }
       }
@@ -549,28 +672,36 @@ static bool make_plan(const void* logits, int dtype, int64_t total_rows, int64_t
 
 template <int DT, int VEC>
 static void launch_partial(dim3 grid, hipStream_t st, const void* logits, const VerifyParams& vp, Part1* p1, Part2* p2) {
-  hipLaunchKernelGGL((row_partial_kernel<DT, VEC, 4>), grid, dim3(kRowThreads), 0, st, logits, vp, p1, p2);
+  if (vp.temperature.t != 1.0f)
+    hipLaunchKernelGGL((row_partial_kernel<DT, VEC, 4, true>), grid, dim3(kRowThreads), 0, st, logits, vp, p1, p2);
+  else
+    hipLaunchKernelGGL((row_partial_kernel<DT, VEC, 4, false>), grid, dim3(kRowThreads), 0, st, logits, vp, p1, p2);
 }
 
 template <int DT>
 static int run_verify(const void* logits, int64_t batch, int64_t rows, int64_t vocab, const Plan& pl,
-                      const VerifyParams& vp, const TreeParams& tp, Part1* p1, Part2* p2,
+                      const VerifyParams& vp, const TreeParams& tp, Part1* p1, Part2* p2, Part3* p3,
                       const int32_t* token_ids, const int32_t* parents, int64_t* out_tokens, int64_t* out_ctx,
                       int32_t* out_counts, int64_t* node_target, float* node_entropy, float* node_child_prob,
                       hipStream_t st) {
   const dim3 grid(pl.splits, (unsigned)(batch * rows));
-  {
-    DominantKernelTimer timer(st);
+  auto partial = [&] {
     if (pl.vec == 1) launch_partial<DT, 1>(grid, st, logits, vp, p1, p2);
     else launch_partial<DT, (DT == SUBSPEC_F32 ? 4 : 8)>(grid, st, logits, vp, p1, p2);
-  }
+  };
+  // the timed kernel is the longest one: the statistics pass, or the draw when sampling
+  if (vp.sample) partial(); else { DominantKernelTimer timer(st); partial(); }
   if (pl.splits > 1) hipLaunchKernelGGL((row_exact_kernel<DT>), grid, dim3(kRowThreads), 0, st, logits, vp, p1, p2);
+  if (vp.sample) {
+    DominantKernelTimer timer(st);
+    hipLaunchKernelGGL((row_sample_kernel<DT>), grid, dim3(kRowThreads), 0, st, logits, vp, p1, p3);
+  }
   const int64_t widest = std::max<int64_t>(rows, tp.n_nodes);
   const int slots = widest <= kWave ? 1 : widest <= 2 * kWave ? 2 : 4;
   const bool lossy = tp.method == SUBSPEC_VERIFY_LOSSY;
 #define SUBSPEC_LAUNCH_TAIL(SLOTS, LOSSY)                                                                        \
   hipLaunchKernelGGL((tree_accept_kernel<DT, SLOTS, LOSSY>), dim3((unsigned)batch), dim3(kTailThreads), 0, st,    \
-                     logits, vp, tp, p1, p2, token_ids, parents, out_tokens, out_ctx, out_counts, node_target,   \
+                     logits, vp, tp, p1, p2, p3, token_ids, parents, out_tokens, out_ctx, out_counts, node_target,   \
                      node_entropy, node_child_prob)
   if (slots == 1) { if (lossy) SUBSPEC_LAUNCH_TAIL(1, true); else SUBSPEC_LAUNCH_TAIL(1, false); }
   else if (slots == 2) { if (lossy) SUBSPEC_LAUNCH_TAIL(2, true); else SUBSPEC_LAUNCH_TAIL(2, false); }
@@ -588,17 +719,19 @@ extern "C" size_t subspec_tree_verify_workspace(int64_t batch, int64_t rows, int
   (void)vocab; (void)dtype;
   if (batch <= 0 || rows <= 0) return 256;
   const size_t n = (size_t)batch * rows * kMaxSplits;
-  return align_up(n * sizeof(Part1), 256) + align_up(n * sizeof(Part2), 256);
+  return align_up(n * sizeof(Part1), 256) + align_up(n * sizeof(Part2), 256) + align_up(n * sizeof(Part3), 256);
 }
 
-extern "C" int subspec_tree_verify(const void* logits, int dtype, int64_t batch, int64_t rows, int64_t vocab,
-                                   const int32_t* token_ids, const int32_t* parents, int64_t n_nodes,
-                                   int32_t root, int32_t skip_nodes, int64_t eos_token_id,
-                                   int verify_method, int threshold_method, double threshold, int32_t window_size,
-                                   int entropy_policy, void* workspace, size_t workspace_bytes,
-                                   int64_t* out_tokens, int64_t* out_ctx, int32_t* out_counts,
-                                   int64_t* node_target, float* node_entropy, float* node_child_prob,
-                                   void* stream) {
+struct SampleArgs { int sample; float temperature; uint64_t seed, offset; };
+
+static int tree_verify_impl(const void* logits, int dtype, int64_t batch, int64_t rows, int64_t vocab,
+                            const int32_t* token_ids, const int32_t* parents, int64_t n_nodes,
+                            int32_t root, int32_t skip_nodes, int64_t eos_token_id,
+                            int verify_method, int threshold_method, double threshold, int32_t window_size,
+                            int entropy_policy, void* workspace, size_t workspace_bytes,
+                            int64_t* out_tokens, int64_t* out_ctx, int32_t* out_counts,
+                            int64_t* node_target, float* node_entropy, float* node_child_prob,
+                            const SampleArgs& sa, void* stream) {
   if (!dtype_ok(dtype)) SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "tree_verify: unknown dtype %d", dtype);
   if (!logits || !token_ids || !parents || !workspace || !out_tokens || !out_ctx || !out_counts || !node_target ||
       !node_entropy || !node_child_prob)
@@ -631,6 +764,7 @@ extern "C" int subspec_tree_verify(const void* logits, int dtype, int64_t batch,
   const size_t n = (size_t)batch * rows * kMaxSplits;
   Part1* p1 = (Part1*)workspace;
   Part2* p2 = (Part2*)((char*)workspace + align_up(n * sizeof(Part1), 256));
+  Part3* p3 = (Part3*)((char*)p2 + align_up(n * sizeof(Part2), 256));
 
   VerifyParams vp;
   vp.vocab = vocab;
@@ -640,6 +774,12 @@ extern "C" int subspec_tree_verify(const void* logits, int dtype, int64_t batch,
   vp.entropy_policy = entropy_policy;
   vp.theta = (float)threshold;
   vp.ln_vocab = vocab > 1 ? (float)log((double)vocab) : 1.0f;
+  vp.sample = sa.sample;
+  vp.temperature = make_divisor(sa.temperature);
+  vp.key[0] = (uint32_t)sa.seed;
+  vp.key[1] = (uint32_t)(sa.seed >> 32);
+  vp.offset[0] = (uint32_t)sa.offset;
+  vp.offset[1] = (uint32_t)(sa.offset >> 32);
   TreeParams tp;
   tp.rows = rows;
   tp.n_nodes = n_nodes;
@@ -653,13 +793,46 @@ extern "C" int subspec_tree_verify(const void* logits, int dtype, int64_t batch,
   hipStream_t st = (hipStream_t)stream;
   switch (dtype) {
     case SUBSPEC_F32:
-      return run_verify<SUBSPEC_F32>(logits, batch, rows, vocab, pl, vp, tp, p1, p2, token_ids, parents, out_tokens,
+      return run_verify<SUBSPEC_F32>(logits, batch, rows, vocab, pl, vp, tp, p1, p2, p3, token_ids, parents, out_tokens,
                                      out_ctx, out_counts, node_target, node_entropy, node_child_prob, st);
     case SUBSPEC_F16:
-      return run_verify<SUBSPEC_F16>(logits, batch, rows, vocab, pl, vp, tp, p1, p2, token_ids, parents, out_tokens,
+      return run_verify<SUBSPEC_F16>(logits, batch, rows, vocab, pl, vp, tp, p1, p2, p3, token_ids, parents, out_tokens,
                                      out_ctx, out_counts, node_target, node_entropy, node_child_prob, st);
     default:
-      return run_verify<SUBSPEC_BF16>(logits, batch, rows, vocab, pl, vp, tp, p1, p2, token_ids, parents, out_tokens,
+      return run_verify<SUBSPEC_BF16>(logits, batch, rows, vocab, pl, vp, tp, p1, p2, p3, token_ids, parents, out_tokens,
                                       out_ctx, out_counts, node_target, node_entropy, node_child_prob, st);
   }
+}
+
+extern "C" int subspec_tree_verify(const void* logits, int dtype, int64_t batch, int64_t rows, int64_t vocab,
+                                   const int32_t* token_ids, const int32_t* parents, int64_t n_nodes,
+                                   int32_t root, int32_t skip_nodes, int64_t eos_token_id,
+                                   int verify_method, int threshold_method, double threshold, int32_t window_size,
+                                   int entropy_policy, void* workspace, size_t workspace_bytes,
+                                   int64_t* out_tokens, int64_t* out_ctx, int32_t* out_counts,
+                                   int64_t* node_target, float* node_entropy, float* node_child_prob,
+                                   void* stream) {
+  const SampleArgs greedy{0, 1.0f, 0, 0};
+  return tree_verify_impl(logits, dtype, batch, rows, vocab, token_ids, parents, n_nodes, root, skip_nodes,
+                          eos_token_id, verify_method, threshold_method, threshold, window_size, entropy_policy,
+                          workspace, workspace_bytes, out_tokens, out_ctx, out_counts, node_target, node_entropy,
+                          node_child_prob, greedy, stream);
+}
+
+extern "C" int subspec_tree_verify_sample(const void* logits, int dtype, int64_t batch, int64_t rows, int64_t vocab,
+                                          const int32_t* token_ids, const int32_t* parents, int64_t n_nodes,
+                                          int32_t root, int32_t skip_nodes, int64_t eos_token_id,
+                                          int verify_method, int threshold_method, double threshold,
+                                          int32_t window_size, int entropy_policy, float temperature, uint64_t seed,
+                                          uint64_t offset, void* workspace, size_t workspace_bytes,
+                                          int64_t* out_tokens, int64_t* out_ctx, int32_t* out_counts,
+                                          int64_t* node_target, float* node_entropy, float* node_child_prob,
+                                          void* stream) {
+  if (!(temperature > 0.f) || temperature == INFINITY)
+    SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "tree_verify_sample: temperature=%g must be positive and finite", (double)temperature);
+  const SampleArgs drawn{1, temperature, seed, offset};
+  return tree_verify_impl(logits, dtype, batch, rows, vocab, token_ids, parents, n_nodes, root, skip_nodes,
+                          eos_token_id, verify_method, threshold_method, threshold, window_size, entropy_policy,
+                          workspace, workspace_bytes, out_tokens, out_ctx, out_counts, node_target, node_entropy,
+                          node_child_prob, drawn, stream);
 }

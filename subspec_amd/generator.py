@@ -2,7 +2,8 @@
 
 Keeps the reference's generator surface (specdecodes/models/generators/base.py:156-197 ``generate``,
 classic_sd.py:12-134 ``ClassicSDGeneratorBase`` incl. ``generator_kwargs = {prefill_chunk_size,
-verify_method, verify_kwargs}``, subspec_sd.py:10-126 ``_generate``) for the greedy target, and the
+verify_method, verify_kwargs}``, subspec_sd.py:10-126 ``_generate``) for the greedy and the sampling
+target (``do_sample``, ``temperature``, ``top_k``, ``top_p``: base.py:42-64,156-197), and the
 metrics contract of ``SDProfilingMixin`` (specdecodes/models/utils/mixin.py:181-224,267-269,318-349:
 ``avg_draft_time``, ``avg_target_time``, ``avg_verify_time``, ``avg_sampled``, ``n_iter``,
 ``n_tokens``, ``elapsed_time``, ``tput``).
@@ -21,7 +22,7 @@ import torch
 from . import ops
 from .cache import KVManager
 from .lossy_diagnostics import record_lossy_diagnostics
-from .tree_verify import verify_tree_device
+from .tree_verify import SampleStream, sample_token, verify_tree_device
 from .utils import DraftParams
 from .wandb_logger import wandb_logger
 
@@ -41,6 +42,8 @@ class SubSpecSDGenerator:
         self.prefill_chunk_size = self.generator_kwargs.get("prefill_chunk_size", None)
         self.eos_token_id = eos_token_id if eos_token_id is not None else getattr(tokenizer, "eos_token_id", None)
         self.draft_model.eos_token_id = self.eos_token_id
+        # Philox stream of the sampling target; generator_kwargs["seed"] fixes it, else torch's seed
+        self.sample_stream = SampleStream(self.generator_kwargs.get("seed"))
 
     # ------------------------------------------------------------------ pieces of one cycle
     def _speculate(self, input_ids):
@@ -53,15 +56,33 @@ class SubSpecSDGenerator:
         both = torch.stack([packed["token_ids"].long(), packed["depths"].long(), anc]).to(dev, non_blocking=True)
         return self.target_model.tree_forward(both[0], both[1], both[2], position_offset)
 
+    def _get_logits_processor(self, temperature: float = 1.0, top_k: Optional[int] = None, top_p: Optional[float] = None):
+        """The HuggingFace warpers of multinomial sampling, in the reference's order and under its
+        conditions (generators/base.py:42-64): temperature unless None or 1, top-k unless None or
+        0, top-p unless None or >= 1."""
+        from transformers.generation.logits_process import (LogitsProcessorList, TemperatureLogitsWarper,
+                                                            TopKLogitsWarper, TopPLogitsWarper)
+        warpers = LogitsProcessorList()
+        if temperature is not None and temperature != 1.0:
+            warpers.append(TemperatureLogitsWarper(temperature))
+        if top_k is not None and top_k != 0:
+            warpers.append(TopKLogitsWarper(top_k=top_k))
+        if top_p is not None and top_p < 1.0:
+            warpers.append(TopPLogitsWarper(top_p=top_p))
+        return warpers
+
+    def _sample_token(self, logits, logits_processor, do_sample: bool, return_probs: bool = False):
+        return sample_token(logits, logits_processor, do_sample, return_probs, stream=self.sample_stream)
+
     def _verify(self, tree, root_ind, logits, logits_processor=None, do_sample=False, skip_nodes=0):
-        if do_sample:
-            raise NotImplementedError("the HIP verifier implements the greedy target (do_sample=False) only")
         method = str(self.generator_kwargs.get("verify_method", "exact") or "exact").strip().lower()
         if method not in ("exact", "lossy"):
             raise ValueError(f"Unsupported verify_method: {method!r} (supported: 'exact', 'lossy')")
         return verify_tree_device(tree=tree, root_ind=int(root_ind), logits=logits, eos_token_id=self.eos_token_id,
                                   skip_nodes=int(skip_nodes), verify_method=method,
-                                  verify_kwargs=dict(self.generator_kwargs.get("verify_kwargs") or {}))
+                                  verify_kwargs=dict(self.generator_kwargs.get("verify_kwargs") or {}),
+                                  logits_processor=logits_processor, do_sample=bool(do_sample),
+                                  stream=self.sample_stream)
 
     def _chunked_prefill_forward(self, input_ids: torch.Tensor, past_key_values: KVManager):
         """Prefill in chunks of ``prefill_chunk_size`` (generators/base.py:204-263); returns the last logits."""
@@ -79,8 +100,6 @@ class SubSpecSDGenerator:
     @torch.no_grad()
     def generate(self, input_ids: torch.LongTensor, temperature=None, top_p=None, top_k=None, max_new_tokens=None,
                  max_length=None, do_sample=False, stop_strings=None, stream_callback=None, **model_kwargs):
-        if do_sample:
-            raise NotImplementedError("do_sample=True is not implemented (greedy target only)")
         if stop_strings is not None:
             raise NotImplementedError("stop_strings need a tokenizer; not available in this build")
         if max_new_tokens is not None:
@@ -91,9 +110,13 @@ class SubSpecSDGenerator:
         if past_key_values is None:
             raise ValueError("past_key_values is not provided")
         assert input_ids.shape[0] == 1, "Only support batch_size=1 for now."
-        return self._generate(input_ids.clone(), int(max_length), past_key_values, stream_callback)
+        logits_processor = (self._get_logits_processor(temperature=temperature, top_p=top_p, top_k=top_k)
+                            if do_sample else None)
+        return self._generate(input_ids.clone(), int(max_length), past_key_values, stream_callback,
+                              logits_processor=logits_processor, do_sample=bool(do_sample))
 
-    def _generate(self, input_ids, max_length: int, past_key_values: KVManager, stream_callback=None):
+    def _generate(self, input_ids, max_length: int, past_key_values: KVManager, stream_callback=None,
+                  logits_processor=None, do_sample: bool = False):
         dev = self.target_model.device
         input_ids = input_ids.to(dev)
         self.draft_model.set_past_key_values(past_key_values)
@@ -104,7 +127,7 @@ class SubSpecSDGenerator:
         org_len = input_ids.shape[1]
 
         logits = self._chunked_prefill_forward(input_ids, past_key_values)
-        sampled = logits.argmax(-1).view(1, 1)
+        sampled = self._sample_token(logits.view(1, 1, -1), logits_processor, do_sample).view(1, 1)
         input_ids = torch.cat([input_ids, sampled], dim=-1)
         if stream_callback is not None:
             stream_callback(sampled)
@@ -119,7 +142,7 @@ class SubSpecSDGenerator:
             prev_kv_len = past_key_values.get_seq_length()
             logits = self._tree_decoding(tree, past_key_values, position_offset=input_ids.shape[1] - 1)
             e[2].record()
-            out = self._verify(tree, 0, logits)
+            out = self._verify(tree, 0, logits, logits_processor, do_sample)
             # KV rows of the accepted path move up right behind the verifier, count read on the device
             past_key_values.reorder_cache_with_offset(out["contexts"][0], new_chunk_len=p.max_verify_tokens,
                                                       offset=prev_kv_len, dim=2, count_dev=out["counts"][0, 0:1])

@@ -50,8 +50,15 @@ def tree_verify(
     window_size: int = 1,
     exact_entropy: bool = False,
     workspace: Optional[torch.Tensor] = None,
+    do_sample: bool = False,
+    temperature: float = 1.0,
+    seed: int = 0,
+    offset: int = 0,
 ) -> Dict[str, torch.Tensor]:
     """Runs the fused verifier; everything stays on the device (no synchronisation here).
+
+    ``do_sample=True`` draws the target token of every row from ``softmax(logits / temperature)``
+    (Philox stream ``seed`` / ``offset``) instead of taking the argmax.
 
     Returns device tensors: ``tokens`` / ``contexts`` int64 [B, n+1], ``counts`` int32 [B, 4]
     (emitted, accept_len, total_len, status) and the per-node ``target`` int64 / ``entropy`` /
@@ -89,16 +96,37 @@ def tree_verify(
         "entropy": torch.zeros((B, rows), dtype=torch.float32, device=dev),
         "child_prob": torch.empty((B, rows), dtype=torch.float32, device=dev),
     }
-    code = lib.subspec_tree_verify(
-        logits.data_ptr(), _dtype_code(logits), B, rows, V, token_ids.data_ptr(), parents.data_ptr(), n,
-        int(root), int(skip_nodes), -1 if eos_token_id is None else int(eos_token_id),
-        method, gate, float(threshold), int(window_size),
-        L.ENTROPY_ALWAYS if exact_entropy else L.ENTROPY_GUARD,
-        workspace.data_ptr(), workspace.numel() * workspace.element_size(),
-        out["tokens"].data_ptr(), out["contexts"].data_ptr(), out["counts"].data_ptr(),
-        out["target"].data_ptr(), out["entropy"].data_ptr(), out["child_prob"].data_ptr(), _stream(dev))
-    L.check(code, "subspec_tree_verify")
+    head = (logits.data_ptr(), _dtype_code(logits), B, rows, V, token_ids.data_ptr(), parents.data_ptr(), n,
+            int(root), int(skip_nodes), -1 if eos_token_id is None else int(eos_token_id),
+            method, gate, float(threshold), int(window_size),
+            L.ENTROPY_ALWAYS if exact_entropy else L.ENTROPY_GUARD)
+    tail = (workspace.data_ptr(), workspace.numel() * workspace.element_size(),
+            out["tokens"].data_ptr(), out["contexts"].data_ptr(), out["counts"].data_ptr(),
+            out["target"].data_ptr(), out["entropy"].data_ptr(), out["child_prob"].data_ptr(), _stream(dev))
+    if do_sample:
+        mask = (1 << 64) - 1
+        code = lib.subspec_tree_verify_sample(*head, float(temperature), int(seed) & mask, int(offset) & mask, *tail)
+        L.check(code, "subspec_tree_verify_sample")
+    else:
+        code = lib.subspec_tree_verify(*head, *tail)
+        L.check(code, "subspec_tree_verify")
     return out
+
+
+def sample_tokens(logits: torch.Tensor, temperature: float = 1.0, seed: int = 0, offset: int = 0) -> torch.Tensor:
+    """One token per row of ``logits [rows, V]`` drawn from ``softmax(logits / temperature)`` (rounded to the
+    logits dtype) with the verifier's Philox race: ``GeneratorBase._sample_token(do_sample=True)`` for
+    the rows outside a tree, e.g. the first token after the prefill
+    (specdecodes/models/generators/base.py:116-132).  Returns int64 ``[rows]`` on the device."""
+    lg = logits.reshape(-1, logits.shape[-1])
+    rows = lg.shape[0]
+    if rows > L.MAX_TREE_NODES:
+        raise ValueError(f"at most {L.MAX_TREE_NODES} rows per call")
+    # a parentless forest: no node has children, so the verifier only reports each row's draw
+    tok = torch.zeros(rows, dtype=torch.int32, device=lg.device)
+    par = torch.full((rows,), -1, dtype=torch.int32, device=lg.device)
+    out = tree_verify(lg, tok, par, do_sample=True, temperature=temperature, seed=seed, offset=offset)
+    return out["target"][0]
 
 
 def kv_compact_(
@@ -279,6 +307,17 @@ def softmax_temperature(logits: torch.Tensor, temperature: float) -> torch.Tenso
 
 
 # ---------------------------------------------------------------------------------------------- decoder layer
+def temperature_warp(logits: torch.Tensor, temperature: float) -> torch.Tensor:
+    """``logits / temperature`` in the logits dtype (TemperatureLogitsWarper; generators/base.py:57-58)."""
+    dev = _require_gpu(logits)
+    logits = logits.contiguous()
+    out = torch.empty_like(logits)
+    code = L.lib().subspec_temperature_warp(logits.data_ptr(), out.data_ptr(), _dtype_code(logits), logits.numel(),
+                                            float(temperature), _stream(dev))
+    L.check(code, "subspec_temperature_warp")
+    return out
+
+
 def decoder_layer_dims(dtype: torch.dtype, n_rows: int, hidden: int, intermediate: int, n_q_heads: int, n_kv_heads: int,
                        head_dim: int, kv_seq_stride: int, prefix_len: int, n_tree_slots: int, rms_eps: float,
                        rope_theta: float) -> "L.DecoderLayerDims":

@@ -130,10 +130,65 @@ def test_generator_argument_errors():
     with pytest.raises(ValueError):
         gen.generate(ids, max_new_tokens=4, do_sample=False)                    # no cache
     with pytest.raises(NotImplementedError):
-        gen.generate(ids, max_new_tokens=4, do_sample=True, past_key_values=kv)
+        gen.generate(ids, max_new_tokens=4, do_sample=False, stop_strings=["x"], past_key_values=kv)
+    with pytest.raises(ValueError):                                             # the warper rejects T <= 0
+        gen.generate(ids, max_new_tokens=4, do_sample=True, temperature=0.0, past_key_values=kv)
     with pytest.raises(ValueError):
         create_kv_cache("dynamic", max_cache_len=8, config=CFG)
     bad = SubSpecSDGenerator(target, None, SubSpecSDDraftModel(draft), DraftParams(max_depth=2, topk_len=2),
                              generator_kwargs=dict(verify_method="bogus"))
     with pytest.raises(ValueError):
         bad.generate(ids, max_new_tokens=4, do_sample=False, past_key_values=kv)
+
+
+def _sampled_run(seed, max_new=20, **sampling):
+    kv, target, draft, _ = _models()
+    gen = SubSpecSDGenerator(target, None, SubSpecSDDraftModel(draft), DraftParams(temperature=0.2, max_depth=4, topk_len=4),
+                             generator_kwargs=dict(seed=seed))
+    prompt = torch.randint(0, CFG.vocab_size, (1, 32), generator=torch.Generator().manual_seed(4)).to(DEV)
+    out = gen.generate(prompt, max_new_tokens=max_new, past_key_values=kv, **sampling)
+    assert out.shape[1] == 32 + max_new and kv.get_seq_length() == out.shape[1] - 1
+    return out[0, 32:].cpu()
+
+
+def test_sampling_cycle_is_seeded_and_top_k_one_is_greedy():
+    a = _sampled_run(11, do_sample=True, temperature=0.9)
+    b = _sampled_run(11, do_sample=True, temperature=0.9)
+    c = _sampled_run(12, do_sample=True, temperature=0.9)
+    assert torch.equal(a, b) and not torch.equal(a, c)
+    assert int(a.min()) >= 0 and int(a.max()) < CFG.vocab_size
+    # the other warpers run through the same cycle
+    d = _sampled_run(5, do_sample=True, temperature=0.8, top_k=5, top_p=0.9)
+    assert int(d.min()) >= 0 and int(d.max()) < CFG.vocab_size
+
+
+def test_one_sampling_cycle_against_the_oracle():
+    from oracle import sampling as osamp
+    kv, target, draft, _ = _models()
+    prompt = torch.randint(0, CFG.vocab_size, (48,), generator=torch.Generator().manual_seed(6)).to(DEV)
+    lg = target.prefill(prompt, 0)
+    kv.seq_len = 48
+    dm = SubSpecSDDraftModel(draft)
+    gen = SubSpecSDGenerator(target, None, dm, DraftParams(temperature=0.2, max_depth=5, topk_len=4),
+                             generator_kwargs=dict(seed=77))
+    dm.set_past_key_values(kv)
+    proc = gen._get_logits_processor(temperature=0.5)
+    first = gen._sample_token(lg.view(1, 1, -1), proc, True)          # stream offset 0
+    want, margin = osamp.draw_tokens(osamp.warp_probs(lg.cpu(), 0.5), seed=77, offset=0)
+    assert first.item() == want[0] or margin[0] < 2.0 ** -6
+    tree = dm.speculate(first.view(1, 1))
+    logits = gen._tree_decoding(tree, kv, position_offset=48)
+    out = gen._verify(tree, 0, logits, proc, True)                     # stream offset 1
+    torch.cuda.synchronize()
+    d = tree.get_tree_data()
+    drawn = out["target"][0].cpu()
+    ref_draw, margins = osamp.draw_tokens(osamp.warp_probs(logits.cpu(), 0.5), seed=77, offset=1)
+    for g, w, m in zip(drawn.tolist(), ref_draw, margins):
+        assert g == w or m < 2.0 ** -6
+    exp_t, exp_c, (_, exp_a) = ov.verify_logits(logits.cpu(), d["token_ids"].tolist(), d["parent_indices"].tolist(),
+                                               temperature=0.5, target_tokens=drawn.tolist())
+    emitted, accept = int(out["counts"][0, 0]), int(out["counts"][0, 1])
+    assert out["tokens"][0, :emitted].tolist() == exp_t and out["contexts"][0, :emitted].tolist() == exp_c
+    assert accept == exp_a
+    # every emitted token is the draw of its context (exact verifier)
+    assert out["tokens"][0, :emitted].tolist() == [int(drawn[c]) for c in exp_c]

@@ -7,6 +7,11 @@
   * permutation: reordering the trees reorders the outputs;
   * planted flavours: trees built with an all-exact depth-8 path accept all 8 draft tokens, trees
     with nothing planted accept none;
+  * sampling verifier at the same size: seeded draws are reproducible, a tree's draws do not depend
+    on the trees around it once its global row numbers are the same, every emitted token of the
+    exact verifier is the draw of its context, a sample of rows equals the oracle's draws, and the
+    drawn tokens' mean log-probability sits at minus the mean row entropy (what sampling from
+    the rows themselves gives, and what neither argmax nor uniform draws give);
   * top-k: every value is the rounded product of its (row, token) probability and the parent
     probability, values are sorted (ties by index), and the count of strictly larger / larger-or-equal
     products brackets k for every row (checked with torch on the device)."""
@@ -70,6 +75,54 @@ def test_verify_full_batch_properties():
     shuffled = _verify(cfg["logits"][perm], [cfg["tokens"][i] for i in perm], [cfg["parents"][i] for i in perm], cfg)
     for k in KEYS:
         assert torch.equal(shuffled[k], full[k][perm]), k
+
+
+def test_sampling_verify_full_batch_properties():
+    from oracle import sampling as osamp
+    print("full-size sampling verify: 32 x 64 x 152064 bf16, T = 0.8", flush=True)
+    cfg = W.lossy_config(seed=1, batch=32, device=DEV)
+    tok = torch.tensor(cfg["tokens"], dtype=torch.int32, device=DEV)
+    par = torch.tensor(cfg["parents"], dtype=torch.int32, device=DEV)
+    T = 0.8
+
+    def run(logits, tok, par, seed, offset):
+        out = ops.tree_verify(logits, tok, par, verify_method="exact", do_sample=True, temperature=T, seed=seed,
+                              offset=offset)
+        torch.cuda.synchronize()
+        return out
+
+    full = run(cfg["logits"], tok, par, 17, 3)
+    again = run(cfg["logits"], tok, par, 17, 3)
+    other = run(cfg["logits"], tok, par, 17, 4)
+    assert torch.equal(full["target"], again["target"]) and torch.equal(full["counts"], again["counts"])
+    assert (full["target"] != other["target"]).float().mean().item() > 0.3
+    counts = full["counts"].cpu()
+    assert int(counts[:, 3].abs().sum()) == 0
+    # every emitted token is the draw of its context node (exact verifier, skip_nodes = 0)
+    for b in range(32):
+        n = int(counts[b, 0])
+        ctx = full["contexts"][b, :n]
+        assert torch.equal(full["tokens"][b, :n], full["target"][b][ctx]), b
+        assert n == int(counts[b, 1]) + 1
+    # tree 0 alone occupies the same global rows 0..63: identical draws and walk
+    alone = run(cfg["logits"][:1], tok[:1], par[:1], 17, 3)
+    assert torch.equal(alone["target"][0], full["target"][0])
+    assert torch.equal(alone["counts"][0], full["counts"][0])
+    # the oracle on a sample of rows of trees 0 and 31 (global row = 64 * tree + row)
+    for b, rows in ((0, [0, 1, 17, 63]), (31, [0, 5, 62])):
+        lg = cfg["logits"][b][rows].cpu()
+        for j, r in enumerate(rows):
+            want, margin = osamp.draw_tokens(osamp.warp_probs(lg[j:j + 1], T), 17, 3, first_row=64 * b + r)
+            assert int(full["target"][b, r]) == want[0] or margin[0] < 2.0 ** -6, (b, r)
+    # distribution-level check over all 2048 draws: E[log p(draw)] = -H(row), both estimated in fp32
+    lp_sum = ent_sum = 0.0
+    for b in range(32):
+        logp = torch.log_softmax((cfg["logits"][b].float() / T).to(torch.bfloat16).float(), -1)
+        lp_sum += float(torch.gather(logp, 1, full["target"][b].unsqueeze(1)).sum())
+        ent_sum += float(-(logp.exp() * logp).sum())
+    mean_lp, mean_h = lp_sum / 2048, ent_sum / 2048
+    print("mean log p(draw)", mean_lp, "mean entropy", mean_h, flush=True)
+    assert abs(mean_lp + mean_h) < 0.05 * max(1.0, mean_h)
 
 
 def test_topk_full_size_properties():

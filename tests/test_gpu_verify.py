@@ -214,8 +214,14 @@ def test_verify_tree_host_interface_and_errors():
     with pytest.raises(ValueError):
         verify_tree(tree=tree, root_ind=0, logits=logits.to(DEV), eos_token_id=None, verify_method="lossy",
                     verify_kwargs=dict(threshold_method="bogus"))
-    with pytest.raises(NotImplementedError):
-        verify_tree(tree=tree, root_ind=0, logits=logits.to(DEV), eos_token_id=None, do_sample=True)
+    # sampling target through the same interface: the planted logits (+9 over N(0,1) rows) make the
+    # drafted path the overwhelmingly likely draw at a low temperature
+    from subspec_amd.tree_verify import SampleStream
+    from transformers.generation.logits_process import LogitsProcessorList, TemperatureLogitsWarper
+    toks, ctx, (total, acc) = verify_tree(tree=tree, root_ind=0, logits=logits.to(DEV), eos_token_id=None,
+                                          logits_processor=LogitsProcessorList([TemperatureLogitsWarper(0.25)]),
+                                          do_sample=True, stream=SampleStream(1))
+    assert toks.tolist() == [[11, 13, 40]] and ctx.tolist() == [0, 1, 3] and (total, acc) == (2, 2)
     with pytest.raises(ValueError):            # more nodes than the kernels are built for
         ops.tree_verify(torch.zeros(300, 64, device=DEV), torch.zeros(300, dtype=torch.int32, device=DEV),
                         torch.zeros(300, dtype=torch.int32, device=DEV))
