@@ -169,8 +169,10 @@ def bench_e2e(args):
         line = {"metric": "accepted tokens/sec, end-to-end speculative cycle", "value": round(log["tput"], 2),
                 "unit": "tokens/s", "n_gpus": 1, "higher_is_better": True, "dtype": "bf16",
                 "data": "synthetic prompt, weights from " + args.checkpoint if args.checkpoint else "synthetic",
-                "config": {"workload": f"BASELINE config 5: {'checkpoint' if args.checkpoint else 'Qwen2.5-7B shape'}, layers "
-                                       f"{min(args.keep_layers, cfg.num_hidden_layers)}-{cfg.num_hidden_layers - 1} streamed, int4 draft, depth 8, k 8, "
+                "config": {"workload": f"BASELINE config 5: {'checkpoint' if args.checkpoint else 'Qwen2.5-7B shape'}, "
+                                       + ("all layers resident" if args.keep_layers >= cfg.num_hidden_layers else
+                                          f"layers {args.keep_layers}-{cfg.num_hidden_layers - 1} streamed")
+                                       + f", int4 draft, depth 8, k 8, "
                                        f"<=64 nodes, prompt 2048, {args.new_tokens} new tokens, verify {method}",
                            "verify_method": method, "n_iter": log["n_iter"], "n_tokens": log["n_tokens"],
                            "tokens_per_cycle": round(log["avg_sampled"], 3),

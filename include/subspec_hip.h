@@ -216,9 +216,15 @@ int subspec_tree_attention(const void* q, const void* k_cache, const void* v_cac
  *           specdecodes/models/draft_models/classic_sd.py:10-16
  *
  * logits, out  device [rows, vocab], same dtype (fp32 / fp16 / bf16); out may alias logits.
+ * workspace    device, 8-byte aligned, subspec_softmax_temperature_workspace(rows, vocab) bytes, or
+ *              NULL.  With few rows (a draft step has 1 to 16) one workgroup per row leaves the chip
+ *              idle; given the workspace, rows are cut into slices over two launches.  NULL (or a
+ *              size of 0 returned by the query) selects the one-workgroup-per-row kernel.
  */
+size_t subspec_softmax_temperature_workspace(int64_t rows, int64_t vocab);
+
 int subspec_softmax_temperature(const void* logits, void* out, int dtype, int64_t rows, int64_t vocab,
-                                float temperature, void* stream);
+                                float temperature, void* workspace, size_t workspace_bytes, void* stream);
 
 /* TemperatureLogitsWarper alone: out[i] = logits[i] / temperature, the IEEE quotient rounded once to
  * the logits dtype (what ``scores / temperature`` gives for a tensor in that dtype).
@@ -309,6 +315,40 @@ size_t subspec_int4_decoder_layer_workspace(const subspec_decoder_layer_dims* di
 int subspec_int4_decoder_layer(const subspec_decoder_layer_dims* dims, const subspec_decoder_layer_weights* weights,
                                void* x, const int32_t* positions, const int32_t* cache_rows, const uint64_t* anc_bits,
                                void* k_cache, void* v_cache, void* workspace, size_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Dense 16-bit linear for few activation rows:  y[M, N] = x[M, K] * W[N, K]^T (+ bias), 1 <= M <= 64.
+ *
+ * Replaces  the nn.Linear projections (q/k/v, o, gate/up, down) of the TARGET model's decoder layers in
+ *           the tree-decoding forward: ClassicSDGeneratorBase._tree_decoding -> self.target_model(...)
+ *           specdecodes/models/generators/classic_sd.py:75-109 (at most max_verify_tokens = 64 rows).
+ *
+ * x  device [M, K], w  device [N, K] row-major, bias [N] or NULL, y [M, N]: all bf16 or all fp16.
+ * N % 16 == 0, K % 64 == 0; x and w 16-byte aligned.  Products accumulate in fp32 and are rounded once.
+ * workspace  subspec_dense_linear_workspace(M, N, K) bytes (fp32 partials when K is split).
+ */
+size_t subspec_dense_linear_workspace(int64_t M, int64_t N, int64_t K);
+
+int subspec_dense_linear(const void* x, const void* w, const void* bias, void* y, int dtype, int64_t M, int64_t N,
+                         int64_t K, void* workspace, size_t workspace_bytes, void* stream);
+
+/* One decoder layer with dense 16-bit projections: same sequence of kernels, arguments, workspace
+ * (subspec_int4_decoder_layer_workspace) and limits as subspec_int4_decoder_layer, for the target
+ * model's layers (HF Qwen2DecoderLayer inside the forward named above); q|k|v and gate|up rows are
+ * stored fused.  Weight matrices are row-major [N, K] in the activation dtype. */
+typedef struct subspec_dense_layer_weights {
+  const void* input_norm;   /* [hidden] */
+  const void* post_norm;    /* [hidden] */
+  const void* qkv_w;        /* [(n_q_heads + 2 n_kv_heads) * head_dim, hidden] */
+  const void* qkv_bias;     /* [N] or NULL */
+  const void* o_w;          /* [hidden, n_q_heads * head_dim] */
+  const void* gate_up_w;    /* [2 * intermediate, hidden] */
+  const void* down_w;       /* [hidden, intermediate] */
+} subspec_dense_layer_weights;
+
+int subspec_dense_decoder_layer(const subspec_decoder_layer_dims* dims, const subspec_dense_layer_weights* weights,
+                                void* x, const int32_t* positions, const int32_t* cache_rows, const uint64_t* anc_bits,
+                                void* k_cache, void* v_cache, void* workspace, size_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------------------------------
  * Layer streaming: asynchronous copy of one weight slab from pinned host memory to its device

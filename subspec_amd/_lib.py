@@ -38,6 +38,11 @@ class DecoderLayerWeights(C.Structure):
                                   "gate_up_wq", "gate_up_sz", "down_wq", "down_sz")]
 
 
+class DenseLayerWeights(C.Structure):
+    """subspec_dense_layer_weights"""
+    _fields_ = [(n, _p) for n in ("input_norm", "post_norm", "qkv_w", "qkv_bias", "o_w", "gate_up_w", "down_w")]
+
+
 _SIGNATURES = {
     "subspec_abi_version": (C.c_int, []),
     "subspec_last_error": (C.c_char_p, []),
@@ -56,13 +61,18 @@ _SIGNATURES = {
     "subspec_tree_attention_workspace": (_sz, [_i64, _i64, _i64, _i64]),
     "subspec_tree_attention": (C.c_int, [_p, _p, _p, _p, C.c_int, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _p, _i64,
                                          C.c_float, _p, _sz, _p]),
-    "subspec_softmax_temperature": (C.c_int, [_p, _p, C.c_int, _i64, _i64, C.c_float, _p]),
+    "subspec_softmax_temperature_workspace": (_sz, [_i64, _i64]),
+    "subspec_softmax_temperature": (C.c_int, [_p, _p, C.c_int, _i64, _i64, C.c_float, _p, _sz, _p]),
     "subspec_temperature_warp": (C.c_int, [_p, _p, C.c_int, _i64, C.c_float, _p]),
     "subspec_int4_linear_workspace": (_sz, [_i64, _i64, _i64]),
     "subspec_int4_linear": (C.c_int, [_p, _p, _p, _p, _p, C.c_int, _i64, _i64, _i64, _i64, _p, _sz, _p]),
     "subspec_int4_decoder_layer_workspace": (_sz, [C.POINTER(DecoderLayerDims)]),
     "subspec_int4_decoder_layer": (C.c_int, [C.POINTER(DecoderLayerDims), C.POINTER(DecoderLayerWeights), _p, _p, _p, _p,
                                              _p, _p, _p, _sz, _p]),
+    "subspec_dense_linear_workspace": (_sz, [_i64, _i64, _i64]),
+    "subspec_dense_linear": (C.c_int, [_p, _p, _p, _p, C.c_int, _i64, _i64, _i64, _p, _sz, _p]),
+    "subspec_dense_decoder_layer": (C.c_int, [C.POINTER(DecoderLayerDims), C.POINTER(DenseLayerWeights), _p, _p, _p, _p,
+                                              _p, _p, _p, _sz, _p]),
     "subspec_stream_copy_h2d": (C.c_int, [_p, _p, _sz, _p]),
     "subspec_kv_compact": (C.c_int, [_p, _p, _i64, _i64, _i64, _i64, _i64, _p, _p, _i32, _i32, _p]),
 }

@@ -1,4 +1,5 @@
-// One int4 decoder layer of the substitute draft over the tree rows, launched from one host call.
+// One decoder layer over the tree rows, launched from one host call: the substitute draft's int4
+// layer, and the target's layer with dense 16-bit projections (same sequence, see the end).
 //
 // The reference runs the draft as a HuggingFace Qwen2 / Llama decoder layer whose seven projections
 // were replaced by HQQ int4 linears (specdecodes/helpers/recipes/subspec/hqq_4bit_postspec.py:17-58)
@@ -16,6 +17,10 @@
 // Rounding follows the eager torch layer: every intermediate tensor is rounded to the activation
 // dtype where torch would materialise it (normalised activations before the weight product, the
 // two rotary products and their sum, silu before the product with `up`, both residual sums).
+//
+// The target model's layer in the tree-decoding forward (HF Qwen2DecoderLayer under
+// ClassicSDGeneratorBase._tree_decoding, specdecodes/models/generators/classic_sd.py:75-109) is the
+// same sequence with dense 16-bit projections (dense.hip) in place of the int4 ones.
 #include "common.h"
 #include <algorithm>
 
@@ -184,6 +189,10 @@ static LayerPlan layer_plan(const subspec_decoder_layer_dims& s) {
   sub = std::max(sub, subspec_int4_linear_workspace(s.n_rows, H, Q));
   sub = std::max(sub, subspec_int4_linear_workspace(s.n_rows, 2 * F, H));
   sub = std::max(sub, subspec_int4_linear_workspace(s.n_rows, H, F));
+  sub = std::max(sub, subspec_dense_linear_workspace(s.n_rows, Q + 2 * KV, H));
+  sub = std::max(sub, subspec_dense_linear_workspace(s.n_rows, H, Q));
+  sub = std::max(sub, subspec_dense_linear_workspace(s.n_rows, 2 * F, H));
+  sub = std::max(sub, subspec_dense_linear_workspace(s.n_rows, H, F));
   sub = std::max(sub, subspec_tree_attention_workspace(1, s.n_q_heads, s.prefix_len, s.n_tree_slots));
   p.sub_bytes = align_up(sub, 256);
   p.sub = take(p.sub_bytes);
@@ -211,8 +220,22 @@ static int check_dims(const subspec_decoder_layer_dims* s) {
   return SUBSPEC_OK;
 }
 
+// The four projections of a layer in either storage: int4 codes + (scale, zero) words, or a dense
+// row-major 16-bit matrix (then the second pointer is unused).
+struct Projection { const void* w; const void* sz; };
+struct LayerWeights {
+  const void *input_norm, *post_norm, *qkv_bias;
+  Projection qkv, o, gate_up, down;
+  bool dense;
+};
+static int project(const LayerWeights& w, const Projection& p, const void* x, const void* bias, void* y, int dtype, int64_t M,
+                   int64_t N, int64_t K, void* sub, size_t sub_bytes, hipStream_t st) {
+  if (w.dense) return subspec_dense_linear(x, p.w, bias, y, dtype, M, N, K, sub, sub_bytes, st);
+  return subspec_int4_linear(x, (const uint32_t*)p.w, (const uint32_t*)p.sz, bias, y, dtype, M, N, K, 64, sub, sub_bytes, st);
+}
+
 template <int DT>
-static int run_layer(const subspec_decoder_layer_dims& s, const subspec_decoder_layer_weights& w, uint16_t* x,
+static int run_layer(const subspec_decoder_layer_dims& s, const LayerWeights& w, uint16_t* x,
                      const int32_t* positions, const int32_t* cache_rows, const uint64_t* anc_bits, uint16_t* k_cache,
                      uint16_t* v_cache, char* ws, hipStream_t st) {
   const LayerPlan p = layer_plan(s);
@@ -225,20 +248,19 @@ static int run_layer(const subspec_decoder_layer_dims& s, const subspec_decoder_
   int rc;
   hipLaunchKernelGGL((add_rmsnorm_kernel<DT, false>), dim3(M), dim3(kNormThreads), 0, st, x, (const uint16_t*)nullptr,
                      (const uint16_t*)w.input_norm, h, H, s.rms_eps);
-  if ((rc = subspec_int4_linear(h, w.qkv_wq, w.qkv_sz, w.qkv_bias, qkv, DT, M, Q + 2 * KV, H, 64, sub, p.sub_bytes, st))) return rc;
+  if ((rc = project(w, w.qkv, h, w.qkv_bias, qkv, DT, M, Q + 2 * KV, H, sub, p.sub_bytes, st))) return rc;
   hipLaunchKernelGGL((rope_write_kernel<DT>), dim3(M, Hq + 2 * Hkv), dim3(64), 0, st, qkv, positions, cache_rows, q, k_cache,
                      v_cache, M, Hq, Hkv, D, s.kv_seq_stride, log2f(s.rope_theta));
   if ((rc = subspec_tree_attention(q, k_cache, v_cache, a, DT, 1, Hq, Hkv, M, s.n_tree_slots, D, s.kv_seq_stride, s.prefix_len,
                                    anc_bits, 0, 1.f / sqrtf((float)D), sub, p.sub_bytes, st)))
     return rc;
-  if ((rc = subspec_int4_linear(a, w.o_wq, w.o_sz, nullptr, o, DT, M, H, Q, 64, sub, p.sub_bytes, st))) return rc;
+  if ((rc = project(w, w.o, a, nullptr, o, DT, M, H, Q, sub, p.sub_bytes, st))) return rc;
   hipLaunchKernelGGL((add_rmsnorm_kernel<DT, true>), dim3(M), dim3(kNormThreads), 0, st, x, o, (const uint16_t*)w.post_norm, h, H,
                      s.rms_eps);
-  if ((rc = subspec_int4_linear(h, w.gate_up_wq, w.gate_up_sz, nullptr, gu, DT, M, 2 * (int64_t)F, H, 64, sub, p.sub_bytes, st)))
-    return rc;
+  if ((rc = project(w, w.gate_up, h, nullptr, gu, DT, M, 2 * (int64_t)F, H, sub, p.sub_bytes, st))) return rc;
   const int64_t act_pieces = (int64_t)M * F / 8;
   hipLaunchKernelGGL((silu_mul_kernel<DT>), dim3((unsigned)((act_pieces + 255) / 256)), dim3(256), 0, st, gu, act, F, act_pieces);
-  if ((rc = subspec_int4_linear(act, w.down_wq, w.down_sz, nullptr, d, DT, M, H, F, 64, sub, p.sub_bytes, st))) return rc;
+  if ((rc = project(w, w.down, act, nullptr, d, DT, M, H, F, sub, p.sub_bytes, st))) return rc;
   const int64_t x_pieces = (int64_t)M * H / 8;
   hipLaunchKernelGGL((add_kernel<DT>), dim3((unsigned)((x_pieces + 255) / 256)), dim3(256), 0, st, x, d, x_pieces);
   SUBSPEC_CHECK_HIP(hipGetLastError());
@@ -254,17 +276,15 @@ extern "C" size_t subspec_int4_decoder_layer_workspace(const subspec_decoder_lay
   return layer_plan(*dims).total;
 }
 
-extern "C" int subspec_int4_decoder_layer(const subspec_decoder_layer_dims* dims, const subspec_decoder_layer_weights* weights,
-                                          void* x, const int32_t* positions, const int32_t* cache_rows,
-                                          const uint64_t* anc_bits, void* k_cache, void* v_cache, void* workspace,
-                                          size_t workspace_bytes, void* stream) {
+static int decoder_layer_entry(const subspec_decoder_layer_dims* dims, const LayerWeights& w, void* x, const int32_t* positions,
+                               const int32_t* cache_rows, const uint64_t* anc_bits, void* k_cache, void* v_cache,
+                               void* workspace, size_t workspace_bytes, void* stream) {
   const int rc = check_dims(dims);
   if (rc != SUBSPEC_OK) return rc;
-  if (!weights || !x || !positions || !cache_rows || !anc_bits || !k_cache || !v_cache)
+  if (!x || !positions || !cache_rows || !anc_bits || !k_cache || !v_cache)
     SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "decoder_layer: null pointer argument");
-  const subspec_decoder_layer_weights& w = *weights;
-  if (!w.input_norm || !w.post_norm || !w.qkv_wq || !w.qkv_sz || !w.o_wq || !w.o_sz || !w.gate_up_wq || !w.gate_up_sz ||
-      !w.down_wq || !w.down_sz)
+  if (!w.input_norm || !w.post_norm || !w.qkv.w || !w.o.w || !w.gate_up.w || !w.down.w ||
+      (!w.dense && (!w.qkv.sz || !w.o.sz || !w.gate_up.sz || !w.down.sz)))
     SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "decoder_layer: null weight pointer");
   if ((uintptr_t)x % 16 || (uintptr_t)w.input_norm % 16 || (uintptr_t)w.post_norm % 16 || (uintptr_t)k_cache % 16 ||
       (uintptr_t)v_cache % 16)
@@ -278,4 +298,26 @@ extern "C" int subspec_int4_decoder_layer(const subspec_decoder_layer_dims* dims
                                    (char*)workspace, (hipStream_t)stream);
   return run_layer<SUBSPEC_F16>(*dims, w, (uint16_t*)x, positions, cache_rows, anc_bits, (uint16_t*)k_cache, (uint16_t*)v_cache,
                                 (char*)workspace, (hipStream_t)stream);
+}
+
+extern "C" int subspec_int4_decoder_layer(const subspec_decoder_layer_dims* dims, const subspec_decoder_layer_weights* weights,
+                                          void* x, const int32_t* positions, const int32_t* cache_rows,
+                                          const uint64_t* anc_bits, void* k_cache, void* v_cache, void* workspace,
+                                          size_t workspace_bytes, void* stream) {
+  if (!weights) SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "decoder_layer: null weights");
+  const subspec_decoder_layer_weights& s = *weights;
+  const LayerWeights w{s.input_norm, s.post_norm, s.qkv_bias, {s.qkv_wq, s.qkv_sz}, {s.o_wq, s.o_sz},
+                       {s.gate_up_wq, s.gate_up_sz}, {s.down_wq, s.down_sz}, false};
+  return decoder_layer_entry(dims, w, x, positions, cache_rows, anc_bits, k_cache, v_cache, workspace, workspace_bytes, stream);
+}
+
+extern "C" int subspec_dense_decoder_layer(const subspec_decoder_layer_dims* dims, const subspec_dense_layer_weights* weights,
+                                           void* x, const int32_t* positions, const int32_t* cache_rows,
+                                           const uint64_t* anc_bits, void* k_cache, void* v_cache, void* workspace,
+                                           size_t workspace_bytes, void* stream) {
+  if (!weights) SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "decoder_layer: null weights");
+  const subspec_dense_layer_weights& s = *weights;
+  const LayerWeights w{s.input_norm, s.post_norm, s.qkv_bias, {s.qkv_w, nullptr}, {s.o_w, nullptr},
+                       {s.gate_up_w, nullptr}, {s.down_w, nullptr}, true};
+  return decoder_layer_entry(dims, w, x, positions, cache_rows, anc_bits, k_cache, v_cache, workspace, workspace_bytes, stream);
 }

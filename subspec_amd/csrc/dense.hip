@@ -1,0 +1,279 @@
+// Dense 16-bit linear layers for few activation rows on gfx950:
+//   y[M, N] = x[M, K] * W[N, K]^T (+ bias),   1 <= M <= 64,   W row-major bf16 / fp16
+//
+// Replaces the nn.Linear modules of the target model's decoder layers in the tree-decoding forward
+// (ClassicSDGeneratorBase._tree_decoding -> self.target_model(...),
+// specdecodes/models/generators/classic_sd.py:75-109): at most max_verify_tokens = 64 tree nodes go
+// through the layer at once, so every projection streams its whole weight matrix for a handful of
+// rows and is bound by HBM (algorithmic bytes = N*K*2 + (M*K + M*N)*2).  A library GEMM tiled for
+// large M leaves more than half of that bandwidth unused at this shape.
+//
+// Same skeleton as the int4 kernel next door: the activations are the MFMA A operand, a 16-row
+// weight tile the B operand (v_mfma_f32_16x16x32, k permutation "step s, lane group c, element e ->
+// k = 16c + 8s + e" on both operands), a workgroup owns up to RT consecutive tiles, its four
+// wavefronts split K in groups of 64 and run as independent software pipelines (weights two groups
+// ahead in registers, activation block through a wavefront-private LDS stage), partial sums are
+// added in wavefront order at the end and split-K partials in split order by a second launch.
+// With the permutation above lane (ln, c) reads the 32 contiguous bytes of row ln, k = 64g + 16c ..
+// + 15: a wavefront's weight request covers whole 128-byte lines of 16 rows.
+#include "common.h"
+#include <algorithm>
+
+namespace subspec {
+
+constexpr int kDnThreads = 256;
+constexpr int kDnGroup = 64;
+constexpr int kDnXlStride = kDnGroup + 8;                      // LDS row stride (elements) of a parked activation block
+
+typedef float dn_v4f __attribute__((ext_vector_type(4)));
+typedef uint32_t dn_u4 __attribute__((ext_vector_type(4)));
+typedef __bf16 dn_v8bf __attribute__((ext_vector_type(8)));
+typedef _Float16 dn_v8h __attribute__((ext_vector_type(8)));
+
+template <int DT>
+__device__ __forceinline__ dn_v4f dn_mfma32(dn_u4 a, dn_u4 b, dn_v4f c) {
+  if constexpr (DT == SUBSPEC_BF16)
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(dn_v8bf, a), __builtin_bit_cast(dn_v8bf, b), c, 0, 0, 0);
+  else
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(dn_v8h, a), __builtin_bit_cast(dn_v8h, b), c, 0, 0, 0);
+}
+
+template <int DT, int MT, int RT>
+__global__ __launch_bounds__(kDnThreads) void dense_gemm_kernel(
+    const uint16_t* __restrict__ x, const uint16_t* __restrict__ w, const uint16_t* __restrict__ bias,
+    uint16_t* __restrict__ y, float* __restrict__ partial, int M, int64_t N, int K, int splits, int groups_per_split) {
+  // 4 wavefronts x 2 stages of a [16*MT][64] activation block; reused for the final reduction
+  constexpr int kStageBytes = 4 * 2 * MT * 16 * kDnXlStride * 2, kRedBytes = 2 * 4 * MT * 256 * 4;
+  __shared__ __attribute__((aligned(16))) unsigned char lds_raw[kStageBytes > kRedBytes ? kStageBytes : kRedBytes];
+  uint16_t* const xstage = (uint16_t*)lds_raw;
+  float* const red = (float*)lds_raw;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int ln = lane & 15, c = lane >> 4;
+  const int G = K / kDnGroup;
+  const int n_tiles = (int)(N / 16);
+  const int ks = blockIdx.y;
+  const int g_begin = ks * groups_per_split, g_end = min(G, g_begin + groups_per_split);
+  const int g_first = g_begin + wave;                            // this wavefront's groups: g_first + 4j
+  const int nj = g_first < g_end ? (g_end - g_first + 3) / 4 : 0;
+
+  // tiles [tile0, tile0 + ntl) of this workgroup: an even split of all tiles over the grid
+  const int tile0 = (int)((int64_t)blockIdx.x * n_tiles / gridDim.x);
+  const int ntl = (int)((int64_t)(blockIdx.x + 1) * n_tiles / gridDim.x) - tile0;     // 1 .. RT
+
+  dn_v4f acc[RT][MT];
+#pragma unroll
+  for (int t = 0; t < RT; ++t)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[t][mt] = dn_v4f{0.f, 0.f, 0.f, 0.f};
+
+  // Buffer-descriptor loads keep their place in the program (plain loads that feed a loop-carried
+  // value are merged into one load at the loop head, which would undo the prefetch distance) and
+  // return zeros outside the tensor.  The weight descriptor starts at this workgroup's first tile,
+  // so its offsets stay far below the 2 GiB range whatever the size of the matrix.
+  const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)x, 0, M * K * 2, 0x00027000);
+  const int64_t w_bytes = (int64_t)ntl * 16 * K * 2;
+  const __amdgpu_buffer_rsrc_t w_rsrc =
+      __builtin_amdgcn_make_buffer_rsrc((void*)(w + (int64_t)tile0 * 16 * K), 0, (int)w_bytes, 0x00027000);
+  constexpr int kXg = MT * 2;                                    // 16-byte pieces per lane of one group block
+  const int xg_off = ((lane >> 3) * K + (lane & 7) * 8) * 2;     // byte offset of piece 0; piece i is 8 rows further
+  uint16_t* const xl = xstage + wave * (2 * MT * 16 * kDnXlStride);  // this wavefront's two stages
+  const int xl_write = (lane >> 3) * kDnXlStride + (lane & 7) * 8;
+  const int xl_read = ln * kDnXlStride + c * 16;
+  const int w_lane = (ln * K + c * 16) * 2;                      // byte offset of this lane's 32 bytes inside a tile
+  int wofs[RT];                                                  // byte offset of (tile t, k = 0) from the first tile
+#pragma unroll
+  for (int t = 0; t < RT; ++t) wofs[t] = min(t, ntl - 1) * 16 * K * 2;
+
+  dn_u4 xg[kXg];                                                 // block on its way from global memory to LDS
+  dn_u4 wbuf[2][RT][2];
+
+#define SUBSPEC_DN_FETCH_X(J)                                                                           \
+  {                                                                                                     \
+    const int kc = min(g_first + 4 * (J), G - 1) * (kDnGroup * 2);                                      \
+    _Pragma("unroll") for (int i = 0; i < kXg; ++i)                                                     \
+      xg[i] = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, xg_off + i * 16 * K, kc, 0);                \
+  }
+#define SUBSPEC_DN_PARK_X(SLOT)                                                                         \
+  _Pragma("unroll") for (int i = 0; i < kXg; ++i)                                                       \
+    *(dn_u4*)(&xl[(SLOT) * (MT * 16 * kDnXlStride) + i * 8 * kDnXlStride + xl_write]) = xg[i];
+#define SUBSPEC_DN_FETCH_W(SLOT, J, T)                                                                  \
+  {                                                                                                     \
+    const int kc = wofs[T] + min(g_first + 4 * (J), G - 1) * (kDnGroup * 2);                            \
+    wbuf[SLOT][T][0] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, w_lane, kc, 0);                    \
+    wbuf[SLOT][T][1] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, w_lane + 16, kc, 0);               \
+  }
+  // Step J works on LDS stage SLOT = J & 1.  Once its operands are in registers the stage is free:
+  // the block of group J + 2 (requested one step ago) is parked there and group J + 3 requested.
+  // A step past the wavefront's last group multiplies activations that were replaced by zeros.
+#define SUBSPEC_DN_STEP(SLOT, J)                                                                        \
+  {                                                                                                     \
+    const bool step_live = (J) < nj;                                                                    \
+    dn_u4 xa[MT][2];                                                                                    \
+    _Pragma("unroll") for (int mt = 0; mt < MT; ++mt) {                                                 \
+      const uint16_t* xr = &xl[(SLOT) * (MT * 16 * kDnXlStride) + mt * 16 * kDnXlStride + xl_read];     \
+      const dn_u4 a0 = *(const dn_u4*)xr, a1 = *(const dn_u4*)(xr + 8);                                 \
+      xa[mt][0] = step_live ? a0 : dn_u4{0u, 0u, 0u, 0u};                                               \
+      xa[mt][1] = step_live ? a1 : dn_u4{0u, 0u, 0u, 0u};                                               \
+    }                                                                                                   \
+    SUBSPEC_DN_PARK_X(SLOT);                                                                            \
+    SUBSPEC_DN_FETCH_X((J) + 3);                                                                        \
+    __builtin_amdgcn_sched_barrier(0);              /* keep the requests here: a full step ahead of their use */ \
+    _Pragma("unroll") for (int t = 0; t < RT; ++t) {                                                    \
+      const dn_u4 b0 = wbuf[SLOT][t][0], b1 = wbuf[SLOT][t][1];                                         \
+      SUBSPEC_DN_FETCH_W(SLOT, (J) + 2, t);                                                             \
+      _Pragma("unroll") for (int mt = 0; mt < MT; ++mt) {                                               \
+        acc[t][mt] = dn_mfma32<DT>(xa[mt][0], b0, acc[t][mt]);                                          \
+        acc[t][mt] = dn_mfma32<DT>(xa[mt][1], b1, acc[t][mt]);                                          \
+      }                                                                                                 \
+    }                                                                                                   \
+    __builtin_amdgcn_sched_barrier(0);                                                                  \
+  }
+
+  SUBSPEC_DN_FETCH_X(0);
+#pragma unroll
+  for (int t = 0; t < RT; ++t) SUBSPEC_DN_FETCH_W(0, 0, t);
+  SUBSPEC_DN_PARK_X(0);
+  SUBSPEC_DN_FETCH_X(1);
+#pragma unroll
+  for (int t = 0; t < RT; ++t) SUBSPEC_DN_FETCH_W(1, 1, t);
+  SUBSPEC_DN_PARK_X(1);
+  SUBSPEC_DN_FETCH_X(2);
+  for (int j = 0; j < nj; j += 2) {
+    SUBSPEC_DN_STEP(0, j);
+    SUBSPEC_DN_STEP(1, j + 1);
+  }
+  __syncthreads();                                               // the stages are reused for the reduction below
+#undef SUBSPEC_DN_PARK_X
+#undef SUBSPEC_DN_FETCH_X
+#undef SUBSPEC_DN_FETCH_W
+#undef SUBSPEC_DN_STEP
+
+  // ---- sum the four wavefronts' partial accumulators in wavefront order (0, 1, 2, 3), one tile per
+  // round.  LDS holds two rounds, so a round needs one barrier; wavefront w finishes the activation
+  // row blocks mt = w, w + 4, ... of the tile.  Accumulator layout: rows m = 16*mt + 4*c + rr,
+  // column n = 16*tile + ln.
+#pragma unroll
+  for (int t = 0; t < RT; ++t) {
+    if (t >= ntl) break;                                         // uniform
+    float* stage = red + (t & 1) * (4 * MT * 256);
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) *(dn_v4f*)(&stage[((wave * MT + mt) * 64 + lane) * 4]) = acc[t][mt];
+    __syncthreads();                                             // round t written; round t - 1 fully read
+    const int64_t n = (int64_t)(tile0 + t) * 16 + ln;
+    const float bv = (splits == 1 && bias) ? Elem<DT>::load(bias, n) : 0.f;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      if ((mt & 3) != wave) continue;                            // uniform
+      dn_v4f v = *(const dn_v4f*)(&stage[((0 * MT + mt) * 64 + lane) * 4]);
+#pragma unroll
+      for (int wv = 1; wv < 4; ++wv) {
+        const dn_v4f o = *(const dn_v4f*)(&stage[((wv * MT + mt) * 64 + lane) * 4]);
+#pragma unroll
+        for (int rr = 0; rr < 4; ++rr) v[rr] += o[rr];
+      }
+#pragma unroll
+      for (int rr = 0; rr < 4; ++rr) {
+        const int m = mt * 16 + c * 4 + rr;
+        if (m >= M) continue;
+        if (splits == 1) Elem<DT>::store(y, (int64_t)m * N + n, v[rr] + bv);
+        else partial[((int64_t)ks * M + m) * N + n] = v[rr];
+      }
+    }
+  }
+}
+
+template <int DT>
+__global__ __launch_bounds__(256) void dense_reduce_kernel(const float* __restrict__ partial, const uint16_t* __restrict__ bias,
+                                                           uint16_t* __restrict__ y, int64_t M, int64_t N, int splits) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= M * N) return;
+  float v = 0.f;
+  for (int s = 0; s < splits; ++s) v += partial[(int64_t)s * M * N + i];
+  if (bias) v += Elem<DT>::load(bias, i % N);
+  Elem<DT>::store(y, i, v);
+}
+
+struct DnPlan { int wgs, row_tiles, splits, groups_per_split; };
+// Workgroups are balanced for two resident per CU (512).  A tile row group is 2 KB per 64 k, four times
+// the int4 kernel's, so fewer tiles per workgroup keep as many bytes in flight.
+static DnPlan dn_plan(int64_t M, int64_t N, int64_t K) {
+  (void)M;
+  const int G = (int)(K / kDnGroup);
+  const int64_t tiles = N / 16, slots = 512;
+  const int64_t want = (tiles + slots - 1) / slots;
+  const int row_tiles = want <= 1 ? 1 : want <= 2 ? 2 : 4;
+  const int64_t wgs = (tiles + row_tiles - 1) / row_tiles;
+  int splits = (int)std::max<int64_t>(1, (slots + wgs / 2) / wgs);
+  splits = std::min(splits, std::max(1, G / 56));              // a split costs a second launch: only for long K
+  splits = std::min(splits, 16);
+  int gps = (G + splits - 1) / splits;
+  gps = (gps + 3) / 4 * 4;
+  splits = (G + gps - 1) / gps;
+  return DnPlan{(int)wgs, row_tiles, splits, gps};
+}
+
+template <int DT>
+static int run_dense(const void* x, const void* w, const void* bias, void* y, int64_t M, int64_t N, int64_t K,
+                     void* workspace, hipStream_t st) {
+  const DnPlan pl = dn_plan(M, N, K);
+  float* partial = (float*)workspace;
+  const dim3 grid((unsigned)pl.wgs, (unsigned)pl.splits);
+#define SUBSPEC_DN_LAUNCH(MT, RT)                                                                                  \
+  hipLaunchKernelGGL((dense_gemm_kernel<DT, MT, RT>), grid, dim3(kDnThreads), 0, st, (const uint16_t*)x,           \
+                     (const uint16_t*)w, (const uint16_t*)bias, (uint16_t*)y, partial, (int)M, N, (int)K,          \
+                     pl.splits, pl.groups_per_split)
+#define SUBSPEC_DN_LAUNCH_MT(MT)                                                                                   \
+  do {                                                                                                             \
+    if (pl.row_tiles == 1) SUBSPEC_DN_LAUNCH(MT, 1);                                                               \
+    else if (pl.row_tiles == 2) SUBSPEC_DN_LAUNCH(MT, 2);                                                          \
+    else SUBSPEC_DN_LAUNCH(MT, 4);                                                                                 \
+  } while (0)
+  {
+    DominantKernelTimer timer(st);
+    if (M <= 16) SUBSPEC_DN_LAUNCH_MT(1);
+    else if (M <= 32) SUBSPEC_DN_LAUNCH_MT(2);
+    else SUBSPEC_DN_LAUNCH_MT(4);
+  }
+#undef SUBSPEC_DN_LAUNCH_MT
+#undef SUBSPEC_DN_LAUNCH
+  if (pl.splits > 1)
+    hipLaunchKernelGGL((dense_reduce_kernel<DT>), dim3((unsigned)((M * N + 255) / 256)), dim3(256), 0, st, partial,
+                       (const uint16_t*)bias, (uint16_t*)y, M, N, pl.splits);
+  SUBSPEC_CHECK_HIP(hipGetLastError());
+  return SUBSPEC_OK;
+}
+
+}  // namespace subspec
+
+using namespace subspec;
+
+extern "C" size_t subspec_dense_linear_workspace(int64_t M, int64_t N, int64_t K) {
+  if (M <= 0 || N <= 0 || K <= 0) return 256;
+  const DnPlan pl = dn_plan(M, N, K);
+  return (pl.splits > 1 ? align_up((size_t)pl.splits * M * N * sizeof(float), 256) : 0) + 256;
+}
+
+extern "C" int subspec_dense_linear(const void* x, const void* w, const void* bias, void* y, int dtype, int64_t M,
+                                    int64_t N, int64_t K, void* workspace, size_t workspace_bytes, void* stream) {
+  if (dtype != SUBSPEC_BF16 && dtype != SUBSPEC_F16)
+    SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "dense_linear: dtype %d not supported (bf16 / fp16 only)", dtype);
+  if (!x || !w || !y) SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "dense_linear: null pointer argument");
+  if (M <= 0 || N <= 0 || K <= 0 || N % 16 != 0 || K % kDnGroup != 0)
+    SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "dense_linear: M=%lld N=%lld K=%lld; N must be a multiple of 16 and K of 64",
+                 (long long)M, (long long)N, (long long)K);
+  if (M > 64) SUBSPEC_FAIL(SUBSPEC_ERR_LIMIT, "dense_linear: M=%lld exceeds the 64-row limit (tree width)", (long long)M);
+  if (K > 65536) SUBSPEC_FAIL(SUBSPEC_ERR_LIMIT, "dense_linear: K=%lld too large", (long long)K);
+  if ((uintptr_t)x % 16 || (uintptr_t)w % 16 || (uintptr_t)y % 2)
+    SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "dense_linear: x and w must be 16-byte aligned");
+  const size_t need = subspec_dense_linear_workspace(M, N, K);
+  if (need > 256) {
+    if (!workspace || workspace_bytes < need)
+      SUBSPEC_FAIL(SUBSPEC_ERR_WORKSPACE, "dense_linear: workspace of %zu bytes is smaller than the %zu required",
+                   workspace_bytes, need);
+    if ((uintptr_t)workspace % 16) SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "dense_linear: workspace must be 16-byte aligned");
+  }
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == SUBSPEC_BF16) return run_dense<SUBSPEC_BF16>(x, w, bias, y, M, N, K, workspace, st);
+  return run_dense<SUBSPEC_F16>(x, w, bias, y, M, N, K, workspace, st);
+}

@@ -126,15 +126,19 @@ class Decoder:
         self.cos = torch.cat([freqs, freqs], -1).cos()
         self.sin = torch.cat([freqs, freqs], -1).sin()
 
-    # ------------------------------------------------------------------ native int4 layers
+    # ------------------------------------------------------------------ native layers
     @property
     def native_layers(self) -> bool:
-        """True when every layer is int4-packed, i.e. the stack can run through the library's decoder-layer
-        entry point (one host call per layer instead of one per module)."""
+        """True when the stack can run through the library's decoder-layer entry points (one host call
+        per layer instead of one per module): every layer int4-packed, or every layer dense 16-bit."""
         if self._native is None:
-            self._native = bool(self.layers) and all("qkv_proj.wq" in w for w in self.layers)
+            packed = [("qkv_proj.wq" in w) for w in self.layers]
+            self._native = bool(self.layers) and (all(packed) or not any(packed)) and self.dtype != torch.float32
             if self._native:
-                self._native_weights = [ops.decoder_layer_weights(w) for w in self.layers]
+                make = ops.decoder_layer_weights if packed[0] else ops.dense_layer_weights
+                self._native_make = make
+                resident = min(self.first_streamed, len(self.layers))
+                self._native_weights = [make(w) for w in self.layers[:resident]]
                 self._native_ws = {}
         return self._native
 
@@ -152,7 +156,14 @@ class Decoder:
         pos32, rows32 = positions.to(torch.int32), rows.to(torch.int32)
         bits = anc_bits.to(torch.int64).contiguous()
         for i, w in enumerate(self._native_weights):
-            ops.int4_decoder_layer_(x, dims, w, pos32, rows32, bits, cache.k(i), cache.v(i), ws)
+            ops.decoder_layer_(x, dims, w, pos32, rows32, bits, cache.k(i), cache.v(i), ws)
+        if self.streamer is not None and self.streamer.n:
+            base = self.first_streamed
+
+            def step(j, w):                       # w: views into the device slab that holds layer base + j right now
+                ops.decoder_layer_(x, dims, self._native_make(w), pos32, rows32, bits, cache.k(base + j), cache.v(base + j), ws)
+
+            self.streamer.run(step)
         return x
 
     # ------------------------------------------------------------------ pieces
@@ -225,7 +236,7 @@ class Decoder:
         positions = depths.to(self.device) + prefix_len
         rows = torch.arange(prefix_len + first_slot, prefix_len + first_slot + n, device=self.device)
         cfg = self.cfg
-        if self.use_native_layers and self.native_layers and self.streamer is None and n <= 64 and slots <= 64:
+        if self.use_native_layers and self.native_layers and n <= 64 and slots <= 128:
             return self.logits(self._run_native_layers(self.embed[token_ids], positions, rows, anc_bits, prefix_len, slots))
 
         def attn(i, q):

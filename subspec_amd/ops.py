@@ -300,8 +300,12 @@ def softmax_temperature(logits: torch.Tensor, temperature: float) -> torch.Tenso
     x = logits.contiguous()
     out = torch.empty_like(x)
     vocab = x.shape[-1]
-    code = L.lib().subspec_softmax_temperature(x.data_ptr(), out.data_ptr(), _dtype_code(x), x.numel() // vocab, vocab,
-                                               float(temperature), _stream(dev))
+    rows = x.numel() // vocab
+    lib = L.lib()
+    need = lib.subspec_softmax_temperature_workspace(rows, vocab)
+    ws = torch.empty(need, dtype=torch.uint8, device=dev) if need else None
+    code = lib.subspec_softmax_temperature(x.data_ptr(), out.data_ptr(), _dtype_code(x), rows, vocab, float(temperature),
+                                           ws.data_ptr() if need else None, need, _stream(dev))
     L.check(code, "subspec_softmax_temperature")
     return out
 
@@ -343,6 +347,23 @@ def decoder_layer_weights(w: dict) -> "L.DecoderLayerWeights":
                                  ptr("down_proj.wq"), ptr("down_proj.sz"))
 
 
+def dense_layer_weights(w: dict) -> "L.DenseLayerWeights":
+    """Pointer table of one layer's dense tensors (``qkv_proj.weight`` ... in the fused layout of
+    ``subspec_amd.model.init_weights``).  The caller keeps the tensors alive."""
+    def ptr(name, required=True):
+        t = w.get(name)
+        if t is None:
+            if required:
+                raise ValueError(f"decoder layer: {name} missing")
+            return None
+        if not t.is_contiguous():
+            raise ValueError(f"decoder layer: {name} must be contiguous")
+        return t.data_ptr()
+    return L.DenseLayerWeights(ptr("input_layernorm.weight"), ptr("post_attention_layernorm.weight"),
+                               ptr("qkv_proj.weight"), ptr("qkv_proj.bias", False), ptr("o_proj.weight"),
+                               ptr("gate_up_proj.weight"), ptr("down_proj.weight"))
+
+
 def decoder_layer_workspace(dims: "L.DecoderLayerDims") -> int:
     need = L.lib().subspec_int4_decoder_layer_workspace(ctypes.byref(dims))
     if need == 0:
@@ -364,9 +385,36 @@ def int4_decoder_layer_(x: torch.Tensor, dims: "L.DecoderLayerDims", weights: "L
     if x.shape != (dims.n_rows, dims.hidden) or positions.numel() != dims.n_rows or cache_rows.numel() != dims.n_rows \
             or anc_bits.numel() != dims.n_rows * (2 if dims.n_tree_slots > 64 else 1):
         raise ValueError("decoder layer: tensor shapes do not match the dimensions given")
-    code = L.lib().subspec_int4_decoder_layer(
-        ctypes.byref(dims), ctypes.byref(weights), x.data_ptr(), positions.data_ptr(), cache_rows.data_ptr(),
-        anc_bits.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), workspace.data_ptr(),
-        workspace.numel() * workspace.element_size(), _stream(dev))
-    L.check(code, "subspec_int4_decoder_layer")
+    dense = isinstance(weights, L.DenseLayerWeights)
+    fn = L.lib().subspec_dense_decoder_layer if dense else L.lib().subspec_int4_decoder_layer
+    code = fn(ctypes.byref(dims), ctypes.byref(weights), x.data_ptr(), positions.data_ptr(), cache_rows.data_ptr(),
+              anc_bits.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), workspace.data_ptr(),
+              workspace.numel() * workspace.element_size(), _stream(dev))
+    L.check(code, "subspec_dense_decoder_layer" if dense else "subspec_int4_decoder_layer")
     return x
+
+
+decoder_layer_ = int4_decoder_layer_     # either weight storage: the pointer table's type selects the entry point
+
+
+def dense_linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``F.linear(x, weight, bias)`` for at most 64 rows of bf16 / fp16 activations: x [..., K], weight [N, K]."""
+    dev = _require_gpu(x, weight)
+    N, K = weight.shape
+    if x.shape[-1] != K or x.dtype != weight.dtype:
+        raise ValueError("dense_linear: x [..., K] and weight [N, K] must agree in K and dtype")
+    M = x.numel() // K
+    x2 = x.reshape(M, K).contiguous()
+    weight = weight.contiguous()
+    if bias is not None:
+        if bias.dtype != x.dtype or bias.numel() != N:
+            raise ValueError("dense_linear: bias must be [N] in the activation dtype")
+        bias = bias.contiguous()
+    lib = L.lib()
+    need = lib.subspec_dense_linear_workspace(M, N, K)
+    ws = torch.empty(need, dtype=torch.uint8, device=dev)
+    y = torch.empty((M, N), dtype=x.dtype, device=dev)
+    code = lib.subspec_dense_linear(x2.data_ptr(), weight.data_ptr(), None if bias is None else bias.data_ptr(), y.data_ptr(),
+                                    _dtype_code(x), M, N, K, ws.data_ptr(), need, _stream(dev))
+    L.check(code, "subspec_dense_linear")
+    return y.reshape(*x.shape[:-1], N)

@@ -94,7 +94,8 @@ def test_draft_probabilities_softmax_with_temperature(dtype):
     the last place of exp and of the row sum, so values agree to one unit in the last place of the
     dtype (tolerance 2^-7 relative for bf16, 2^-10 for fp16, 1e-5 for fp32) and nearly all are equal."""
     g = torch.Generator().manual_seed(11)
-    for rows, V, T in ((8, 152064, 0.2), (1, 152064, 1.0), (5, 1000, 0.7), (3, 77, 0.2)):
+    # few rows x several slices (two launches), one slice, and many rows (one workgroup per row)
+    for rows, V, T in ((8, 152064, 0.2), (1, 152064, 1.0), (5, 1000, 0.7), (3, 77, 0.2), (3, 9001, 0.5), (300, 5000, 0.3)):
         print("softmax_temperature", dtype, rows, V, T, flush=True)
         logits = (torch.randn(rows, V, generator=g) * 3).to(dtype)
         logits[0, 3] = float("-inf")                                  # masked entry
