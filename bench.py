@@ -112,6 +112,17 @@ def bench_attention(args):
         _kernel_line("tree-masked GQA attention latency",
                      f"BASELINE config 3, B={B}: q [B,28,64,128], KV [B,4,4160,128] bf16", call_us, kernel_us, nbytes,
                      B * 4 * 64 * 28 * 4160 * 128, "subspec::tree_attention_kernel", bound="mfma", extra={"batch": B})
+    # the same sequence out of a paged pool (16-token pages in shuffled order)
+    page_len, n_pages, max_pages = 16, 4160 // 16, 300
+    layer = torch.randn(max_pages, 2, page_len, 4, 128, device=dev).to(torch.bfloat16)
+    pages = torch.randperm(max_pages, device=dev)[:n_pages].to(torch.int32)
+    q = torch.randn(1, 28, 64, 128, device=dev).to(torch.bfloat16)
+    need = ops.L.lib().subspec_tree_attention_workspace(1, 28, 4096, 64)
+    ws = torch.empty(max(need, 256), dtype=torch.uint8, device=dev)
+    call_us, kernel_us = _time_us(lambda: ops.tree_attention_paged(q, layer, pages, anc, 4096, workspace=ws), args.steps, args.warmup)
+    _kernel_line("tree-masked GQA attention latency, paged KV", "config 3 shape, B=1, KV pool [300,2,16,4,128] bf16, shuffled pages",
+                 call_us, kernel_us, 2 * 4 * 4160 * 128 * 2 + 2 * 28 * 64 * 128 * 2, 4 * 64 * 28 * 4160 * 128,
+                 "subspec::tree_attention_kernel", bound="mfma", extra={"batch": 1, "page_len": page_len})
 
 
 def bench_int4(args):

@@ -208,6 +208,41 @@ int subspec_tree_attention(const void* q, const void* k_cache, const void* v_cac
                            void* stream);
 
 /* ------------------------------------------------------------------------------------------
+ * Paged KV cache (one request): the same attention and compaction over the page pool of the
+ * reference's FlashInfer path instead of the contiguous static cache.
+ *
+ * Pool layout  [layers][max_pages][2 (K, V)][page_len][n_kv_heads][head_dim]   ("NHD" pages):
+ *           KvCachePool.cache_data    specdecodes/models/utils/flashinfer/cache_manager.py:35-52
+ * page_indices  device int32 [n_pages]: the request's pages in sequence order
+ *           RequestKvCache.kv_page_indices / KvCacheBatchPosition.kv_page_indices   cache_manager.py:9-25,218-240,350-372
+ * Cache row p lives in page page_indices[p / page_len] at token p % page_len; page_len must be a power
+ * of two.  Page numbers are clamped to [0, max_pages) on the device, so a corrupt table reads wrong
+ * rows but never leaves the pool.
+ *
+ * subspec_tree_attention_paged replaces
+ *   flashinfer.BatchPrefillWithPagedKVCacheWrapper.run with custom_mask (mode "tree")
+ *           specdecodes/models/utils/flashinfer/attention_wrapper.py:104-137 and its forward call
+ * kv_pool_layer = one layer of the pool; every other argument as in subspec_tree_attention (batch 1,
+ * workspace = subspec_tree_attention_workspace(1, n_q_heads, prefix_len, n_tree_slots)).
+ *
+ * subspec_kv_compact_paged replaces
+ *   KvCachePool.reorder_cache_with_offset (clone of every layer, index_select / index_copy_, copy back)
+ *           cache_manager.py:120-213
+ * for all layers, K and V, in one launch: row offset + j <- row offset + ctx[j], j < count, rows
+ * addressed through page_indices (the reference indexes the pool as if the request's pages were
+ * 0, 1, 2, ...: the identity table).  token_bytes = n_kv_heads * head_dim * sizeof(dtype).
+ */
+int subspec_tree_attention_paged(const void* q, const void* kv_pool_layer, const int32_t* page_indices, int64_t n_pages,
+                                 int64_t max_pages, int64_t page_len, void* out, int dtype, int64_t n_q_heads,
+                                 int64_t n_kv_heads, int64_t n_rows, int64_t n_tree_slots, int64_t head_dim,
+                                 int64_t prefix_len, const uint64_t* anc_bits, float scale, void* workspace,
+                                 size_t workspace_bytes, void* stream);
+
+int subspec_kv_compact_paged(void* pool, int64_t n_layers, int64_t max_pages, int64_t page_len, int64_t token_bytes,
+                             const int32_t* page_indices, int64_t n_pages, int64_t offset, const int64_t* ctx,
+                             const int32_t* count_dev, int32_t count_host, int32_t max_count, void* stream);
+
+/* ------------------------------------------------------------------------------------------
  * Draft probabilities: out = softmax(round(logits / temperature)) over the last axis, in the logits
  * dtype (the quotient is rounded to the dtype first, the softmax is evaluated in fp32 and each
  * probability rounded once).

@@ -61,6 +61,9 @@ _SIGNATURES = {
     "subspec_tree_attention_workspace": (_sz, [_i64, _i64, _i64, _i64]),
     "subspec_tree_attention": (C.c_int, [_p, _p, _p, _p, C.c_int, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _p, _i64,
                                          C.c_float, _p, _sz, _p]),
+    "subspec_tree_attention_paged": (C.c_int, [_p, _p, _p, _i64, _i64, _i64, _p, C.c_int, _i64, _i64, _i64, _i64, _i64, _i64, _p,
+                                               C.c_float, _p, _sz, _p]),
+    "subspec_kv_compact_paged": (C.c_int, [_p, _i64, _i64, _i64, _i64, _p, _i64, _i64, _p, _p, _i32, _i32, _p]),
     "subspec_softmax_temperature_workspace": (_sz, [_i64, _i64]),
     "subspec_softmax_temperature": (C.c_int, [_p, _p, C.c_int, _i64, _i64, C.c_float, _p, _sz, _p]),
     "subspec_temperature_warp": (C.c_int, [_p, _p, C.c_int, _i64, C.c_float, _p]),

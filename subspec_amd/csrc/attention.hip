@@ -88,9 +88,14 @@ struct AttnParams {
   int pairs_per_kv;            // workgroups (head pairs) per KV head
   int64_t units;               // batch * hkv * chunks
   float scale_log2;            // softmax scale * log2(e)
+  // paged cache (one request): row p of K lives at page_table[p >> page_shift], token p & (page_len - 1) of
+  // a pool layer [max_pages][2 (K, V)][page_len][hkv][128]; V is v_delta elements behind K
+  const int32_t* page_table;
+  int page_shift, max_pages;
+  int64_t page_stride, tok_stride, v_delta;   // elements
 };
 
-template <int DT>
+template <int DT, bool PAGED>
 __global__ __launch_bounds__(kAttnThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void tree_attention_kernel(
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ kc, const uint16_t* __restrict__ vc,
     const uint64_t* __restrict__ anc, AttnParams ap, uint16_t* __restrict__ out, float* __restrict__ part_o,
@@ -148,8 +153,17 @@ __global__ __launch_bounds__(kAttnThreads) __attribute__((amdgpu_waves_per_eu(2,
     for (int mt = 0; mt < kAttnD / 16; ++mt) oacc[nt][mt] = v4f{0.f, 0.f, 0.f, 0.f};
   }
 
-  const uint16_t* kbase = kc + ((int64_t)b * ap.hkv + kvh) * ap.seq_stride * kAttnD;
-  const uint16_t* vbase = vc + ((int64_t)b * ap.hkv + kvh) * ap.seq_stride * kAttnD;
+  // contiguous cache [B, Hkv, S, 128]: row p of this head at base + p * 128.  Paged pool: see AttnParams.
+  const uint16_t* kbase = PAGED ? kc + (int64_t)kvh * kAttnD : kc + ((int64_t)b * ap.hkv + kvh) * ap.seq_stride * kAttnD;
+  const uint16_t* vbase = PAGED ? kbase + ap.v_delta : vc + ((int64_t)b * ap.hkv + kvh) * ap.seq_stride * kAttnD;
+  auto row_offset = [&](int64_t p) -> int64_t {          // element offset of cache row p from kbase / vbase
+    if constexpr (PAGED) {
+      const int page = min(max(ap.page_table[p >> ap.page_shift], 0), ap.max_pages - 1);   // a bad table must not fault
+      return (int64_t)page * ap.page_stride + (p & ((1 << ap.page_shift) - 1)) * ap.tok_stride;
+    } else {
+      return p * kAttnD;
+    }
+  };
   const int64_t key0 = (int64_t)chunk * ap.chunk_keys;
   const int64_t key1 = min(key0 + ap.chunk_keys, kv_len);
 
@@ -161,11 +175,12 @@ __global__ __launch_bounds__(kAttnThreads) __attribute__((amdgpu_waves_per_eu(2,
   const int skey = tid >> 4, sdc = tid & 15;           // this thread stages keys skey, skey + 32, d-chunk sdc
 #define SUBSPEC_ATTN_FETCH(KB)                                                                   \
   do {                                                                                           \
-    const int64_t p0_ = min((KB) + skey, kv_len - 1), p1_ = min((KB) + 32 + skey, kv_len - 1);   \
-    k0 = *(const uint4*)(kbase + p0_ * kAttnD + sdc * 8);                                        \
-    k1 = *(const uint4*)(kbase + p1_ * kAttnD + sdc * 8);                                        \
-    v0 = *(const uint4*)(vbase + p0_ * kAttnD + sdc * 8);                                        \
-    v1 = *(const uint4*)(vbase + p1_ * kAttnD + sdc * 8);                                        \
+    const int64_t p0_ = row_offset(min((KB) + skey, kv_len - 1));                                \
+    const int64_t p1_ = row_offset(min((KB) + 32 + skey, kv_len - 1));                           \
+    k0 = *(const uint4*)(kbase + p0_ + sdc * 8);                                                 \
+    k1 = *(const uint4*)(kbase + p1_ + sdc * 8);                                                 \
+    v0 = *(const uint4*)(vbase + p0_ + sdc * 8);                                                 \
+    v1 = *(const uint4*)(vbase + p1_ + sdc * 8);                                                 \
   } while (0)
 #define SUBSPEC_ATTN_STAGE(BUF)                                                                  \
   do {                                                                                           \
@@ -372,34 +387,47 @@ extern "C" size_t subspec_tree_attention_workspace(int64_t batch, int64_t n_q_he
   return align_up(slots * kAttnD * sizeof(float), 256) + align_up(slots * 2 * sizeof(float), 256);
 }
 
-extern "C" int subspec_tree_attention(const void* q, const void* k_cache, const void* v_cache, void* out, int dtype,
-                                      int64_t batch, int64_t n_q_heads, int64_t n_kv_heads, int64_t n_rows,
-                                      int64_t n_tree_slots, int64_t head_dim, int64_t kv_seq_stride, int64_t prefix_len,
-                                      const uint64_t* anc_bits, int64_t anc_batch_stride, float scale,
-                                      void* workspace, size_t workspace_bytes, void* stream) {
+struct PagedArgs { const int32_t* page_table; int64_t n_pages, max_pages, page_len; };
+
+static int tree_attention_impl(const char* what, const void* q, const void* k_cache, const void* v_cache, void* out, int dtype,
+                               int64_t batch, int64_t n_q_heads, int64_t n_kv_heads, int64_t n_rows, int64_t n_tree_slots,
+                               int64_t head_dim, int64_t kv_seq_stride, int64_t prefix_len, const uint64_t* anc_bits,
+                               int64_t anc_batch_stride, float scale, const PagedArgs* paged, void* workspace,
+                               size_t workspace_bytes, void* stream) {
   if (dtype != SUBSPEC_BF16 && dtype != SUBSPEC_F16)
-    SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "tree_attention: dtype %d not supported (bf16 / fp16 only)", dtype);
-  if (!q || !k_cache || !v_cache || !out || !anc_bits) SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "tree_attention: null pointer argument");
-  if (head_dim != kAttnD) SUBSPEC_FAIL(SUBSPEC_ERR_LIMIT, "tree_attention: head_dim=%lld (built for 128)", (long long)head_dim);
+    SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "%s: dtype %d not supported (bf16 / fp16 only)", what, dtype);
+  if (!q || !k_cache || !v_cache || !out || !anc_bits) SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "%s: null pointer argument", what);
+  if (head_dim != kAttnD) SUBSPEC_FAIL(SUBSPEC_ERR_LIMIT, "%s: head_dim=%lld (built for 128)", what, (long long)head_dim);
   if (batch <= 0 || n_q_heads <= 0 || n_kv_heads <= 0 || n_q_heads % n_kv_heads != 0)
-    SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "tree_attention: batch=%lld heads=%lld/%lld", (long long)batch, (long long)n_q_heads,
+    SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "%s: batch=%lld heads=%lld/%lld", what, (long long)batch, (long long)n_q_heads,
                  (long long)n_kv_heads);
   if (n_rows <= 0 || n_rows > kAttnRows)
-    SUBSPEC_FAIL(SUBSPEC_ERR_LIMIT, "tree_attention: n_rows=%lld outside [1, %d]", (long long)n_rows, kAttnRows);
+    SUBSPEC_FAIL(SUBSPEC_ERR_LIMIT, "%s: n_rows=%lld outside [1, %d]", what, (long long)n_rows, kAttnRows);
   if (n_tree_slots < 1 || n_tree_slots > 128)
-    SUBSPEC_FAIL(SUBSPEC_ERR_LIMIT, "tree_attention: n_tree_slots=%lld outside [1, 128] (at most two 64-bit mask words per row)",
+    SUBSPEC_FAIL(SUBSPEC_ERR_LIMIT, "%s: n_tree_slots=%lld outside [1, 128] (at most two 64-bit mask words per row)", what,
                  (long long)n_tree_slots);
   if (prefix_len < 0 || prefix_len + n_tree_slots > kv_seq_stride)
-    SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "tree_attention: prefix_len=%lld + n_tree_slots=%lld exceeds the cache length %lld",
+    SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "%s: prefix_len=%lld + n_tree_slots=%lld exceeds the cache length %lld", what,
                  (long long)prefix_len, (long long)n_tree_slots, (long long)kv_seq_stride);
-  if (batch * n_q_heads > 65535) SUBSPEC_FAIL(SUBSPEC_ERR_LIMIT, "tree_attention: batch*heads=%lld too large", (long long)(batch * n_q_heads));
+  if (batch * n_q_heads > 65535) SUBSPEC_FAIL(SUBSPEC_ERR_LIMIT, "%s: batch*heads=%lld too large", what, (long long)(batch * n_q_heads));
   if ((uintptr_t)q % 8 || (uintptr_t)k_cache % 16 || (uintptr_t)v_cache % 16 || (uintptr_t)out % 8)
-    SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "tree_attention: q/out must be 8-byte and k/v 16-byte aligned");
+    SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "%s: q/out must be 8-byte and k/v 16-byte aligned", what);
   AttnParams ap;
   ap.batch = batch; ap.hq = n_q_heads; ap.hkv = n_kv_heads; ap.n_rows = n_rows; ap.n_slots = n_tree_slots;
   ap.seq_stride = kv_seq_stride;
   ap.prefix = prefix_len; ap.anc_batch_stride = anc_batch_stride;
   ap.mask_words = n_tree_slots > 64 ? 2 : 1;
+  ap.page_table = nullptr; ap.page_shift = 0; ap.max_pages = 0; ap.page_stride = ap.tok_stride = ap.v_delta = 0;
+  if (paged) {
+    int shift = 0;
+    while ((1ll << shift) < paged->page_len) ++shift;
+    ap.page_table = paged->page_table;
+    ap.page_shift = shift;
+    ap.max_pages = (int)paged->max_pages;
+    ap.tok_stride = n_kv_heads * kAttnD;
+    ap.v_delta = paged->page_len * ap.tok_stride;
+    ap.page_stride = 2 * ap.v_delta;
+  }
   const int64_t kv_len = prefix_len + n_tree_slots;
   ap.chunks = attn_chunks(batch, n_q_heads, kv_len);
   const int64_t blocks = (kv_len + kKeyBlock - 1) / kKeyBlock;
@@ -415,34 +443,57 @@ extern "C" int subspec_tree_attention(const void* q, const void* k_cache, const 
     const size_t slots = (size_t)batch * n_q_heads * ap.chunks * kAttnRows;
     const size_t need = align_up(slots * kAttnD * sizeof(float), 256) + align_up(slots * 2 * sizeof(float), 256);
     if (!workspace || workspace_bytes < need)
-      SUBSPEC_FAIL(SUBSPEC_ERR_WORKSPACE, "tree_attention: workspace of %zu bytes is smaller than the %zu required",
+      SUBSPEC_FAIL(SUBSPEC_ERR_WORKSPACE, "%s: workspace of %zu bytes is smaller than the %zu required", what,
                    workspace_bytes, need);
-    if ((uintptr_t)workspace % 16) SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "tree_attention: workspace must be 16-byte aligned");
+    if ((uintptr_t)workspace % 16) SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "%s: workspace must be 16-byte aligned", what);
     part_o = (float*)workspace;
     part_ml = (float*)((char*)workspace + align_up(slots * kAttnD * sizeof(float), 256));
   }
   hipStream_t st = (hipStream_t)stream;
   const dim3 grid((unsigned)((ap.units + kXcds - 1) / kXcds * kXcds * ap.pairs_per_kv));
   const int64_t merge_rows = batch * n_q_heads * n_rows / 8 >= 1024 ? 8 : 2;   // rows per merge workgroup
-  if (dtype == SUBSPEC_BF16) {
-    {
-      DominantKernelTimer timer(st);
-      hipLaunchKernelGGL((tree_attention_kernel<SUBSPEC_BF16>), grid, dim3(kAttnThreads), 0, st, (const uint16_t*)q,
-                         (const uint16_t*)k_cache, (const uint16_t*)v_cache, anc_bits, ap, (uint16_t*)out, part_o, part_ml);
-    }
-    if (ap.chunks > 1)
-      hipLaunchKernelGGL((tree_attention_merge_kernel<SUBSPEC_BF16>), dim3((unsigned)((n_rows + merge_rows - 1) / merge_rows), (unsigned)(batch * n_q_heads)),
-                         dim3(merge_rows * 32), 0, st, part_o, part_ml, ap, (uint16_t*)out);
-  } else {
-    {
-      DominantKernelTimer timer(st);
-      hipLaunchKernelGGL((tree_attention_kernel<SUBSPEC_F16>), grid, dim3(kAttnThreads), 0, st, (const uint16_t*)q,
-                         (const uint16_t*)k_cache, (const uint16_t*)v_cache, anc_bits, ap, (uint16_t*)out, part_o, part_ml);
-    }
-    if (ap.chunks > 1)
-      hipLaunchKernelGGL((tree_attention_merge_kernel<SUBSPEC_F16>), dim3((unsigned)((n_rows + merge_rows - 1) / merge_rows), (unsigned)(batch * n_q_heads)),
-                         dim3(merge_rows * 32), 0, st, part_o, part_ml, ap, (uint16_t*)out);
-  }
+  const dim3 merge_grid((unsigned)((n_rows + merge_rows - 1) / merge_rows), (unsigned)(batch * n_q_heads));
+#define SUBSPEC_ATTN_LAUNCH(DT, PAGED)                                                                             \
+  do {                                                                                                             \
+    {                                                                                                              \
+      DominantKernelTimer timer(st);                                                                               \
+      hipLaunchKernelGGL((tree_attention_kernel<DT, PAGED>), grid, dim3(kAttnThreads), 0, st, (const uint16_t*)q,  \
+                         (const uint16_t*)k_cache, (const uint16_t*)v_cache, anc_bits, ap, (uint16_t*)out, part_o, part_ml); \
+    }                                                                                                              \
+    if (ap.chunks > 1)                                                                                             \
+      hipLaunchKernelGGL((tree_attention_merge_kernel<DT>), merge_grid, dim3(merge_rows * 32), 0, st, part_o, part_ml, ap, \
+                         (uint16_t*)out);                                                                          \
+  } while (0)
+  if (dtype == SUBSPEC_BF16) { if (paged) SUBSPEC_ATTN_LAUNCH(SUBSPEC_BF16, true); else SUBSPEC_ATTN_LAUNCH(SUBSPEC_BF16, false); }
+  else { if (paged) SUBSPEC_ATTN_LAUNCH(SUBSPEC_F16, true); else SUBSPEC_ATTN_LAUNCH(SUBSPEC_F16, false); }
+#undef SUBSPEC_ATTN_LAUNCH
   SUBSPEC_CHECK_HIP(hipGetLastError());
   return SUBSPEC_OK;
+}
+
+extern "C" int subspec_tree_attention(const void* q, const void* k_cache, const void* v_cache, void* out, int dtype,
+                                      int64_t batch, int64_t n_q_heads, int64_t n_kv_heads, int64_t n_rows,
+                                      int64_t n_tree_slots, int64_t head_dim, int64_t kv_seq_stride, int64_t prefix_len,
+                                      const uint64_t* anc_bits, int64_t anc_batch_stride, float scale,
+                                      void* workspace, size_t workspace_bytes, void* stream) {
+  return tree_attention_impl("tree_attention", q, k_cache, v_cache, out, dtype, batch, n_q_heads, n_kv_heads, n_rows,
+                             n_tree_slots, head_dim, kv_seq_stride, prefix_len, anc_bits, anc_batch_stride, scale, nullptr,
+                             workspace, workspace_bytes, stream);
+}
+
+extern "C" int subspec_tree_attention_paged(const void* q, const void* kv_pool_layer, const int32_t* page_indices,
+                                            int64_t n_pages, int64_t max_pages, int64_t page_len, void* out, int dtype,
+                                            int64_t n_q_heads, int64_t n_kv_heads, int64_t n_rows, int64_t n_tree_slots,
+                                            int64_t head_dim, int64_t prefix_len, const uint64_t* anc_bits, float scale,
+                                            void* workspace, size_t workspace_bytes, void* stream) {
+  if (!page_indices) SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "tree_attention_paged: null page table");
+  if (page_len <= 0 || (page_len & (page_len - 1)) != 0 || page_len > 4096)
+    SUBSPEC_FAIL(SUBSPEC_ERR_LIMIT, "tree_attention_paged: page_len=%lld must be a power of two up to 4096", (long long)page_len);
+  if (n_pages <= 0 || max_pages < n_pages || max_pages > 0x7fffffff)
+    SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "tree_attention_paged: n_pages=%lld max_pages=%lld", (long long)n_pages, (long long)max_pages);
+  const PagedArgs pg{page_indices, n_pages, max_pages, page_len};
+  // the request's pages play the part of the cache length: rows beyond them do not exist
+  return tree_attention_impl("tree_attention_paged", q, kv_pool_layer, kv_pool_layer, out, dtype, 1, n_q_heads, n_kv_heads,
+                             n_rows, n_tree_slots, head_dim, n_pages * page_len, prefix_len, anc_bits, 0, scale, &pg, workspace,
+                             workspace_bytes, stream);
 }

@@ -261,6 +261,74 @@ def tree_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
     return out
 
 
+def _page_shape(pool_layer_or_pool: torch.Tensor, page_indices: torch.Tensor):
+    if page_indices.dtype != torch.int32 or page_indices.dim() != 1 or not page_indices.is_contiguous():
+        raise ValueError("page_indices must be a contiguous int32 vector")
+    if not pool_layer_or_pool.is_contiguous() or pool_layer_or_pool.shape[-4] != 2:
+        raise ValueError("expected a contiguous pool [..., max_pages, 2, page_len, kv_heads, head_dim]")
+    return pool_layer_or_pool.shape[-5], pool_layer_or_pool.shape[-3], pool_layer_or_pool.shape[-2], pool_layer_or_pool.shape[-1]
+
+
+def tree_attention_paged(q: torch.Tensor, pool_layer: torch.Tensor, page_indices: torch.Tensor, anc_bits: torch.Tensor,
+                         prefix_len: int, scale: Optional[float] = None, workspace: Optional[torch.Tensor] = None,
+                         n_tree_slots: Optional[int] = None):
+    """``tree_attention`` over one request's pages: ``q`` [1, Hq, n, D], ``pool_layer``
+    [max_pages, 2, page_len, Hkv, D] (one layer of ``KvCachePool.cache_data``), ``page_indices`` int32
+    [n_pages] in sequence order; tree K/V already appended at rows prefix_len...  Returns [1, n, Hq * D]."""
+    dev = _require_gpu(q, pool_layer, page_indices, anc_bits)
+    if q.dim() != 4 or q.shape[0] != 1 or pool_layer.dim() != 5:
+        raise ValueError("expected q [1, Hq, n, D] and a pool layer [max_pages, 2, page_len, Hkv, D]")
+    max_pages, page_len, Hkv, D = _page_shape(pool_layer, page_indices)
+    _, Hq, n, Dq = q.shape
+    if Dq != D or q.dtype != pool_layer.dtype:
+        raise ValueError("q and the pool must share head_dim and dtype")
+    slots = n if n_tree_slots is None else int(n_tree_slots)
+    words = 2 if slots > 64 else 1
+    if anc_bits.dtype != torch.int64 or anc_bits.numel() != n * words:
+        raise ValueError("anc_bits must be int64 [n] ([n, 2] above 64 tree slots)")
+    q, anc_bits = q.contiguous(), anc_bits.contiguous()
+    lib = L.lib()
+    need = lib.subspec_tree_attention_workspace(1, Hq, int(prefix_len), slots)
+    if workspace is None and need > 256:
+        workspace = torch.empty(need, dtype=torch.uint8, device=dev)
+    out = torch.empty((1, n, Hq * D), dtype=q.dtype, device=dev)
+    code = lib.subspec_tree_attention_paged(
+        q.data_ptr(), pool_layer.data_ptr(), page_indices.data_ptr(), page_indices.numel(), max_pages, page_len,
+        out.data_ptr(), _dtype_code(q), Hq, Hkv, n, slots, D, int(prefix_len), anc_bits.data_ptr(),
+        float(D ** -0.5 if scale is None else scale), None if workspace is None else workspace.data_ptr(),
+        0 if workspace is None else workspace.numel() * workspace.element_size(), _stream(dev))
+    L.check(code, "subspec_tree_attention_paged")
+    return out
+
+
+def kv_compact_paged_(pool: torch.Tensor, page_indices: torch.Tensor, contexts: torch.Tensor, offset: int,
+                      count: Optional[int] = None, count_dev: Optional[torch.Tensor] = None,
+                      max_count: Optional[int] = None) -> torch.Tensor:
+    """In place, for every layer and K / V of ``pool`` [L, max_pages, 2, page_len, Hkv, D]:
+    logical row offset + j <- logical row offset + contexts[j], j < count, rows addressed through ``page_indices``."""
+    dev = _require_gpu(pool, page_indices, contexts)
+    if pool.dim() != 6:
+        raise ValueError("expected a pool [L, max_pages, 2, page_len, Hkv, D]")
+    max_pages, page_len, Hkv, D = _page_shape(pool, page_indices)
+    if contexts.dtype != torch.int64 or not contexts.is_contiguous():
+        raise ValueError("kv_compact_paged_: contexts must be a contiguous int64 tensor")
+    if count_dev is None:
+        count = int(contexts.numel()) if count is None else int(count)
+    else:
+        _require_gpu(count_dev)
+        if count_dev.dtype != torch.int32:
+            raise ValueError("kv_compact_paged_: count_dev must be int32")
+        count = 0
+    if max_count is None:
+        max_count = min(int(contexts.numel()), L.MAX_TREE_NODES) if count_dev is not None else count
+    code = L.lib().subspec_kv_compact_paged(
+        pool.data_ptr(), pool.shape[0], max_pages, page_len, Hkv * D * pool.element_size(), page_indices.data_ptr(),
+        page_indices.numel(), int(offset), contexts.data_ptr(), None if count_dev is None else count_dev.data_ptr(), count,
+        int(max_count), _stream(dev))
+    L.check(code, "subspec_kv_compact_paged")
+    return pool
+
+
 def int4_linear(x: torch.Tensor, wq: torch.Tensor, sz: torch.Tensor, out_features: int,
                 bias: Optional[torch.Tensor] = None, workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``x`` [..., K] (bf16 / fp16, at most 64 rows in total) times the tiled int4 weight
