@@ -260,3 +260,39 @@ def test_kv_compaction_count_from_device_follows_verifier():
     assert torch.equal(dev.cpu(), okv.compact_static(cache, ctx, 2048))
     with pytest.raises(ValueError):
         ops.kv_compact_(dev[..., :7], out["contexts"][0], 0)                 # non-contiguous
+
+
+@pytest.mark.parametrize("n", [65, 128, 129, 200, 256])
+def test_large_trees_up_to_the_node_limit(n):
+    """Trees beyond one node per lane (2 and 4 nodes per lane in the acceptance step), greedy and sampled
+    targets, exact walk and both lossy gates, against the oracle; rows may be fewer than nodes."""
+    g = torch.Generator().manual_seed(n)
+    vocab = 777
+    parents, toks, depths = W.random_tree(g, n=n, max_depth=12, max_children=4, vocab=vocab, chain_depth=10)
+    kids = ov.children_from_parents(parents)
+    for rows, dtype in ((n, torch.bfloat16), (n, torch.float32), (max(1, n - 40), torch.bfloat16)):
+        logits = (torch.randn(rows, vocab, generator=g) * 2).to(dtype)
+        for u in range(rows):                              # make drafted children frequent targets: deep walks
+            if kids[u] and float(torch.rand(1, generator=g)) < 0.8:
+                pick = kids[u][int(torch.randint(0, len(kids[u]), (1,), generator=g))]
+                logits[u, toks[pick]] += 8.0
+        for method, vk in (("exact", {}),
+                           ("lossy", {"threshold_method": "prob", "threshold": 0.02, "window_size": 1}),
+                           ("lossy", {"threshold_method": "entropy", "threshold": 0.7, "window_size": 2})):
+            print("large tree", n, rows, dtype, method, vk, flush=True)
+            out = _run(logits, toks, parents, verify_method=method, exact_entropy=True,
+                       threshold_method=vk.get("threshold_method", "prob"), threshold=vk.get("threshold", 0.0),
+                       window_size=vk.get("window_size", 1))
+            want = ov.verify_logits(logits, toks, parents, verify_method=method, verify_kwargs=vk)
+            got_t, got_c, got_m = _unpack(out)
+            assert (got_t, got_c, got_m) == (want[0], want[1], want[2]), (n, rows, method)
+            assert out["target"][0].tolist() == ov.target_probs(logits).argmax(-1).tolist()
+            # sampled target: the walk / DP must follow the device's own draws exactly
+            smp = _run(logits, toks, parents, verify_method=method, exact_entropy=True,
+                       threshold_method=vk.get("threshold_method", "prob"), threshold=vk.get("threshold", 0.0),
+                       window_size=vk.get("window_size", 1), do_sample=True, temperature=0.9, seed=n, offset=rows)
+            drawn = smp["target"][0].tolist()
+            want = ov.verify_logits(logits, toks, parents, verify_method=method, verify_kwargs=vk, temperature=0.9,
+                                    target_tokens=drawn)
+            got_t, got_c, got_m = _unpack(smp)
+            assert (got_t, got_c, got_m) == (want[0], want[1], want[2]), (n, rows, method, "sampled")
