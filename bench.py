@@ -43,7 +43,7 @@ def parse():
                     help="e2e workload: local HuggingFace checkpoint directory (config.json + *.safetensors, Qwen2 / "
                          "Llama naming) to use instead of random-init weights of the Qwen2.5-7B shape")
     ap.add_argument("--keep-layers", type=int, default=14, help="e2e workload: target layers kept resident; the rest stream")
-    ap.add_argument("--workload", default="verify-cycle", choices=["verify-cycle", "attention", "int4", "greedy", "sampling", "e2e"],
+    ap.add_argument("--workload", default="verify-cycle", choices=["verify-cycle", "attention", "int4", "dense", "greedy", "sampling", "e2e"],
                     help="verify-cycle (default, BASELINE config 2) is the benchmark line; the others time one "
                          "kernel family of configs 1, 3 and 4 and print one JSON line per shape")
     return ap.parse_args()
@@ -125,6 +125,21 @@ def bench_attention(args):
                  "subspec::tree_attention_kernel", bound="mfma", extra={"batch": 1, "page_len": page_len})
 
 
+def _rotating(make_call, n_copies):
+    """fn() that uses copy 0, 1, 2, ... of the weights in turn: with enough copies (more bytes than the 256 MB
+    memory-side cache plus the L2s hold) every call streams its weights from HBM, as inside a model where the
+    other layers' weights pass through the caches between two uses of the same matrix."""
+    state = [0]
+
+    def fn():
+        make_call(state[0] % n_copies)
+        state[0] += 1
+    return fn
+
+
+COLD_BYTES = 640 << 20
+
+
 def bench_int4(args):
     import torch
     from subspec_amd import ops, quant
@@ -133,15 +148,42 @@ def bench_int4(args):
         W_ = torch.randn(N, K, device=dev) * 0.02
         wq, sz = quant.pack_tiled(*quant.quantize_int4_g64(W_))
         del W_
+        copies = max(2, COLD_BYTES // (wq.numel() * 4) + 1)
+        wqs, szs = [wq.clone() for _ in range(copies)], [sz.clone() for _ in range(copies)]
         for M in (1, 16, 64):
             x = torch.randn(M, K, device=dev).to(torch.bfloat16)
             ws = torch.empty(max(ops.L.lib().subspec_int4_linear_workspace(M, N, K), 256), dtype=torch.uint8, device=dev)
-            call_us, kernel_us = _time_us(lambda: ops.int4_linear(x, wq, sz, N, workspace=ws), args.steps, args.warmup)
+            warm_us, warm_kernel_us = _time_us(lambda: ops.int4_linear(x, wq, sz, N, workspace=ws), args.steps, args.warmup)
+            call_us, kernel_us = _time_us(_rotating(lambda i: ops.int4_linear(x, wqs[i], szs[i], N, workspace=ws), copies),
+                                          max(args.steps, copies), args.warmup)
             nbytes = N * K // 2 + N * (K // 64) * 4 + M * (K + N) * 2
-            _kernel_line("int4 g64 linear latency", f"BASELINE config 4: {K}->{N}, M={M}, bf16 activations", call_us,
-                         kernel_us, nbytes, 2 * M * N * K,
+            _kernel_line("int4 g64 linear latency", f"BASELINE config 4: {K}->{N}, M={M}, bf16 activations, weights streamed "
+                         f"from HBM (rotating over {copies} copies)", call_us, kernel_us, nbytes, 2 * M * N * K,
                          "subspec::int4_gemv_kernel" if M == 1 else "subspec::int4_gemm_kernel",
-                         extra={"N": N, "K": K, "M": M})
+                         extra={"N": N, "K": K, "M": M, "same_weights_every_call_us": round(warm_us, 2),
+                                "same_weights_every_call_kernel_us": round(warm_kernel_us, 2)})
+        del wqs, szs
+
+
+def bench_dense(args):
+    """The target model's projections in the tree-decoding forward (bf16, at most 64 rows), next to the
+    library GEMM (torch F.linear) on the same operands; weights streamed from HBM as in bench_int4."""
+    import torch
+    import torch.nn.functional as F
+    from subspec_amd import ops
+    dev = torch.device("cuda:0")
+    for N, K in ((4608, 3584), (3584, 3584), (37888, 3584), (3584, 18944)):
+        copies = max(2, COLD_BYTES // (N * K * 2) + 1)
+        wl = [(torch.randn(N, K, device=dev) * 0.02).to(torch.bfloat16) for _ in range(copies)]
+        for M in (8, 64):
+            x = torch.randn(M, K, device=dev).to(torch.bfloat16)
+            steps = max(args.steps, copies)
+            call_us, kernel_us = _time_us(_rotating(lambda i: ops.dense_linear(x, wl[i]), copies), steps, args.warmup)
+            lib_us, _ = _time_us(_rotating(lambda i: F.linear(x, wl[i]), copies), steps, args.warmup)
+            _kernel_line("dense 16-bit linear latency", f"target layer projection {K}->{N}, M={M}, bf16, weights streamed from "
+                         f"HBM (rotating over {copies} copies)", call_us, kernel_us, N * K * 2 + M * (K + N) * 2, 2 * M * N * K,
+                         "subspec::dense_gemm_kernel", extra={"N": N, "K": K, "M": M, "library_gemm_call_us": round(lib_us, 2)})
+        del wl
 
 
 def bench_e2e(args):
@@ -287,7 +329,7 @@ def main():
         sys.exit(1)
     L.lib()                                            # fail loudly when the HIP library is missing
     if args.workload != "verify-cycle":
-        {"attention": bench_attention, "int4": bench_int4, "greedy": bench_greedy, "sampling": bench_sampling,
+        {"attention": bench_attention, "int4": bench_int4, "dense": bench_dense, "greedy": bench_greedy, "sampling": bench_sampling,
          "e2e": bench_e2e}[args.workload](args)
         return
     dev = torch.device("cuda:0")

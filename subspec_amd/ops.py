@@ -348,7 +348,7 @@ def int4_linear(x: torch.Tensor, wq: torch.Tensor, sz: torch.Tensor, out_feature
         bias = bias.contiguous()
     lib = L.lib()
     need = lib.subspec_int4_linear_workspace(M, N, K)
-    if workspace is None and M > 1:
+    if workspace is None:
         workspace = torch.empty(need, dtype=torch.uint8, device=dev)
     y = torch.empty((M, N), dtype=x.dtype, device=dev)
     code = lib.subspec_int4_linear(
