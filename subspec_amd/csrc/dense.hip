@@ -206,7 +206,7 @@ static DnPlan dn_plan(int64_t M, int64_t N, int64_t K) {
   const int row_tiles = want <= 1 ? 1 : want <= 2 ? 2 : 4;
   const int64_t wgs = (tiles + row_tiles - 1) / row_tiles;
   int splits = (int)std::max<int64_t>(1, (slots + wgs / 2) / wgs);
-  splits = std::min(splits, std::max(1, G / 56));              // a split costs a second launch: only for long K
+  splits = std::min(splits, std::max(1, G / 112));             // a split costs a second launch: only for long K (two at K = 18944)
   splits = std::min(splits, 16);
   int gps = (G + splits - 1) / splits;
   gps = (gps + 3) / 4 * 4;
