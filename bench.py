@@ -93,38 +93,6 @@ def _kernel_line(name, workload, call_us, kernel_us, nbytes, flops, kernel, boun
     print(json.dumps(line), flush=True)
 
 
-def bench_attention(args):
-    import torch
-    from subspec_amd import ops, workloads as W
-    dev = torch.device("cuda:0")
-    g = torch.Generator().manual_seed(0)
-    parents, _, _ = W.random_tree(g, n=64, max_depth=8, max_children=4, vocab=1000, chain_depth=8)
-    anc = ops.ancestor_bits_tensor(parents, device=dev)
-    for B in (1, 8):
-        q = torch.randn(B, 28, 64, 128, device=dev).to(torch.bfloat16)
-        k = torch.randn(B, 4, 4160, 128, device=dev).to(torch.bfloat16)
-        v = torch.randn(B, 4, 4160, 128, device=dev).to(torch.bfloat16)
-        need = ops.L.lib().subspec_tree_attention_workspace(B, 28, 4096, 64)
-        ws = torch.empty(max(need, 256), dtype=torch.uint8, device=dev)
-        call_us, kernel_us = _time_us(lambda: ops.tree_attention(q, k, v, anc, 4096, workspace=ws), args.steps, args.warmup)
-        nbytes = B * (2 * 4 * 4160 * 128 * 2 + 2 * 28 * 64 * 128 * 2)
-        # 3.82 GFLOP per sequence over 9.44 MB: at 405 FLOP/B the shape sits above the ridge (310 FLOP/B)
-        _kernel_line("tree-masked GQA attention latency",
-                     f"BASELINE config 3, B={B}: q [B,28,64,128], KV [B,4,4160,128] bf16", call_us, kernel_us, nbytes,
-                     B * 4 * 64 * 28 * 4160 * 128, "subspec::tree_attention_kernel", bound="mfma", extra={"batch": B})
-    # the same sequence out of a paged pool (16-token pages in shuffled order)
-    page_len, n_pages, max_pages = 16, 4160 // 16, 300
-    layer = torch.randn(max_pages, 2, page_len, 4, 128, device=dev).to(torch.bfloat16)
-    pages = torch.randperm(max_pages, device=dev)[:n_pages].to(torch.int32)
-    q = torch.randn(1, 28, 64, 128, device=dev).to(torch.bfloat16)
-    need = ops.L.lib().subspec_tree_attention_workspace(1, 28, 4096, 64)
-    ws = torch.empty(max(need, 256), dtype=torch.uint8, device=dev)
-    call_us, kernel_us = _time_us(lambda: ops.tree_attention_paged(q, layer, pages, anc, 4096, workspace=ws), args.steps, args.warmup)
-    _kernel_line("tree-masked GQA attention latency, paged KV", "config 3 shape, B=1, KV pool [300,2,16,4,128] bf16, shuffled pages",
-                 call_us, kernel_us, 2 * 4 * 4160 * 128 * 2 + 2 * 28 * 64 * 128 * 2, 4 * 64 * 28 * 4160 * 128,
-                 "subspec::tree_attention_kernel", bound="mfma", extra={"batch": 1, "page_len": page_len})
-
-
 def _rotating(make_call, n_copies):
     """fn() that uses copy 0, 1, 2, ... of the weights in turn: with enough copies (more bytes than the 256 MB
     memory-side cache plus the L2s hold) every call streams its weights from HBM, as inside a model where the
@@ -138,6 +106,43 @@ def _rotating(make_call, n_copies):
 
 
 COLD_BYTES = 640 << 20
+
+
+def bench_attention(args):
+    import torch
+    from subspec_amd import ops, workloads as W
+    dev = torch.device("cuda:0")
+    g = torch.Generator().manual_seed(0)
+    parents, _, _ = W.random_tree(g, n=64, max_depth=8, max_children=4, vocab=1000, chain_depth=8)
+    anc = ops.ancestor_bits_tensor(parents, device=dev)
+    for B in (1, 8):
+        q = torch.randn(B, 28, 64, 128, device=dev).to(torch.bfloat16)
+        # a different layer's cache on every call (rotation over > 640 MB), as in a forward through 28 layers
+        copies = max(2, COLD_BYTES // (2 * B * 4 * 4160 * 128 * 2) + 1)
+        ks = [torch.randn(B, 4, 4160, 128, device=dev).to(torch.bfloat16) for _ in range(copies)]
+        vs = [torch.randn(B, 4, 4160, 128, device=dev).to(torch.bfloat16) for _ in range(copies)]
+        need = ops.L.lib().subspec_tree_attention_workspace(B, 28, 4096, 64)
+        ws = torch.empty(max(need, 256), dtype=torch.uint8, device=dev)
+        call_us, kernel_us = _time_us(_rotating(lambda i: ops.tree_attention(q, ks[i], vs[i], anc, 4096, workspace=ws), copies),
+                                      max(args.steps, copies), args.warmup)
+        nbytes = B * (2 * 4 * 4160 * 128 * 2 + 2 * 28 * 64 * 128 * 2)
+        # 3.82 GFLOP per sequence over 9.44 MB: at 405 FLOP/B the shape sits above the ridge (310 FLOP/B)
+        _kernel_line("tree-masked GQA attention latency",
+                     f"BASELINE config 3, B={B}: q [B,28,64,128], KV [B,4,4160,128] bf16, another cache every call ({copies} copies)",
+                     call_us, kernel_us, nbytes, B * 4 * 64 * 28 * 4160 * 128, "subspec::tree_attention_kernel", bound="mfma",
+                     extra={"batch": B})
+        del ks, vs
+    # the same sequence out of a paged pool (16-token pages in shuffled order)
+    page_len, n_pages, max_pages = 16, 4160 // 16, 300
+    layer = torch.randn(max_pages, 2, page_len, 4, 128, device=dev).to(torch.bfloat16)
+    pages = torch.randperm(max_pages, device=dev)[:n_pages].to(torch.int32)
+    q = torch.randn(1, 28, 64, 128, device=dev).to(torch.bfloat16)
+    need = ops.L.lib().subspec_tree_attention_workspace(1, 28, 4096, 64)
+    ws = torch.empty(max(need, 256), dtype=torch.uint8, device=dev)
+    call_us, kernel_us = _time_us(lambda: ops.tree_attention_paged(q, layer, pages, anc, 4096, workspace=ws), args.steps, args.warmup)
+    _kernel_line("tree-masked GQA attention latency, paged KV", "config 3 shape, B=1, KV pool [300,2,16,4,128] bf16, shuffled pages",
+                 call_us, kernel_us, 2 * 4 * 4160 * 128 * 2 + 2 * 28 * 64 * 128 * 2, 4 * 64 * 28 * 4160 * 128,
+                 "subspec::tree_attention_kernel", bound="mfma", extra={"batch": 1, "page_len": page_len})
 
 
 def bench_int4(args):
