@@ -14,15 +14,18 @@
 //                                     (the node in slot j is the row's node or one of its ancestors);
 //                                     words = 1 for up to 64 tree slots, 2 for up to 128
 //   out      [B, n, Hq, D]
-// One workgroup (8 wavefronts) owns FOUR query heads of one KV head (256 rows) and one chunk of
-// the keys, so a staged K/V tile feeds four heads' worth of matrix work; wavefront w owns 32 rows
-// (two 16-row tiles) of head w/2.  Scores are produced TRANSPOSED, S^T = K Q^T, with v_mfma_f32_16x16x32: the
+// One workgroup (8 wavefronts) owns several query heads of one KV head and one chunk of the keys, so
+// a staged K/V tile feeds several heads' worth of matrix work.  With 33 to 64 query rows it owns
+// FOUR heads (256 rows): wavefront w takes 32 rows (two 16-row tiles) of head w/2.  With fewer rows
+// (17 to 32: two tiles, up to 16 -- one level of the draft tree --: one tile) a wavefront is a
+// whole head and the workgroup owns EIGHT heads, all of a 7:1 GQA group, so K/V are staged once per
+// KV head and no wavefront multiplies padding rows.  Scores are produced TRANSPOSED, S^T = K Q^T, with v_mfma_f32_16x16x32: the
 // accumulator then holds, per lane, four consecutive keys of one query, and two such tiles are
 // exactly the eight-key B operand of the second product O^T = V^T P^T (with the matching key
 // permutation applied to the V^T operand), so probabilities go from one MFMA to the next without
 // leaving registers and the row maximum / sum need only two cross-lane steps.  The ancestor bitset
-// of a lane's query sits in a register pair; prefix keys need no mask at all.  K is staged
-// row-major in LDS, V transposed; the global loads of the next 64-key block are issued before the
+// of a lane's query sits in a register pair; prefix keys need no mask at all.  K and V are staged
+// row-major in LDS (V^T operands come from transposing LDS reads); the global loads of the next 64-key block are issued before the
 // current block is multiplied.  Workgroups that share a KV chunk get consecutive slots on the same
 // XCD (linear id modulo 8), so the chunk is fetched from HBM once and served from that XCD's L2.
 // When the keys are split over several workgroups the partial (O, max, sum) triples are merged by
@@ -36,7 +39,6 @@ namespace subspec {
 
 constexpr int kAttnThreads = 512;
 constexpr int kAttnRows = 64;          // query rows per head
-constexpr int kHeadsPerWG = 4;
 constexpr int kAttnD = 128;
 constexpr int kKeyBlock = 64;
 constexpr int kKStride = kAttnD + 8;   // LDS row stride (elements) of the K tile
@@ -85,7 +87,7 @@ struct AttnParams {
   int mask_words;              // 64-bit words per ancestor bitset: 1 (<= 64 tree slots) or 2 (<= 128)
   int chunks;
   int64_t chunk_keys;          // multiple of kKeyBlock
-  int pairs_per_kv;            // workgroups (head pairs) per KV head
+  int pairs_per_kv;            // workgroups (groups of 4 or 8 query heads) per KV head
   int64_t units;               // batch * hkv * chunks
   float scale_log2;            // softmax scale * log2(e)
   // paged cache (one request): row p of K lives at page_table[p >> page_shift], token p & (page_len - 1) of
@@ -95,7 +97,7 @@ struct AttnParams {
   int64_t page_stride, tok_stride, v_delta;   // elements
 };
 
-template <int DT, bool PAGED>
+template <int DT, bool PAGED, int ROWT, int WPH>
 __global__ __launch_bounds__(kAttnThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void tree_attention_kernel(
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ kc, const uint16_t* __restrict__ vc,
     const uint64_t* __restrict__ anc, AttnParams ap, uint16_t* __restrict__ out, float* __restrict__ part_o,
@@ -118,7 +120,8 @@ __global__ __launch_bounds__(kAttnThreads) __attribute__((amdgpu_waves_per_eu(2,
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int lq = lane & 15, lg = lane >> 4;            // query column of the lane, lane group
-  const int head_in_group = pair * kHeadsPerWG + (wave >> 1);
+  constexpr int kHeadsPerWG = 8 / WPH;                 // heads of one KV head that share a workgroup's K / V stages
+  const int head_in_group = pair * kHeadsPerWG + wave / WPH;
   const bool head_ok = head_in_group < group;
   const int qh = kvh * group + (head_ok ? head_in_group : 0);
   const int bh = b * (int)ap.hq + qh;
@@ -126,13 +129,13 @@ __global__ __launch_bounds__(kAttnThreads) __attribute__((amdgpu_waves_per_eu(2,
   const int64_t kv_len = ap.prefix + ap.n_slots;
 
   // ---- Q^T operands of the wave's two 16-row tiles: Q[row][32*ks + 8*lg .. +7]
-  int row[2];
-  bool row_ok[2];
-  uint4 qreg[2][kAttnD / 32];
-  uint64_t bits[2][2];                                  // [row tile][mask word]
+  int row[ROWT];
+  bool row_ok[ROWT];
+  uint4 qreg[ROWT][kAttnD / 32];
+  uint64_t bits[ROWT][2];                                  // [row tile][mask word]
 #pragma unroll
-  for (int nt = 0; nt < 2; ++nt) {
-    row[nt] = (wave & 1) * 32 + nt * 16 + lq;
+  for (int nt = 0; nt < ROWT; ++nt) {
+    row[nt] = (wave % WPH) * (16 * ROWT) + nt * 16 + lq;
     row_ok[nt] = head_ok && row[nt] < n;
     const uint16_t* qp = q + ((int64_t)bh * n + (row_ok[nt] ? row[nt] : 0)) * kAttnD;
 #pragma unroll
@@ -143,10 +146,10 @@ __global__ __launch_bounds__(kAttnThreads) __attribute__((amdgpu_waves_per_eu(2,
     bits[nt][1] = (row_ok[nt] && ap.mask_words > 1) ? ap_bits[1] : 0ull;
   }
 
-  v4f oacc[2][kAttnD / 16];
-  float m_run[2], l_run[2];
+  v4f oacc[ROWT][kAttnD / 16];
+  float m_run[ROWT], l_run[ROWT];
 #pragma unroll
-  for (int nt = 0; nt < 2; ++nt) {
+  for (int nt = 0; nt < ROWT; ++nt) {
     m_run[nt] = -INFINITY;
     l_run[nt] = 0.f;
 #pragma unroll
@@ -209,20 +212,24 @@ __global__ __launch_bounds__(kAttnThreads) __attribute__((amdgpu_waves_per_eu(2,
 
     // ---- S^T tiles: 4 x (16 keys x 16 queries) per row tile; lane holds keys 16*kt + 4*lg + r of query lq.
     //      Scores stay unscaled; the softmax scale is folded into the exp2 argument.
-    float s[2][4][4];
-    float mloc[2] = {-INFINITY, -INFINITY};
-    const bool plain = kb + kKeyBlock <= ap.prefix;    // block lies entirely in the prefix: no mask (uniform)
-    v4f acc[4][2];
+    float s[ROWT][4][4];
+    float mloc[ROWT];
 #pragma unroll
-    for (int kt = 0; kt < 4; ++kt) acc[kt][0] = acc[kt][1] = v4f{0.f, 0.f, 0.f, 0.f};
+    for (int nt = 0; nt < ROWT; ++nt) mloc[nt] = -INFINITY;
+    const bool plain = kb + kKeyBlock <= ap.prefix;    // block lies entirely in the prefix: no mask (uniform)
+    v4f acc[4][ROWT];
+#pragma unroll
+    for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+      for (int nt = 0; nt < ROWT; ++nt) acc[kt][nt] = v4f{0.f, 0.f, 0.f, 0.f};
     // eight independent accumulator chains (4 key tiles x 2 row tiles) keep the matrix pipe busy
 #pragma unroll
     for (int ks = 0; ks < kAttnD / 32; ++ks) {
 #pragma unroll
       for (int kt = 0; kt < 4; ++kt) {
         const uint4 a = *(const uint4*)(Ks + (kt * 16 + lq) * kKStride + ks * 32 + lg * 8);
-        acc[kt][0] = mfma32<DT>(a, qreg[0][ks], acc[kt][0]);
-        acc[kt][1] = mfma32<DT>(a, qreg[1][ks], acc[kt][1]);
+#pragma unroll
+        for (int nt = 0; nt < ROWT; ++nt) acc[kt][nt] = mfma32<DT>(a, qreg[nt][ks], acc[kt][nt]);
       }
     }
 #pragma unroll
@@ -231,7 +238,7 @@ __global__ __launch_bounds__(kAttnThreads) __attribute__((amdgpu_waves_per_eu(2,
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
 #pragma unroll
-          for (int nt = 0; nt < 2; ++nt) {
+          for (int nt = 0; nt < ROWT; ++nt) {
             s[nt][kt][r] = acc[kt][nt][r];
             mloc[nt] = fmaxf(mloc[nt], acc[kt][nt][r]);
           }
@@ -245,7 +252,7 @@ __global__ __launch_bounds__(kAttnThreads) __attribute__((amdgpu_waves_per_eu(2,
           const int rel = tree ? (int)(pos - ap.prefix) : 0;   // tree slot, < 64 * mask_words
           const int sh = rel & 63;
 #pragma unroll
-          for (int nt = 0; nt < 2; ++nt) {
+          for (int nt = 0; nt < ROWT; ++nt) {
             const uint64_t word = rel < 64 ? bits[nt][0] : bits[nt][1];
             const bool ok = in_range && (!tree || ((word >> sh) & 1ull));
             const float t = ok ? acc[kt][nt][r] : -INFINITY;
@@ -256,9 +263,9 @@ __global__ __launch_bounds__(kAttnThreads) __attribute__((amdgpu_waves_per_eu(2,
       }
     }
     // running maximum in units of raw scores (the scale is positive, so the order is the same)
-    float mneg[2];                                     // -max * scale_log2, the additive term of the exp2 argument
+    float mneg[ROWT];                                     // -max * scale_log2, the additive term of the exp2 argument
 #pragma unroll
-    for (int nt = 0; nt < 2; ++nt) {
+    for (int nt = 0; nt < ROWT; ++nt) {
       float mx = mloc[nt];
       mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
       mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
@@ -275,9 +282,9 @@ __global__ __launch_bounds__(kAttnThreads) __attribute__((amdgpu_waves_per_eu(2,
     }
     // ---- P^T as B operands straight from the accumulators: k index 8*lg + e of step j is key
     //      32*j + 16*(e/4) + 4*lg + e%4, i.e. registers of score tiles 2j and 2j+1
-    uint4 pb[2][2];
+    uint4 pb[ROWT][2];
 #pragma unroll
-    for (int nt = 0; nt < 2; ++nt) {
+    for (int nt = 0; nt < ROWT; ++nt) {
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
         float p[8];
@@ -302,14 +309,14 @@ __global__ __launch_bounds__(kAttnThreads) __attribute__((amdgpu_waves_per_eu(2,
         const uint16_t* vp = vlane + (j * 32) * kVStride + mt * 16;
         const uint2 lo = lds_read_tr16(vp), hi = lds_read_tr16(vp + 16 * kVStride);
         const uint4 a = make_uint4(lo.x, lo.y, hi.x, hi.y);
-        oacc[0][mt] = mfma32<DT>(a, pb[0][j], oacc[0][mt]);
-        oacc[1][mt] = mfma32<DT>(a, pb[1][j], oacc[1][mt]);
+#pragma unroll
+        for (int nt = 0; nt < ROWT; ++nt) oacc[nt][mt] = mfma32<DT>(a, pb[nt][j], oacc[nt][mt]);
       }
     }
   }
 
 #pragma unroll
-  for (int nt = 0; nt < 2; ++nt) {
+  for (int nt = 0; nt < ROWT; ++nt) {
     // the four lane groups hold disjoint keys of the same query
     float l = l_run[nt];
     l += __shfl_xor(l, 16, kWave);
@@ -369,7 +376,7 @@ __global__ __launch_bounds__(256) void tree_attention_merge_kernel(
 
 static int attn_chunks(int64_t batch, int64_t hq, int64_t kv_len) {
   const int64_t blocks = (kv_len + kKeyBlock - 1) / kKeyBlock;
-  // one workgroup per two query heads; aim at roughly one workgroup per compute unit
+  // aim at roughly one workgroup per compute unit
   int64_t chunks = std::max<int64_t>(1, 1024 / std::max<int64_t>(1, batch * hq));
   chunks = std::min<int64_t>(chunks, std::max<int64_t>(1, blocks / 2));   // at least 128 keys per chunk
   return (int)std::min<int64_t>(chunks, 64);
@@ -435,7 +442,11 @@ static int tree_attention_impl(const char* what, const void* q, const void* k_ca
   ap.chunks = (int)((kv_len + ap.chunk_keys - 1) / ap.chunk_keys);
   ap.scale_log2 = scale * kLog2e;
   const int group = (int)(n_q_heads / n_kv_heads);
-  ap.pairs_per_kv = (group + kHeadsPerWG - 1) / kHeadsPerWG;
+  // wavefront = ROWT 16-row tiles of one head; WPH wavefronts per head; 8 / WPH heads share a workgroup's K / V stages:
+  // up to 16 rows (a draft level): 1 tile, 8 heads; up to 32 rows: 2 tiles, 8 heads; up to 64 rows: 2 tiles x 2 wavefronts, 4 heads
+  const int wph = n_rows <= 32 ? 1 : 2, rowt = n_rows <= 16 ? 1 : 2;
+  const int heads_per_wg = 8 / wph;
+  ap.pairs_per_kv = (group + heads_per_wg - 1) / heads_per_wg;
   ap.units = batch * n_kv_heads * ap.chunks;
   float* part_o = nullptr;
   float* part_ml = nullptr;
@@ -453,12 +464,16 @@ static int tree_attention_impl(const char* what, const void* q, const void* k_ca
   const dim3 grid((unsigned)((ap.units + kXcds - 1) / kXcds * kXcds * ap.pairs_per_kv));
   const int64_t merge_rows = batch * n_q_heads * n_rows / 8 >= 1024 ? 8 : 2;   // rows per merge workgroup
   const dim3 merge_grid((unsigned)((n_rows + merge_rows - 1) / merge_rows), (unsigned)(batch * n_q_heads));
+#define SUBSPEC_ATTN_KERNEL(DT, PAGED, ROWT, WPH)                                                                  \
+  hipLaunchKernelGGL((tree_attention_kernel<DT, PAGED, ROWT, WPH>), grid, dim3(kAttnThreads), 0, st, (const uint16_t*)q, \
+                     (const uint16_t*)k_cache, (const uint16_t*)v_cache, anc_bits, ap, (uint16_t*)out, part_o, part_ml)
 #define SUBSPEC_ATTN_LAUNCH(DT, PAGED)                                                                             \
   do {                                                                                                             \
     {                                                                                                              \
       DominantKernelTimer timer(st);                                                                               \
-      hipLaunchKernelGGL((tree_attention_kernel<DT, PAGED>), grid, dim3(kAttnThreads), 0, st, (const uint16_t*)q,  \
-                         (const uint16_t*)k_cache, (const uint16_t*)v_cache, anc_bits, ap, (uint16_t*)out, part_o, part_ml); \
+      if (rowt == 1) SUBSPEC_ATTN_KERNEL(DT, PAGED, 1, 1);                                                         \
+      else if (wph == 1) SUBSPEC_ATTN_KERNEL(DT, PAGED, 2, 1);                                                     \
+      else SUBSPEC_ATTN_KERNEL(DT, PAGED, 2, 2);                                                                   \
     }                                                                                                              \
     if (ap.chunks > 1)                                                                                             \
       hipLaunchKernelGGL((tree_attention_merge_kernel<DT>), merge_grid, dim3(merge_rows * 32), 0, st, part_o, part_ml, ap, \
@@ -467,6 +482,7 @@ static int tree_attention_impl(const char* what, const void* q, const void* k_ca
   if (dtype == SUBSPEC_BF16) { if (paged) SUBSPEC_ATTN_LAUNCH(SUBSPEC_BF16, true); else SUBSPEC_ATTN_LAUNCH(SUBSPEC_BF16, false); }
   else { if (paged) SUBSPEC_ATTN_LAUNCH(SUBSPEC_F16, true); else SUBSPEC_ATTN_LAUNCH(SUBSPEC_F16, false); }
 #undef SUBSPEC_ATTN_LAUNCH
+#undef SUBSPEC_ATTN_KERNEL
   SUBSPEC_CHECK_HIP(hipGetLastError());
   return SUBSPEC_OK;
 }

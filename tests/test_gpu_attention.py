@@ -37,7 +37,9 @@ def _check(parents, q, k, v, P, tag):
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_small_shapes(dtype):
     for seed, (B, Hq, Hkv, n, P, S) in enumerate([(1, 4, 2, 9, 0, 16), (2, 7, 1, 17, 5, 64), (1, 28, 4, 64, 100, 200),
-                                                  (3, 8, 8, 33, 63, 128), (1, 14, 2, 1, 300, 301), (2, 4, 4, 64, 64, 128)]):
+                                                  (3, 8, 8, 33, 63, 128), (1, 14, 2, 1, 300, 301), (2, 4, 4, 64, 64, 128),
+                                                  # more heads per KV head than one workgroup takes, few rows
+                                                  (1, 16, 1, 8, 40, 64), (1, 12, 1, 24, 10, 64), (2, 20, 2, 16, 130, 160)]):
         parents, q, k, v = _case(seed, B, Hq, Hkv, n, P, S, dtype, depth=6)
         _check(parents, q, k, v, P, f"small{seed}")
 
