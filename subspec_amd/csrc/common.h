@@ -102,6 +102,16 @@ __device__ __forceinline__ float div_rn(float x, const Divisor& d) {
   return fabsf(q) == INFINITY ? q : q1;
 }
 
+// Output element of a linear layer: v = accumulator (+ bias), optionally followed by a residual add with
+// the rounding points of the separate tensor ops it replaces: out = round(round(v) + residual[i]).
+// `residual` may be the output itself (in-place update of the residual stream): the element is read and
+// written by the same thread.
+template <int DT>
+__device__ __forceinline__ void store_linear_out(void* y, int64_t i, float v, const void* residual) {
+  if (residual) v = Elem<DT>::round(v) + Elem<DT>::load(residual, i);
+  Elem<DT>::store(y, i, v);
+}
+
 // ---------------------------------------------------------------- wave / block reductions
 __device__ __forceinline__ float wave_max(float v) {
 #pragma unroll
@@ -161,5 +171,14 @@ __device__ __forceinline__ int block_min_i(int v, int* scratch) {
 
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
+
+// Linear layers with a fused residual add (y = x W^T + bias + residual; residual may alias y); the C entry points
+// are these with residual = NULL.  Used by the decoder-layer sequence.
+int int4_linear_ex(const void* x, const uint32_t* wq, const uint32_t* sz, const void* bias, const void* residual, void* y,
+                   int dtype, int64_t M, int64_t N, int64_t K, int64_t group_size, void* workspace, size_t workspace_bytes,
+                   void* stream);
+int dense_linear_ex(const void* x, const void* w, const void* bias, const void* residual, void* y, int dtype, int64_t M,
+                    int64_t N, int64_t K, void* workspace, size_t workspace_bytes, void* stream);
+
 
 }  // namespace subspec

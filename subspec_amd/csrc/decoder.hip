@@ -13,7 +13,7 @@
 //   x     += int4(a)                            (o_proj; the add is fused into the next rmsnorm)
 //   h      = rmsnorm(x) * w_post
 //   act    = silu(gate) * up,  gate|up = int4(h)
-//   x     += int4(act)                          (down_proj)
+//   x     += int4(act)                          (down_proj; the add is fused into its output stage)
 // Rounding follows the eager torch layer: every intermediate tensor is rounded to the activation
 // dtype where torch would materialise it (normalised activations before the weight product, the
 // two rotary products and their sum, silu before the product with `up`, both residual sums).
@@ -104,19 +104,6 @@ __global__ __launch_bounds__(kNormThreads) void add_rmsnorm_kernel(uint16_t* __r
   }
 }
 
-// x += delta (rounded), 8 elements per thread
-template <int DT>
-__global__ __launch_bounds__(256) void add_kernel(uint16_t* __restrict__ x, const uint16_t* __restrict__ delta, int64_t pieces) {
-  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (i >= pieces) return;
-  float a[8], d[8];
-  unpack8<DT>(((const dec_u4*)x)[i], a);
-  unpack8<DT>(((const dec_u4*)delta)[i], d);
-#pragma unroll
-  for (int j = 0; j < 8; ++j) a[j] = Elem<DT>::round(a[j] + d[j]);
-  ((dec_u4*)x)[i] = pack8<DT>(a);
-}
-
 // act[m, f] = round(silu(gate)) * up with gate = gu[m, f], up = gu[m, F + f]
 template <int DT>
 __global__ __launch_bounds__(256) void silu_mul_kernel(const uint16_t* __restrict__ gu, uint16_t* __restrict__ act, int F,
@@ -169,7 +156,7 @@ __global__ __launch_bounds__(64) void rope_write_kernel(const uint16_t* __restri
 }
 
 struct LayerPlan {
-  size_t h, qkv, q, a, o, gu, act, d, sub, sub_bytes, total;
+  size_t h, qkv, q, a, o, gu, act, sub, sub_bytes, total;
 };
 static LayerPlan layer_plan(const subspec_decoder_layer_dims& s) {
   LayerPlan p;
@@ -184,7 +171,6 @@ static LayerPlan layer_plan(const subspec_decoder_layer_dims& s) {
   p.o = take(M * H * es);
   p.gu = take(M * 2 * F * es);
   p.act = take(M * F * es);
-  p.d = take(M * H * es);
   size_t sub = subspec_int4_linear_workspace(s.n_rows, Q + 2 * KV, H);
   sub = std::max(sub, subspec_int4_linear_workspace(s.n_rows, H, Q));
   sub = std::max(sub, subspec_int4_linear_workspace(s.n_rows, 2 * F, H));
@@ -228,10 +214,10 @@ struct LayerWeights {
   Projection qkv, o, gate_up, down;
   bool dense;
 };
-static int project(const LayerWeights& w, const Projection& p, const void* x, const void* bias, void* y, int dtype, int64_t M,
-                   int64_t N, int64_t K, void* sub, size_t sub_bytes, hipStream_t st) {
-  if (w.dense) return subspec_dense_linear(x, p.w, bias, y, dtype, M, N, K, sub, sub_bytes, st);
-  return subspec_int4_linear(x, (const uint32_t*)p.w, (const uint32_t*)p.sz, bias, y, dtype, M, N, K, 64, sub, sub_bytes, st);
+static int project(const LayerWeights& w, const Projection& p, const void* x, const void* bias, const void* residual, void* y,
+                   int dtype, int64_t M, int64_t N, int64_t K, void* sub, size_t sub_bytes, hipStream_t st) {
+  if (w.dense) return dense_linear_ex(x, p.w, bias, residual, y, dtype, M, N, K, sub, sub_bytes, st);
+  return int4_linear_ex(x, (const uint32_t*)p.w, (const uint32_t*)p.sz, bias, residual, y, dtype, M, N, K, 64, sub, sub_bytes, st);
 }
 
 template <int DT>
@@ -243,26 +229,25 @@ static int run_layer(const subspec_decoder_layer_dims& s, const LayerWeights& w,
             F = (int)s.intermediate;
   const int64_t Q = (int64_t)Hq * D, KV = (int64_t)Hkv * D;
   uint16_t *h = (uint16_t*)(ws + p.h), *qkv = (uint16_t*)(ws + p.qkv), *q = (uint16_t*)(ws + p.q), *a = (uint16_t*)(ws + p.a),
-           *o = (uint16_t*)(ws + p.o), *gu = (uint16_t*)(ws + p.gu), *act = (uint16_t*)(ws + p.act), *d = (uint16_t*)(ws + p.d);
+           *o = (uint16_t*)(ws + p.o), *gu = (uint16_t*)(ws + p.gu), *act = (uint16_t*)(ws + p.act);
   void* sub = ws + p.sub;
   int rc;
   hipLaunchKernelGGL((add_rmsnorm_kernel<DT, false>), dim3(M), dim3(kNormThreads), 0, st, x, (const uint16_t*)nullptr,
                      (const uint16_t*)w.input_norm, h, H, s.rms_eps);
-  if ((rc = project(w, w.qkv, h, w.qkv_bias, qkv, DT, M, Q + 2 * KV, H, sub, p.sub_bytes, st))) return rc;
+  if ((rc = project(w, w.qkv, h, w.qkv_bias, nullptr, qkv, DT, M, Q + 2 * KV, H, sub, p.sub_bytes, st))) return rc;
   hipLaunchKernelGGL((rope_write_kernel<DT>), dim3(M, Hq + 2 * Hkv), dim3(64), 0, st, qkv, positions, cache_rows, q, k_cache,
                      v_cache, M, Hq, Hkv, D, s.kv_seq_stride, log2f(s.rope_theta));
   if ((rc = subspec_tree_attention(q, k_cache, v_cache, a, DT, 1, Hq, Hkv, M, s.n_tree_slots, D, s.kv_seq_stride, s.prefix_len,
                                    anc_bits, 0, 1.f / sqrtf((float)D), sub, p.sub_bytes, st)))
     return rc;
-  if ((rc = project(w, w.o, a, nullptr, o, DT, M, H, Q, sub, p.sub_bytes, st))) return rc;
+  if ((rc = project(w, w.o, a, nullptr, nullptr, o, DT, M, H, Q, sub, p.sub_bytes, st))) return rc;
   hipLaunchKernelGGL((add_rmsnorm_kernel<DT, true>), dim3(M), dim3(kNormThreads), 0, st, x, o, (const uint16_t*)w.post_norm, h, H,
                      s.rms_eps);
-  if ((rc = project(w, w.gate_up, h, nullptr, gu, DT, M, 2 * (int64_t)F, H, sub, p.sub_bytes, st))) return rc;
+  if ((rc = project(w, w.gate_up, h, nullptr, nullptr, gu, DT, M, 2 * (int64_t)F, H, sub, p.sub_bytes, st))) return rc;
   const int64_t act_pieces = (int64_t)M * F / 8;
   hipLaunchKernelGGL((silu_mul_kernel<DT>), dim3((unsigned)((act_pieces + 255) / 256)), dim3(256), 0, st, gu, act, F, act_pieces);
-  if ((rc = project(w, w.down, act, nullptr, d, DT, M, H, F, sub, p.sub_bytes, st))) return rc;
-  const int64_t x_pieces = (int64_t)M * H / 8;
-  hipLaunchKernelGGL((add_kernel<DT>), dim3((unsigned)((x_pieces + 255) / 256)), dim3(256), 0, st, x, d, x_pieces);
+  // down projection with the residual add in its output stage: x = round(round(down(act)) + x)
+  if ((rc = project(w, w.down, act, nullptr, x, x, DT, M, H, F, sub, p.sub_bytes, st))) return rc;
   SUBSPEC_CHECK_HIP(hipGetLastError());
   return SUBSPEC_OK;
 }

@@ -41,7 +41,8 @@ __device__ __forceinline__ dn_v4f dn_mfma32(dn_u4 a, dn_u4 b, dn_v4f c) {
 template <int DT, int MT, int RT>
 __global__ __launch_bounds__(kDnThreads) void dense_gemm_kernel(
     const uint16_t* __restrict__ x, const uint16_t* __restrict__ w, const uint16_t* __restrict__ bias,
-    uint16_t* __restrict__ y, float* __restrict__ partial, int M, int64_t N, int K, int splits, int groups_per_split) {
+    const uint16_t* residual, uint16_t* y, float* __restrict__ partial, int M, int64_t N, int K, int splits,
+    int groups_per_split) {
   // 4 wavefronts x 2 stages of a [16*MT][64] activation block; reused for the final reduction
   constexpr int kStageBytes = 4 * 2 * MT * 16 * kDnXlStride * 2, kRedBytes = 2 * 4 * MT * 256 * 4;
   __shared__ __attribute__((aligned(16))) unsigned char lds_raw[kStageBytes > kRedBytes ? kStageBytes : kRedBytes];
@@ -176,7 +177,7 @@ __global__ __launch_bounds__(kDnThreads) void dense_gemm_kernel(
       for (int rr = 0; rr < 4; ++rr) {
         const int m = mt * 16 + c * 4 + rr;
         if (m >= M) continue;
-        if (splits == 1) Elem<DT>::store(y, (int64_t)m * N + n, v[rr] + bv);
+        if (splits == 1) store_linear_out<DT>(y, (int64_t)m * N + n, v[rr] + bv, residual);
         else partial[((int64_t)ks * M + m) * N + n] = v[rr];
       }
     }
@@ -185,13 +186,14 @@ __global__ __launch_bounds__(kDnThreads) void dense_gemm_kernel(
 
 template <int DT>
 __global__ __launch_bounds__(256) void dense_reduce_kernel(const float* __restrict__ partial, const uint16_t* __restrict__ bias,
-                                                           uint16_t* __restrict__ y, int64_t M, int64_t N, int splits) {
+                                                           const uint16_t* residual, uint16_t* y, int64_t M, int64_t N,
+                                                           int splits) {
   const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (i >= M * N) return;
   float v = 0.f;
   for (int s = 0; s < splits; ++s) v += partial[(int64_t)s * M * N + i];
   if (bias) v += Elem<DT>::load(bias, i % N);
-  Elem<DT>::store(y, i, v);
+  store_linear_out<DT>(y, i, v, residual);
 }
 
 struct DnPlan { int wgs, row_tiles, splits, groups_per_split; };
@@ -215,14 +217,14 @@ static DnPlan dn_plan(int64_t M, int64_t N, int64_t K) {
 }
 
 template <int DT>
-static int run_dense(const void* x, const void* w, const void* bias, void* y, int64_t M, int64_t N, int64_t K,
-                     void* workspace, hipStream_t st) {
+static int run_dense(const void* x, const void* w, const void* bias, const void* residual, void* y, int64_t M, int64_t N,
+                     int64_t K, void* workspace, hipStream_t st) {
   const DnPlan pl = dn_plan(M, N, K);
   float* partial = (float*)workspace;
   const dim3 grid((unsigned)pl.wgs, (unsigned)pl.splits);
 #define SUBSPEC_DN_LAUNCH(MT, RT)                                                                                  \
   hipLaunchKernelGGL((dense_gemm_kernel<DT, MT, RT>), grid, dim3(kDnThreads), 0, st, (const uint16_t*)x,           \
-                     (const uint16_t*)w, (const uint16_t*)bias, (uint16_t*)y, partial, (int)M, N, (int)K,          \
+                     (const uint16_t*)w, (const uint16_t*)bias, (const uint16_t*)residual, (uint16_t*)y, partial, (int)M, N, (int)K, \
                      pl.splits, pl.groups_per_split)
 #define SUBSPEC_DN_LAUNCH_MT(MT)                                                                                   \
   do {                                                                                                             \
@@ -240,7 +242,7 @@ static int run_dense(const void* x, const void* w, const void* bias, void* y, in
 #undef SUBSPEC_DN_LAUNCH
   if (pl.splits > 1)
     hipLaunchKernelGGL((dense_reduce_kernel<DT>), dim3((unsigned)((M * N + 255) / 256)), dim3(256), 0, st, partial,
-                       (const uint16_t*)bias, (uint16_t*)y, M, N, pl.splits);
+                       (const uint16_t*)bias, (const uint16_t*)residual, (uint16_t*)y, M, N, pl.splits);
   SUBSPEC_CHECK_HIP(hipGetLastError());
   return SUBSPEC_OK;
 }
@@ -257,6 +259,11 @@ extern "C" size_t subspec_dense_linear_workspace(int64_t M, int64_t N, int64_t K
 
 extern "C" int subspec_dense_linear(const void* x, const void* w, const void* bias, void* y, int dtype, int64_t M,
                                     int64_t N, int64_t K, void* workspace, size_t workspace_bytes, void* stream) {
+  return dense_linear_ex(x, w, bias, nullptr, y, dtype, M, N, K, workspace, workspace_bytes, stream);
+}
+
+int subspec::dense_linear_ex(const void* x, const void* w, const void* bias, const void* residual, void* y, int dtype, int64_t M,
+                             int64_t N, int64_t K, void* workspace, size_t workspace_bytes, void* stream) {
   if (dtype != SUBSPEC_BF16 && dtype != SUBSPEC_F16)
     SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "dense_linear: dtype %d not supported (bf16 / fp16 only)", dtype);
   if (!x || !w || !y) SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "dense_linear: null pointer argument");
@@ -275,6 +282,6 @@ extern "C" int subspec_dense_linear(const void* x, const void* w, const void* bi
     if ((uintptr_t)workspace % 16) SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "dense_linear: workspace must be 16-byte aligned");
   }
   hipStream_t st = (hipStream_t)stream;
-  if (dtype == SUBSPEC_BF16) return run_dense<SUBSPEC_BF16>(x, w, bias, y, M, N, K, workspace, st);
-  return run_dense<SUBSPEC_F16>(x, w, bias, y, M, N, K, workspace, st);
+  if (dtype == SUBSPEC_BF16) return run_dense<SUBSPEC_BF16>(x, w, bias, residual, y, M, N, K, workspace, st);
+  return run_dense<SUBSPEC_F16>(x, w, bias, residual, y, M, N, K, workspace, st);
 }

@@ -58,7 +58,7 @@ __device__ __forceinline__ uint32_t code_pair(uint32_t w, int shift, uint32_t ma
 template <int DT>
 __global__ __launch_bounds__(kI4Threads) void int4_gemv_kernel(
     const uint16_t* __restrict__ x, const uint2* __restrict__ wq, const uint32_t* __restrict__ sz,
-    const uint16_t* __restrict__ bias, uint16_t* __restrict__ y, int64_t N, int64_t K) {
+    const uint16_t* __restrict__ bias, const uint16_t* residual, uint16_t* y, int64_t N, int64_t K) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   uint16_t* xs = (uint16_t*)smem;                               // [K]
   float* xsum16 = (float*)(smem + K * 2);                       // [K / 16]
@@ -119,7 +119,7 @@ __global__ __launch_bounds__(kI4Threads) void int4_gemv_kernel(
     float v = red[tid] + red[16 + tid] + red[32 + tid] + red[48 + tid];
     const int64_t n = nt * 16 + tid;
     if (bias) v += I4<DT>::to_float(bias[n]);
-    Elem<DT>::store(y, n, v);
+    store_linear_out<DT>(y, n, v, residual);
   }
 }
 
@@ -153,7 +153,7 @@ __device__ __forceinline__ i4_v4f i4_mfma32(i4_u4 a, i4_u4 b, i4_v4f c) {
 template <int DT, int MT, int RT>
 __global__ __launch_bounds__(kI4Threads) void int4_gemm_kernel(
     const uint16_t* __restrict__ x, const uint2* __restrict__ wq, const uint32_t* __restrict__ sz,
-    const uint16_t* __restrict__ bias, uint16_t* __restrict__ y, float* __restrict__ partial, int M, int64_t N,
+    const uint16_t* __restrict__ bias, const uint16_t* residual, uint16_t* y, float* __restrict__ partial, int M, int64_t N,
     int K, int splits, int groups_per_split) {
   // 4 wavefronts x 2 stages of a [16*MT][64] activation block; reused for the final reduction
   // (two rounds of one accumulator tile set per wavefront)
@@ -316,7 +316,7 @@ __global__ __launch_bounds__(kI4Threads) void int4_gemm_kernel(
       for (int rr = 0; rr < 4; ++rr) {
         const int m = mt * 16 + c * 4 + rr;
         if (m >= M) continue;
-        if (splits == 1) Elem<DT>::store(y, (int64_t)m * N + n, v[rr] + bv);
+        if (splits == 1) store_linear_out<DT>(y, (int64_t)m * N + n, v[rr] + bv, residual);
         else partial[((int64_t)ks * M + m) * N + n] = v[rr];
       }
     }
@@ -325,14 +325,14 @@ __global__ __launch_bounds__(kI4Threads) void int4_gemm_kernel(
 
 template <int DT>
 __global__ __launch_bounds__(256) void int4_reduce_kernel(const float* __restrict__ partial,
-                                                          const uint16_t* __restrict__ bias, uint16_t* __restrict__ y,
-                                                          int64_t M, int64_t N, int splits) {
+                                                          const uint16_t* __restrict__ bias, const uint16_t* residual,
+                                                          uint16_t* y, int64_t M, int64_t N, int splits) {
   const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (i >= M * N) return;
   float v = 0.f;
   for (int s = 0; s < splits; ++s) v += partial[(int64_t)s * M * N + i];
   if (bias) v += I4<DT>::to_float(bias[i % N]);
-  Elem<DT>::store(y, i, v);
+  store_linear_out<DT>(y, i, v, residual);
 }
 
 struct I4Plan { int wgs, row_tiles, splits, groups_per_split; };
@@ -360,22 +360,22 @@ static I4Plan i4_plan(int64_t M, int64_t N, int64_t K) {
 }
 
 template <int DT>
-static int run_int4(const void* x, const uint32_t* wq, const uint32_t* sz, const void* bias, void* y, int64_t M,
-                    int64_t N, int64_t K, void* workspace, hipStream_t st) {
+static int run_int4(const void* x, const uint32_t* wq, const uint32_t* sz, const void* bias, const void* residual, void* y,
+                    int64_t M, int64_t N, int64_t K, void* workspace, hipStream_t st) {
   // One row: the GEMV kernel, unless the matrix has few rows and a long K (down projection): then its one workgroup
   // per 16-row tile leaves most of the chip idle and the split-K GEMM path is faster (3584x18944 from HBM: 22 against 32 us).
   if (M == 1 && i4_plan(M, N, K).splits == 1) {
     const size_t smem = (size_t)K * 2 + (size_t)(K / 16) * 4 + 64 * 4;
     DominantKernelTimer timer(st);
     hipLaunchKernelGGL((int4_gemv_kernel<DT>), dim3((unsigned)(N / 16)), dim3(kI4Threads), smem, st, (const uint16_t*)x,
-                       (const uint2*)wq, sz, (const uint16_t*)bias, (uint16_t*)y, N, K);
+                       (const uint2*)wq, sz, (const uint16_t*)bias, (const uint16_t*)residual, (uint16_t*)y, N, K);
   } else {
     const I4Plan pl = i4_plan(M, N, K);
     float* partial = (float*)workspace;
     const dim3 grid((unsigned)pl.wgs, (unsigned)pl.splits);
 #define SUBSPEC_I4_LAUNCH(MT, RT)                                                                                  \
   hipLaunchKernelGGL((int4_gemm_kernel<DT, MT, RT>), grid, dim3(kI4Threads), 0, st, (const uint16_t*)x,            \
-                     (const uint2*)wq, sz, (const uint16_t*)bias, (uint16_t*)y, partial, (int)M, N, (int)K,        \
+                     (const uint2*)wq, sz, (const uint16_t*)bias, (const uint16_t*)residual, (uint16_t*)y, partial, (int)M, N, (int)K, \
                      pl.splits, pl.groups_per_split)
 #define SUBSPEC_I4_LAUNCH_MT(MT)                                                                                   \
   do {                                                                                                             \
@@ -394,7 +394,7 @@ static int run_int4(const void* x, const uint32_t* wq, const uint32_t* sz, const
 #undef SUBSPEC_I4_LAUNCH
     if (pl.splits > 1)
       hipLaunchKernelGGL((int4_reduce_kernel<DT>), dim3((unsigned)((M * N + 255) / 256)), dim3(256), 0, st, partial,
-                         (const uint16_t*)bias, (uint16_t*)y, M, N, pl.splits);
+                         (const uint16_t*)bias, (const uint16_t*)residual, (uint16_t*)y, M, N, pl.splits);
   }
   SUBSPEC_CHECK_HIP(hipGetLastError());
   return SUBSPEC_OK;
@@ -404,15 +404,21 @@ static int run_int4(const void* x, const uint32_t* wq, const uint32_t* sz, const
 
 using namespace subspec;
 
+extern "C" int subspec_int4_linear(const void* x, const uint32_t* wq, const uint32_t* sz, const void* bias, void* y,
+                                   int dtype, int64_t M, int64_t N, int64_t K, int64_t group_size, void* workspace,
+                                   size_t workspace_bytes, void* stream) {
+  return int4_linear_ex(x, wq, sz, bias, nullptr, y, dtype, M, N, K, group_size, workspace, workspace_bytes, stream);
+}
+
 extern "C" size_t subspec_int4_linear_workspace(int64_t M, int64_t N, int64_t K) {
   if (M <= 0 || N <= 0 || K <= 0) return 256;
   const I4Plan pl = i4_plan(M, N, K);
   return (pl.splits > 1 ? align_up((size_t)pl.splits * M * N * sizeof(float), 256) : 0) + 256;
 }
 
-extern "C" int subspec_int4_linear(const void* x, const uint32_t* wq, const uint32_t* sz, const void* bias, void* y,
-                                   int dtype, int64_t M, int64_t N, int64_t K, int64_t group_size, void* workspace,
-                                   size_t workspace_bytes, void* stream) {
+int subspec::int4_linear_ex(const void* x, const uint32_t* wq, const uint32_t* sz, const void* bias, const void* residual,
+                            void* y, int dtype, int64_t M, int64_t N, int64_t K, int64_t group_size, void* workspace,
+                            size_t workspace_bytes, void* stream) {
   if (dtype != SUBSPEC_BF16 && dtype != SUBSPEC_F16)
     SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "int4_linear: dtype %d not supported (bf16 / fp16 activations only)", dtype);
   if (!x || !wq || !sz || !y) SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "int4_linear: null pointer argument");
@@ -433,6 +439,6 @@ extern "C" int subspec_int4_linear(const void* x, const uint32_t* wq, const uint
                    workspace_bytes, need);
     if ((uintptr_t)workspace % 16) SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "int4_linear: workspace must be 16-byte aligned");
   }
-  if (dtype == SUBSPEC_BF16) return run_int4<SUBSPEC_BF16>(x, wq, sz, bias, y, M, N, K, workspace, (hipStream_t)stream);
-  return run_int4<SUBSPEC_F16>(x, wq, sz, bias, y, M, N, K, workspace, (hipStream_t)stream);
+  if (dtype == SUBSPEC_BF16) return run_int4<SUBSPEC_BF16>(x, wq, sz, bias, residual, y, M, N, K, workspace, (hipStream_t)stream);
+  return run_int4<SUBSPEC_F16>(x, wq, sz, bias, residual, y, M, N, K, workspace, (hipStream_t)stream);
 }
