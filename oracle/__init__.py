@@ -31,8 +31,17 @@ How each function is pinned (so a wrong sign / index / dropped term fails a test
 * ``int4.linear``                          – closed form x @ ((Wq - z) * s).T; the special case
   s=1, z=0 reduces to an integer matmul.  The HQQ *quantizer* itself (hqq==0.2.6, absent) is
   **parity unpinned**: parity is defined on the linear given identical (Wq, scale, zero).
-* ``decoder.decoder_layer``                – float32 restatement of the published Qwen2 decoder layer
-  (transformers 4.52.3, not in the reference tree) with the affine int4 linears; **parity
-  unpinned** beyond closed forms: rotary is a rotation, identity at position 0 and relative; zero
-  output projections leave the residual stream; its attention block equals ``attention.tree_attention``.
+* ``decoder.decoder_layer``                – float32 restatement of the Qwen2 decoder layer the reference runs
+  through HuggingFace; equals ``transformers``' own Qwen2 decoder (small random-weight model built in the
+  test, called with a cached prefix, ``position_ids = prefix + depth`` and the additive ancestor mask, as
+  ``_tree_decoding`` does) to 2e-4 in every layer's hidden state, the logits and the cached K / V rows;
+  plus closed forms (rotary is a rotation, identity at position 0 and relative; zero output projections
+  leave the residual stream; its attention block equals ``attention.tree_attention``).
+* ``kv.compact_paged``                     – the reference's pool reorder restated literally
+  (``compact_paged_reference``) for the identity page table; gather / compact / scatter equivalence for a
+  permuted table.
+* ``sampling``                             – Philox4x32-10 against Random123's known-answer vectors; the
+  exponential race against a per-element loop and a chi-square test; the verifiers with pre-drawn target
+  tokens against brute force and hand-built walks.  The random stream is this build's contract (torch's is
+  not an interface); the distribution and the use of the draw are the reference's.
 """

@@ -5,8 +5,12 @@ draft: the HuggingFace Qwen2 layer whose projections are the affine int4 linears
 ancestor mask of ``cpu_tree.py:263-286``.  Everything is float32 on dequantized weights; the device
 layer rounds intermediates to bf16, so comparisons use a relative tolerance.
 
-Pinned by: closed form only (textbook RMSNorm / rotary / softmax attention / SwiGLU); the
-arithmetic of the HuggingFace layer itself is not part of the reference tree.
+Pinned by: the HuggingFace Qwen2 decoder itself (transformers is importable in the build image; a small
+random-weight model, nothing downloaded), called as the reference calls it -- prefix in a KV cache, tree tokens
+with ``position_ids = prefix + depth`` and the additive ancestor mask (generators/classic_sd.py:75-109): hidden
+states of every layer, final logits and the cached K / V rows agree to 2e-4 in fp32
+(tests/test_oracle_hf_layer.py, which also shows that a causal mask or slot-index positions are detected);
+plus closed forms (rotary is a rotation, identity at position 0, relative).
 """
 import torch
 

@@ -283,13 +283,20 @@ def load_hf_checkpoint(path: str, device="cpu", dtype=torch.bfloat16):
             for key in sf.keys():
                 tensors[key] = sf.get_tensor(key)
 
+    return cfg, weights_from_tensors(cfg, tensors, device, dtype, where=f"the checkpoint in {path}")
+
+
+def weights_from_tensors(cfg: DecoderConfig, tensors: Dict[str, torch.Tensor], device="cpu", dtype=torch.bfloat16,
+                         where: str = "the state dict") -> dict:
+    """HuggingFace-named tensors (``model.layers.N.self_attn.q_proj.weight`` ..., Qwen2 or Llama) -> this package's
+    fused layout (``qkv_proj = q|k|v`` rows, ``gate_up_proj = gate|up`` rows), as produced by ``init_weights``."""
     def take(name: str, required: bool = True) -> Optional[torch.Tensor]:
         t = tensors.get(name)
         if t is None:
             if required:
-                raise KeyError(f"{name} missing from the checkpoint in {path}")
+                raise KeyError(f"{name} missing from {where}")
             return None
-        return t.to(device=device, dtype=dtype)
+        return t.detach().to(device=device, dtype=dtype)
 
     layers = []
     for i in range(cfg.num_hidden_layers):
@@ -313,7 +320,7 @@ def load_hf_checkpoint(path: str, device="cpu", dtype=torch.bfloat16):
     head = take("lm_head.weight", required=False)
     if head is None:                                              # tie_word_embeddings
         head = embed
-    return cfg, {"embed": embed, "layers": layers, "norm": take("model.norm.weight"), "lm_head": head}
+    return {"embed": embed, "layers": layers, "norm": take("model.norm.weight"), "lm_head": head}
 
 
 def build_models(cfg: DecoderConfig, kv: KVManager, seed: int = 0, device="cuda:0", dtype=torch.bfloat16,

@@ -1,0 +1,121 @@
+"""GPU: the product decoder (bf16 target on one-call dense layers, int4 substitute draft on one-call int4
+layers, torch prefill) against a HuggingFace Qwen2 model with the same weights, called the way the
+reference calls it: prefill into a KV cache, then the draft tree as one sequence with
+``position_ids = prefix + depth`` and the additive ancestor mask
+(specdecodes/models/generators/classic_sd.py:75-109).  The HuggingFace side runs in fp32 on the CPU on
+the bf16-rounded weights; tolerance 3e-2 of the logit scale for two bf16 layers."""
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+transformers = pytest.importorskip("transformers")
+from transformers import Qwen2Config, Qwen2ForCausalLM  # noqa: E402
+from transformers.cache_utils import DynamicCache  # noqa: E402
+
+from oracle import int4 as oi
+from subspec_amd import ops, workloads as W
+from subspec_amd.cache import create_kv_cache
+from subspec_amd.model import DecoderConfig, build_models, weights_from_tensors
+
+DEV = "cuda:0"
+CFG = DecoderConfig(num_hidden_layers=2, hidden_size=256, num_attention_heads=2, num_key_value_heads=1, head_dim=128,
+                    intermediate_size=512, vocab_size=1024, rms_norm_eps=1e-6, rope_theta=1e6)
+
+
+def _hf(seed):
+    torch.manual_seed(seed)
+    cfg = Qwen2Config(vocab_size=CFG.vocab_size, hidden_size=CFG.hidden_size, intermediate_size=CFG.intermediate_size,
+                      num_hidden_layers=CFG.num_hidden_layers, num_attention_heads=CFG.num_attention_heads,
+                      num_key_value_heads=CFG.num_key_value_heads, max_position_embeddings=512, rope_theta=CFG.rope_theta,
+                      rms_norm_eps=CFG.rms_norm_eps, tie_word_embeddings=False)
+    cfg._attn_implementation = "eager"
+    model = Qwen2ForCausalLM(cfg).eval()
+    with torch.no_grad():
+        for p in model.parameters():                       # livelier than the 0.02 init, and exactly representable in bf16
+            if p.dim() == 2:
+                p.mul_(3.0)
+            p.copy_(p.to(torch.bfloat16).float())
+        for layer in model.model.layers:
+            for proj in (layer.self_attn.q_proj, layer.self_attn.k_proj, layer.self_attn.v_proj):
+                proj.bias.copy_((torch.randn_like(proj.bias) * 0.1).to(torch.bfloat16).float())
+    return model
+
+
+def _tree_call(model, prefix, tree, parents, depths):
+    P, n = prefix.numel(), tree.numel()
+    mask = torch.full((1, 1, n, P + n), torch.finfo(torch.float32).min)
+    mask[..., :P] = 0
+    for i in range(n):
+        j = i
+        while j >= 0:
+            mask[0, 0, i, P + j] = 0
+            j = parents[j]
+    with torch.no_grad():
+        cache = DynamicCache()
+        pre = model(prefix[None], past_key_values=cache, use_cache=True)
+        out = model(tree[None], past_key_values=cache, attention_mask=mask, position_ids=torch.tensor([[P + d for d in depths]]),
+                    cache_position=torch.arange(P, P + n), use_cache=True)
+    return pre.logits[0, -1], out.logits[0]
+
+
+def _close(got, ref, tag, tol=3e-2):
+    scale = ref.abs().amax().item()
+    err = (got.float().cpu() - ref).abs().amax().item()
+    assert err <= tol * scale, (tag, err, scale)
+    assert (got.float().cpu().argmax(-1) == ref.argmax(-1)).float().mean().item() >= 0.8, tag
+
+
+@pytest.mark.parametrize("n,P", [(9, 23), (64, 150), (1, 40)])
+def test_target_and_draft_match_huggingface(n, P):
+    print("hf model", n, P, flush=True)
+    model = _hf(n)
+    g = torch.Generator().manual_seed(n)
+    prefix = torch.randint(0, CFG.vocab_size, (P,), generator=g)
+    parents, _, depths = W.random_tree(g, n=n, max_depth=6, max_children=3, vocab=CFG.vocab_size, chain_depth=3)
+    tree = torch.randint(0, CFG.vocab_size, (n,), generator=g)
+    ref_last, ref_tree = _tree_call(model, prefix, tree, parents, depths)
+
+    kv = create_kv_cache("static", max_cache_len=256, config=CFG, device=DEV, dtype=torch.bfloat16)
+    weights = weights_from_tensors(CFG, model.state_dict(), device=DEV, dtype=torch.bfloat16)
+    target, draft, _ = build_models(CFG, kv, device=DEV, weights=weights)
+    anc = ops.ancestor_bits_tensor(parents, device=DEV)
+    dep = torch.tensor(depths, device=DEV)
+    _close(target.prefill(prefix.to(DEV), 0)[0], ref_last, "prefill")
+    assert target.native_layers
+    _close(target.tree_forward(tree.to(DEV), dep, anc, P), ref_tree, "target tree")
+
+    # the substitute draft against HuggingFace running the SAME dequantized int4 weights
+    sd = dict(model.state_dict())
+    q, kvs, F = CFG.q_size, CFG.kv_size, CFG.intermediate_size
+    for i, w in enumerate(draft.layers):
+        def deq(name, N, K):
+            return oi.dequant(*oi.unpack_tiled(w[name + ".wq"].cpu(), w[name + ".sz"].cpu(), N, K)).float()
+        qkv = deq("qkv_proj", q + 2 * kvs, CFG.hidden_size)
+        gu = deq("gate_up_proj", 2 * F, CFG.hidden_size)
+        pre = f"model.layers.{i}."
+        sd[pre + "self_attn.q_proj.weight"], sd[pre + "self_attn.k_proj.weight"], sd[pre + "self_attn.v_proj.weight"] = \
+            qkv[:q], qkv[q:q + kvs], qkv[q + kvs:]
+        sd[pre + "self_attn.o_proj.weight"] = deq("o_proj", CFG.hidden_size, q)
+        sd[pre + "mlp.gate_proj.weight"], sd[pre + "mlp.up_proj.weight"] = gu[:F], gu[F:]
+        sd[pre + "mlp.down_proj.weight"] = deq("down_proj", CFG.hidden_size, F)
+    qmodel = _hf(n)
+    qmodel.load_state_dict(sd)
+    # the draft shares the cache the target's prefill wrote (bf16 weights), as in the reference; HuggingFace's
+    # quantized model therefore also gets the prefix K/V of the unquantized model
+    P_, n_ = prefix.numel(), tree.numel()
+    mask = torch.full((1, 1, n_, P_ + n_), torch.finfo(torch.float32).min)
+    mask[..., :P_] = 0
+    for i in range(n_):
+        j = i
+        while j >= 0:
+            mask[0, 0, i, P_ + j] = 0
+            j = parents[j]
+    with torch.no_grad():
+        cache = DynamicCache()
+        model(prefix[None], past_key_values=cache, use_cache=True)
+        ref_draft = qmodel(tree[None], past_key_values=cache, attention_mask=mask,
+                           position_ids=torch.tensor([[P_ + d for d in depths]]), cache_position=torch.arange(P_, P_ + n_),
+                           use_cache=True).logits[0]
+    assert draft.native_layers
+    _close(draft.tree_forward(tree.to(DEV), dep, anc, P), ref_draft, "draft tree")
