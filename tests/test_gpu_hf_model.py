@@ -119,3 +119,37 @@ def test_target_and_draft_match_huggingface(n, P):
                            use_cache=True).logits[0]
     assert draft.native_layers
     _close(draft.tree_forward(tree.to(DEV), dep, anc, P), ref_draft, "draft tree")
+
+
+@pytest.mark.parametrize("method,kwargs", [("exact", None), ("lossy", dict(threshold=0.0, window_size=3, threshold_method="entropy"))])
+def test_speculative_generation_is_huggingface_greedy_decoding(method, kwargs):
+    """Exact verification (and the lossy verifier with a gate that blocks everything) must emit exactly what greedy
+    decoding of the target emits.  Checked by teacher forcing: HuggingFace scores the produced sequence in one
+    fp32 forward, and every produced token must be its argmax there -- or, where two logits are closer than bf16
+    can tell apart, within that margin of the maximum."""
+    from subspec_amd.draft import SubSpecSDDraftModel
+    from subspec_amd.generator import SubSpecSDGenerator
+    from subspec_amd.utils import DraftParams
+    model = _hf(5)
+    g = torch.Generator().manual_seed(5)
+    prompt = torch.randint(0, CFG.vocab_size, (1, 20), generator=g)
+    kv = create_kv_cache("static", max_cache_len=256, config=CFG, device=DEV, dtype=torch.bfloat16)
+    weights = weights_from_tensors(CFG, model.state_dict(), device=DEV, dtype=torch.bfloat16)
+    target, draft, _ = build_models(CFG, kv, device=DEV, weights=weights)
+    gen = SubSpecSDGenerator(target, None, SubSpecSDDraftModel(draft), DraftParams(temperature=0.2, max_depth=4, topk_len=4),
+                             generator_kwargs=dict(verify_method=method, verify_kwargs=kwargs))
+    out = gen.generate(prompt.to(DEV), max_new_tokens=40, do_sample=False, past_key_values=kv).cpu()
+    assert out.shape[1] == 60
+    with torch.no_grad():
+        logits = model(out).logits[0]                      # row t scores token t + 1
+    scale = logits.abs().amax().item()
+    exact = 0
+    for t in range(19, 59):
+        row = logits[t]
+        tok = int(out[0, t + 1])
+        if tok == int(row.argmax()):
+            exact += 1
+        else:
+            assert float(row.max() - row[tok]) <= 3e-2 * scale, (t, tok, int(row.argmax()), float(row.max() - row[tok]))
+    print("greedy agreement", exact, "of 40", flush=True)
+    assert exact >= 34
