@@ -1,7 +1,9 @@
-"""Static KV cache shared by the target and the substitute draft, with the reference's
+"""KV caches shared by the target and the substitute draft, with the reference's
 ``KVManager`` interface (specdecodes/models/utils/cache_utils.py:41-60): ``seq_len``,
 ``get_seq_length()``, ``crop()``, ``reorder_cache_with_offset(beam_idx, new_chunk_len, offset, dim)``,
-``reset()``.
+``reset()``.  ``StaticKVCache`` stands for ``TreeStaticCache`` (:113-208), ``DynamicKVCache`` for
+``TreeDynamicCache`` (:62-110): no fixed length, storage grows as rows are written, and a reorder
+truncates to the kept rows.
 
 Layout: ONE tensor ``[layers, 2 (K, V), batch, kv_heads, max_cache_len, head_dim]`` so that
 compaction after verification is a single kernel launch over ``layers * 2 * batch * kv_heads`` slabs
@@ -30,6 +32,11 @@ class StaticKVCache:
     def v(self, layer: int) -> torch.Tensor:
         return self.data[layer, 1]
 
+    def ensure(self, n_rows: int) -> None:
+        """Called before a forward that touches cache rows below ``n_rows``."""
+        if n_rows > self.max_cache_len:
+            raise ValueError(f"the static cache holds {self.max_cache_len} rows, {n_rows} are needed")
+
     def write(self, layer: int, positions: torch.Tensor, k: torch.Tensor, v: torch.Tensor) -> None:
         """k, v: [B, Hkv, n, D] written at cache rows ``positions`` (int64 [n])."""
         self.data[layer, 0].index_copy_(2, positions, k)
@@ -54,6 +61,46 @@ class StaticKVCache:
                         max_count=None if count_dev is None else min(int(beam_idx.numel()), 256))
 
 
+class DynamicKVCache(StaticKVCache):
+    """The same single-tensor layout without a fixed length (``TreeDynamicCache``, cache_utils.py:62-110): the
+    capacity doubles whenever a forward needs more rows (one reallocation and copy, amortised), ``crop`` and
+    ``reorder_cache_with_offset`` set the number of rows seen, as the reference's slicing / index_select do;
+    the kernels are the static cache's.  ``max_cache_len`` is the current capacity."""
+
+    def __init__(self, n_layers: int, n_kv_heads: int, head_dim: int, device, dtype, max_batch_size: int = 1,
+                 initial_len: int = 1024):
+        super().__init__(n_layers, n_kv_heads, head_dim, max(64, int(initial_len)), device, dtype, max_batch_size)
+        self._seen_tokens = 0
+
+    def ensure(self, n_rows: int) -> None:
+        if n_rows <= self.max_cache_len:
+            return
+        new_len = max(2 * self.max_cache_len, (int(n_rows) + 255) // 256 * 256)
+        shape = list(self.data.shape)
+        shape[-2] = new_len
+        grown = torch.zeros(shape, device=self.data.device, dtype=self.data.dtype)
+        grown[..., :self.max_cache_len, :] = self.data
+        self.data, self.max_cache_len = grown, new_len
+
+    def get_seq_length(self) -> int:
+        return self._seen_tokens
+
+    def reset(self) -> None:
+        self._seen_tokens = 0
+
+    def crop(self, start: int, end: Optional[int] = None, dim: int = 2) -> None:
+        if end is not None and start < 0:
+            start = end - abs(start)
+        self._seen_tokens = start                            # rows beyond are simply no longer part of the cache
+
+    def reorder_cache_with_offset(self, beam_idx: torch.Tensor, new_chunk_len: int = 1, offset: int = 0, dim: int = 2,
+                                  count_dev: Optional[torch.Tensor] = None) -> None:
+        """[:offset] unchanged, rows offset + beam_idx[j] follow, everything else is dropped (:92-110)."""
+        super().reorder_cache_with_offset(beam_idx, new_chunk_len, offset, dim, count_dev=count_dev)
+        if count_dev is None:                                # with a device-side count the caller sets the length
+            self._seen_tokens = int(offset) + int(beam_idx.numel())
+
+
 class KVManager:
     def __init__(self, cache: StaticKVCache):
         self.cache = cache
@@ -75,15 +122,20 @@ class KVManager:
 
 def create_kv_cache(cache_implementation: str = "static", max_cache_len: Optional[int] = None,
                     max_batch_size: Optional[int] = 1, config=None, device="cuda:0", dtype=torch.bfloat16) -> KVManager:
-    """Factory with the reference's signature (cache_utils.py:6-39); only the static cache exists here."""
+    """Factory with the reference's signature (cache_utils.py:6-39).  For the dynamic cache ``max_cache_len`` is only
+    the initial capacity."""
     if isinstance(dtype, str):
         if not hasattr(torch, dtype):
             raise ValueError(f"Unsupported dtype string: {dtype}")
         dtype = getattr(torch, dtype)
-    if cache_implementation != "static":
-        raise ValueError(f"Unsupported cache_implementation: {cache_implementation} (this build keeps the static cache)")
+    if cache_implementation not in ("static", "dynamic"):
+        raise ValueError(f"Unsupported cache_implementation: {cache_implementation}")
     if config is None:
-        raise ValueError("config must be provided for static cache")
+        # the reference's dynamic cache learns its shapes from the first update; this one allocates up front
+        raise ValueError("config must be provided (layer count and head shapes of the cache)")
+    if cache_implementation == "dynamic":
+        return KVManager(DynamicKVCache(config.num_hidden_layers, config.num_key_value_heads, config.head_dim, device, dtype,
+                                        max_batch_size or 1, initial_len=max_cache_len or 1024))
     if max_cache_len is None:
         raise ValueError("max_cache_len must be provided for static cache")
     return KVManager(StaticKVCache(config.num_hidden_layers, config.num_key_value_heads, config.head_dim,

@@ -20,7 +20,7 @@ from typing import Any, Optional
 import torch
 
 from . import ops
-from .cache import KVManager
+from .cache import DynamicKVCache, KVManager
 from .lossy_diagnostics import record_lossy_diagnostics
 from .tree_verify import SampleStream, sample_token, verify_tree_device
 from .utils import DraftParams
@@ -34,8 +34,8 @@ class SubSpecSDGenerator:
         self.target_model, self.tokenizer, self.draft_model = target_model, tokenizer, draft_model
         self.draft_params = draft_params or DraftParams()
         self.draft_model.draft_params = self.draft_params
-        if cache_implementation != "static":
-            raise ValueError("only the static KV cache is implemented")
+        if cache_implementation not in ("static", "dynamic"):
+            raise ValueError(f"Unsupported cache_implementation: {cache_implementation}")
         self.cache_implementation = cache_implementation
         self.profiling = profiling
         self.generator_kwargs = generator_kwargs or {}
@@ -104,18 +104,19 @@ class SubSpecSDGenerator:
             raise NotImplementedError("stop_strings need a tokenizer; not available in this build")
         if max_new_tokens is not None:
             max_length = input_ids.shape[1] + int(max_new_tokens)
-        if max_length is None:
-            raise ValueError("max_length is not set. Only 'dynamic' kv-cache is supported when max_length is unspecified.")
         past_key_values = model_kwargs.get("past_key_values")
+        if max_length is None and (self.cache_implementation == "static" or
+                                   not isinstance(getattr(past_key_values, "cache", None), DynamicKVCache)):
+            raise ValueError("max_length is not set. Only 'dynamic' kv-cache is supported when max_length is unspecified.")
         if past_key_values is None:
             raise ValueError("past_key_values is not provided")
         assert input_ids.shape[0] == 1, "Only support batch_size=1 for now."
         logits_processor = (self._get_logits_processor(temperature=temperature, top_p=top_p, top_k=top_k)
                             if do_sample else None)
-        return self._generate(input_ids.clone(), int(max_length), past_key_values, stream_callback,
+        return self._generate(input_ids.clone(), None if max_length is None else int(max_length), past_key_values, stream_callback,
                               logits_processor=logits_processor, do_sample=bool(do_sample))
 
-    def _generate(self, input_ids, max_length: int, past_key_values: KVManager, stream_callback=None,
+    def _generate(self, input_ids, max_length: Optional[int], past_key_values: KVManager, stream_callback=None,
                   logits_processor=None, do_sample: bool = False):
         dev = self.target_model.device
         input_ids = input_ids.to(dev)
@@ -194,7 +195,8 @@ class SubSpecSDGenerator:
         toks = sampled_tokens[0].tolist()
         for j, t in enumerate(toks):
             cur_len = base + j + 1
-            if cur_len >= max_length or (self.eos_token_id is not None and t == int(self.eos_token_id)):
+            if (max_length is not None and cur_len >= max_length) or \
+                    (self.eos_token_id is not None and t == int(self.eos_token_id)):
                 prune = len(toks) - j - 1
                 if prune > 0:
                     input_ids = input_ids[:, :-prune]

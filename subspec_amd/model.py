@@ -120,11 +120,19 @@ class Decoder:
         self.device, self.dtype = embed.device, embed.dtype
         self._native = None
         self.use_native_layers = True            # False: run every module through its own torch / library call
-        inv = 1.0 / (cfg.rope_theta ** (torch.arange(0, cfg.head_dim, 2, device=self.device, dtype=torch.float32) / cfg.head_dim))
-        pos = torch.arange(kv.cache.max_cache_len + 8, device=self.device, dtype=torch.float32)
-        freqs = torch.outer(pos, inv)
+        self._inv_freq = 1.0 / (cfg.rope_theta ** (torch.arange(0, cfg.head_dim, 2, device=self.device, dtype=torch.float32)
+                                                   / cfg.head_dim))
+        self._rope_len = 0
+        self._rope_tables(kv.cache.max_cache_len + 8)
+
+    def _rope_tables(self, n: int) -> None:
+        """cos / sin of positions 0 .. n - 1 (rebuilt when a growing cache passes their length)."""
+        if n <= self._rope_len:
+            return
+        freqs = torch.outer(torch.arange(n, device=self.device, dtype=torch.float32), self._inv_freq)
         self.cos = torch.cat([freqs, freqs], -1).cos()
         self.sin = torch.cat([freqs, freqs], -1).sin()
+        self._rope_len = n
 
     # ------------------------------------------------------------------ native layers
     @property
@@ -212,6 +220,8 @@ class Decoder:
     def prefill(self, token_ids: torch.Tensor, start: int) -> torch.Tensor:
         """Causal forward of ``token_ids`` [n] at cache rows start..start+n-1; returns the last logits [1, V]."""
         n = token_ids.numel()
+        self.kv.cache.ensure(start + n)
+        self._rope_tables(start + n)
         positions = torch.arange(start, start + n, device=self.device)
         cfg = self.cfg
         rep = cfg.num_attention_heads // cfg.num_key_value_heads
@@ -233,6 +243,8 @@ class Decoder:
         slots.  Returns logits [n, V]."""
         n = token_ids.numel()
         slots = first_slot + n if n_tree_slots is None else n_tree_slots
+        self.kv.cache.ensure(prefix_len + max(slots, first_slot + n))
+        self._rope_tables(prefix_len + n + 8)
         positions = depths.to(self.device) + prefix_len
         rows = torch.arange(prefix_len + first_slot, prefix_len + first_slot + n, device=self.device)
         cfg = self.cfg

@@ -134,7 +134,7 @@ def test_generator_argument_errors():
     with pytest.raises(ValueError):                                             # the warper rejects T <= 0
         gen.generate(ids, max_new_tokens=4, do_sample=True, temperature=0.0, past_key_values=kv)
     with pytest.raises(ValueError):
-        create_kv_cache("dynamic", max_cache_len=8, config=CFG)
+        create_kv_cache("paged", max_cache_len=8, config=CFG)
     bad = SubSpecSDGenerator(target, None, SubSpecSDDraftModel(draft), DraftParams(max_depth=2, topk_len=2),
                              generator_kwargs=dict(verify_method="bogus"))
     with pytest.raises(ValueError):
@@ -192,3 +192,46 @@ def test_one_sampling_cycle_against_the_oracle():
     assert accept == exp_a
     # every emitted token is the draw of its context (exact verifier)
     assert out["tokens"][0, :emitted].tolist() == [int(drawn[c]) for c in exp_c]
+
+
+def test_dynamic_cache_grows_and_matches_the_static_cache():
+    """``create_kv_cache("dynamic")``: no fixed length, storage grows during generation, reorder truncates
+    (TreeDynamicCache, cache_utils.py:62-110).  Same tokens as with the static cache; generation without a
+    length limit stops at EOS."""
+    from subspec_amd.cache import DynamicKVCache
+
+    def run(kind, **gen_kwargs):
+        kv = create_kv_cache(kind, max_cache_len=256 if kind == "static" else 64, config=CFG, device=DEV, dtype=torch.bfloat16)
+        target, draft, _ = build_models(CFG, kv, seed=3, device=DEV)
+        gen = SubSpecSDGenerator(target, None, SubSpecSDDraftModel(draft), DraftParams(temperature=0.2, max_depth=4, topk_len=4),
+                                 cache_implementation=kind, eos_token_id=gen_kwargs.pop("eos", None))
+        prompt = torch.randint(0, CFG.vocab_size, (1, 40), generator=torch.Generator().manual_seed(4)).to(DEV)
+        out = gen.generate(prompt, do_sample=False, past_key_values=kv, **gen_kwargs)
+        return out[0, 40:].cpu(), kv
+
+    static_tokens, _ = run("static", max_new_tokens=60)
+    dyn_tokens, kv = run("dynamic", max_new_tokens=60)
+    assert isinstance(kv.cache, DynamicKVCache) and kv.cache.max_cache_len >= 128       # grew from 64 rows
+    assert torch.equal(static_tokens, dyn_tokens)
+    assert kv.get_seq_length() == 40 + 60 - 1
+    # no length limit: allowed with the dynamic cache only, ends at EOS (here: a token the run above produced)
+    eos = int(static_tokens[17])
+    first = static_tokens.tolist().index(eos)
+    toks, _ = run("dynamic", eos=eos)
+    assert toks.tolist() == static_tokens[:first + 1].tolist()
+    with pytest.raises(ValueError):
+        run("static")
+
+    # reorder keeps [:offset] and the selected rows and drops the rest (oracle: compact_dynamic)
+    kv = create_kv_cache("dynamic", max_cache_len=64, config=CFG, device=DEV, dtype=torch.bfloat16)
+    kv.cache.ensure(100)
+    kv.cache.data.copy_(torch.randn(kv.cache.data.shape, generator=torch.Generator().manual_seed(1)).to(torch.bfloat16))
+    before = kv.cache.data.clone().cpu()
+    idx = torch.tensor([0, 3, 4, 9])
+    kv.cache.reorder_cache_with_offset(idx, new_chunk_len=16, offset=70, dim=2)
+    assert kv.cache.get_seq_length() == 74
+    assert torch.equal(kv.cache.data[..., :74, :].cpu(), okv.compact_dynamic(before, idx.tolist(), 70))
+    kv.cache.crop(50)
+    assert kv.cache.get_seq_length() == 50
+    kv.cache.crop(-5, end=50)
+    assert kv.cache.get_seq_length() == 45

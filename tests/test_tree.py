@@ -82,3 +82,35 @@ def test_tree_errors():
         t.get_node(5)
     with pytest.raises(AssertionError):
         t.add_nodes(torch.zeros(2, 1, 1, dtype=torch.long), torch.zeros(2, 1, 1), torch.zeros(2, 1, 1, dtype=torch.long))
+
+
+def test_dynamic_cache_bookkeeping_on_the_host():
+    import torch
+    from subspec_amd.cache import DynamicKVCache, create_kv_cache
+    from subspec_amd.model import DecoderConfig
+    cfg = DecoderConfig(num_hidden_layers=2, hidden_size=256, num_attention_heads=2, num_key_value_heads=1, head_dim=128,
+                        intermediate_size=512, vocab_size=64)
+    kv = create_kv_cache("dynamic", max_cache_len=None, config=cfg, device="cpu", dtype=torch.float32)
+    c = kv.cache
+    assert isinstance(c, DynamicKVCache) and c.max_cache_len == 1024 and c.get_seq_length() == 0
+    c.data[..., :10, :] = 1.0
+    c.ensure(1000)
+    assert c.max_cache_len == 1024
+    c.ensure(1025)
+    assert c.max_cache_len == 2048 and c.data.shape[-2] == 2048
+    assert float(c.data[..., :10, :].min()) == 1.0 and float(c.data[..., 10:, :].abs().max()) == 0.0   # contents carried over
+    c.ensure(10000)
+    assert c.max_cache_len == 10240
+    c.crop(7)
+    assert c.get_seq_length() == 7
+    kv.reset()
+    assert c.get_seq_length() == 0 and kv.get_seq_length() == 0
+    import pytest
+    with pytest.raises(ValueError):
+        create_kv_cache("paged", config=cfg)
+    with pytest.raises(ValueError):
+        create_kv_cache("dynamic", config=None)
+    static = create_kv_cache("static", max_cache_len=32, config=cfg, device="cpu", dtype=torch.float32)
+    static.cache.ensure(32)
+    with pytest.raises(ValueError):
+        static.cache.ensure(33)
