@@ -42,6 +42,10 @@ def parse():
     ap.add_argument("--checkpoint", default=None,
                     help="e2e workload: local HuggingFace checkpoint directory (config.json + *.safetensors, Qwen2 / "
                          "Llama naming) to use instead of random-init weights of the Qwen2.5-7B shape")
+    ap.add_argument("--agreeing-draft", action="store_true",
+                    help="e2e workload: give the target the draft's dequantized int4 weights, so that draft and target agree "
+                         "except for rounding: the high-acceptance end of the cycle (random weights alone accept about one "
+                         "token per cycle)")
     ap.add_argument("--keep-layers", type=int, default=14, help="e2e workload: target layers kept resident; the rest stream")
     ap.add_argument("--workload", default="verify-cycle", choices=["verify-cycle", "attention", "int4", "dense", "greedy", "sampling", "e2e"],
                     help="verify-cycle (default, BASELINE config 2) is the benchmark line; the others time one "
@@ -199,7 +203,8 @@ def bench_e2e(args):
     from subspec_amd.cache import create_kv_cache
     from subspec_amd.draft import SubSpecSDDraftModel
     from subspec_amd.generator import SubSpecSDGenerator
-    from subspec_amd.model import DecoderConfig, build_models, load_hf_checkpoint
+    from subspec_amd import quant
+    from subspec_amd.model import QUANTIZED, DecoderConfig, build_models, init_weights, load_hf_checkpoint
     from subspec_amd.utils import DraftParams
     from subspec_amd.wandb_logger import wandb_logger
     dev = "cuda:0"
@@ -209,6 +214,12 @@ def bench_e2e(args):
         cfg, weights = load_hf_checkpoint(args.checkpoint, device=dev)
     else:
         cfg = DecoderConfig()
+    if args.agreeing_draft:
+        weights = weights or init_weights(cfg, 0, dev)
+        for w in weights["layers"]:
+            for name in QUANTIZED:
+                t = w[name + ".weight"]
+                w[name + ".weight"] = quant.dequantize(*quant.quantize_int4_g64(t)).to(t.dtype)
     kv = create_kv_cache("static", max_cache_len=2048 + args.new_tokens + 64 + 8, config=cfg, device=dev, dtype=torch.bfloat16)
     target, draft, _ = build_models(cfg, kv, seed=0, device=dev, first_streamed=min(args.keep_layers, cfg.num_hidden_layers),
                                     weights=weights)
@@ -226,7 +237,8 @@ def bench_e2e(args):
         log = dict(wandb_logger.log_data)
         line = {"metric": "accepted tokens/sec, end-to-end speculative cycle", "value": round(log["tput"], 2),
                 "unit": "tokens/s", "n_gpus": 1, "higher_is_better": True, "dtype": "bf16",
-                "data": "synthetic prompt, weights from " + args.checkpoint if args.checkpoint else "synthetic",
+                "data": ("synthetic prompt, weights from " + args.checkpoint if args.checkpoint else "synthetic")
+                        + (", target = the draft's dequantized int4 weights" if args.agreeing_draft else ""),
                 "config": {"workload": f"BASELINE config 5: {'checkpoint' if args.checkpoint else 'Qwen2.5-7B shape'}, "
                                        + ("all layers resident" if args.keep_layers >= cfg.num_hidden_layers else
                                           f"layers {args.keep_layers}-{cfg.num_hidden_layers - 1} streamed")

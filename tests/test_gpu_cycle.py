@@ -235,3 +235,33 @@ def test_dynamic_cache_grows_and_matches_the_static_cache():
     assert kv.cache.get_seq_length() == 50
     kv.cache.crop(-5, end=50)
     assert kv.cache.get_seq_length() == 45
+
+
+def test_agreeing_draft_accepts_deep_paths():
+    """With the target running the draft's own dequantized weights the two agree except for rounding: most cycles
+    accept the whole depth-4 chain plus the bonus token, the KV rows of long accepted paths are compacted, and the
+    output is still the target's greedy continuation (checked against a run without speculation help: depth 1)."""
+    from subspec_amd import quant
+    from subspec_amd.model import QUANTIZED, init_weights
+    weights = init_weights(CFG, 9, DEV)
+    for w in weights["layers"]:
+        for name in QUANTIZED:
+            t = w[name + ".weight"]
+            w[name + ".weight"] = quant.dequantize(*quant.quantize_int4_g64(t)).to(t.dtype)
+
+    def run(depth):
+        kv = create_kv_cache("static", max_cache_len=256, config=CFG, device=DEV, dtype=torch.bfloat16)
+        target, draft, _ = build_models(CFG, kv, device=DEV, weights=weights)
+        gen = SubSpecSDGenerator(target, None, SubSpecSDDraftModel(draft), DraftParams(temperature=0.2, max_depth=depth, topk_len=4))
+        prompt = torch.randint(0, CFG.vocab_size, (1, 32), generator=torch.Generator().manual_seed(4)).to(DEV)
+        wandb_logger.clear_log_data()
+        out = gen.generate(prompt, max_new_tokens=48, do_sample=False, past_key_values=kv)
+        return out[0, 32:].cpu(), dict(wandb_logger.log_data), kv
+
+    deep, log, kv = run(4)
+    assert log["avg_sampled"] >= 3.0, log["avg_sampled"]            # at most 5 per cycle
+    assert kv.get_seq_length() == 32 + 48 - 1
+    shallow, log1, _ = run(1)
+    assert log1["avg_sampled"] <= 2.0
+    agree = (deep == shallow).float().mean().item()
+    assert agree >= 0.9, agree                                      # bf16 near-ties may flip a token late in the sequence
