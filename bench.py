@@ -46,6 +46,12 @@ def parse():
                     help="e2e workload: give the target the draft's dequantized int4 weights, so that draft and target agree "
                          "except for rounding: the high-acceptance end of the cycle (random weights alone accept about one "
                          "token per cycle)")
+    ap.add_argument("--generator", default="v1", choices=["v1", "v2"],
+                    help="e2e workload: v1 = speculate / verify cycle; v2 = the draft keeps extending the tree while the "
+                         "target waits for streamed layers (post-speculation)")
+    ap.add_argument("--postspec-steps", type=int, default=None,
+                    help="e2e workload, generator v2: force this many post-speculation steps per target forward "
+                         "(default: as many as fit into the waits for streamed layers)")
     ap.add_argument("--keep-layers", type=int, default=14, help="e2e workload: target layers kept resident; the rest stream")
     ap.add_argument("--workload", default="verify-cycle", choices=["verify-cycle", "attention", "int4", "dense", "greedy", "sampling", "e2e"],
                     help="verify-cycle (default, BASELINE config 2) is the benchmark line; the others time one "
@@ -203,6 +209,7 @@ def bench_e2e(args):
     from subspec_amd.cache import create_kv_cache
     from subspec_amd.draft import SubSpecSDDraftModel
     from subspec_amd.generator import SubSpecSDGenerator
+    from subspec_amd.generator_v2 import SubSpecSDGeneratorV2
     from subspec_amd import quant
     from subspec_amd.model import QUANTIZED, DecoderConfig, build_models, init_weights, load_hf_checkpoint
     from subspec_amd.utils import DraftParams
@@ -220,15 +227,20 @@ def bench_e2e(args):
             for name in QUANTIZED:
                 t = w[name + ".weight"]
                 w[name + ".weight"] = quant.dequantize(*quant.quantize_int4_g64(t)).to(t.dtype)
-    kv = create_kv_cache("static", max_cache_len=2048 + args.new_tokens + 64 + 8, config=cfg, device=dev, dtype=torch.bfloat16)
+    kv = create_kv_cache("static", max_cache_len=2048 + args.new_tokens + 128 + 8, config=cfg, device=dev, dtype=torch.bfloat16)
     target, draft, _ = build_models(cfg, kv, seed=0, device=dev, first_streamed=min(args.keep_layers, cfg.num_hidden_layers),
                                     weights=weights)
     print(f"# models built in {time.perf_counter() - t0:.1f} s", file=sys.stderr, flush=True)
     prompt = torch.randint(0, cfg.vocab_size, (1, 2048), generator=torch.Generator().manual_seed(0)).to(dev)
     for method, vk in (("exact", None), ("lossy", dict(threshold=0.3, window_size=6, threshold_method="entropy"))):
-        gen = SubSpecSDGenerator(target, None, SubSpecSDDraftModel(draft),
-                                 DraftParams(temperature=0.2, max_depth=8, topk_len=8, max_verify_tokens=64),
-                                 generator_kwargs=dict(verify_method=method, verify_kwargs=vk))
+        # the post-speculating driver decodes the tree in one window of at most 64 nodes: depth 7 x k 8 + root = 57
+        v2 = args.generator == "v2"
+        depth = 7 if v2 else 8
+        gen = (SubSpecSDGeneratorV2 if v2 else SubSpecSDGenerator)(
+            target, None, SubSpecSDDraftModel(draft),
+            DraftParams(temperature=0.2, max_depth=depth, topk_len=8, max_verify_tokens=64),
+            generator_kwargs=dict(verify_method=method, verify_kwargs=vk,
+                                  **(dict(postspec_steps=args.postspec_steps) if v2 else {})))
         kv.reset()
         wandb_logger.clear_log_data()
         if target.streamer is not None:
@@ -242,9 +254,11 @@ def bench_e2e(args):
                 "config": {"workload": f"BASELINE config 5: {'checkpoint' if args.checkpoint else 'Qwen2.5-7B shape'}, "
                                        + ("all layers resident" if args.keep_layers >= cfg.num_hidden_layers else
                                           f"layers {args.keep_layers}-{cfg.num_hidden_layers - 1} streamed")
-                                       + f", int4 draft, depth 8, k 8, "
-                                       f"<=64 nodes, prompt 2048, {args.new_tokens} new tokens, verify {method}",
-                           "verify_method": method, "n_iter": log["n_iter"], "n_tokens": log["n_tokens"],
+                                       + f", int4 draft, depth {depth}, k 8, "
+                                       f"<=64 nodes, prompt 2048, {args.new_tokens} new tokens, verify {method}"
+                                       + (", post-speculating driver" if v2 else ""),
+                           "verify_method": method, "generator": args.generator,
+                           **({"post_verify_count": log["post_verify_count"], "speculate_count": log["speculate_count"]} if v2 else {}), "n_iter": log["n_iter"], "n_tokens": log["n_tokens"],
                            "tokens_per_cycle": round(log["avg_sampled"], 3),
                            "avg_draft_s": round(log.get("avg_draft_time", 0), 5),
                            "avg_target_s": round(log.get("avg_target_time", 0), 5),

@@ -20,6 +20,8 @@ from . import ops
 
 
 class StaticKVCache:
+    growable = False
+
     def __init__(self, n_layers: int, n_kv_heads: int, head_dim: int, max_cache_len: int, device, dtype,
                  max_batch_size: int = 1):
         self.max_cache_len = int(max_cache_len)
@@ -66,6 +68,8 @@ class DynamicKVCache(StaticKVCache):
     capacity doubles whenever a forward needs more rows (one reallocation and copy, amortised), ``crop`` and
     ``reorder_cache_with_offset`` set the number of rows seen, as the reference's slicing / index_select do;
     the kernels are the static cache's.  ``max_cache_len`` is the current capacity."""
+
+    growable = True
 
     def __init__(self, n_layers: int, n_kv_heads: int, head_dim: int, device, dtype, max_batch_size: int = 1,
                  initial_len: int = 1024):

@@ -9,7 +9,8 @@ classic_sd.py:10-118, base.py:268-305).  Differences in mechanism:
 * softmax(logits / T) stays a torch call, the cumulative-probability product and the global top-k
   over (leaves x vocab) are one fused HIP launch (no ``[1, k, V]`` product buffer);
 * the incremental ``[1, 1, k, max_cache_len]`` boolean mask of ``TreeMaskCache`` (base.py:49-117) is
-  replaced by one 64-bit ancestor bitset per node, updated on the device with a gather and an OR;
+  replaced by an ancestor bitset per node (two 64-bit words: up to 128 tree slots, enough for a 64-node
+  tree extended by post-speculation), updated on the device with a gather and an OR;
 * nothing is copied to the host until the tree is assembled (one small copy, as in
   ``Tree.add_nodes``).
 """
@@ -63,13 +64,14 @@ class SubSpecSDDraftModel:
                                          torch.ones(1, dtype=torch.int64, device=dev), self.prefix_len)
         self.tree = Tree(input_ids[0, -1], self.model.dtype)
         self.levels = []
-        self.level_bits = torch.ones(1, dtype=torch.int64, device=dev)             # root: slot 0
+        self.level_state = {}                                                      # depth -> what speculate_once needs
+        self.level_bits = torch.tensor([[1, 0]], dtype=torch.int64, device=dev)    # root: slot 0 (words 0 and 1)
         self.next_slot = 1
         self.depth = 0
         self._expand(self._probs(logits).unsqueeze(0), torch.ones((1, 1), device=dev, dtype=logits.dtype))
         for _ in range(p.max_depth - 1):
             self.speculate_once()
-        return self.update_tree()
+        return self.update_tree(cap=True)
 
     def _expand(self, sampled_probs: torch.Tensor, parent_probs: torch.Tensor) -> None:
         k = self.draft_params.topk_len
@@ -77,49 +79,90 @@ class SubSpecSDDraftModel:
         self.levels.append((token_ids, child_probs, parent_indices))
         self.token_ids, self.parent_probs = token_ids, child_probs
         slots = torch.arange(self.next_slot, self.next_slot + token_ids.shape[1], device=token_ids.device)
-        usable = slots < 64                                                        # one mask word per node
-        self_bit = torch.where(usable, torch.ones_like(slots) << slots.clamp(max=62), torch.zeros_like(slots))
-        self_bit = torch.where(slots == 63, torch.full_like(slots, -(1 << 63)), self_bit)
-        self.level_bits = self.level_bits[parent_indices[0]] | self_bit
+        # own bit of slot s: word s // 64, bit s % 64 (bit 63 is the sign bit of the signed word)
+        low = slots % 64
+        bit = torch.where(low == 63, torch.full_like(slots, -(1 << 63)), torch.ones_like(slots) << low.clamp(max=62))
+        own = torch.zeros((slots.numel(), 2), dtype=torch.int64, device=slots.device)
+        own[:, 0] = torch.where(slots < 64, bit, torch.zeros_like(bit))
+        own[:, 1] = torch.where((slots >= 64) & (slots < 128), bit, torch.zeros_like(bit))
+        self.level_bits = self.level_bits[parent_indices[0]] | own
         self.first_slot = self.next_slot
         self.next_slot += token_ids.shape[1]
         self.depth += 1
+        self.level_state[self.depth] = (self.first_slot, self.token_ids, self.parent_probs, self.level_bits)
 
     @torch.no_grad()
     def speculate_once(self, **kwargs) -> None:
         """One more level: draft forward on the newest k nodes, then top-k over (k x vocab)."""
         dev = self.model.device
         n = self.token_ids.shape[1]
-        if self.first_slot + n > 64:
-            raise ValueError("draft tree exceeds 64 slots (max_depth * topk_len must stay below 64 for fed levels)")
+        total = self.first_slot + n
+        if total > 128:
+            raise ValueError("draft tree exceeds the 128 tree slots of the attention mask")
         depths = torch.full((n,), self.depth, dtype=torch.long, device=dev)
-        logits = self.model.tree_forward(self.token_ids[0], depths, self.level_bits, self.prefix_len,
+        bits = self.level_bits if total > 64 else self.level_bits[:, 0].contiguous()
+        logits = self.model.tree_forward(self.token_ids[0], depths, bits, self.prefix_len,
                                          first_slot=self.first_slot)
         self._expand(self._probs(logits).unsqueeze(0), self.parent_probs)
 
-    def update_tree(self) -> Tree:
+    def update_tree(self, cap: bool = False) -> Tree:
         tok = torch.stack([lv[0][0] for lv in self.levels]).unsqueeze(0)
         prob = torch.stack([lv[1][0] for lv in self.levels]).unsqueeze(0)
         par = torch.stack([lv[2][0] for lv in self.levels]).unsqueeze(0)
         packed = torch.stack([tok.double(), prob.double(), par.double()]).cpu()     # one device-to-host copy
         self.tree.add_nodes(packed[0].long(), packed[1].to(self.model.dtype), packed[2].long())
         self.levels = []
-        cap = self.draft_params.max_verify_tokens
-        if cap is not None and self.tree.size() > cap:
-            self.tree.truncate(cap)
+        limit = self.draft_params.max_verify_tokens if cap else None
+        if limit is not None and self.tree.size() > limit:
+            self.tree.truncate(limit)
         return self.tree
 
     # ------------------------------------------------------------------ post-speculation hooks
-    def init_postspec(self) -> None:
-        self.levels = []
+    def init_postspec(self, keep_pending: bool = False) -> None:
+        """Start counting post-speculation steps; levels not yet attached to the tree are dropped unless kept."""
+        if not keep_pending:
+            self.levels = []
         self.postspec_count = 0
 
     @torch.no_grad()
+    def prefeed(self) -> bool:
+        """Runs the deepest level of the tree through the draft now and keeps the level it yields pending.  Done before
+        the target decodes that level: a post-speculation step that fed it later would overwrite, in the layers the
+        target has already passed, the target's K / V rows of nodes that may be accepted."""
+        if not self._room_for_level():
+            return False
+        self.speculate_once()
+        return True
+
+    def _room_for_level(self) -> bool:
+        """One more level needs tree slots (the masks describe 128) and, once it is decoded, cache rows."""
+        n = self.token_ids.shape[1]
+        if self.first_slot + n > 128 or self.next_slot + n > 128:
+            return False
+        cache = self.model.kv.cache
+        return cache.growable or self.prefix_len + self.next_slot + n <= cache.max_cache_len
+
+    @torch.no_grad()
     def postspec(self) -> None:
+        """One more level while the target is busy (subspec_sd.py:133-140); also a no-op once the 128 tree slots
+        the masks can describe, or the rows of a fixed-length cache, are used up."""
         if not self.had_first_speculate or self.postspec_count > (self.draft_params.max_depth - 1):
+            return
+        if not self._room_for_level():
             return
         self.speculate_once()
         self.postspec_count += 1
+
+    def resync_to_depth(self, depth: int) -> None:
+        """After the tree was pruned to ``depth``: continue from that level (its tokens, cumulative probabilities,
+        masks and slots) instead of from the deeper level that no longer exists, and make exactly that level the
+        tree's expandable frontier."""
+        first, tokens, probs, bits = self.level_state[int(depth)]
+        self.token_ids, self.parent_probs, self.level_bits = tokens, probs, bits
+        self.first_slot, self.next_slot, self.depth = first, first + tokens.shape[1], int(depth)
+        self.level_state = {d: v for d, v in self.level_state.items() if d <= depth}
+        self.levels = []
+        self.tree.available_leaves = list(range(first, first + tokens.shape[1]))
 
     def update_tree_after_post(self) -> Tree:
         return self.update_tree() if self.levels else self.tree

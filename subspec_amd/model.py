@@ -217,8 +217,9 @@ class Decoder:
         return F.linear(rms_norm(x, self.norm, self.cfg.rms_norm_eps), self.lm_head)
 
     # ------------------------------------------------------------------ forwards
-    def prefill(self, token_ids: torch.Tensor, start: int) -> torch.Tensor:
-        """Causal forward of ``token_ids`` [n] at cache rows start..start+n-1; returns the last logits [1, V]."""
+    def prefill(self, token_ids: torch.Tensor, start: int, all_logits: bool = False) -> torch.Tensor:
+        """Causal forward of ``token_ids`` [n] at cache rows start..start+n-1; returns the last logits [1, V]
+        (``all_logits``: the logits of every position [n, V], e.g. to score a sequence by teacher forcing)."""
         n = token_ids.numel()
         self.kv.cache.ensure(start + n)
         self._rope_tables(start + n)
@@ -234,7 +235,7 @@ class Decoder:
             return o.transpose(1, 2).reshape(n, cfg.q_size)
 
         x = self._run_layers(self.embed[token_ids], positions, positions, attn)
-        return self.logits(x[-1:])
+        return self.logits(x if all_logits else x[-1:])
 
     def tree_forward(self, token_ids: torch.Tensor, depths: torch.Tensor, anc_bits: torch.Tensor, prefix_len: int,
                      first_slot: int = 0, n_tree_slots: Optional[int] = None) -> torch.Tensor:

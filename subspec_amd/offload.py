@@ -17,7 +17,7 @@ explicit schedule:
 """
 from __future__ import annotations
 
-from typing import Callable, Dict, List, Sequence, Tuple
+from typing import Optional, Callable, Dict, List, Sequence, Tuple
 
 import torch
 
@@ -76,6 +76,10 @@ class LayerStreamer:
         self._visit = 0                 # visits computed so far (visit v = layer v % n, slab v % n_slabs)
         self._issued = 0                # visits whose copy has been issued
         self.bytes_streamed = 0
+        # Called as idle_hook(copy_done_event) right before the compute stream has to wait for a slab whose copy is
+        # still running: work queued by the hook runs in the gap (post-speculation of the draft, as the reference's
+        # wait hook does, prefetch_offloader_postspec.py:193-232).
+        self.idle_hook: Optional[Callable[[torch.cuda.Event], None]] = None
 
     def _issue_until(self, visit: int) -> None:
         """Issue the copies of all visits up to and including ``visit``."""
@@ -102,6 +106,8 @@ class LayerStreamer:
             v = self._visit
             slot = v % self.n_slabs
             self._issue_until(v + self.n_slabs - 1)
+            if self.idle_hook is not None and not self.copied[slot].query():
+                self.idle_hook(self.copied[slot])
             compute.wait_event(self.copied[slot])
             fn(i, self.slab_views[slot])
             self.released[slot].record(compute)

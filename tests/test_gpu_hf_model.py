@@ -121,14 +121,17 @@ def test_target_and_draft_match_huggingface(n, P):
     _close(draft.tree_forward(tree.to(DEV), dep, anc, P), ref_draft, "draft tree")
 
 
+@pytest.mark.parametrize("driver", ["v1", "v2"])
 @pytest.mark.parametrize("method,kwargs", [("exact", None), ("lossy", dict(threshold=0.0, window_size=3, threshold_method="entropy"))])
-def test_speculative_generation_is_huggingface_greedy_decoding(method, kwargs):
+def test_speculative_generation_is_huggingface_greedy_decoding(method, kwargs, driver):
     """Exact verification (and the lossy verifier with a gate that blocks everything) must emit exactly what greedy
-    decoding of the target emits.  Checked by teacher forcing: HuggingFace scores the produced sequence in one
+    decoding of the target emits, with the plain cycle driver and with the post-speculating one (two forced
+    post-speculation steps per target forward).  Checked by teacher forcing: HuggingFace scores the produced sequence in one
     fp32 forward, and every produced token must be its argmax there -- or, where two logits are closer than bf16
     can tell apart, within that margin of the maximum."""
     from subspec_amd.draft import SubSpecSDDraftModel
     from subspec_amd.generator import SubSpecSDGenerator
+    from subspec_amd.generator_v2 import SubSpecSDGeneratorV2
     from subspec_amd.utils import DraftParams
     model = _hf(5)
     g = torch.Generator().manual_seed(5)
@@ -136,8 +139,9 @@ def test_speculative_generation_is_huggingface_greedy_decoding(method, kwargs):
     kv = create_kv_cache("static", max_cache_len=256, config=CFG, device=DEV, dtype=torch.bfloat16)
     weights = weights_from_tensors(CFG, model.state_dict(), device=DEV, dtype=torch.bfloat16)
     target, draft, _ = build_models(CFG, kv, device=DEV, weights=weights)
-    gen = SubSpecSDGenerator(target, None, SubSpecSDDraftModel(draft), DraftParams(temperature=0.2, max_depth=4, topk_len=4),
-                             generator_kwargs=dict(verify_method=method, verify_kwargs=kwargs))
+    cls, extra = (SubSpecSDGenerator, {}) if driver == "v1" else (SubSpecSDGeneratorV2, dict(postspec_steps=2))
+    gen = cls(target, None, SubSpecSDDraftModel(draft), DraftParams(temperature=0.2, max_depth=4, topk_len=4),
+              generator_kwargs=dict(verify_method=method, verify_kwargs=kwargs, **extra))
     out = gen.generate(prompt.to(DEV), max_new_tokens=40, do_sample=False, past_key_values=kv).cpu()
     assert out.shape[1] == 60
     with torch.no_grad():
