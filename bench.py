@@ -52,6 +52,11 @@ def parse():
     ap.add_argument("--postspec-steps", type=int, default=None,
                     help="e2e workload, generator v2: force this many post-speculation steps per target forward "
                          "(default: as many as fit into the waits for streamed layers)")
+    ap.add_argument("--tree-depth", type=int, default=None, help="e2e workload: draft tree depth (default 8; 7 for generator v2)")
+    ap.add_argument("--tree-k", type=int, default=8, help="e2e workload: children kept per level")
+    ap.add_argument("--max-verify-tokens", type=int, default=64,
+                    help="e2e workload: cap on the nodes verified per cycle (0: the whole tree); the reference's offloading "
+                         "configurations use depth 48, k 6 and no cap: --tree-depth 48 --tree-k 6 --max-verify-tokens 0")
     ap.add_argument("--keep-layers", type=int, default=14, help="e2e workload: target layers kept resident; the rest stream")
     ap.add_argument("--workload", default="verify-cycle", choices=["verify-cycle", "attention", "int4", "dense", "greedy", "sampling", "e2e"],
                     help="verify-cycle (default, BASELINE config 2) is the benchmark line; the others time one "
@@ -227,18 +232,18 @@ def bench_e2e(args):
             for name in QUANTIZED:
                 t = w[name + ".weight"]
                 w[name + ".weight"] = quant.dequantize(*quant.quantize_int4_g64(t)).to(t.dtype)
-    kv = create_kv_cache("static", max_cache_len=2048 + args.new_tokens + 128 + 8, config=cfg, device=dev, dtype=torch.bfloat16)
+    kv = create_kv_cache("static", max_cache_len=2048 + args.new_tokens + 512 + 8, config=cfg, device=dev, dtype=torch.bfloat16)
     target, draft, _ = build_models(cfg, kv, seed=0, device=dev, first_streamed=min(args.keep_layers, cfg.num_hidden_layers),
                                     weights=weights)
     print(f"# models built in {time.perf_counter() - t0:.1f} s", file=sys.stderr, flush=True)
     prompt = torch.randint(0, cfg.vocab_size, (1, 2048), generator=torch.Generator().manual_seed(0)).to(dev)
     for method, vk in (("exact", None), ("lossy", dict(threshold=0.3, window_size=6, threshold_method="entropy"))):
-        # the post-speculating driver decodes the tree in one window of at most 64 nodes: depth 7 x k 8 + root = 57
         v2 = args.generator == "v2"
-        depth = 7 if v2 else 8
+        depth = args.tree_depth or (7 if v2 else 8)
+        cap = args.max_verify_tokens or None
         gen = (SubSpecSDGeneratorV2 if v2 else SubSpecSDGenerator)(
             target, None, SubSpecSDDraftModel(draft),
-            DraftParams(temperature=0.2, max_depth=depth, topk_len=8, max_verify_tokens=64),
+            DraftParams(temperature=0.2, max_depth=depth, topk_len=args.tree_k, max_verify_tokens=cap),
             generator_kwargs=dict(verify_method=method, verify_kwargs=vk,
                                   **(dict(postspec_steps=args.postspec_steps) if v2 else {})))
         kv.reset()
@@ -254,8 +259,8 @@ def bench_e2e(args):
                 "config": {"workload": f"BASELINE config 5: {'checkpoint' if args.checkpoint else 'Qwen2.5-7B shape'}, "
                                        + ("all layers resident" if args.keep_layers >= cfg.num_hidden_layers else
                                           f"layers {args.keep_layers}-{cfg.num_hidden_layers - 1} streamed")
-                                       + f", int4 draft, depth {depth}, k 8, "
-                                       f"<=64 nodes, prompt 2048, {args.new_tokens} new tokens, verify {method}"
+                                       + f", int4 draft, depth {depth}, k {args.tree_k}, "
+                                       + (f"<={cap} nodes" if cap else f"{1 + depth * args.tree_k} nodes") + f", prompt 2048, {args.new_tokens} new tokens, verify {method}"
                                        + (", post-speculating driver" if v2 else ""),
                            "verify_method": method, "generator": args.generator,
                            **({"post_verify_count": log["post_verify_count"], "speculate_count": log["speculate_count"]} if v2 else {}), "n_iter": log["n_iter"], "n_tokens": log["n_tokens"],

@@ -47,7 +47,10 @@ extern "C" {
 #define SUBSPEC_ENTROPY_GUARD 0
 #define SUBSPEC_ENTROPY_ALWAYS 1
 
-#define SUBSPEC_MAX_TREE_NODES 256
+/* Largest tree: nodes the verifier walks, tree slots (and query rows) attention takes, rows one
+ * compaction moves.  The reference's offloading configurations draft 1 + 48 * 6 = 289 nodes
+ * (configs/exp_offloading/subspec_sd_qwen_7b.yaml:16-19). */
+#define SUBSPEC_MAX_TREE_NODES 512
 
 int subspec_abi_version(void);
 const char* subspec_last_error(void);
@@ -178,10 +181,10 @@ int subspec_topk_expand(const void* probs, const void* parent_probs, int dtype, 
 /* ------------------------------------------------------------------------------------------
  * Tree-masked GQA attention of the draft tree against the static KV cache:
  * out = softmax(q k^T * scale + mask) v, where query row i attends to cache rows [0, prefix_len) and
- * to tree slot prefix_len + j (j < n_tree_slots <= 128) iff bit j of row i's ancestor bitset is set (the
+ * to tree slot prefix_len + j (j < n_tree_slots <= SUBSPEC_MAX_TREE_NODES) iff bit j of row i's ancestor bitset is set (the
  * node in slot j is row i's node or one of its ancestors).  The verify forward has one query row per
  * slot; a draft step queries only the newest level (n_rows < n_tree_slots); a tree extended during
- * the target forward (post-speculation) may occupy up to 128 slots.
+ * the target forward (post-speculation) occupies more slots than the tree that is being verified.
  *
  * Replaces  HF sdpa_attention_forward under SDPBackend.MATH with the additive finfo.min mask and
  *           repeat_kv, as reached from _tree_decoding   specdecodes/models/generators/classic_sd.py:57-109
@@ -190,11 +193,12 @@ int subspec_topk_expand(const void* probs, const void* parent_probs, int dtype, 
  *           generators/classic_sd.py:33-55, utils/utils.py:4-6.  The FlashInfer form is
  *           flashinfer/attention_wrapper.py:116-151,288-316.
  *
- * q          device [batch, n_q_heads, n_rows, head_dim]      bf16 / fp16, head_dim = 128, n_rows <= 64
+ * q          device [batch, n_q_heads, n_rows, head_dim]      bf16 / fp16, head_dim = 128, n_rows <= SUBSPEC_MAX_TREE_NODES
+ *            (64 rows per launch; more rows are further launches on the same stream)
  * k_cache    device [batch, n_kv_heads, kv_seq_stride, head_dim]  (HF static-cache layout); the K/V of
  * v_cache    the tree nodes must already sit in rows prefix_len .. prefix_len + n_tree_slots - 1
  * out        device [batch, n_rows, n_q_heads, head_dim]       (= [batch, n_rows, hidden])
- * anc_bits   device uint64 [*, n_rows, words], words = 1 for n_tree_slots <= 64, else 2 (bit j of a row is bit
+ * anc_bits   device uint64 [*, n_rows, words], words = ceil(n_tree_slots / 64) (bit j of a row is bit
  *            j % 64 of word j / 64); batch element b uses rows from b * anc_batch_stride (0: shared tree)
  * workspace  partial results when the keys are split over workgroups (may be NULL if the size is 256)
  */
@@ -281,7 +285,8 @@ int subspec_temperature_warp(const void* logits, void* out, int dtype, int64_t n
  *           quantizers/hqq/hf/base.py:94-230) for BaseQuantizeConfig(nbits=4, group_size=64, axis=1)
  *           specdecodes/helpers/recipes/subspec/hqq_4bit_postspec.py:17-58.
  *
- * x     device [M, K]  bf16 / fp16, 1 <= M <= 64 (tree width), K % 64 == 0
+ * x     device [M, K]  bf16 / fp16, K % 64 == 0; one pass over the weights serves 64 rows (a tree window),
+ *       more rows are further passes on the same stream
  * wq    device uint32, tiled codes: [N/16][K/64][4][16] entries of 8 bytes; entry (c, r) holds the 16
  *       codes of row 16*nt + r for k = 64*g + 16*c .. +15, word j the codes of k = .. + 8j .. +7
  *       with code(8j + 2i) in bits 4i..4i+3 and code(8j + 2i + 1) in bits 16+4i..16+4i+3
@@ -317,9 +322,9 @@ int subspec_int4_linear(const void* x, const uint32_t* wq, const uint32_t* sz, c
  * x           device [n_rows, hidden], updated in place (the residual stream)
  * positions   device int32 [n_rows]   rotary position of each row (prefix_len + node depth)
  * cache_rows  device int32 [n_rows]   cache row each row's K / V is written to (prefix_len + slot)
- * anc_bits    device uint64 [n_rows, words]  as for subspec_tree_attention (words = 2 above 64 tree slots)
+ * anc_bits    device uint64 [n_rows, words]  as for subspec_tree_attention (words = ceil(n_tree_slots / 64))
  * k_cache, v_cache  device [n_kv_heads, kv_seq_stride, head_dim] of THIS layer (batch 1)
- * Limits: n_rows <= 64, n_tree_slots <= 128, head_dim 128, hidden % 64 == 0 and <= 16384,
+ * Limits: n_rows <= 64, n_tree_slots <= SUBSPEC_MAX_TREE_NODES, head_dim 128, hidden % 64 == 0 and <= 16384,
  *         intermediate % 64 == 0.
  */
 typedef struct subspec_decoder_layer_dims {

@@ -17,7 +17,7 @@ F32, F16, BF16 = 0, 1, 2
 VERIFY_EXACT, VERIFY_LOSSY = 0, 1
 GATE_ENTROPY, GATE_PROB = 0, 1
 ENTROPY_GUARD, ENTROPY_ALWAYS = 0, 1
-MAX_TREE_NODES = 256
+MAX_TREE_NODES = 512
 
 _lib = None
 

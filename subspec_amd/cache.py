@@ -60,7 +60,7 @@ class StaticKVCache:
         if beam_idx.device != self.data.device:
             beam_idx = beam_idx.to(self.data.device)
         ops.kv_compact_(self.data, beam_idx.to(torch.int64).contiguous(), int(offset), count_dev=count_dev,
-                        max_count=None if count_dev is None else min(int(beam_idx.numel()), 256))
+                        max_count=None if count_dev is None else min(int(beam_idx.numel()), ops.L.MAX_TREE_NODES))
 
 
 class DynamicKVCache(StaticKVCache):

@@ -7,12 +7,12 @@
 // among the tree slots, only node i and its ancestors.
 //
 // Layout and mapping
-//   q        [B, Hq, n, D]            (n <= 64 query rows, D = 128)
+//   q        [B, Hq, n, D]            (D = 128; a launch takes 64 query rows, more rows are more launches)
 //   k, v     [B, Hkv, S, D]           static cache; rows [0, prefix) are the prompt, rows
-//                                     [prefix, prefix + slots) hold the tree nodes (slots <= 128)
+//                                     [prefix, prefix + slots) hold the tree nodes (slots <= 512)
 //   anc      [B or 1, n, words] u64   bit j of row i (word j / 64): query row i may attend to tree slot j
 //                                     (the node in slot j is the row's node or one of its ancestors);
-//                                     words = 1 for up to 64 tree slots, 2 for up to 128
+//                                     words = ceil(slots / 64), at most 8
 //   out      [B, n, Hq, D]
 // One workgroup (8 wavefronts) owns several query heads of one KV head and one chunk of the keys, so
 // a staged K/V tile feeds several heads' worth of matrix work.  With 33 to 64 query rows it owns
@@ -84,7 +84,8 @@ __device__ __forceinline__ uint2 lds_read_tr16(const uint16_t* p) {
 
 struct AttnParams {
   int64_t batch, hq, hkv, n_rows, n_slots, seq_stride, prefix, anc_batch_stride;
-  int mask_words;              // 64-bit words per ancestor bitset: 1 (<= 64 tree slots) or 2 (<= 128)
+  int mask_words;              // 64-bit words per ancestor bitset: ceil(n_slots / 64)
+  int row0, win_rows;          // this launch covers query rows row0 .. row0 + win_rows - 1 (win_rows <= 64) of n_rows
   int chunks;
   int64_t chunk_keys;          // multiple of kKeyBlock
   int pairs_per_kv;            // workgroups (groups of 4 or 8 query heads) per KV head
@@ -132,18 +133,17 @@ __global__ __launch_bounds__(kAttnThreads) __attribute__((amdgpu_waves_per_eu(2,
   int row[ROWT];
   bool row_ok[ROWT];
   uint4 qreg[ROWT][kAttnD / 32];
-  uint64_t bits[ROWT][2];                                  // [row tile][mask word]
+  const uint64_t* row_bits[ROWT];                          // the row's ancestor bitset (mask_words words)
 #pragma unroll
   for (int nt = 0; nt < ROWT; ++nt) {
-    row[nt] = (wave % WPH) * (16 * ROWT) + nt * 16 + lq;
-    row_ok[nt] = head_ok && row[nt] < n;
-    const uint16_t* qp = q + ((int64_t)bh * n + (row_ok[nt] ? row[nt] : 0)) * kAttnD;
+    row[nt] = (wave % WPH) * (16 * ROWT) + nt * 16 + lq;   // row inside this launch's window
+    row_ok[nt] = head_ok && row[nt] < ap.win_rows;
+    const int grow = ap.row0 + (row_ok[nt] ? row[nt] : 0);
+    const uint16_t* qp = q + ((int64_t)bh * n + grow) * kAttnD;
 #pragma unroll
     for (int ks = 0; ks < kAttnD / 32; ++ks)
       qreg[nt][ks] = row_ok[nt] ? *(const uint4*)(qp + ks * 32 + lg * 8) : make_uint4(0, 0, 0, 0);
-    const uint64_t* ap_bits = anc + ((int64_t)b * ap.anc_batch_stride + row[nt]) * ap.mask_words;
-    bits[nt][0] = row_ok[nt] ? ap_bits[0] : 0ull;
-    bits[nt][1] = (row_ok[nt] && ap.mask_words > 1) ? ap_bits[1] : 0ull;
+    row_bits[nt] = anc + ((int64_t)b * ap.anc_batch_stride + grow) * ap.mask_words;
   }
 
   v4f oacc[ROWT][kAttnD / 16];
@@ -195,6 +195,18 @@ __global__ __launch_bounds__(kAttnThreads) __attribute__((amdgpu_waves_per_eu(2,
     *(uint4*)(vsw_ + (skey + 32) * kVStride + sdc * 8) = v1;                                     \
   } while (0)
 
+  // mask words of the first block of this chunk that reaches into the tree (none does: the loads are harmless)
+  uint64_t bits[ROWT][2];
+  auto load_bits = [&](int w) {
+#pragma unroll
+    for (int nt = 0; nt < ROWT; ++nt) {
+      bits[nt][0] = (row_ok[nt] && w < ap.mask_words) ? row_bits[nt][w] : 0ull;
+      bits[nt][1] = (row_ok[nt] && w + 1 < ap.mask_words) ? row_bits[nt][w + 1] : 0ull;
+    }
+  };
+  int held_word = (int)(max(max(key0, ap.prefix / kKeyBlock * kKeyBlock) - ap.prefix, (int64_t)0) >> 6);
+  load_bits(held_word);
+
   SUBSPEC_ATTN_FETCH(key0);
   SUBSPEC_ATTN_STAGE(0);
   if (key0 + kKeyBlock < key1) SUBSPEC_ATTN_FETCH(key0 + kKeyBlock);
@@ -217,6 +229,13 @@ __global__ __launch_bounds__(kAttnThreads) __attribute__((amdgpu_waves_per_eu(2,
 #pragma unroll
     for (int nt = 0; nt < ROWT; ++nt) mloc[nt] = -INFINITY;
     const bool plain = kb + kKeyBlock <= ap.prefix;    // block lies entirely in the prefix: no mask (uniform)
+    // a 64-key block touches at most two consecutive words of the bitsets: word0 and word0 + 1.  They were
+    // fetched before the loop for the first masked block; trees beyond 128 slots fetch again as the blocks move on.
+    const int word0 = (int)(max(kb - ap.prefix, (int64_t)0) >> 6);
+    if (!plain && word0 != held_word) {                // uniform
+      held_word = word0;
+      load_bits(word0);
+    }
     v4f acc[4][ROWT];
 #pragma unroll
     for (int kt = 0; kt < 4; ++kt)
@@ -249,11 +268,12 @@ __global__ __launch_bounds__(kAttnThreads) __attribute__((amdgpu_waves_per_eu(2,
           const int64_t pos = kb + kt * 16 + lg * 4 + r;
           const bool in_range = pos < kv_len;
           const bool tree = pos >= ap.prefix;
-          const int rel = tree ? (int)(pos - ap.prefix) : 0;   // tree slot, < 64 * mask_words
+          const int rel = tree ? (int)(pos - ap.prefix) : 0;   // tree slot, < 64 * mask_words when in range
           const int sh = rel & 63;
+          const bool first_word = (rel >> 6) == word0;
 #pragma unroll
           for (int nt = 0; nt < ROWT; ++nt) {
-            const uint64_t word = rel < 64 ? bits[nt][0] : bits[nt][1];
+            const uint64_t word = first_word ? bits[nt][0] : bits[nt][1];
             const bool ok = in_range && (!tree || ((word >> sh) & 1ull));
             const float t = ok ? acc[kt][nt][r] : -INFINITY;
             s[nt][kt][r] = t;
@@ -324,7 +344,7 @@ __global__ __launch_bounds__(kAttnThreads) __attribute__((amdgpu_waves_per_eu(2,
     if (!row_ok[nt]) continue;
     if (ap.chunks == 1) {
       const float inv = l > 0.f ? 1.0f / l : 0.f;
-      uint16_t* op = out + (((int64_t)b * n + row[nt]) * ap.hq + qh) * kAttnD;
+      uint16_t* op = out + (((int64_t)b * n + ap.row0 + row[nt]) * ap.hq + qh) * kAttnD;
 #pragma unroll
       for (int mt = 0; mt < kAttnD / 16; ++mt) {
         const v4f o = oacc[nt][mt];
@@ -348,7 +368,7 @@ template <int DT>
 __global__ __launch_bounds__(256) void tree_attention_merge_kernel(
     const float* __restrict__ part_o, const float* __restrict__ part_ml, AttnParams ap, uint16_t* __restrict__ out) {
   const int row = blockIdx.x * (blockDim.x >> 5) + (threadIdx.x >> 5), bh = blockIdx.y;
-  if (row >= ap.n_rows) return;
+  if (row >= ap.win_rows) return;
   const int b = bh / (int)ap.hq, qh = bh % (int)ap.hq;
   const int d4 = threadIdx.x & 31;
   const int64_t slot0 = (int64_t)bh * ap.chunks * kAttnRows + row;     // chunk c: slot0 + c * kAttnRows
@@ -371,7 +391,7 @@ __global__ __launch_bounds__(256) void tree_attention_merge_kernel(
   uint2 packed;
   packed.x = pack2<DT>(num[0] * inv, num[1] * inv);
   packed.y = pack2<DT>(num[2] * inv, num[3] * inv);
-  *(uint2*)(out + (((int64_t)b * ap.n_rows + row) * ap.hq + qh) * kAttnD + d4 * 4) = packed;
+  *(uint2*)(out + (((int64_t)b * ap.n_rows + ap.row0 + row) * ap.hq + qh) * kAttnD + d4 * 4) = packed;
 }
 
 static int attn_chunks(int64_t batch, int64_t hq, int64_t kv_len) {
@@ -408,11 +428,11 @@ static int tree_attention_impl(const char* what, const void* q, const void* k_ca
   if (batch <= 0 || n_q_heads <= 0 || n_kv_heads <= 0 || n_q_heads % n_kv_heads != 0)
     SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "%s: batch=%lld heads=%lld/%lld", what, (long long)batch, (long long)n_q_heads,
                  (long long)n_kv_heads);
-  if (n_rows <= 0 || n_rows > kAttnRows)
-    SUBSPEC_FAIL(SUBSPEC_ERR_LIMIT, "%s: n_rows=%lld outside [1, %d]", what, (long long)n_rows, kAttnRows);
-  if (n_tree_slots < 1 || n_tree_slots > 128)
-    SUBSPEC_FAIL(SUBSPEC_ERR_LIMIT, "%s: n_tree_slots=%lld outside [1, 128] (at most two 64-bit mask words per row)", what,
-                 (long long)n_tree_slots);
+  if (n_rows <= 0 || n_rows > SUBSPEC_MAX_TREE_NODES)
+    SUBSPEC_FAIL(SUBSPEC_ERR_LIMIT, "%s: n_rows=%lld outside [1, %d]", what, (long long)n_rows, SUBSPEC_MAX_TREE_NODES);
+  if (n_tree_slots < 1 || n_tree_slots > SUBSPEC_MAX_TREE_NODES)
+    SUBSPEC_FAIL(SUBSPEC_ERR_LIMIT, "%s: n_tree_slots=%lld outside [1, %d] (at most %d 64-bit mask words per row)", what,
+                 (long long)n_tree_slots, SUBSPEC_MAX_TREE_NODES, SUBSPEC_MAX_TREE_NODES / 64);
   if (prefix_len < 0 || prefix_len + n_tree_slots > kv_seq_stride)
     SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "%s: prefix_len=%lld + n_tree_slots=%lld exceeds the cache length %lld", what,
                  (long long)prefix_len, (long long)n_tree_slots, (long long)kv_seq_stride);
@@ -423,7 +443,8 @@ static int tree_attention_impl(const char* what, const void* q, const void* k_ca
   ap.batch = batch; ap.hq = n_q_heads; ap.hkv = n_kv_heads; ap.n_rows = n_rows; ap.n_slots = n_tree_slots;
   ap.seq_stride = kv_seq_stride;
   ap.prefix = prefix_len; ap.anc_batch_stride = anc_batch_stride;
-  ap.mask_words = n_tree_slots > 64 ? 2 : 1;
+  ap.mask_words = (int)((n_tree_slots + 63) / 64);
+  ap.row0 = 0; ap.win_rows = (int)std::min<int64_t>(n_rows, kAttnRows);
   ap.page_table = nullptr; ap.page_shift = 0; ap.max_pages = 0; ap.page_stride = ap.tok_stride = ap.v_delta = 0;
   if (paged) {
     int shift = 0;
@@ -444,9 +465,6 @@ static int tree_attention_impl(const char* what, const void* q, const void* k_ca
   const int group = (int)(n_q_heads / n_kv_heads);
   // wavefront = ROWT 16-row tiles of one head; WPH wavefronts per head; 8 / WPH heads share a workgroup's K / V stages:
   // up to 16 rows (a draft level): 1 tile, 8 heads; up to 32 rows: 2 tiles, 8 heads; up to 64 rows: 2 tiles x 2 wavefronts, 4 heads
-  const int wph = n_rows <= 32 ? 1 : 2, rowt = n_rows <= 16 ? 1 : 2;
-  const int heads_per_wg = 8 / wph;
-  ap.pairs_per_kv = (group + heads_per_wg - 1) / heads_per_wg;
   ap.units = batch * n_kv_heads * ap.chunks;
   float* part_o = nullptr;
   float* part_ml = nullptr;
@@ -461,9 +479,16 @@ static int tree_attention_impl(const char* what, const void* q, const void* k_ca
     part_ml = (float*)((char*)workspace + align_up(slots * kAttnD * sizeof(float), 256));
   }
   hipStream_t st = (hipStream_t)stream;
+  // more than 64 query rows: one launch (pair) per window of 64, in stream order, sharing the partial buffers
+  for (int64_t row0 = 0; row0 < n_rows; row0 += kAttnRows) {
+  ap.row0 = (int)row0;
+  ap.win_rows = (int)std::min<int64_t>(n_rows - row0, kAttnRows);
+  const int wph = ap.win_rows <= 32 ? 1 : 2, rowt = ap.win_rows <= 16 ? 1 : 2;
+  const int heads_per_wg = 8 / wph;
+  ap.pairs_per_kv = (group + heads_per_wg - 1) / heads_per_wg;
   const dim3 grid((unsigned)((ap.units + kXcds - 1) / kXcds * kXcds * ap.pairs_per_kv));
-  const int64_t merge_rows = batch * n_q_heads * n_rows / 8 >= 1024 ? 8 : 2;   // rows per merge workgroup
-  const dim3 merge_grid((unsigned)((n_rows + merge_rows - 1) / merge_rows), (unsigned)(batch * n_q_heads));
+  const int64_t merge_rows = batch * n_q_heads * ap.win_rows / 8 >= 1024 ? 8 : 2;   // rows per merge workgroup
+  const dim3 merge_grid((unsigned)((ap.win_rows + merge_rows - 1) / merge_rows), (unsigned)(batch * n_q_heads));
 #define SUBSPEC_ATTN_KERNEL(DT, PAGED, ROWT, WPH)                                                                  \
   hipLaunchKernelGGL((tree_attention_kernel<DT, PAGED, ROWT, WPH>), grid, dim3(kAttnThreads), 0, st, (const uint16_t*)q, \
                      (const uint16_t*)k_cache, (const uint16_t*)v_cache, anc_bits, ap, (uint16_t*)out, part_o, part_ml)
@@ -483,6 +508,7 @@ static int tree_attention_impl(const char* what, const void* q, const void* k_ca
   else { if (paged) SUBSPEC_ATTN_LAUNCH(SUBSPEC_F16, true); else SUBSPEC_ATTN_LAUNCH(SUBSPEC_F16, false); }
 #undef SUBSPEC_ATTN_LAUNCH
 #undef SUBSPEC_ATTN_KERNEL
+  }
   SUBSPEC_CHECK_HIP(hipGetLastError());
   return SUBSPEC_OK;
 }

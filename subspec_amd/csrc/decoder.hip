@@ -199,7 +199,7 @@ static int check_dims(const subspec_decoder_layer_dims* s) {
     SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "decoder_layer: intermediate=%lld must be a multiple of 64", (long long)s->intermediate);
   if (s->n_q_heads <= 0 || s->n_kv_heads <= 0 || s->n_q_heads % s->n_kv_heads != 0)
     SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "decoder_layer: %lld query heads over %lld kv heads", (long long)s->n_q_heads, (long long)s->n_kv_heads);
-  if (s->n_tree_slots < 1 || s->n_tree_slots > 128 || s->prefix_len < 0 || s->prefix_len + s->n_tree_slots > s->kv_seq_stride)
+  if (s->n_tree_slots < 1 || s->n_tree_slots > SUBSPEC_MAX_TREE_NODES || s->prefix_len < 0 || s->prefix_len + s->n_tree_slots > s->kv_seq_stride)
     SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "decoder_layer: prefix_len=%lld, n_tree_slots=%lld do not fit a cache of %lld rows",
                  (long long)s->prefix_len, (long long)s->n_tree_slots, (long long)s->kv_seq_stride);
   if (!(s->rope_theta > 1.f) || !(s->rms_eps > 0.f)) SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "decoder_layer: rope_theta / rms_eps out of range");

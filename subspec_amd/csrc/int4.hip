@@ -407,13 +407,31 @@ using namespace subspec;
 extern "C" int subspec_int4_linear(const void* x, const uint32_t* wq, const uint32_t* sz, const void* bias, void* y,
                                    int dtype, int64_t M, int64_t N, int64_t K, int64_t group_size, void* workspace,
                                    size_t workspace_bytes, void* stream) {
-  return int4_linear_ex(x, wq, sz, bias, nullptr, y, dtype, M, N, K, group_size, workspace, workspace_bytes, stream);
+  if (M <= 64) return int4_linear_ex(x, wq, sz, bias, nullptr, y, dtype, M, N, K, group_size, workspace, workspace_bytes, stream);
+  // more than 64 rows (a whole large tree through the draft): 64 rows per pass over the weights, in stream order
+  if (!x || !y) SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "int4_linear: null pointer argument");
+  if (dtype != SUBSPEC_BF16 && dtype != SUBSPEC_F16)
+    SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "int4_linear: dtype %d not supported (bf16 / fp16 activations only)", dtype);
+  if (M > 65536) SUBSPEC_FAIL(SUBSPEC_ERR_LIMIT, "int4_linear: M=%lld too large", (long long)M);
+  for (int64_t m0 = 0; m0 < M; m0 += 64) {
+    const int64_t m = std::min<int64_t>(64, M - m0);
+    const int rc = int4_linear_ex((const uint16_t*)x + m0 * K, wq, sz, bias, nullptr, (uint16_t*)y + m0 * N, dtype, m, N, K,
+                                  group_size, workspace, workspace_bytes, stream);
+    if (rc) return rc;
+  }
+  return SUBSPEC_OK;
+}
+
+static size_t i4_workspace_one(int64_t M, int64_t N, int64_t K) {
+  const I4Plan pl = i4_plan(M, N, K);
+  return (pl.splits > 1 ? align_up((size_t)pl.splits * M * N * sizeof(float), 256) : 0) + 256;
 }
 
 extern "C" size_t subspec_int4_linear_workspace(int64_t M, int64_t N, int64_t K) {
   if (M <= 0 || N <= 0 || K <= 0) return 256;
-  const I4Plan pl = i4_plan(M, N, K);
-  return (pl.splits > 1 ? align_up((size_t)pl.splits * M * N * sizeof(float), 256) : 0) + 256;
+  if (M <= 64) return i4_workspace_one(M, N, K);
+  const size_t full = i4_workspace_one(64, N, K);
+  return M % 64 ? std::max(full, i4_workspace_one(M % 64, N, K)) : full;
 }
 
 int subspec::int4_linear_ex(const void* x, const uint32_t* wq, const uint32_t* sz, const void* bias, const void* residual,
@@ -426,7 +444,7 @@ int subspec::int4_linear_ex(const void* x, const uint32_t* wq, const uint32_t* s
   if (M <= 0 || N <= 0 || K <= 0 || N % 16 != 0 || K % kGroup != 0)
     SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "int4_linear: M=%lld N=%lld K=%lld; N must be a multiple of 16 and K of 64",
                  (long long)M, (long long)N, (long long)K);
-  if (M > 64) SUBSPEC_FAIL(SUBSPEC_ERR_LIMIT, "int4_linear: M=%lld exceeds the 64-row limit (tree width)", (long long)M);
+  if (M > 64) SUBSPEC_FAIL(SUBSPEC_ERR_LIMIT, "int4_linear: M=%lld exceeds the 64 rows of one pass", (long long)M);
   if (K > 65536) SUBSPEC_FAIL(SUBSPEC_ERR_LIMIT, "int4_linear: K=%lld too large", (long long)K);
   if (N * K / 2 >= ((int64_t)1 << 31))
     SUBSPEC_FAIL(SUBSPEC_ERR_LIMIT, "int4_linear: N*K/2=%lld bytes of codes exceed the 2 GiB descriptor range", (long long)(N * K / 2));

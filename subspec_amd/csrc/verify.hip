@@ -428,7 +428,7 @@ __device__ __forceinline__ T pick_slot(const T (&a)[kSlots], int slot) {
   return r;
 }
 
-// kSlots = nodes per lane (1, 2 or 4: trees of up to 64, 128, 256 nodes); LOSSY selects the
+// kSlots = nodes per lane (1, 2, 4 or 8: trees of up to 64, 128, 256, 512 nodes); LOSSY selects the
 // verifier.  Both are compile-time so that the common 64-node case stays a few hundred
 // instructions: a single wavefront pays for every instruction-cache miss it takes.
 template <int DT, int kSlots, bool LOSSY>
@@ -697,7 +697,7 @@ static int run_verify(const void* logits, int64_t batch, int64_t rows, int64_t v
     hipLaunchKernelGGL((row_sample_kernel<DT>), grid, dim3(kRowThreads), 0, st, logits, vp, p1, p3);
   }
   const int64_t widest = std::max<int64_t>(rows, tp.n_nodes);
-  const int slots = widest <= kWave ? 1 : widest <= 2 * kWave ? 2 : 4;
+  const int slots = widest <= kWave ? 1 : widest <= 2 * kWave ? 2 : widest <= 4 * kWave ? 4 : 8;
   const bool lossy = tp.method == SUBSPEC_VERIFY_LOSSY;
 #define SUBSPEC_LAUNCH_TAIL(SLOTS, LOSSY)                                                                        \
   hipLaunchKernelGGL((tree_accept_kernel<DT, SLOTS, LOSSY>), dim3((unsigned)batch), dim3(kTailThreads), 0, st,    \
@@ -705,7 +705,8 @@ static int run_verify(const void* logits, int64_t batch, int64_t rows, int64_t v
                      node_entropy, node_child_prob)
   if (slots == 1) { if (lossy) SUBSPEC_LAUNCH_TAIL(1, true); else SUBSPEC_LAUNCH_TAIL(1, false); }
   else if (slots == 2) { if (lossy) SUBSPEC_LAUNCH_TAIL(2, true); else SUBSPEC_LAUNCH_TAIL(2, false); }
-  else { if (lossy) SUBSPEC_LAUNCH_TAIL(4, true); else SUBSPEC_LAUNCH_TAIL(4, false); }
+  else if (slots == 4) { if (lossy) SUBSPEC_LAUNCH_TAIL(4, true); else SUBSPEC_LAUNCH_TAIL(4, false); }
+  else { if (lossy) SUBSPEC_LAUNCH_TAIL(8, true); else SUBSPEC_LAUNCH_TAIL(8, false); }
 #undef SUBSPEC_LAUNCH_TAIL
   SUBSPEC_CHECK_HIP(hipGetLastError());
   return SUBSPEC_OK;

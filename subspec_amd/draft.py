@@ -9,8 +9,9 @@ classic_sd.py:10-118, base.py:268-305).  Differences in mechanism:
 * softmax(logits / T) stays a torch call, the cumulative-probability product and the global top-k
   over (leaves x vocab) are one fused HIP launch (no ``[1, k, V]`` product buffer);
 * the incremental ``[1, 1, k, max_cache_len]`` boolean mask of ``TreeMaskCache`` (base.py:49-117) is
-  replaced by an ancestor bitset per node (two 64-bit words: up to 128 tree slots, enough for a 64-node
-  tree extended by post-speculation), updated on the device with a gather and an OR;
+  replaced by an ancestor bitset per node (eight 64-bit words: up to 512 tree slots, the 289 nodes of the
+  reference's depth-48 x 6 trees plus what post-speculation adds), updated on the device with a gather
+  and an OR; a forward is handed only the words its occupied slots need;
 * nothing is copied to the host until the tree is assembled (one small copy, as in
   ``Tree.add_nodes``).
 """
@@ -24,6 +25,9 @@ from . import ops
 from .cpu_tree import Tree
 from .model import Decoder
 from .utils import DraftParams
+
+MAX_SLOTS = ops.L.MAX_TREE_NODES          # tree slots the attention masks describe
+MASK_WORDS = MAX_SLOTS // 64
 
 
 class SubSpecSDDraftModel:
@@ -65,7 +69,8 @@ class SubSpecSDDraftModel:
         self.tree = Tree(input_ids[0, -1], self.model.dtype)
         self.levels = []
         self.level_state = {}                                                      # depth -> what speculate_once needs
-        self.level_bits = torch.tensor([[1, 0]], dtype=torch.int64, device=dev)    # root: slot 0 (words 0 and 1)
+        self.level_bits = torch.zeros((1, MASK_WORDS), dtype=torch.int64, device=dev)
+        self.level_bits[0, 0] = 1                                                  # root: slot 0
         self.next_slot = 1
         self.depth = 0
         self._expand(self._probs(logits).unsqueeze(0), torch.ones((1, 1), device=dev, dtype=logits.dtype))
@@ -82,9 +87,8 @@ class SubSpecSDDraftModel:
         # own bit of slot s: word s // 64, bit s % 64 (bit 63 is the sign bit of the signed word)
         low = slots % 64
         bit = torch.where(low == 63, torch.full_like(slots, -(1 << 63)), torch.ones_like(slots) << low.clamp(max=62))
-        own = torch.zeros((slots.numel(), 2), dtype=torch.int64, device=slots.device)
-        own[:, 0] = torch.where(slots < 64, bit, torch.zeros_like(bit))
-        own[:, 1] = torch.where((slots >= 64) & (slots < 128), bit, torch.zeros_like(bit))
+        words = torch.arange(MASK_WORDS, device=slots.device)
+        own = torch.where((slots // 64).unsqueeze(1) == words, bit.unsqueeze(1), torch.zeros_like(bit).unsqueeze(1))
         self.level_bits = self.level_bits[parent_indices[0]] | own
         self.first_slot = self.next_slot
         self.next_slot += token_ids.shape[1]
@@ -97,10 +101,10 @@ class SubSpecSDDraftModel:
         dev = self.model.device
         n = self.token_ids.shape[1]
         total = self.first_slot + n
-        if total > 128:
-            raise ValueError("draft tree exceeds the 128 tree slots of the attention mask")
+        if total > MAX_SLOTS:
+            raise ValueError(f"draft tree exceeds the {MAX_SLOTS} tree slots of the attention mask")
         depths = torch.full((n,), self.depth, dtype=torch.long, device=dev)
-        bits = self.level_bits if total > 64 else self.level_bits[:, 0].contiguous()
+        bits = self.level_bits[:, 0].contiguous() if total <= 64 else self.level_bits[:, :(total + 63) // 64].contiguous()
         logits = self.model.tree_forward(self.token_ids[0], depths, bits, self.prefix_len,
                                          first_slot=self.first_slot)
         self._expand(self._probs(logits).unsqueeze(0), self.parent_probs)
@@ -135,16 +139,16 @@ class SubSpecSDDraftModel:
         return True
 
     def _room_for_level(self) -> bool:
-        """One more level needs tree slots (the masks describe 128) and, once it is decoded, cache rows."""
+        """One more level needs tree slots (the masks describe ``MAX_SLOTS``) and, once it is decoded, cache rows."""
         n = self.token_ids.shape[1]
-        if self.first_slot + n > 128 or self.next_slot + n > 128:
+        if self.first_slot + n > MAX_SLOTS or self.next_slot + n > MAX_SLOTS:
             return False
         cache = self.model.kv.cache
         return cache.growable or self.prefix_len + self.next_slot + n <= cache.max_cache_len
 
     @torch.no_grad()
     def postspec(self) -> None:
-        """One more level while the target is busy (subspec_sd.py:133-140); also a no-op once the 128 tree slots
+        """One more level while the target is busy (subspec_sd.py:133-140); also a no-op once the tree slots
         the masks can describe, or the rows of a fixed-length cache, are used up."""
         if not self.had_first_speculate or self.postspec_count > (self.draft_params.max_depth - 1):
             return

@@ -53,8 +53,12 @@ class SubSpecSDGenerator:
         dev = self.target_model.device
         packed = tree.packed()
         anc = ops.ancestor_bits_tensor(packed["parent_indices"].tolist())
-        both = torch.stack([packed["token_ids"].long(), packed["depths"].long(), anc]).to(dev, non_blocking=True)
-        return self.target_model.tree_forward(both[0], both[1], both[2], position_offset)
+        n = anc.shape[0]
+        # one host-to-device copy: token ids, depths and the mask words of every node side by side
+        both = torch.cat([packed["token_ids"].long().view(n, 1), packed["depths"].long().view(n, 1), anc.view(n, -1)],
+                         dim=1).to(dev, non_blocking=True)
+        bits = both[:, 2].contiguous() if both.shape[1] == 3 else both[:, 2:].contiguous()
+        return self.target_model.tree_forward(both[:, 0].contiguous(), both[:, 1].contiguous(), bits, position_offset)
 
     def _get_logits_processor(self, temperature: float = 1.0, top_k: Optional[int] = None, top_p: Optional[float] = None):
         """The HuggingFace warpers of multinomial sampling, in the reference's order and under its

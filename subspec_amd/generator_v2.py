@@ -28,8 +28,8 @@ Three things are not carried over as they are, and are decided here:
   deepest level and attaches the new nodes to whatever leaves come first in index order.  Here the draft state is
   first set back to the deepest level that survived (``resync_to_depth``), so new levels hang below it.
 
-The tree may grow to 128 nodes (two mask words per row); a window of at most 64 nodes is decoded per forward,
-so ``1 + max_depth * topk_len`` must not exceed 64.
+Tree and extension together may occupy 512 tree slots (eight mask words per row); once they are used up, or a
+fixed-length cache has no rows left, post-speculation simply stops adding levels.
 """
 from __future__ import annotations
 
@@ -133,9 +133,8 @@ class SubSpecSDGeneratorV2(SubSpecSDGenerator):
     def _generate(self, input_ids, max_length: Optional[int], past_key_values: KVManager, stream_callback=None,
                   logits_processor=None, do_sample: bool = False):
         p = self.draft_params
-        if 1 + p.max_depth * p.topk_len > 64:
-            raise ValueError("post-speculation decodes the tree in windows of at most 64 nodes: "
-                             "1 + max_depth * topk_len must not exceed 64")
+        if 1 + p.max_depth * p.topk_len > ops.L.MAX_TREE_NODES:
+            raise ValueError(f"1 + max_depth * topk_len must not exceed the {ops.L.MAX_TREE_NODES} tree slots of the masks")
         dev = self.target_model.device
         input_ids = input_ids.to(dev)
         self.draft_model.set_past_key_values(past_key_values)

@@ -241,15 +241,17 @@ class Decoder:
                      first_slot: int = 0, n_tree_slots: Optional[int] = None) -> torch.Tensor:
         """Forward of tree nodes occupying cache rows prefix_len+first_slot.. ; ``depths`` are the node
         depths (rotary position = prefix_len + depth), ``anc_bits`` int64 [n] bitsets over tree
-        slots.  Returns logits [n, V]."""
+        slots ([n, ceil(slots / 64)] words above 64 slots).  Up to 64 rows go through the one-call layers; a larger
+        window (a whole large tree in the target) runs module by module, so that every weight matrix is read once
+        for all rows (library GEMMs) and only attention is split into launches of 64 rows.  Returns logits [n, V]."""
         n = token_ids.numel()
         slots = first_slot + n if n_tree_slots is None else n_tree_slots
         self.kv.cache.ensure(prefix_len + max(slots, first_slot + n))
-        self._rope_tables(prefix_len + n + 8)
+        self._rope_tables(prefix_len + max(slots, first_slot + n) + 8)
         positions = depths.to(self.device) + prefix_len
         rows = torch.arange(prefix_len + first_slot, prefix_len + first_slot + n, device=self.device)
         cfg = self.cfg
-        if self.use_native_layers and self.native_layers and n <= 64 and slots <= 128:
+        if self.use_native_layers and self.native_layers and n <= 64 and slots <= ops.L.MAX_TREE_NODES:
             return self.logits(self._run_native_layers(self.embed[token_ids], positions, rows, anc_bits, prefix_len, slots))
 
         def attn(i, q):

@@ -195,21 +195,22 @@ def topk_expand(sampled_probs: torch.Tensor, parent_probs: torch.Tensor, k: int,
 
 
 def bits_to_words(bits, n_slots: int, device=None) -> torch.Tensor:
-    """Python-int bitsets -> int64 tensor [n] (up to 64 slots) or [n, 2] (up to 128 slots): bit j of a row is
+    """Python-int bitsets -> int64 tensor [n] (up to 64 slots) or [n, ceil(n_slots / 64)]: bit j of a row is
     bit j % 64 of word j // 64."""
     def signed(w):
         return w - (1 << 64) if w >= (1 << 63) else w
     mask = (1 << 64) - 1
     if n_slots <= 64:
         return torch.tensor([signed(int(b) & mask) for b in bits], dtype=torch.int64, device=device)
-    if n_slots > 128:
-        raise ValueError(f"{n_slots} tree slots exceed the 128 the attention kernel masks")
-    return torch.tensor([[signed(int(b) & mask), signed((int(b) >> 64) & mask)] for b in bits], dtype=torch.int64,
+    if n_slots > L.MAX_TREE_NODES:
+        raise ValueError(f"{n_slots} tree slots exceed the {L.MAX_TREE_NODES} the attention kernel masks")
+    words = (n_slots + 63) // 64
+    return torch.tensor([[signed((int(b) >> (64 * w)) & mask) for w in range(words)] for b in bits], dtype=torch.int64,
                         device=device)
 
 
 def ancestor_bits_tensor(parents, device=None) -> torch.Tensor:
-    """uint64 ancestor-or-self bitsets (as an int64 tensor, [n] or [n, 2] above 64 nodes) from a parent
+    """uint64 ancestor-or-self bitsets (as an int64 tensor, [n] or [n, ceil(n / 64)] above 64 nodes) from a parent
     array with parent < child."""
     bits = []
     for i, p in enumerate(parents):
@@ -222,9 +223,9 @@ def tree_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
                    prefix_len: int, scale: Optional[float] = None, workspace: Optional[torch.Tensor] = None,
                    n_tree_slots: Optional[int] = None):
     """``q`` [B, Hq, n, D], caches [B, Hkv, S, D] (tree K/V already written at rows prefix_len..),
-    ``anc_bits`` int64 [n] (shared tree) or [B, n], with a trailing dimension of 2 words when more than 64
-    tree slots are occupied: bit j = row may attend to tree slot j.  ``n_tree_slots`` (default n) is the
-    number of occupied tree slots (<= 128).  Returns [B, n, Hq * D]."""
+    ``anc_bits`` int64 [n] (shared tree) or [B, n], with a trailing dimension of ceil(slots / 64) words when
+    more than 64 tree slots are occupied: bit j = row may attend to tree slot j.  ``n_tree_slots`` (default n) is
+    the number of occupied tree slots (<= 512); n may be as large (64 rows per launch).  Returns [B, n, Hq * D]."""
     dev = _require_gpu(q, k_cache, v_cache, anc_bits)
     if q.dim() != 4 or k_cache.dim() != 4 or v_cache.shape != k_cache.shape:
         raise ValueError("expected q [B, Hq, n, D] and k/v caches [B, Hkv, S, D]")
@@ -237,11 +238,12 @@ def tree_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
     if not (k_cache.is_contiguous() and v_cache.is_contiguous()):
         raise ValueError("tree_attention: the KV caches must be contiguous [B, Hkv, S, D]")
     slots = n if n_tree_slots is None else int(n_tree_slots)
-    words = 2 if slots > 64 else 1
-    rows_shape = anc_bits.shape[:-1] if words == 2 else anc_bits.shape       # [n] or [B, n]
-    if anc_bits.dtype != torch.int64 or (words == 2 and anc_bits.shape[-1] != 2) or len(rows_shape) not in (1, 2) \
+    words = (slots + 63) // 64
+    rows_shape = anc_bits.shape[:-1] if words > 1 else anc_bits.shape       # [n] or [B, n]
+    if anc_bits.dtype != torch.int64 or (words > 1 and anc_bits.shape[-1] != words) or len(rows_shape) not in (1, 2) \
             or rows_shape[-1] != n:
-        raise ValueError("anc_bits must be int64 [n] / [B, n] (two words per row, [..., n, 2], above 64 tree slots)")
+        raise ValueError("anc_bits must be int64 [n] / [B, n] (ceil(slots / 64) words per row, [..., n, words], above 64 "
+                         "tree slots)")
     q = q.contiguous()
     anc_bits = anc_bits.contiguous()
     if len(rows_shape) == 2 and rows_shape[0] not in (1, B):
@@ -283,9 +285,9 @@ def tree_attention_paged(q: torch.Tensor, pool_layer: torch.Tensor, page_indices
     if Dq != D or q.dtype != pool_layer.dtype:
         raise ValueError("q and the pool must share head_dim and dtype")
     slots = n if n_tree_slots is None else int(n_tree_slots)
-    words = 2 if slots > 64 else 1
+    words = (slots + 63) // 64
     if anc_bits.dtype != torch.int64 or anc_bits.numel() != n * words:
-        raise ValueError("anc_bits must be int64 [n] ([n, 2] above 64 tree slots)")
+        raise ValueError("anc_bits must be int64 [n] ([n, ceil(slots / 64)] above 64 tree slots)")
     q, anc_bits = q.contiguous(), anc_bits.contiguous()
     lib = L.lib()
     need = lib.subspec_tree_attention_workspace(1, Hq, int(prefix_len), slots)
@@ -331,7 +333,7 @@ def kv_compact_paged_(pool: torch.Tensor, page_indices: torch.Tensor, contexts: 
 
 def int4_linear(x: torch.Tensor, wq: torch.Tensor, sz: torch.Tensor, out_features: int,
                 bias: Optional[torch.Tensor] = None, workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """``x`` [..., K] (bf16 / fp16, at most 64 rows in total) times the tiled int4 weight
+    """``x`` [..., K] (bf16 / fp16; 64 rows per pass over the weights, more rows are more passes) times the tiled int4 weight
     (``wq`` int32, ``sz`` int32 as produced by ``subspec_amd.quant.pack_tiled``) -> [..., N]."""
     dev = _require_gpu(x, wq, sz)
     K = x.shape[-1]
@@ -451,7 +453,7 @@ def int4_decoder_layer_(x: torch.Tensor, dims: "L.DecoderLayerDims", weights: "L
     if not (x.is_contiguous() and k_cache.is_contiguous() and v_cache.is_contiguous()):
         raise ValueError("decoder layer: x and the layer's cache views must be contiguous")
     if x.shape != (dims.n_rows, dims.hidden) or positions.numel() != dims.n_rows or cache_rows.numel() != dims.n_rows \
-            or anc_bits.numel() != dims.n_rows * (2 if dims.n_tree_slots > 64 else 1):
+            or anc_bits.numel() != dims.n_rows * ((dims.n_tree_slots + 63) // 64):
         raise ValueError("decoder layer: tensor shapes do not match the dimensions given")
     dense = isinstance(weights, L.DenseLayerWeights)
     fn = L.lib().subspec_dense_decoder_layer if dense else L.lib().subspec_int4_decoder_layer

@@ -74,7 +74,7 @@ class KvCachePool:
             page_indices = torch.arange(min(need, self.max_pages), dtype=torch.int32, device=self.device)
         beam_idx = beam_idx.to(self.device).to(torch.int64).contiguous()
         ops.kv_compact_paged_(self.cache_data, page_indices, beam_idx, int(offset), count_dev=count_dev,
-                              max_count=None if count_dev is None else min(int(beam_idx.numel()), 256))
+                              max_count=None if count_dev is None else min(int(beam_idx.numel()), ops.L.MAX_TREE_NODES))
 
 
 class RequestKvCache:

@@ -86,8 +86,38 @@ def test_extended_tree_up_to_128_slots(dtype):
             want = ref[:, lo:hi]
             assert (out - want).abs().amax().item() <= 1e-2 * want.abs().amax().item()
             assert torch.allclose(out, want, rtol=1e-2, atol=2e-2)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_large_trees_up_to_512_slots(dtype):
+    """Trees of the reference's offloading configurations (1 + 48 * 6 = 289 nodes) and the largest the masks describe
+    (512 slots, eight words per row): all rows in one call (windows of 64 rows inside), and windows of few rows
+    as a draft step or a post-speculation window queries them.  Prefixes that are and are not multiples of 64, so
+    that a 64-key block straddles two mask words."""
+    for seed, (B, n_slots, P, S, depth) in enumerate([(1, 289, 70, 400, 48), (2, 512, 1000, 1600, 60), (1, 200, 0, 256, 30),
+                                                      (1, 130, 64, 320, 20)]):
+        g = torch.Generator().manual_seed(90 + seed)
+        parents, _, _ = W.random_tree(g, n=n_slots, max_depth=depth, max_children=6, vocab=1000, chain_depth=depth)
+        q = torch.randn(B, 8, n_slots, 128, generator=g).to(dtype)
+        k = torch.randn(B, 2, S, 128, generator=g).to(dtype)
+        v = torch.randn(B, 2, S, 128, generator=g).to(dtype)
+        k[:, :, P + n_slots:] = 1e3                                   # stale rows beyond the tree
+        ref = oa.tree_attention(q, k, v, parents, P)
+        anc = ops.ancestor_bits_tensor(parents, device=DEV)
+        assert anc.shape == (n_slots, (n_slots + 63) // 64)
+        print("attention large tree", dtype, B, n_slots, P, "all rows", flush=True)
+        out = ops.tree_attention(q.to(DEV), k.to(DEV), v.to(DEV), anc, P).float().cpu()
+        assert (out - ref).abs().amax().item() <= 1e-2 * ref.abs().amax().item()
+        assert torch.allclose(out, ref, rtol=1e-2, atol=2e-2)
+        for lo, hi in ((n_slots - 6, n_slots), (100, 164), (n_slots - 70, n_slots - 3)):
+            print("attention large tree", dtype, B, n_slots, P, lo, hi, flush=True)
+            out = ops.tree_attention(q[:, :, lo:hi].contiguous().to(DEV), k.to(DEV), v.to(DEV), anc[lo:hi].contiguous(), P,
+                                     n_tree_slots=n_slots).float().cpu()
+            want = ref[:, lo:hi]
+            assert (out - want).abs().amax().item() <= 1e-2 * want.abs().amax().item()
+            assert torch.allclose(out, want, rtol=1e-2, atol=2e-2)
     with pytest.raises(ValueError):
-        ops.ancestor_bits_tensor([-1] + list(range(128)))              # 129 nodes
+        ops.ancestor_bits_tensor([-1] + list(range(512)))              # 513 nodes
 
 
 def test_argument_errors():

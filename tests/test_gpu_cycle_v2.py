@@ -95,6 +95,33 @@ def test_v2_emits_what_v1_emits(agreeing, first_streamed):
             assert log["speculate_count"] < ref_log["n_iter"]
 
 
+@pytest.mark.parametrize("cls,steps", [(SubSpecSDGenerator, None), (SubSpecSDGeneratorV2, 3), (SubSpecSDGeneratorV2, None)])
+def test_deep_trees_beyond_one_window(cls, steps):
+    """Depth 20 x 6 = 121 nodes (the shape of the reference's depth-48 x 6 trees at test size): the target decodes
+    the tree in two windows of rows and the draft's masks take more than one word."""
+    w = _weights(True)
+    kv = create_kv_cache("static", max_cache_len=1024, config=CFG, device=DEV, dtype=torch.bfloat16)
+    target, draft, _ = build_models(CFG, kv, device=DEV, weights=w, first_streamed=2)
+    gk = {} if steps is None and cls is SubSpecSDGenerator else dict(postspec_steps=steps)
+    gen = cls(target, None, SubSpecSDDraftModel(draft), DraftParams(temperature=0.2, max_depth=20, topk_len=6),
+              generator_kwargs=dict(verify_method="exact", **gk))
+    prompt = torch.randint(0, CFG.vocab_size, (1, 32), generator=torch.Generator().manual_seed(4)).to(DEV)
+    wandb_logger.clear_log_data()
+    out = gen.generate(prompt, max_new_tokens=120, do_sample=False, past_key_values=kv)[0].cpu()
+    log = dict(wandb_logger.log_data)
+    print("deep trees", cls.__name__, steps, log["n_iter"], log["avg_sampled"], flush=True)
+    assert out.numel() == 152
+    _assert_greedy_continuation(w, out, 32, (cls.__name__, steps))
+    assert log["avg_sampled"] > 3.0, log
+    L = kv.get_seq_length()
+    assert L == out.numel() - 1
+    kv2 = create_kv_cache("static", max_cache_len=512, config=CFG, device=DEV, dtype=torch.bfloat16)
+    t2, _, _ = build_models(CFG, kv2, device=DEV, weights=w)
+    t2.prefill(out[:-1].to(DEV), 0)
+    a, b = kv.cache.data[..., :L, :].float(), kv2.cache.data[..., :L, :].float()
+    assert (a - b).abs().amax().item() <= 5e-2 * b.abs().amax().item()
+
+
 def test_v2_lossy_and_sampling_targets_run_through_the_same_loop():
     w = _weights(True)
     ref, _, _, _ = _run(SubSpecSDGenerator, w, 2, verify="lossy")
@@ -112,10 +139,10 @@ def test_v2_lossy_and_sampling_targets_run_through_the_same_loop():
     assert a.shape[1] == 62 and kv.get_seq_length() == 61
 
 
-def test_v2_rejects_trees_wider_than_one_window():
+def test_v2_rejects_trees_beyond_the_slot_limit():
     w = _weights(False)
     kv = create_kv_cache("static", max_cache_len=512, config=CFG, device=DEV, dtype=torch.bfloat16)
     target, draft, _ = build_models(CFG, kv, device=DEV, weights=w)
-    gen = SubSpecSDGeneratorV2(target, None, SubSpecSDDraftModel(draft), DraftParams(max_depth=8, topk_len=8))
+    gen = SubSpecSDGeneratorV2(target, None, SubSpecSDDraftModel(draft), DraftParams(max_depth=64, topk_len=8))
     with pytest.raises(ValueError):
         gen.generate(torch.zeros(1, 4, dtype=torch.long, device=DEV), max_new_tokens=4, do_sample=False, past_key_values=kv)

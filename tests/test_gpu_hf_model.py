@@ -66,7 +66,7 @@ def _close(got, ref, tag, tol=3e-2):
     assert (got.float().cpu().argmax(-1) == ref.argmax(-1)).float().mean().item() >= 0.8, tag
 
 
-@pytest.mark.parametrize("n,P", [(9, 23), (64, 150), (1, 40)])
+@pytest.mark.parametrize("n,P", [(9, 23), (64, 150), (1, 40), (150, 60)])       # 150 rows: beyond one 64-row window
 def test_target_and_draft_match_huggingface(n, P):
     print("hf model", n, P, flush=True)
     model = _hf(n)

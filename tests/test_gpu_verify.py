@@ -223,8 +223,8 @@ def test_verify_tree_host_interface_and_errors():
                                           do_sample=True, stream=SampleStream(1))
     assert toks.tolist() == [[11, 13, 40]] and ctx.tolist() == [0, 1, 3] and (total, acc) == (2, 2)
     with pytest.raises(ValueError):            # more nodes than the kernels are built for
-        ops.tree_verify(torch.zeros(300, 64, device=DEV), torch.zeros(300, dtype=torch.int32, device=DEV),
-                        torch.zeros(300, dtype=torch.int32, device=DEV))
+        ops.tree_verify(torch.zeros(513, 64, device=DEV), torch.zeros(513, dtype=torch.int32, device=DEV),
+                        torch.zeros(513, dtype=torch.int32, device=DEV))
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
@@ -246,6 +246,19 @@ def test_kv_compaction_bit_exact(dtype):
         assert torch.equal(got[..., : offset + len(ctx), :], okv.compact_dynamic(cache, ctx, offset))
 
 
+@pytest.mark.parametrize("count", [257, 300, 512])
+def test_kv_compaction_of_long_paths(count):
+    """More rows than a 256-node tree could accept: the accumulated contexts of consecutive post-verified cycles."""
+    g = torch.Generator().manual_seed(count)
+    cache = torch.randn(2, 2, 1, 2, 1200, 128, generator=g).to(torch.bfloat16)
+    ctx = sorted(torch.randperm(1000, generator=g)[:count].tolist())
+    exp = okv.compact_static(cache, ctx, 150)
+    dev = cache.to(DEV)
+    ops.kv_compact_(dev, torch.tensor(ctx, dtype=torch.int64, device=DEV), 150)
+    torch.cuda.synchronize()
+    assert torch.equal(dev.cpu(), exp)
+
+
 def test_kv_compaction_count_from_device_follows_verifier():
     cfg = W.greedy_config(9)
     out = ops.tree_verify(cfg["logits"].to(DEV), torch.tensor(cfg["tokens"], dtype=torch.int32, device=DEV),
@@ -262,13 +275,16 @@ def test_kv_compaction_count_from_device_follows_verifier():
         ops.kv_compact_(dev[..., :7], out["contexts"][0], 0)                 # non-contiguous
 
 
-@pytest.mark.parametrize("n", [65, 128, 129, 200, 256])
+@pytest.mark.parametrize("n", [65, 128, 129, 200, 256, 257, 289, 512])
 def test_large_trees_up_to_the_node_limit(n):
-    """Trees beyond one node per lane (2 and 4 nodes per lane in the acceptance step), greedy and sampled
-    targets, exact walk and both lossy gates, against the oracle; rows may be fewer than nodes."""
+    """Trees beyond one node per lane (2, 4 and 8 nodes per lane in the acceptance step; 289 = the reference's
+    depth-48 x 6 tree), greedy and sampled targets, exact walk and both lossy gates, against the oracle; rows may be
+    fewer than nodes."""
     g = torch.Generator().manual_seed(n)
     vocab = 777
-    parents, toks, depths = W.random_tree(g, n=n, max_depth=12, max_children=4, vocab=vocab, chain_depth=10)
+    deep = n > 256
+    parents, toks, depths = W.random_tree(g, n=n, max_depth=48 if deep else 12, max_children=6 if deep else 4, vocab=vocab,
+                                          chain_depth=40 if deep else 10)
     kids = ov.children_from_parents(parents)
     for rows, dtype in ((n, torch.bfloat16), (n, torch.float32), (max(1, n - 40), torch.bfloat16)):
         logits = (torch.randn(rows, vocab, generator=g) * 2).to(dtype)
