@@ -1,5 +1,6 @@
 """Pins the attention oracle: explicit softmax(QK^T)V == F.scaled_dot_product_attention with the
 additive mask; mask == the host tree's create_attention_mask; single-key special case.  No GPU."""
+import pytest
 import torch
 
 from oracle import attention as oa
@@ -37,3 +38,20 @@ def test_mask_matches_host_tree_and_bitsets():
     assert bits == t.ancestor_bits()
     for i, w in enumerate(bits):
         assert [bool((w >> j) & 1) for j in range(t.size())] == m[i, 3:].tolist()
+
+
+def test_mask_words_of_large_trees():
+    """Trees beyond 64 nodes: word w of row i holds the slots 64 w .. 64 w + 63 (as signed 64-bit integers) of the
+    same ancestor-or-self relation the dense mask of the oracle describes."""
+    from subspec_amd import workloads as W
+    for n, depth in ((65, 10), (289, 48), (512, 60)):
+        parents, _, _ = W.random_tree(torch.Generator().manual_seed(n), n=n, max_depth=depth, max_children=6, vocab=1000,
+                                      chain_depth=depth)
+        words = ops.ancestor_bits_tensor(parents)
+        assert words.shape == (n, (n + 63) // 64) and words.dtype == torch.int64
+        m = oa.allowed_mask(parents, 0, n)
+        for i in (0, 1, 63, 64, n // 2, n - 1):
+            row = [bool((int(words[i, j // 64]) >> (j % 64)) & 1) for j in range(n)]
+            assert row == m[i].tolist(), (n, i)
+    with pytest.raises(ValueError):
+        ops.ancestor_bits_tensor([-1] + list(range(512)))
