@@ -44,6 +44,15 @@ class StaticKVCache:
         self.data[layer, 0].index_copy_(2, positions, k)
         self.data[layer, 1].index_copy_(2, positions, v)
 
+    contiguous = True                          # k(i) / v(i) are [B, Hkv, S, D] views the one-call layers can take
+
+    def prefix_kv(self, layer: int, n_rows: int):
+        """K and V of rows 0 .. n_rows - 1 as [B, Hkv, n_rows, D] (the causal prefill reads them)."""
+        return self.data[layer, 0][:, :, :n_rows], self.data[layer, 1][:, :, :n_rows]
+
+    def tree_attention(self, layer: int, q: torch.Tensor, anc_bits: torch.Tensor, prefix_len: int, n_tree_slots: int):
+        return ops.tree_attention(q, self.k(layer), self.v(layer), anc_bits, prefix_len, n_tree_slots=n_tree_slots)
+
     def reset(self) -> None:
         self.data.zero_()
 
@@ -127,12 +136,13 @@ class KVManager:
 def create_kv_cache(cache_implementation: str = "static", max_cache_len: Optional[int] = None,
                     max_batch_size: Optional[int] = 1, config=None, device="cuda:0", dtype=torch.bfloat16) -> KVManager:
     """Factory with the reference's signature (cache_utils.py:6-39).  For the dynamic cache ``max_cache_len`` is only
-    the initial capacity."""
+    the initial capacity.  ``"paged"`` (not a choice of the reference's factory, whose paged path has generators of
+    its own) puts the same interface over a page pool: one request's pages, 16 tokens each."""
     if isinstance(dtype, str):
         if not hasattr(torch, dtype):
             raise ValueError(f"Unsupported dtype string: {dtype}")
         dtype = getattr(torch, dtype)
-    if cache_implementation not in ("static", "dynamic"):
+    if cache_implementation not in ("static", "dynamic", "paged"):
         raise ValueError(f"Unsupported cache_implementation: {cache_implementation}")
     if config is None:
         # the reference's dynamic cache learns its shapes from the first update; this one allocates up front
@@ -140,6 +150,12 @@ def create_kv_cache(cache_implementation: str = "static", max_cache_len: Optiona
     if cache_implementation == "dynamic":
         return KVManager(DynamicKVCache(config.num_hidden_layers, config.num_key_value_heads, config.head_dim, device, dtype,
                                         max_batch_size or 1, initial_len=max_cache_len or 1024))
+    if cache_implementation == "paged":
+        if max_cache_len is None:
+            raise ValueError("max_cache_len must be provided for the paged cache (it sizes the page pool)")
+        from .paged_cache import PagedKVCache
+        return KVManager(PagedKVCache(config.num_hidden_layers, config.num_key_value_heads, config.head_dim,
+                                      max_cache_len, device, dtype))
     if max_cache_len is None:
         raise ValueError("max_cache_len must be provided for static cache")
     return KVManager(StaticKVCache(config.num_hidden_layers, config.num_key_value_heads, config.head_dim,

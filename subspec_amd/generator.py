@@ -34,7 +34,7 @@ class SubSpecSDGenerator:
         self.target_model, self.tokenizer, self.draft_model = target_model, tokenizer, draft_model
         self.draft_params = draft_params or DraftParams()
         self.draft_model.draft_params = self.draft_params
-        if cache_implementation not in ("static", "dynamic"):
+        if cache_implementation not in ("static", "dynamic", "paged"):
             raise ValueError(f"Unsupported cache_implementation: {cache_implementation}")
         self.cache_implementation = cache_implementation
         self.profiling = profiling

@@ -141,7 +141,8 @@ class Decoder:
         per layer instead of one per module): every layer int4-packed, or every layer dense 16-bit."""
         if self._native is None:
             packed = [("qkv_proj.wq" in w) for w in self.layers]
-            self._native = bool(self.layers) and (all(packed) or not any(packed)) and self.dtype != torch.float32
+            self._native = (bool(self.layers) and (all(packed) or not any(packed)) and self.dtype != torch.float32
+                            and self.kv.cache.contiguous)
             if self._native:
                 make = ops.decoder_layer_weights if packed[0] else ops.dense_layer_weights
                 self._native_make = make
@@ -228,8 +229,8 @@ class Decoder:
         rep = cfg.num_attention_heads // cfg.num_key_value_heads
 
         def attn(i, q):
-            k = self.kv.cache.k(i)[:, :, :start + n].repeat_interleave(rep, dim=1)
-            v = self.kv.cache.v(i)[:, :, :start + n].repeat_interleave(rep, dim=1)
+            k, v = self.kv.cache.prefix_kv(i, start + n)
+            k, v = k.repeat_interleave(rep, dim=1), v.repeat_interleave(rep, dim=1)
             mask = torch.ones(n, start + n, dtype=torch.bool, device=self.device).tril(diagonal=start)
             o = F.scaled_dot_product_attention(q, k, v, attn_mask=mask)
             return o.transpose(1, 2).reshape(n, cfg.q_size)
@@ -255,8 +256,7 @@ class Decoder:
             return self.logits(self._run_native_layers(self.embed[token_ids], positions, rows, anc_bits, prefix_len, slots))
 
         def attn(i, q):
-            return ops.tree_attention(q, self.kv.cache.k(i), self.kv.cache.v(i), anc_bits, prefix_len,
-                                      n_tree_slots=slots).reshape(n, cfg.q_size)
+            return self.kv.cache.tree_attention(i, q, anc_bits, prefix_len, slots).reshape(n, cfg.q_size)
 
         return self.logits(self._run_layers(self.embed[token_ids], positions, rows, attn))
 

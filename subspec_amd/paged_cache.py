@@ -164,3 +164,72 @@ class RequestKvCache:
         table = self.page_table(max(0, offset + max(int(beam_idx.numel()), num_new_tokens) - self.kv_len))
         self.kvCachePool.reorder_cache_with_offset(beam_idx, offset, num_new_tokens, page_indices=table)
         self._set_len(offset + int(beam_idx.size(0)), allow_growth=False)
+
+
+class PagedKVCache:
+    """One sequence over a page pool behind the interface the decoder and the cycle drivers use for the static cache
+    (``ensure``, ``write``, ``prefix_kv``, ``tree_attention``, ``reorder_cache_with_offset``, ``crop``, ``reset``):
+    the alternative cache layout of the reference's FlashInfer path serving the same speculative cycle.  Rows are
+    logical positions; pages are taken from the pool as rows are first needed, in whatever order the pool hands them
+    out, and the page table goes to the kernels as it is."""
+    growable = False
+    contiguous = False
+
+    def __init__(self, n_layers: int, n_kv_heads: int, head_dim: int, max_cache_len: int, device, dtype, page_len: int = 16):
+        self.page_len = int(page_len)
+        max_pages = (int(max_cache_len) + self.page_len - 1) // self.page_len
+        self.max_cache_len = max_pages * self.page_len
+        self.pool = KvCachePool(max_pages, n_layers, n_kv_heads, head_dim, self.page_len, dtype, device)
+        self.request = RequestKvCache(self.pool, self.page_len, 0)
+        self._table: Optional[torch.Tensor] = None
+
+    # ---- pages
+    def ensure(self, n_rows: int) -> None:
+        if n_rows > self.max_cache_len:
+            raise ValueError(f"the page pool holds {self.max_cache_len} rows, {n_rows} are needed")
+        need = (int(n_rows) + self.page_len - 1) // self.page_len
+        pages = self.request.kv_page_indices
+        if need > len(pages):
+            pages.extend(self.pool.allocate(need - len(pages)))
+            self._table = None
+
+    def table(self) -> torch.Tensor:
+        if self._table is None or self._table.numel() != len(self.request.kv_page_indices):
+            self._table = torch.tensor(self.request.kv_page_indices, dtype=torch.int32, device=self.pool.device)
+        return self._table
+
+    # ---- rows
+    def write(self, layer: int, positions: torch.Tensor, k: torch.Tensor, v: torch.Tensor) -> None:
+        """k, v: [1, Hkv, n, D] written at logical rows ``positions`` (int64 [n])."""
+        table = self.table().long()                       # the caller has sized the cache with ensure()
+        pages, toks = table[positions // self.page_len], positions % self.page_len
+        data = self.pool.cache_data
+        data[layer, pages, 0, toks] = k[0].transpose(0, 1)
+        data[layer, pages, 1, toks] = v[0].transpose(0, 1)
+
+    def prefix_kv(self, layer: int, n_rows: int):
+        rows = torch.arange(n_rows, device=self.pool.device)
+        table = self.table().long()
+        pages, toks = table[rows // self.page_len], rows % self.page_len
+        kv = self.pool.cache_data[layer, pages, :, toks]                  # [n_rows, 2, Hkv, D]
+        return kv[:, 0].transpose(0, 1).unsqueeze(0), kv[:, 1].transpose(0, 1).unsqueeze(0)
+
+    def tree_attention(self, layer: int, q: torch.Tensor, anc_bits: torch.Tensor, prefix_len: int, n_tree_slots: int):
+        return ops.tree_attention_paged(q, self.pool.cache_data[layer], self.table(), anc_bits, prefix_len,
+                                        n_tree_slots=n_tree_slots)
+
+    def reorder_cache_with_offset(self, beam_idx: torch.Tensor, new_chunk_len: int = 1, offset: int = 0, dim: int = 2,
+                                  count_dev: Optional[torch.Tensor] = None) -> None:
+        self.pool.reorder_cache_with_offset(beam_idx, int(offset), 0, page_indices=self.table(), count_dev=count_dev)
+
+    def crop(self, start: int, end: Optional[int] = None, dim: int = 2) -> None:
+        """Rows from ``start`` on leave the cache: whole pages behind them go back to the pool."""
+        keep = (max(int(start), 0) + self.page_len - 1) // self.page_len
+        pages = self.request.kv_page_indices
+        if keep < len(pages):
+            self.pool.deallocate(pages[keep:])
+            del pages[keep:]
+            self._table = None
+
+    def reset(self) -> None:
+        self.crop(0)

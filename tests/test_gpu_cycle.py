@@ -134,7 +134,7 @@ def test_generator_argument_errors():
     with pytest.raises(ValueError):                                             # the warper rejects T <= 0
         gen.generate(ids, max_new_tokens=4, do_sample=True, temperature=0.0, past_key_values=kv)
     with pytest.raises(ValueError):
-        create_kv_cache("paged", max_cache_len=8, config=CFG)
+        create_kv_cache("sliding", max_cache_len=8, config=CFG)
     bad = SubSpecSDGenerator(target, None, SubSpecSDDraftModel(draft), DraftParams(max_depth=2, topk_len=2),
                              generator_kwargs=dict(verify_method="bogus"))
     with pytest.raises(ValueError):

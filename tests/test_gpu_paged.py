@@ -131,3 +131,49 @@ def test_request_cache_cycle_matches_static_cache():
     want_v = okv.compact_static(vc.cpu(), accepted.tolist(), prefix)[:, :, :prefix + 4]
     assert torch.equal(kk, want_k) and torch.equal(vv, want_v)
     assert len(req.kv_page_indices) == (prefix + 4 + page_len - 1) // page_len
+
+
+@pytest.mark.parametrize("driver", ["v1", "v2"])
+def test_speculative_cycle_over_the_paged_cache_equals_the_static_cache(driver):
+    """The whole cycle (prefill, draft levels, target window, verification, compaction) over a page pool whose pages
+    were handed out in scrambled order, against the same models over the contiguous cache.  Both runs go module by
+    module (the one-call layers take contiguous caches only), so the cache layout is the only difference and
+    tokens and cached K / V must agree bit for bit."""
+    from subspec_amd.cache import create_kv_cache
+    from subspec_amd.draft import SubSpecSDDraftModel
+    from subspec_amd.generator import SubSpecSDGenerator
+    from subspec_amd.generator_v2 import SubSpecSDGeneratorV2
+    from subspec_amd.model import DecoderConfig, build_models, init_weights
+    from subspec_amd.utils import DraftParams
+    cfg = DecoderConfig(num_hidden_layers=3, hidden_size=256, num_attention_heads=2, num_key_value_heads=1,
+                        head_dim=128, intermediate_size=512, vocab_size=2048)
+    w = init_weights(cfg, 3, DEV)
+    prompt = torch.randint(0, cfg.vocab_size, (1, 37), generator=torch.Generator().manual_seed(8)).to(DEV)
+    runs = {}
+    for impl in ("static", "paged"):
+        kv = create_kv_cache(impl, max_cache_len=512, config=cfg, device=DEV, dtype=torch.bfloat16)
+        if impl == "paged":
+            pool = kv.cache.pool
+            held = pool.allocate(9)                               # scramble the order of the request's pages:
+            pool.deallocate(held[::2])                            # gaps in what the pool hands out later, and the
+            kv.cache.request.kv_page_indices.extend(reversed(pool.allocate(3)))   # first three logical pages backwards
+        target, draft, _ = build_models(cfg, kv, device=DEV, weights=w)
+        target.use_native_layers = draft.use_native_layers = False
+        cls, extra = (SubSpecSDGenerator, {}) if driver == "v1" else (SubSpecSDGeneratorV2, dict(postspec_steps=2))
+        gen = cls(target, None, SubSpecSDDraftModel(draft), DraftParams(temperature=0.2, max_depth=5, topk_len=4),
+                  cache_implementation=impl, generator_kwargs=dict(verify_method="exact", **extra))
+        out = gen.generate(prompt, max_new_tokens=40, do_sample=False, past_key_values=kv)[0].cpu()
+        L = kv.get_seq_length()
+        k, v = kv.cache.prefix_kv(1, L)
+        runs[impl] = (out, L, k.cpu().clone(), v.cpu().clone(), kv)
+    (a, La, ka, va, _), (b, Lb, kb, vb, kvp) = runs["static"], runs["paged"]
+    assert a.numel() == 77 and torch.equal(a, b) and La == Lb == 76
+    assert torch.equal(ka, kb) and torch.equal(va, vb)
+    table = kvp.cache.table().tolist()
+    assert table != sorted(table)                                   # the pages really were out of order
+    # rows leave the cache: whole pages go back to the pool
+    free = int(kvp.cache.pool.num_free_pages())
+    kvp.cache.crop(20)
+    assert int(kvp.cache.pool.num_free_pages()) == free + (len(table) - 2) and kvp.cache.table().tolist() == table[:2]
+    with pytest.raises(ValueError):
+        kvp.cache.ensure(100000)

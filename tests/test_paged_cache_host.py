@@ -90,3 +90,38 @@ def test_paged_compaction_oracle_pins(seed):
     logical_in = pool[:, perm].clone()                         # pages in sequence order
     logical_out = okv.compact_paged_reference(logical_in, ctx, offset)
     assert torch.equal(got[:, perm], logical_out)
+
+
+def test_paged_cache_behind_the_static_cache_interface():
+    """PagedKVCache on the CPU: pages are taken as rows are first needed, writes land where the page table says,
+    prefix_kv gathers them back in logical order, crop hands whole pages back."""
+    from subspec_amd.cache import create_kv_cache
+    from subspec_amd.model import DecoderConfig
+    cfg = DecoderConfig(num_hidden_layers=2, hidden_size=64, num_attention_heads=2, num_key_value_heads=2, head_dim=8,
+                        intermediate_size=64, vocab_size=50)
+    kv = create_kv_cache("paged", max_cache_len=100, config=cfg, device="cpu", dtype=torch.float32)
+    c = kv.cache
+    assert c.max_cache_len == 112 and not c.contiguous and not c.growable         # 7 pages of 16 rows
+    held = c.pool.allocate(2)
+    c.ensure(40)                                                                   # 3 pages: physical 2, 3, 4
+    assert c.table().tolist() == [2, 3, 4]
+    c.pool.deallocate(held)
+    g = torch.Generator().manual_seed(0)
+    k = torch.randn(1, 2, 40, 8, generator=g)
+    v = torch.randn(1, 2, 40, 8, generator=g)
+    c.write(1, torch.arange(40), k, v)
+    kk, vv = c.prefix_kv(1, 40)
+    assert torch.equal(kk, k) and torch.equal(vv, v)
+    assert torch.equal(c.pool.cache_data[1, 3, 0, 5], k[0, :, 21])                  # row 21 = page 1 (physical 3), token 5
+    c.write(1, torch.arange(33, 36), k[:, :, :3], v[:, :, :3])                     # overwrite rows in the last page
+    assert torch.equal(c.prefix_kv(1, 36)[0][0, :, 33:36], k[0, :, :3])
+    c.ensure(50)                                                                   # a 4th page: the lowest free one
+    assert c.table().tolist() == [2, 3, 4, 0]
+    c.crop(17)
+    assert c.table().tolist() == [2, 3] and int(c.pool.num_free_pages()) == 5
+    with pytest.raises(ValueError):
+        c.ensure(113)
+    kv.reset()
+    assert c.table().numel() == 0 and int(c.pool.num_free_pages()) == 7
+    with pytest.raises(ValueError):
+        create_kv_cache("paged", config=cfg)
