@@ -44,6 +44,7 @@ class SubSpecSDGenerator:
         self.draft_model.eos_token_id = self.eos_token_id
         # Philox stream of the sampling target; generator_kwargs["seed"] fixes it, else torch's seed
         self.sample_stream = SampleStream(self.generator_kwargs.get("seed"))
+        self._stop_strings = None                # HuggingFace StopStringCriteria of the current generate() call
 
     # ------------------------------------------------------------------ pieces of one cycle
     def _speculate(self, input_ids):
@@ -104,8 +105,13 @@ class SubSpecSDGenerator:
     @torch.no_grad()
     def generate(self, input_ids: torch.LongTensor, temperature=None, top_p=None, top_k=None, max_new_tokens=None,
                  max_length=None, do_sample=False, stop_strings=None, stream_callback=None, **model_kwargs):
-        if stop_strings is not None:
-            raise NotImplementedError("stop_strings need a tokenizer; not available in this build")
+        self._stop_strings = None
+        if stop_strings is not None:                          # generators/base.py:94-101
+            if self.tokenizer is None:
+                raise ValueError("There are one or more stop strings in the arguments to `generate`, but the generator has "
+                                 "no tokenizer: pass the model's tokenizer to the generator when generating with stop strings.")
+            from transformers.generation.stopping_criteria import StopStringCriteria
+            self._stop_strings = StopStringCriteria(stop_strings=stop_strings, tokenizer=self.tokenizer)
         if max_new_tokens is not None:
             max_length = input_ids.shape[1] + int(max_new_tokens)
         past_key_values = model_kwargs.get("past_key_values")
@@ -199,8 +205,11 @@ class SubSpecSDGenerator:
         toks = sampled_tokens[0].tolist()
         for j, t in enumerate(toks):
             cur_len = base + j + 1
-            if (max_length is not None and cur_len >= max_length) or \
-                    (self.eos_token_id is not None and t == int(self.eos_token_id)):
+            stop = (max_length is not None and cur_len >= max_length) or \
+                (self.eos_token_id is not None and t == int(self.eos_token_id))
+            if not stop and getattr(self, "_stop_strings", None) is not None:
+                stop = bool(self._stop_strings(input_ids[:, :cur_len], None).any())    # the text so far ends in a stop string
+            if stop:
                 prune = len(toks) - j - 1
                 if prune > 0:
                     input_ids = input_ids[:, :-prune]

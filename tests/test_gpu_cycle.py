@@ -129,7 +129,7 @@ def test_generator_argument_errors():
         gen.generate(ids, do_sample=False, past_key_values=kv)                  # no max_length
     with pytest.raises(ValueError):
         gen.generate(ids, max_new_tokens=4, do_sample=False)                    # no cache
-    with pytest.raises(NotImplementedError):
+    with pytest.raises(ValueError):                                             # stop strings need the tokenizer
         gen.generate(ids, max_new_tokens=4, do_sample=False, stop_strings=["x"], past_key_values=kv)
     with pytest.raises(ValueError):                                             # the warper rejects T <= 0
         gen.generate(ids, max_new_tokens=4, do_sample=True, temperature=0.0, past_key_values=kv)
@@ -265,3 +265,61 @@ def test_agreeing_draft_accepts_deep_paths():
     assert log1["avg_sampled"] <= 2.0
     agree = (deep == shallow).float().mean().item()
     assert agree >= 0.9, agree                                      # bf16 near-ties may flip a token late in the sequence
+
+
+def _letter_tokenizer():
+    """An in-memory tokenizer (nothing is downloaded): single letters plus a few merged pairs, decoded by
+    concatenation."""
+    import string
+    from tokenizers import Tokenizer, decoders, models
+    from transformers import PreTrainedTokenizerFast
+    vocab = {c: i for i, c in enumerate(string.ascii_lowercase + string.ascii_uppercase + " .,;")}
+    merges = [("t", "h"), ("e", "r"), ("S", "T"), ("O", "P"), ("a", "n"), ("i", "n"), ("o", "u"), ("e", "n")]
+    for a, b in merges:
+        vocab[a + b] = len(vocab)
+    tok = Tokenizer(models.BPE(vocab=vocab, merges=merges))
+    tok.decoder = decoders.Fuse()
+    return PreTrainedTokenizerFast(tokenizer_object=tok), len(vocab)
+
+
+@pytest.mark.parametrize("driver", ["v1", "v2"])
+def test_stop_strings_end_generation_where_huggingface_says(driver):
+    """``stop_strings`` go through HuggingFace's StopStringCriteria token by token over each emitted block
+    (generators/base.py:94-101,265-299): the output is the unconstrained output cut right after the first token that
+    completes a stop string -- also when that token sits in the middle of an accepted path."""
+    from subspec_amd.generator_v2 import SubSpecSDGeneratorV2
+    from subspec_amd import quant
+    from subspec_amd.model import QUANTIZED, init_weights
+    tok, n_vocab = _letter_tokenizer()
+    cfg = DecoderConfig(num_hidden_layers=2, hidden_size=256, num_attention_heads=2, num_key_value_heads=1, head_dim=128,
+                        intermediate_size=512, vocab_size=n_vocab)
+    w = init_weights(cfg, 11, DEV)
+    for layer in w["layers"]:                                   # an agreeing draft: long accepted paths
+        for name in QUANTIZED:
+            t = layer[name + ".weight"]
+            layer[name + ".weight"] = quant.dequantize(*quant.quantize_int4_g64(t)).to(t.dtype)
+    prompt = torch.randint(0, n_vocab, (1, 12), generator=torch.Generator().manual_seed(2)).to(DEV)
+
+    def run(stop):
+        kv = create_kv_cache("static", max_cache_len=256, config=cfg, device=DEV, dtype=torch.bfloat16)
+        target, draft, _ = build_models(cfg, kv, device=DEV, weights=w)
+        cls, extra = (SubSpecSDGenerator, {}) if driver == "v1" else (SubSpecSDGeneratorV2, dict(postspec_steps=2))
+        gen = cls(target, tok, SubSpecSDDraftModel(draft), DraftParams(temperature=0.2, max_depth=6, topk_len=4),
+                  generator_kwargs=extra)
+        wandb_logger.clear_log_data()
+        out = gen.generate(prompt, max_new_tokens=48, do_sample=False, stop_strings=stop, past_key_values=kv)[0].cpu()
+        return out, kv.get_seq_length(), dict(wandb_logger.log_data)
+
+    free, _, log = run(None)
+    assert free.numel() == 60 and log["avg_sampled"] > 2.0            # blocks of several tokens
+    text = tok.decode(free[12:].tolist())
+    # a stop string from the middle of the generated text, spanning several tokens
+    stop = tok.decode(free[30:33].tolist())
+    first = text.index(stop) + len(stop)
+    # the token that completes the first occurrence
+    ends = [len(tok.decode(free[12:j + 1].tolist())) for j in range(12, 60)]
+    cut = 12 + next(i for i, e in enumerate(ends) if e >= first)
+    out, seq_len, _ = run([stop, "no such text QQQ"])
+    assert torch.equal(out, free[:cut + 1]), (stop, cut, out.numel())
+    assert tok.decode(out[12:].tolist()).endswith(stop)
+    assert seq_len == out.numel() - 1                                  # the cache holds exactly the kept rows
