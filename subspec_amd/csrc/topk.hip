@@ -10,7 +10,7 @@
 //
 //   1. topk_slice_kernel - grid (slices, B*L), 512 threads.  A workgroup streams its slice of one
 //      row once.  A lower bound of the slice's k-th best is taken from the per-thread maxima of a
-//      16K-element sample; 16-bit rows are then screened eight elements at a time with packed
+//      sample of the first U tiles of every thread; 16-bit rows are then screened eight elements at a time with packed
 //      unsigned maxima against the bit pattern of that bound, and the few survivors go to a
 //      candidate list in LDS.  Two checkpoints tighten the bound to the exact k-th best so far; at
 //      the end the list is pruned to the slice's exact top-k in (key, index) order.
@@ -134,7 +134,7 @@ __device__ int prune_list(uint64_t* list, int count, uint64_t cut, int* counter)
   return *counter;
 }
 
-template <int DT, int VEC>
+template <int DT, int VEC, int U>
 __global__ __launch_bounds__(kTopkThreads) void topk_slice_kernel(
     const void* __restrict__ probs, const void* __restrict__ parent_probs, int64_t vocab, int leaves, int splits,
     int64_t chunk, int k, uint64_t* __restrict__ cand, int32_t* __restrict__ cand_count,
@@ -155,13 +155,14 @@ __global__ __launch_bounds__(kTopkThreads) void topk_slice_kernel(
   const float q = Elem<DT>::load(parent_probs, row);
   const uint32_t flat0 = (uint32_t)((int64_t)leaf * vocab + c0);
 
-  // ---- threshold from a sample: the per-thread maxima over the first 4 tiles.  Each wavefront
+  // ---- threshold from a sample: the per-thread maxima over the first U tiles.  Each wavefront
   // finds, by a 16-step bit search with ballots (no memory traffic), the largest 16-bit key prefix
   // that at least m = ceil(k/4) of its lanes reach; the ceil(k/m)-th largest of those prefixes is
   // reached by at least k elements of the slice, hence a valid lower bound for its k-th best.
-  // The sample IS the first group of the streaming loop below: its four tiles stay in registers
+  // The sample IS the first group of the streaming loop below: its tiles stay in registers
   // and are scanned once the threshold is known, so nothing is read twice.
-  constexpr int U = 4;
+  // U tiles per thread in flight: 8 for whole rows of a large batch (112 against 117 us at 2048 x 152064 bf16),
+  // 4 for the short slices of a draft step, where 8 would mostly re-read the clamped last tile
   PTile<DT, VEC> t[U];
 #pragma unroll
   for (int i = 0; i < U; ++i) {                        // unconditional loads (clamped index): back to back
@@ -222,7 +223,7 @@ __global__ __launch_bounds__(kTopkThreads) void topk_slice_kernel(
       }
     }
   };
-  // fast path: four tiles per thread in flight, no bookkeeping between groups.  For 16-bit rows a
+  // fast path: U tiles per thread in flight, no bookkeeping between groups.  For 16-bit rows a
   // tile is first screened with packed unsigned maxima against the bit pattern of the threshold
   // (five instructions for eight elements); only tiles that may hold a survivor are unpacked.
   uint32_t screen = 0;                                 // (pattern - 1) in both halves; 0: screen nothing out
@@ -386,11 +387,16 @@ static int run_topk(const void* probs, const void* parent_probs, int64_t batch, 
   const dim3 grid(pl.splits, (unsigned)(batch * leaves));
   {
     DominantKernelTimer timer(st);
+    constexpr int kVecFull = DT == SUBSPEC_F32 ? 4 : 8;
     if (pl.vec == 1)
-      hipLaunchKernelGGL((topk_slice_kernel<DT, 1>), grid, dim3(kTopkThreads), 0, st, probs, parent_probs, vocab, leaves,
+      hipLaunchKernelGGL((topk_slice_kernel<DT, 1, 4>), grid, dim3(kTopkThreads), 0, st, probs, parent_probs, vocab, leaves,
                          pl.splits, pl.chunk, k, cand, cand_count, token_ids, topk_probs, parent_indices);
+    else if (pl.chunk / kVecFull >= 2 * (int64_t)kTopkThreads * 8)
+      hipLaunchKernelGGL((topk_slice_kernel<DT, kVecFull, 8>), grid, dim3(kTopkThreads), 0, st, probs,
+                         parent_probs, vocab, leaves, pl.splits, pl.chunk, k, cand, cand_count, token_ids, topk_probs,
+                         parent_indices);
     else
-      hipLaunchKernelGGL((topk_slice_kernel<DT, (DT == SUBSPEC_F32 ? 4 : 8)>), grid, dim3(kTopkThreads), 0, st, probs,
+      hipLaunchKernelGGL((topk_slice_kernel<DT, kVecFull, 4>), grid, dim3(kTopkThreads), 0, st, probs,
                          parent_probs, vocab, leaves, pl.splits, pl.chunk, k, cand, cand_count, token_ids, topk_probs,
                          parent_indices);
   }

@@ -73,6 +73,19 @@ template <int DT> struct Tile16x8 {
   // Makes the packed registers opaque to the optimiser so that the unpacked floats of one pass
   // are not kept alive for the next one (that would double the register footprint of the slice).
   __device__ __forceinline__ void fence() { asm volatile("" : "+v"(r.x), "+v"(r.y), "+v"(r.z), "+v"(r.w)); }
+  // -inf (masked logits) and anything below kFloorBits become a large finite negative, two values per
+  // instruction: as unsigned 16-bit patterns the negative floats are ordered by magnitude, so an unsigned
+  // minimum with the pattern of the floor leaves positive values alone and pulls -inf up to the floor.
+  // bf16: floor -2^100 (its product with log2(e) stays finite in fp32); fp16: the lowest finite value.
+  static constexpr uint32_t kFloorBits = DT == SUBSPEC_BF16 ? 0xf180f180u : 0xfbfffbffu;
+  __device__ __forceinline__ void floor_neg_inf() {
+    typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+    const u16x2 lim = __builtin_bit_cast(u16x2, kFloorBits);
+    r.x = __builtin_bit_cast(uint32_t, __builtin_elementwise_min(__builtin_bit_cast(u16x2, r.x), lim));
+    r.y = __builtin_bit_cast(uint32_t, __builtin_elementwise_min(__builtin_bit_cast(u16x2, r.y), lim));
+    r.z = __builtin_bit_cast(uint32_t, __builtin_elementwise_min(__builtin_bit_cast(u16x2, r.z), lim));
+    r.w = __builtin_bit_cast(uint32_t, __builtin_elementwise_min(__builtin_bit_cast(u16x2, r.w), lim));
+  }
 };
 template <> struct Tile<SUBSPEC_BF16, 8> : Tile16x8<SUBSPEC_BF16> {};
 template <> struct Tile<SUBSPEC_F16, 8> : Tile16x8<SUBSPEC_F16> {};
@@ -215,14 +228,27 @@ template <int DT, int VEC, bool WARP>
 __device__ __forceinline__ float tile_accumulate(const Tile<DT, VEC>& t, float mb, const Divisor& temperature,
                                                  float (&s)[2], float (&u)[2]) {
   float x[VEC];
+  // Packed 16-bit tiles are floored while still packed (half an instruction per element instead of one
+  // fp32 maximum): t stays finite, and whatever lies that far below the reference contributes exp2(t) == 0
+  // and t * 0 == 0 either way.  The maximum of a fully masked tile is then the floor instead of -inf; it
+  // can only surface as a row maximum when the whole row is masked.
+  constexpr bool kPackedFloor = !WARP && DT != SUBSPEC_F32 && VEC == 8;
+  if constexpr (kPackedFloor) {
+    Tile<DT, VEC> tc = t;
+    tc.floor_neg_inf();
 #pragma unroll
-  for (int k = 0; k < VEC; ++k) x[k] = warped<DT, WARP>(t.get(k), temperature);
+    for (int k = 0; k < VEC; ++k) x[k] = tc.get(k);
+  } else {
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) x[k] = warped<DT, WARP>(t.get(k), temperature);
+  }
   float tmax = x[0];
 #pragma unroll
   for (int k = 1; k < VEC; ++k) tmax = fmaxf(tmax, x[k]);
 #pragma unroll
   for (int k = 0; k < VEC; ++k) {
-    const float tt = fmaxf(fmaf(x[k], kLog2e, mb), -200.f);
+    const float raw = fmaf(x[k], kLog2e, mb);
+    const float tt = kPackedFloor ? raw : fmaxf(raw, -200.f);
     const float e = __builtin_amdgcn_exp2f(tt);
     s[k & 1] += e;
     u[k & 1] = fmaf(tt, e, u[k & 1]);
@@ -260,25 +286,39 @@ __global__ __launch_bounds__(kRowThreads) void row_partial_kernel(
   }
 
   float vmax = -INFINITY;
-  int64_t best_tile = 0;
+  int best_tile = 0;                                   // tile index inside the slice (a slice has < 2^31 elements)
   float s[2], u[2];
+  const int nt = (int)ntiles;
+  constexpr int kStep = kRowThreads * U;               // tiles per trip of the whole workgroup
+  const int n_full = nt / kStep;                       // trips in which every thread's U tiles exist
   for (int pass = 0; pass < 2; ++pass) {
     const float mb = -ref * kLog2e;
     s[0] = s[1] = u[0] = u[1] = 0.f;
-    for (int64_t j0 = tid; j0 < ntiles; j0 += (int64_t)kRowThreads * U) {
+    // full trips: no bounds, the U loads of a thread go out back to back
+    for (int it = 0; it < n_full; ++it) {
+      const int j0 = it * kStep + tid;
       Tile<DT, VEC> t[U];
 #pragma unroll
-      for (int i = 0; i < U; ++i) {                    // unconditional loads (clamped index): back to back
-        const int64_t j = j0 + (int64_t)i * kRowThreads;
-        t[i].load(logits, base + min(j, ntiles - 1) * VEC);
-      }
-#pragma unroll
-      for (int i = 0; i < U; ++i)
-        if (j0 + (int64_t)i * kRowThreads >= ntiles) t[i].fill_neg_inf();
+      for (int i = 0; i < U; ++i) t[i].load(logits, base + (int64_t)(j0 + i * kRowThreads) * VEC);
 #pragma unroll
       for (int i = 0; i < U; ++i) {
         const float tmax = tile_accumulate<DT, VEC, WARP>(t[i], mb, vp.temperature, s, u);
-        if (tmax > vmax) { vmax = tmax; best_tile = j0 + (int64_t)i * kRowThreads; }
+        if (tmax > vmax) { vmax = tmax; best_tile = j0 + i * kRowThreads; }
+      }
+    }
+    // the last, ragged trip: clamped loads, missing tiles count as -inf
+    if (n_full * kStep + tid < nt) {
+      const int j0 = n_full * kStep + tid;
+      Tile<DT, VEC> t[U];
+#pragma unroll
+      for (int i = 0; i < U; ++i) t[i].load(logits, base + (int64_t)min(j0 + i * kRowThreads, nt - 1) * VEC);
+#pragma unroll
+      for (int i = 0; i < U; ++i)
+        if (j0 + i * kRowThreads >= nt) t[i].fill_neg_inf();
+#pragma unroll
+      for (int i = 0; i < U; ++i) {
+        const float tmax = tile_accumulate<DT, VEC, WARP>(t[i], mb, vp.temperature, s, u);
+        if (tmax > vmax) { vmax = tmax; best_tile = j0 + i * kRowThreads; }
       }
     }
     if (pass == 1) break;
@@ -291,10 +331,10 @@ __global__ __launch_bounds__(kRowThreads) void row_partial_kernel(
   int idx = 0x7fffffff;
   if (vmax == m && m != -INFINITY) {                  // first index of the maximum inside this thread's tiles
     Tile<DT, VEC> tb;
-    tb.load(logits, base + best_tile * VEC);
+    tb.load(logits, base + (int64_t)best_tile * VEC);
 #pragma unroll
     for (int k = VEC - 1; k >= 0; --k)
-      if (warped<DT, WARP>(tb.get(k), vp.temperature) == m) idx = (int)(c0 + best_tile * VEC + k);
+      if (warped<DT, WARP>(tb.get(k), vp.temperature) == m) idx = (int)(c0 + (int64_t)best_tile * VEC + k);
   }
   const float ssum = block_sum<kRowThreads>(s[0] + s[1], red_f);
   const float usum = block_sum<kRowThreads>(u[0] + u[1], red_f);
@@ -672,8 +712,13 @@ static bool make_plan(const void* logits, int dtype, int64_t total_rows, int64_t
 
 template <int DT, int VEC>
 static void launch_partial(dim3 grid, hipStream_t st, const void* logits, const VerifyParams& vp, Part1* p1, Part2* p2) {
+  // loads in flight per thread: 8 when a slice is long enough for whole trips of that size (whole rows of a
+  // large batch: 111 against 113 us at 2048 x 152064 bf16), 4 for the short slices of a few rows split many ways
+  const bool long_slices = vp.chunk / VEC >= 2 * (int64_t)kRowThreads * 8;
   if (vp.temperature.t != 1.0f)
     hipLaunchKernelGGL((row_partial_kernel<DT, VEC, 4, true>), grid, dim3(kRowThreads), 0, st, logits, vp, p1, p2);
+  else if (long_slices)
+    hipLaunchKernelGGL((row_partial_kernel<DT, VEC, 8, false>), grid, dim3(kRowThreads), 0, st, logits, vp, p1, p2);
   else
     hipLaunchKernelGGL((row_partial_kernel<DT, VEC, 4, false>), grid, dim3(kRowThreads), 0, st, logits, vp, p1, p2);
 }
