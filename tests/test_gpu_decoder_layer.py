@@ -49,6 +49,33 @@ def test_native_layer_stack_matches_module_path(n, prefix):
     assert (got.argmax(-1) == ref.argmax(-1)).float().mean().item() >= 0.9
 
 
+@pytest.mark.parametrize("n_slots,lo,hi", [(289, 283, 289), (289, 225, 289), (400, 130, 190), (512, 448, 512)])
+def test_windows_of_large_trees(n_slots, lo, hi):
+    """A window of rows of a tree with up to 512 occupied slots (a draft level of a depth-48 tree, a
+    post-speculation window): the one-call layers against the whole tree decoded module by module."""
+    print("decoder layer large tree", n_slots, lo, hi, flush=True)
+    prefix = 70
+    kv = create_kv_cache("static", max_cache_len=640, config=CFG, device=DEV, dtype=torch.bfloat16)
+    target, draft, w = build_models(CFG, kv, seed=n_slots, device=DEV)
+    g = torch.Generator().manual_seed(n_slots)
+    target.prefill(torch.randint(0, CFG.vocab_size, (prefix,), generator=g).to(DEV), 0)
+    parents, _, depths = W.random_tree(g, n=n_slots, max_depth=48, max_children=6, vocab=CFG.vocab_size, chain_depth=40)
+    toks = torch.randint(0, CFG.vocab_size, (n_slots,), generator=g).to(DEV)
+    anc = ops.ancestor_bits_tensor(parents, device=DEV)
+    dep = torch.tensor(depths, device=DEV)
+    # the whole tree, module by module (rows beyond one 64-row launch): fills the cache rows of every node
+    ref = draft.tree_forward(toks, dep, anc, prefix)
+    ref_cache = kv.cache.data.clone()
+    # the window again through the one-call layers, over the cache the first pass left
+    got = draft.tree_forward(toks[lo:hi], dep[lo:hi], anc[lo:hi].contiguous(), prefix, first_slot=lo, n_tree_slots=n_slots)
+    scale = ref.float().abs().amax().item()
+    assert (got.float() - ref[lo:hi].float()).abs().amax().item() <= 2e-2 * scale
+    assert (got.argmax(-1) == ref[lo:hi].argmax(-1)).float().mean().item() >= 0.9
+    dc = (kv.cache.data.float() - ref_cache.float()).abs()
+    assert dc[..., :prefix + lo, :].amax().item() == 0 and dc[..., prefix + hi:, :].amax().item() == 0
+    assert dc.amax().item() <= 2e-2 * ref_cache.float().abs().amax().item()
+
+
 def test_single_layer_against_float32_oracle():
     n, prefix = 12, 29
     kv, draft, toks, depths, anc = _setup(5, prefix, n)
