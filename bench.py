@@ -57,6 +57,9 @@ def parse():
     ap.add_argument("--max-verify-tokens", type=int, default=64,
                     help="e2e workload: cap on the nodes verified per cycle (0: the whole tree); the reference's offloading "
                          "configurations use depth 48, k 6 and no cap: --tree-depth 48 --tree-k 6 --max-verify-tokens 0")
+    ap.add_argument("--hqq-optimize", action="store_true",
+                    help="e2e workload: refine the draft's zero points with hqq's proximal solver (what the reference's "
+                         "quantizer does by default; worth it for real weights, --checkpoint)")
     ap.add_argument("--keep-layers", type=int, default=14, help="e2e workload: target layers kept resident; the rest stream")
     ap.add_argument("--workload", default="verify-cycle", choices=["verify-cycle", "attention", "int4", "dense", "greedy", "sampling", "e2e"],
                     help="verify-cycle (default, BASELINE config 2) is the benchmark line; the others time one "
@@ -234,7 +237,7 @@ def bench_e2e(args):
                 w[name + ".weight"] = quant.dequantize(*quant.quantize_int4_g64(t)).to(t.dtype)
     kv = create_kv_cache("static", max_cache_len=2048 + args.new_tokens + 512 + 8, config=cfg, device=dev, dtype=torch.bfloat16)
     target, draft, _ = build_models(cfg, kv, seed=0, device=dev, first_streamed=min(args.keep_layers, cfg.num_hidden_layers),
-                                    weights=weights)
+                                    weights=weights, hqq_optimize=args.hqq_optimize)
     print(f"# models built in {time.perf_counter() - t0:.1f} s", file=sys.stderr, flush=True)
     prompt = torch.randint(0, cfg.vocab_size, (1, 2048), generator=torch.Generator().manual_seed(0)).to(dev)
     for method, vk in (("exact", None), ("lossy", dict(threshold=0.3, window_size=6, threshold_method="entropy"))):

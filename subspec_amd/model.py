@@ -82,13 +82,14 @@ def init_weights(cfg: DecoderConfig, seed: int, device, dtype=torch.bfloat16) ->
             "lm_head": rnd(cfg.vocab_size, cfg.hidden_size)}
 
 
-def quantize_layers(layers: List[Dict[str, torch.Tensor]]) -> List[Dict[str, torch.Tensor]]:
-    """int4 g64 copies of the four projections of every layer (norms and biases are shared)."""
+def quantize_layers(layers: List[Dict[str, torch.Tensor]], optimize: bool = False) -> List[Dict[str, torch.Tensor]]:
+    """int4 g64 copies of the four projections of every layer (norms and biases are shared); ``optimize``
+    refines the zero points as hqq does by default (quant.refine_zero_proximal)."""
     out = []
     for w in layers:
         q = {k: v for k, v in w.items() if not any(k == n + ".weight" for n in QUANTIZED)}
         for n in QUANTIZED:
-            wq, sz = quant.pack_tiled(*quant.quantize_int4_g64(w[n + ".weight"]))
+            wq, sz = quant.pack_tiled(*quant.quantize_int4_g64(w[n + ".weight"], optimize=optimize))
             q[n + ".wq"], q[n + ".sz"] = wq, sz
             q[n + ".out_features"] = w[n + ".weight"].shape[0]
         out.append(q)
@@ -339,11 +340,11 @@ def weights_from_tensors(cfg: DecoderConfig, tensors: Dict[str, torch.Tensor], d
 
 
 def build_models(cfg: DecoderConfig, kv: KVManager, seed: int = 0, device="cuda:0", dtype=torch.bfloat16,
-                 first_streamed: Optional[int] = None, weights: Optional[dict] = None):
+                 first_streamed: Optional[int] = None, weights: Optional[dict] = None, hqq_optimize: bool = False):
     """Target (bf16, layers >= first_streamed in pinned host memory) and substitute draft (same
     weights, int4 g64, resident) over one shared KV cache."""
     w = init_weights(cfg, seed, device, dtype) if weights is None else weights     # e.g. from load_hf_checkpoint
-    draft_layers = quantize_layers(w["layers"])
+    draft_layers = quantize_layers(w["layers"], optimize=hqq_optimize)
     streamer = None
     layers = w["layers"]
     if first_streamed is not None and first_streamed < cfg.num_hidden_layers:

@@ -8,11 +8,15 @@ compute_dtype, device)`` (specdecodes/helpers/quantizers/hqq/__init__.py:17-120)
 specdecodes/helpers/recipes/subspec/hqq_4bit_postspec.py:17-58 (here a plain dict
 ``{"nbits": 4, "group_size": 64, "axis": 1}``).
 
-The quantizer is the plain affine min/max rule of the benchmark definition: per (output row,
+The quantizer starts from the plain affine min/max rule of the benchmark definition: per (output row,
 64-wide input group) ``s = (max - min) / 15``, ``z = -min / s`` (both stored as fp16),
-``Wq = clamp(round(W / s + z), 0, 15)``.  hqq's proximal refinement of the zero point is a
-separate, un-vendored algorithm and is not reproduced; the kernels only rely on the affine
-dequantization ``(Wq - z) * s``.
+``Wq = clamp(round(W / s + z), 0, 15)``.  With ``optimize=True`` the zero point is then refined by the
+half-quadratic proximal iteration that hqq (``hqq==0.2.6`` in the reference's requirements, not part
+of the reference tree and not installed here) applies by default: its published algorithm
+(Badri & Shaji, "Half-Quadratic Quantization of Large Machine Learning Models", 2023;
+``optimize_weights_proximal`` with lp_norm 0.7, beta 10, kappa 1.01, 20 iterations, stop when the mean
+absolute error stops falling) restated, NOT checked against hqq's output: parity unpinned.  The
+kernels only rely on the affine dequantization ``(Wq - z) * s``, whichever zero point is stored.
 """
 from __future__ import annotations
 
@@ -26,8 +30,41 @@ from . import ops
 GROUP = 64
 
 
-def quantize_int4_g64(weight: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
-    """``weight`` [N, K] -> (codes uint8 [N, K] in 0..15, scale fp16 [N, K/64], zero fp16 [N, K/64])."""
+HQQ_OPT_PARAMS = {"lp_norm": 0.7, "beta": 1e1, "kappa": 1.01, "iters": 20}     # hqq's defaults
+
+
+def refine_zero_proximal(w: torch.Tensor, s: torch.Tensor, zero: torch.Tensor, opt_params: Optional[dict] = None) -> torch.Tensor:
+    """hqq's half-quadratic solver for the zero point, scale fixed: ``w`` [N, G, 64] fp32, ``s`` / ``zero`` [N, G] fp32.
+    Alternates  W_e = shrink_lp(W - W_r)  (the generalized soft threshold of the l_p error, p < 1)  and
+    zero = mean(Wq - (W - W_e) / s)  over the group, with beta growing by kappa, until the mean absolute
+    reconstruction error stops falling.  Returns the refined zero [N, G] fp32."""
+    p = dict(HQQ_OPT_PARAMS, **(opt_params or {}))
+    lp, beta, kappa, iters = float(p["lp_norm"]), float(p["beta"]), float(p["kappa"]), int(p["iters"])
+    inv_s = (1.0 / s).unsqueeze(-1)
+    z = zero.unsqueeze(-1).clone()
+    best_err, best_z = float("inf"), z
+    for _ in range(iters):
+        wq = torch.clamp(torch.round(w * inv_s + z), 0, 15)
+        w_r = (wq - z) / inv_s
+        err = float((w - w_r).abs().mean())
+        if err < best_err:
+            best_err, best_z = err, z
+        else:
+            break                                             # the error stopped falling: keep the best zero seen
+        d = w - w_r
+        if lp == 1.0:
+            w_e = torch.sign(d) * torch.relu(d.abs() - 1.0 / beta)
+        else:
+            w_e = torch.sign(d) * torch.relu(d.abs() - (1.0 / beta) * d.abs().clamp_min(1e-30).pow(lp - 1.0))
+        z = (wq - (w - w_e) * inv_s).mean(-1, keepdim=True)
+        beta *= kappa
+    return best_z.squeeze(-1)
+
+
+def quantize_int4_g64(weight: torch.Tensor, optimize: bool = False,
+                      opt_params: Optional[dict] = None) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """``weight`` [N, K] -> (codes uint8 [N, K] in 0..15, scale fp16 [N, K/64], zero fp16 [N, K/64]).
+    ``optimize``: refine the zero point as hqq does (see the module text); the codes then follow the refined zero."""
     N, K = weight.shape
     if K % GROUP:
         raise ValueError(f"in_features={K} must be a multiple of {GROUP}")
@@ -36,6 +73,8 @@ def quantize_int4_g64(weight: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor,
     scale = ((hi - lo) / 15.0).clamp_min(1e-8).to(torch.float16)
     s = scale.float()
     zero = (-lo / s).to(torch.float16)
+    if optimize:
+        zero = refine_zero_proximal(w, s, zero.float(), opt_params).to(torch.float16)
     codes = torch.clamp(torch.round(w / s.unsqueeze(-1) + zero.float().unsqueeze(-1)), 0, 15).to(torch.uint8)
     return codes.reshape(N, K), scale, zero
 
@@ -115,9 +154,10 @@ class HqqInt4Linear(nn.Module):
         self.register_buffer("bias", bias)
 
     @classmethod
-    def from_linear(cls, linear: nn.Linear, compute_dtype: torch.dtype = torch.bfloat16, device=None):
+    def from_linear(cls, linear: nn.Linear, compute_dtype: torch.dtype = torch.bfloat16, device=None,
+                    optimize: bool = False):
         device = device or linear.weight.device
-        codes, scale, zero = quantize_int4_g64(linear.weight.data.to(device))
+        codes, scale, zero = quantize_int4_g64(linear.weight.data.to(device), optimize=optimize)
         wq, sz = pack_tiled(codes, scale, zero)
         bias = None if linear.bias is None else linear.bias.data.to(device=device, dtype=compute_dtype)
         return cls(linear.in_features, linear.out_features, wq.to(device), sz.to(device), bias)
@@ -139,7 +179,8 @@ class HqqInt4Linear(nn.Module):
 class HqqQuantizer:
     """``quantize_model(model, quant_config, compute_dtype, device)`` as the reference recipe calls it
     (specdecodes/helpers/recipes/base_recipe.py:43-52): ``quant_config`` maps module names to a
-    per-layer config; every named ``nn.Linear`` is replaced in place."""
+    per-layer config; every named ``nn.Linear`` is replaced in place.  A config may carry ``"optimize"``
+    (default True, as hqq's ``Quantizer.quantize``): refine the zero points with hqq's proximal solver."""
 
     @classmethod
     def quantize_model(cls, model: nn.Module, quant_config: Dict[str, dict], compute_dtype: torch.dtype, device):
@@ -153,5 +194,6 @@ class HqqQuantizer:
             linear = getattr(parent, child)
             if not isinstance(linear, nn.Linear):
                 raise TypeError(f"{name} is {type(linear).__name__}, expected nn.Linear")
-            setattr(parent, child, HqqInt4Linear.from_linear(linear, compute_dtype, device))
+            optimize = bool(cfg.get("optimize", True)) if isinstance(cfg, dict) else bool(getattr(cfg, "optimize", True))
+            setattr(parent, child, HqqInt4Linear.from_linear(linear, compute_dtype, device, optimize=optimize))
         return model

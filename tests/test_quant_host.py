@@ -75,3 +75,33 @@ def test_hqq_tensor_layout_round_trip():
     assert torch.equal(deq_rows.reshape(N, K), quant.dequantize(codes, scale, zero))
     with pytest.raises(ValueError):
         quant.from_hqq_tensors(packed[:-1], scale, zero, (N, K))
+
+
+def test_proximal_zero_refinement():
+    """The restated hqq solver (parity unpinned against hqq itself): what can be checked is what it promises --
+    the scale and the code range are untouched, the mean absolute reconstruction error never grows against the
+    min/max rule and shrinks on weights with outliers, a group that the min/max rule already reproduces exactly is
+    left alone, and with zero iterations nothing changes."""
+    g = torch.Generator().manual_seed(0)
+    W = torch.randn(96, 512, generator=g) * 0.02
+    W[torch.rand(96, 512, generator=g) < 0.01] *= 6                      # heavy tails, as trained weights have
+    c0, s0, z0 = quant.quantize_int4_g64(W)
+    c1, s1, z1 = quant.quantize_int4_g64(W, optimize=True)
+    assert torch.equal(s0, s1) and int(c1.max()) <= 15 and c1.dtype == torch.uint8
+    e0 = (W - quant.dequantize(c0, s0, z0)).abs().mean().item()
+    e1 = (W - quant.dequantize(c1, s1, z1)).abs().mean().item()
+    assert e1 < 0.99 * e0, (e0, e1)
+    assert not torch.equal(z0, z1)
+    # per group the refined zero is never worse than the starting point by more than fp16 rounding of the zero
+    g0 = (W - quant.dequantize(c0, s0, z0)).abs().reshape(96, 8, 64).mean(-1)
+    g1 = (W - quant.dequantize(c1, s1, z1)).abs().reshape(96, 8, 64).mean(-1)
+    assert (g1 <= g0 * 1.5 + 1e-6).all()
+    # weights that sit exactly on a 16-level grid are reproduced exactly, refined or not
+    levels = torch.randint(0, 16, (8, 128), generator=g).float()
+    levels[:, 0], levels[:, 1], levels[:, 64], levels[:, 65] = 0, 15, 0, 15
+    Wg = (levels - 7.0) * 0.5
+    for opt in (False, True):
+        c, s, z = quant.quantize_int4_g64(Wg, optimize=opt)
+        assert torch.equal(quant.dequantize(c, s, z), Wg)
+    c2, s2, z2 = quant.quantize_int4_g64(W, optimize=True, opt_params={"iters": 0})
+    assert torch.equal(c2, c0) and torch.equal(z2, z0)
