@@ -88,3 +88,29 @@ def test_random_shape_sweep():
     # more than 64 rows (a whole large tree through the draft): several passes of 64 rows
     for i, (N, K, M) in enumerate([(16 * 40, 64 * 9, 65), (4608, 3584, 289), (3584, 18944, 130), (16 * 10, 64 * 3, 512)]):
         _check(N, K, M, torch.bfloat16 if i % 2 == 0 else torch.float16, 950 + i, bias=bool(i % 2))
+
+
+def test_quantizer_default_refines_zero_points():
+    """HqqQuantizer.quantize_model refines the zero points unless told not to (as hqq does); the module then
+    computes the affine dequantization of those tensors, and its output is at least as close to the unquantized
+    layer as with the min/max rule on weights with heavy tails."""
+    g = torch.Generator().manual_seed(12)
+    W = torch.randn(128, 512, generator=g) * 0.02
+    W[torch.rand(128, 512, generator=g) < 0.01] *= 6
+    x = torch.randn(16, 512, generator=g).to(torch.bfloat16)
+    want = x.float() @ W.T
+    errs = {}
+    for optimize in (True, False):
+        model = torch.nn.Sequential()
+        lin = torch.nn.Linear(512, 128, bias=False)
+        lin.weight.data.copy_(W)
+        model.add_module("p", lin)
+        cfg = {"nbits": 4, "group_size": 64, "axis": 1}
+        if not optimize:
+            cfg["optimize"] = False
+        quant.HqqQuantizer.quantize_model(model, {"p": cfg}, torch.bfloat16, DEV)
+        y = model.p(x.to(DEV)).float().cpu()
+        ref = oi.linear(x, *quant.quantize_int4_g64(W, optimize=optimize))
+        assert (y - ref).abs().amax() <= 1e-2 * ref.abs().amax()
+        errs[optimize] = (y - want).pow(2).mean().item()
+    assert errs[True] <= errs[False] * 1.02, errs
