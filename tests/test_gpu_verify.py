@@ -188,6 +188,39 @@ def test_masked_logits_and_single_node_tree():
     assert out["entropy"][0, 0] == 0.0
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("rows,vocab", [(5, 70000), (300, 152064), (3, 8200)])
+def test_mostly_masked_rows(dtype, rows, vocab):
+    """Rows in which almost every logit is -inf (a constrained vocabulary): whole slices and whole trips of a slice
+    hold nothing but -inf, the few finite logits sit in different slices, some next to the slice ends.  Few rows
+    split a row over many workgroups, many rows take one workgroup per row (the long-slice variant of the pass)."""
+    g = torch.Generator().manual_seed(rows + vocab)
+    parents, toks, _ = W.random_tree(g, n=rows, max_depth=6, max_children=4, vocab=vocab, chain_depth=4)
+    kids = ov.children_from_parents(parents)
+    logits = torch.full((rows, vocab), float("-inf"))
+    for r in range(rows):
+        live = torch.randint(0, vocab, (4,), generator=g).tolist() + [0, vocab - 1] + [toks[c] for c in kids[r]]
+        logits[r, live] = torch.randn(len(live), generator=g) * 3
+        if kids[r] and r % 2 == 0:
+            logits[r, toks[kids[r][0]]] = 9.0                      # drafted child wins: walks go deep
+    logits = logits.to(dtype)
+    for method, vk in (("exact", {}), ("lossy", {"threshold_method": "entropy", "threshold": 0.3, "window_size": 2}),
+                       ("lossy", {"threshold_method": "prob", "threshold": 0.05, "window_size": 1})):
+        print("masked rows", dtype, rows, vocab, method, flush=True)
+        out = _run(logits, toks, parents, verify_method=method, exact_entropy=True,
+                   threshold_method=vk.get("threshold_method", "prob"), threshold=vk.get("threshold", 0.0),
+                   window_size=vk.get("window_size", 1))
+        want = ov.verify_logits(logits, toks, parents, verify_method=method, verify_kwargs=vk)
+        assert _unpack(out) == (want[0], want[1], want[2]), (rows, vocab, method)
+        assert out["target"][0].tolist() == ov.target_probs(logits).argmax(-1).tolist()
+        if vk.get("threshold_method") == "entropy":
+            ref_h = torch.tensor(ov.normalized_entropy(ov.target_probs(logits)))
+            if dtype == torch.float32:                       # one fp32 pass against torch's: equal up to summation order
+                assert torch.allclose(out["entropy"][0], ref_h, rtol=1e-4, atol=1e-6)
+            else:
+                _assert_entropy_matches(out["entropy"][0], ref_h, "masked")
+
+
 def test_verify_tree_host_interface_and_errors():
     cfg = W.greedy_config(5)
     tree = Tree(torch.tensor(cfg["tokens"][0]))
