@@ -1,0 +1,98 @@
+"""GPU: seeded random differential run of the verifier and the top-k expansion against the oracle.
+
+Shapes, dtypes, tree forms and parameters are drawn at random (fixed seeds): trees of 1 to 300 nodes, vocabularies
+that are and are not multiples of the vector width, peaked / masked / heavily tied rows, an EOS token that may sit
+on the accepted path, exact and lossy verification with both gates, and windows of a larger tree (``skip_nodes``,
+a root inside the window, fewer scored rows than nodes) as the post-speculating driver verifies them.  Every case
+must reproduce the oracle's tokens, contexts and lengths exactly."""
+import random
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+from oracle import topk as ot
+from oracle import verify as ov
+from subspec_amd import ops, workloads as W
+
+DEV = "cuda:0"
+
+
+def _case(seed):
+    rng = random.Random(seed)
+    g = torch.Generator().manual_seed(seed)
+    n = rng.choice([1, 2, 5, 17, 33, 64, 65, 100, 130, 257, 300])
+    vocab = rng.choice([7, 64, 100, 1000, 4096, 5000, 8191, 8192, 32000, 50257])
+    dtype = rng.choice([torch.bfloat16, torch.float16, torch.float32])
+    depth = rng.choice([2, 4, 8, 16])
+    ch = min(rng.choice([2, 4, 8]), vocab - 1)
+    while sum(ch ** d for d in range(depth + 1)) < n:
+        depth += 1
+    parents, toks, depths = W.random_tree(g, n=n, max_depth=depth, max_children=ch, vocab=vocab,
+                                          chain_depth=rng.choice([0, min(depth, n - 1)]))
+    kids = ov.children_from_parents(parents)
+    skip, root, rows = 0, 0, n
+    if depths[-1] >= 2 and rng.random() < 0.3:
+        # a window of the tree, as after post-speculation: the levels up to d1 were verified before (skip_nodes), the
+        # root is a node behind them, and the levels beyond d2 were added after the forward and have no scored row
+        upto = [sum(1 for d in depths if d <= lv) for lv in range(depths[-1] + 1)]     # level order: nodes of depth <= lv
+        d1 = rng.randrange(0, depths[-1])
+        skip = upto[d1]
+        root = rng.randrange(skip, n)
+        # the reference walks from the root without asking whether its children were scored (tree_verify.py:71-75), so a
+        # window always reaches at least one level below the root
+        d2 = rng.randrange(min(depths[root] + 1, depths[-1]), depths[-1] + 1)
+        rows = upto[d2] - skip
+    logits = torch.randn(rows, vocab, generator=g) * rng.choice([0.3, 1.0, 3.0])
+    mode = rng.choice(["plain", "peaked", "masked", "ties"])
+    for r in range(rows):
+        node = r + skip
+        if mode == "peaked" or (kids[node] and rng.random() < 0.6):
+            j = toks[rng.choice(kids[node])] if kids[node] and rng.random() < 0.8 else rng.randrange(vocab)
+            logits[r, j] += rng.choice([4.0, 8.0, 15.0])
+        if mode == "masked":
+            m = torch.rand(vocab, generator=g) < 0.9
+            m[rng.randrange(vocab)] = False
+            logits[r, m] = float("-inf")
+    logits = logits.to(dtype)
+    if mode == "ties":
+        logits = (logits.float() * 4).round().div(4).to(dtype)          # many exactly equal logits
+    method = rng.choice(["exact", "lossy"])
+    vk = {}
+    if method == "lossy":
+        vk = {"threshold_method": rng.choice(["prob", "entropy"]), "threshold": rng.choice([0.0, 0.05, 0.3, 0.7, 1.5]),
+              "window_size": rng.choice([0, 1, 2, 6])}
+    eos = rng.choice([None, None, toks[rng.randrange(n)]])
+    L = rng.choice([1, 2, 6, 8])
+    k = min(rng.choice([1, 4, 8, 16, 64]), vocab)
+    probs = torch.softmax(torch.randn(1, L, vocab, generator=g) * rng.choice([0.5, 2.0, 6.0]), -1)
+    if mode == "ties":
+        probs = (probs * 64).round() / 64
+    return dict(n=n, vocab=vocab, dtype=dtype, parents=parents, toks=toks, skip=skip, root=root, logits=logits, mode=mode,
+                method=method, vk=vk, eos=eos, probs=probs.to(dtype), parent_probs=torch.rand(1, L, generator=g).to(dtype), k=k)
+
+
+@pytest.mark.parametrize("block", range(4))
+def test_random_cases_match_the_oracle(block):
+    for i in range(100):
+        seed = 7_000_000 + block * 100 + i
+        c = _case(seed)
+        tag = (seed, c["n"], c["vocab"], c["dtype"], c["mode"], c["method"], c["vk"], c["eos"], c["skip"], c["root"],
+               tuple(c["logits"].shape))
+        if i % 20 == 0:
+            print("random case", tag, flush=True)
+        vk = c["vk"]
+        out = ops.tree_verify(c["logits"].to(DEV), torch.tensor(c["toks"], dtype=torch.int32, device=DEV),
+                              torch.tensor(c["parents"], dtype=torch.int32, device=DEV), root=c["root"],
+                              skip_nodes=c["skip"], verify_method=c["method"], exact_entropy=True,
+                              threshold_method=vk.get("threshold_method", "prob"), threshold=vk.get("threshold", 0.0),
+                              window_size=vk.get("window_size", 1), eos_token_id=c["eos"])
+        emitted, accept, total, status = out["counts"][0].tolist()
+        got = (out["tokens"][0, :emitted].tolist(), out["contexts"][0, :emitted].tolist(), (total, accept))
+        want = ov.verify_logits(c["logits"], c["toks"], c["parents"], root=c["root"], eos_token_id=c["eos"],
+                                skip_nodes=c["skip"], verify_method=c["method"], verify_kwargs=vk)
+        assert status == 0 and got == (want[0], want[1], want[2]), tag
+        t, v, p = ops.topk_expand(c["probs"].to(DEV), c["parent_probs"].to(DEV), c["k"])
+        et, ev, ep = ot.topk_expand(c["probs"], c["parent_probs"], c["k"])
+        assert torch.equal(t.cpu(), et) and torch.equal(v.cpu().float(), ev.float()) and torch.equal(p.cpu(), ep), tag
