@@ -96,3 +96,53 @@ def test_random_cases_match_the_oracle(block):
         t, v, p = ops.topk_expand(c["probs"].to(DEV), c["parent_probs"].to(DEV), c["k"])
         et, ev, ep = ot.topk_expand(c["probs"], c["parent_probs"], c["k"])
         assert torch.equal(t.cpu(), et) and torch.equal(v.cpu().float(), ev.float()) and torch.equal(p.cpu(), ep), tag
+
+
+@pytest.mark.parametrize("block", range(2))
+def test_random_attention_and_compaction_cases(block):
+    """Tree attention over random head groupings, prefixes, tree sizes (up to 512 slots) and row windows against the
+    fp32 oracle (1e-2 relative, as the benchmark definition states), contiguous and paged; KV compaction of random
+    ascending contexts bit for bit."""
+    from oracle import attention as oa
+    from oracle import kv as okv
+    for i in range(30):
+        seed = 8_000_000 + block * 100 + i
+        rng = random.Random(seed)
+        g = torch.Generator().manual_seed(seed)
+        dtype = rng.choice([torch.bfloat16, torch.float16])
+        Hkv = rng.choice([1, 2, 4])
+        Hq = Hkv * rng.choice([1, 2, 7, 8])
+        B = rng.choice([1, 1, 2])
+        n_slots = rng.choice([1, 3, 17, 64, 65, 128, 129, 200, 300, 512])
+        P = rng.choice([0, 1, 63, 64, 65, 200, 777])
+        S = P + n_slots + rng.choice([0, 5, 100])
+        depth = rng.choice([3, 8, 40])
+        ch = rng.choice([2, 4, 6])
+        while sum(ch ** d for d in range(depth + 1)) < n_slots:
+            depth += 1
+        parents, _, _ = W.random_tree(g, n=n_slots, max_depth=depth, max_children=ch, vocab=1000,
+                                      chain_depth=min(depth, n_slots - 1))
+        q = torch.randn(B, Hq, n_slots, 128, generator=g).to(dtype)
+        k = torch.randn(B, Hkv, S, 128, generator=g).to(dtype)
+        v = torch.randn(B, Hkv, S, 128, generator=g).to(dtype)
+        k[:, :, P + n_slots:] = 1e3                                   # stale rows beyond the tree must not be read
+        lo = rng.randrange(0, n_slots)
+        hi = rng.randrange(lo + 1, n_slots + 1)
+        tag = (seed, dtype, B, Hq, Hkv, n_slots, P, S, lo, hi)
+        if i % 10 == 0:
+            print("random attention", tag, flush=True)
+        ref = oa.tree_attention(q, k, v, parents, P)[:, lo:hi]
+        anc = ops.ancestor_bits_tensor(parents, device=DEV)
+        out = ops.tree_attention(q[:, :, lo:hi].contiguous().to(DEV), k.to(DEV), v.to(DEV), anc[lo:hi].contiguous(), P,
+                                 n_tree_slots=n_slots).float().cpu()
+        assert (out - ref).abs().amax().item() <= 1e-2 * ref.abs().amax().item(), tag
+        assert torch.allclose(out, ref, rtol=1e-2, atol=2e-2), tag
+        # compaction: ascending contexts of random length behind a random offset
+        L, H2, seq = rng.choice([1, 3]), rng.choice([1, 2]), rng.choice([70, 300, 700])
+        cache = torch.randn(L, 2, 1, H2, seq, 128, generator=g).to(dtype)
+        offset = rng.randrange(0, seq - 1)
+        count = rng.randrange(1, min(512, seq - offset) + 1)
+        ctx = sorted(torch.randperm(seq - offset, generator=g)[:count].tolist())
+        dev = cache.to(DEV)
+        ops.kv_compact_(dev, torch.tensor(ctx, dtype=torch.int64, device=DEV), offset)
+        assert torch.equal(dev.cpu(), okv.compact_static(cache, ctx, offset)), (tag, offset, count)
