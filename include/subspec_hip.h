@@ -90,8 +90,9 @@ float subspec_profile_read_ms(int index);
  *                                      means the tree broke a precondition (see verify.hip)
  * node_target / node_entropy / node_child_prob   device [batch, rows] (int64 / float / float):
  *             argmax token, normalized entropy and p[parent(i), token(i)] per scored node
- *             (what the reference's diagnostics are computed from); node_entropy is only
- *             written for the entropy gate.
+ *             (what the reference's diagnostics are computed from); node_entropy is 0 unless
+ *             the entropy gate is used.  node_target and node_entropy are written for every row,
+ *             node_child_prob for every row that is a node of the tree (the caller need not clear them).
  */
 size_t subspec_tree_verify_workspace(int64_t batch, int64_t rows, int64_t vocab, int dtype);
 

@@ -526,7 +526,7 @@ __global__ __launch_bounds__(kTailThreads) void tree_accept_kernel(
       sm_tgt[r] = tgt;
       sm_h[r] = h;
       node_target[grow] = tgt;
-      if (vp.gate_entropy) node_entropy[grow] = h;
+      node_entropy[grow] = vp.gate_entropy ? h : 0.f;   // always written: the caller need not clear the buffer
     }
   }
   __syncthreads();

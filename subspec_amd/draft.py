@@ -78,17 +78,25 @@ class SubSpecSDDraftModel:
             self.speculate_once()
         return self.update_tree(cap=True)
 
+    def _own_bits(self, device) -> torch.Tensor:
+        """Row s: the mask words with only the bit of slot s set (word s // 64, bit s % 64; bit 63 is the sign bit of
+        the signed word).  Built once, so that a level costs one slice and one OR."""
+        table = getattr(self, "_own_bits_table", None)
+        if table is None or table.device != torch.device(device):
+            slots = torch.arange(MAX_SLOTS)
+            low = slots % 64
+            bit = torch.where(low == 63, torch.full_like(slots, -(1 << 63)), torch.ones_like(slots) << low.clamp(max=62))
+            words = torch.arange(MASK_WORDS)
+            table = torch.where((slots // 64).unsqueeze(1) == words, bit.unsqueeze(1), torch.zeros_like(bit).unsqueeze(1))
+            self._own_bits_table = table = table.to(device)
+        return table
+
     def _expand(self, sampled_probs: torch.Tensor, parent_probs: torch.Tensor) -> None:
         k = self.draft_params.topk_len
         token_ids, child_probs, parent_indices = self.topk_sampling(sampled_probs, parent_probs, k)
         self.levels.append((token_ids, child_probs, parent_indices))
         self.token_ids, self.parent_probs = token_ids, child_probs
-        slots = torch.arange(self.next_slot, self.next_slot + token_ids.shape[1], device=token_ids.device)
-        # own bit of slot s: word s // 64, bit s % 64 (bit 63 is the sign bit of the signed word)
-        low = slots % 64
-        bit = torch.where(low == 63, torch.full_like(slots, -(1 << 63)), torch.ones_like(slots) << low.clamp(max=62))
-        words = torch.arange(MASK_WORDS, device=slots.device)
-        own = torch.where((slots // 64).unsqueeze(1) == words, bit.unsqueeze(1), torch.zeros_like(bit).unsqueeze(1))
+        own = self._own_bits(token_ids.device)[self.next_slot:self.next_slot + token_ids.shape[1]]
         self.level_bits = self.level_bits[parent_indices[0]] | own
         self.first_slot = self.next_slot
         self.next_slot += token_ids.shape[1]

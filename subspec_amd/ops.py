@@ -93,7 +93,7 @@ def tree_verify(
         "contexts": torch.empty((B, n + 1), dtype=torch.int64, device=dev),
         "counts": torch.empty((B, 4), dtype=torch.int32, device=dev),
         "target": torch.empty((B, rows), dtype=torch.int64, device=dev),
-        "entropy": torch.zeros((B, rows), dtype=torch.float32, device=dev),
+        "entropy": torch.empty((B, rows), dtype=torch.float32, device=dev),    # every row is written (0 without the entropy gate)
         "child_prob": torch.empty((B, rows), dtype=torch.float32, device=dev),
     }
     head = (logits.data_ptr(), _dtype_code(logits), B, rows, V, token_ids.data_ptr(), parents.data_ptr(), n,
