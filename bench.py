@@ -403,23 +403,27 @@ def main():
         torch.cuda.synchronize()
         del calib
 
-    # timed region: exactly `steps` steps, synchronised on both sides; per-call durations from events on the
-    # stream the kernels are launched on (torch's current stream)
-    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
+    # timed region: exactly `steps` steps, synchronised on both sides, nothing else on the stream
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for i in range(args.steps):
-        ev[i][0].record()
-        out = ops.tree_verify(cfg["logits"], tok, par, verify_method="lossy", threshold_method="entropy",
-                              threshold=cfg["threshold"], window_size=cfg["window_size"], workspace=ws_v)
-        ev[i][1].record()
-        top = ops.topk_expand(draft, parent_probs, k, workspace=ws_t)
-        ev[i][2].record()
+        out, top = step()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
 
-    # outside the timed region: the same steps again with the library's event pair around the dominant
-    # kernel of every call (the extra event records would otherwise sit inside the timed step)
+    # outside the timed region: the same steps with events around each call (an event record costs the stream about
+    # 5 us, three of them per step would inflate the timed step by 6 %), on the stream the kernels are launched on
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
+    for i in range(args.steps):
+        ev[i][0].record()
+        ops.tree_verify(cfg["logits"], tok, par, verify_method="lossy", threshold_method="entropy",
+                        threshold=cfg["threshold"], window_size=cfg["window_size"], workspace=ws_v)
+        ev[i][1].record()
+        ops.topk_expand(draft, parent_probs, k, workspace=ws_t)
+        ev[i][2].record()
+    torch.cuda.synchronize()
+
+    # and once more with the library's event pair around the dominant kernel of every call
     lib.subspec_profile_enable(1)
     for i in range(args.steps):
         step()
