@@ -392,6 +392,22 @@ int subspec_dense_decoder_layer(const subspec_decoder_layer_dims* dims, const su
                                 void* k_cache, void* v_cache, void* workspace, size_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------------------------------
+ * RMSNorm of [rows, hidden] activations in one launch: y = weight * round(x * rsqrt(mean(x^2) + eps)), the sum
+ * in fp32, the normalized value rounded to the activation dtype before the gain is applied (HuggingFace's
+ * Qwen2RMSNorm / LlamaRMSNorm rounding points).  The decoder-layer entry points run the same kernel
+ * inside a layer; this is the standalone form for the model's final norm and for module-by-module layers.
+ *
+ * Replaces  FiLlamaRMSNorm.forward -> flashinfer.norm.rmsnorm
+ *           specdecodes/models/utils/flashinfer/rms_norm.py:13-41 (the eager module it patches is the
+ *           RMSNorm of the HuggingFace decoder layers).
+ *
+ * x, y   device [rows, hidden] bf16 / fp16 (y may alias x); weight device [hidden], same dtype;
+ *        hidden % 8 == 0 and <= 16384; all pointers 16-byte aligned.
+ */
+int subspec_rms_norm(const void* x, const void* weight, void* y, int dtype, int64_t rows, int64_t hidden, float eps,
+                     void* stream);
+
+/* ------------------------------------------------------------------------------------------
  * Layer streaming: asynchronous copy of one weight slab from pinned host memory to its device
  * slab on the caller's copy stream (hipMemcpyAsync).  Ordering against the compute stream
  * (copy-done before use, last-reader-done before overwrite) is the caller's, with events.

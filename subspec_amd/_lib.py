@@ -76,6 +76,7 @@ _SIGNATURES = {
     "subspec_dense_linear": (C.c_int, [_p, _p, _p, _p, C.c_int, _i64, _i64, _i64, _p, _sz, _p]),
     "subspec_dense_decoder_layer": (C.c_int, [C.POINTER(DecoderLayerDims), C.POINTER(DenseLayerWeights), _p, _p, _p, _p,
                                               _p, _p, _p, _sz, _p]),
+    "subspec_rms_norm": (C.c_int, [_p, _p, _p, C.c_int, _i64, _i64, C.c_float, _p]),
     "subspec_stream_copy_h2d": (C.c_int, [_p, _p, _sz, _p]),
     "subspec_kv_compact": (C.c_int, [_p, _p, _i64, _i64, _i64, _i64, _i64, _p, _p, _i32, _i32, _p]),
 }

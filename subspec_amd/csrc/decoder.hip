@@ -256,6 +256,28 @@ static int run_layer(const subspec_decoder_layer_dims& s, const LayerWeights& w,
 
 using namespace subspec;
 
+extern "C" int subspec_rms_norm(const void* x, const void* weight, void* y, int dtype, int64_t rows, int64_t hidden,
+                                float eps, void* stream) {
+  if (dtype != SUBSPEC_BF16 && dtype != SUBSPEC_F16) SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "rms_norm: dtype %d not supported (bf16 / fp16)", dtype);
+  if (!x || !weight || !y) SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "rms_norm: null pointer argument");
+  if (rows <= 0 || rows > 0x7fffffff) SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "rms_norm: rows=%lld", (long long)rows);
+  if (hidden <= 0 || hidden % 8 != 0 || hidden > 8 * kNormThreads * kNormMaxPieces)
+    SUBSPEC_FAIL(SUBSPEC_ERR_LIMIT, "rms_norm: hidden=%lld must be a multiple of 8 and at most %d", (long long)hidden,
+                 8 * kNormThreads * kNormMaxPieces);
+  if (!(eps > 0.f)) SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "rms_norm: eps out of range");
+  if ((uintptr_t)x % 16 || (uintptr_t)weight % 16 || (uintptr_t)y % 16) SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "rms_norm: pointers must be 16-byte aligned");
+  hipStream_t st = (hipStream_t)stream;
+  // the kernel only writes x when it also adds: here it reads it
+  if (dtype == SUBSPEC_BF16)
+    hipLaunchKernelGGL((add_rmsnorm_kernel<SUBSPEC_BF16, false>), dim3((unsigned)rows), dim3(kNormThreads), 0, st, (uint16_t*)x,
+                       (const uint16_t*)nullptr, (const uint16_t*)weight, (uint16_t*)y, (int)hidden, eps);
+  else
+    hipLaunchKernelGGL((add_rmsnorm_kernel<SUBSPEC_F16, false>), dim3((unsigned)rows), dim3(kNormThreads), 0, st, (uint16_t*)x,
+                       (const uint16_t*)nullptr, (const uint16_t*)weight, (uint16_t*)y, (int)hidden, eps);
+  SUBSPEC_CHECK_HIP(hipGetLastError());
+  return SUBSPEC_OK;
+}
+
 extern "C" size_t subspec_int4_decoder_layer_workspace(const subspec_decoder_layer_dims* dims) {
   if (!dims || check_dims(dims) != SUBSPEC_OK) return 0;
   return layer_plan(*dims).total;

@@ -467,6 +467,21 @@ def int4_decoder_layer_(x: torch.Tensor, dims: "L.DecoderLayerDims", weights: "L
 decoder_layer_ = int4_decoder_layer_     # either weight storage: the pointer table's type selects the entry point
 
 
+def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+    """``weight * (x * rsqrt(mean(x^2) + eps)).to(x.dtype)`` over the last dimension in one launch
+    (bf16 / fp16; hidden a multiple of 8, at most 16384)."""
+    dev = _require_gpu(x, weight)
+    H = x.shape[-1]
+    if weight.numel() != H or weight.dtype != x.dtype:
+        raise ValueError("rms_norm: weight must be [hidden] in the activation dtype")
+    x2 = x.reshape(-1, H).contiguous()
+    y = torch.empty_like(x2)
+    code = L.lib().subspec_rms_norm(x2.data_ptr(), weight.contiguous().data_ptr(), y.data_ptr(), _dtype_code(x2),
+                                    x2.shape[0], H, float(eps), _stream(dev))
+    L.check(code, "subspec_rms_norm")
+    return y.reshape(x.shape)
+
+
 def dense_linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``F.linear(x, weight, bias)`` for at most 64 rows of bf16 / fp16 activations: x [..., K], weight [N, K]."""
     dev = _require_gpu(x, weight)

@@ -116,3 +116,29 @@ def test_rejects_bad_arguments():
     dims = ops.decoder_layer_dims(torch.bfloat16, 8, 256, 512, 2, 1, 64, 256, 10, 8, 1e-6, 1e6)    # head_dim 64
     with pytest.raises(ValueError):
         ops.decoder_layer_workspace(dims)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_rms_norm_matches_the_eager_formula(dtype):
+    """The standalone RMSNorm against HuggingFace's formula (fp32 normalization, rounded, then the gain) evaluated
+    by torch on the same inputs: the only freedom is the order of the fp32 sum of squares, so values agree to a
+    couple of units in the last place of the 16-bit type and almost all agree exactly."""
+    g = torch.Generator().manual_seed(1)
+    for rows, hidden in ((1, 8), (7, 256), (64, 3584), (300, 5120), (3, 16384)):
+        x = (torch.randn(rows, hidden, generator=g) * 3).to(dtype)
+        w = (1 + 0.1 * torch.randn(hidden, generator=g)).to(dtype)
+        got = ops.rms_norm(x.to(DEV), w.to(DEV), 1e-6).cpu()
+        xf = x.float()
+        ref = w * (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + 1e-6)).to(dtype)
+        assert got.shape == ref.shape and got.dtype == dtype
+        same = (got == ref).float().mean().item()
+        assert same >= 0.99, (rows, hidden, same)
+        ulp = 2.0 ** (-7 if dtype == torch.bfloat16 else -10)
+        assert ((got.float() - ref.float()).abs() <= 2.5 * ulp * ref.float().abs() + 1e-6).all()     # a flipped rounding of the normalized value, times the gain, rounded again
+    # leading dimensions are kept, a zero row stays zero
+    x = torch.zeros(2, 3, 64, dtype=dtype, device=DEV)
+    assert ops.rms_norm(x, torch.ones(64, dtype=dtype, device=DEV), 1e-6).abs().max().item() == 0
+    with pytest.raises(ValueError):
+        ops.rms_norm(torch.zeros(2, 12, dtype=dtype, device=DEV), torch.ones(12, dtype=dtype, device=DEV), 1e-6)
+    with pytest.raises(ValueError):
+        ops.rms_norm(torch.zeros(2, 64, device=DEV), torch.ones(64, device=DEV), 1e-6)          # fp32
