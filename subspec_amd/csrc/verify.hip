@@ -8,10 +8,10 @@
 //   2. exact pass          - only for rows that need the reference's per-element rounding
 //      (entropy within the guard band of the threshold, fp16 rows, or a possible tie between
 //      *rounded* probabilities at the row maximum): run by the same workgroup right after step 1
-//      when a row is one slice, otherwise by row_exact_kernel (same grid, exits at once for
-//      rows that do not need it).
+//      when a row is one slice (always, for a greedy target), otherwise by row_exact_kernel (same
+//      grid, exits at once for rows that do not need it; rows are cut into slices for a sampling target).
 //   3. tree_accept_kernel  - one workgroup per tree: combines the partials, gathers
-//      p[parent(i), token(i)], runs the greedy walk or the bottom-up DP on the <= 256 nodes in LDS
+//      p[parent(i), token(i)], runs the greedy walk or the bottom-up DP on the <= 512 nodes in LDS
 //      and writes the accepted path, contexts and bonus token.
 //
 // Sampling target (do_sample=True): the rows are first warped as TemperatureLogitsWarper does
@@ -691,14 +691,19 @@ __global__ __launch_bounds__(kTailThreads) void tree_accept_kernel(
 // ------------------------------------------------------------------ host side
 struct Plan { int vec, splits; int64_t chunk; };
 
-// Slices per row: enough workgroups to cover the chip several times over when there are few
-// rows, one slice per row when there are many; a slice is a whole number of 512-thread tiles.
-static bool make_plan(const void* logits, int dtype, int64_t total_rows, int64_t vocab, Plan* pl) {
+// Slices per row; a slice is a whole number of 512-thread tiles.
+// Greedy target: one slice, whatever the number of rows.  The workgroup that holds a whole row decides by itself
+// whether the row needs the exact pass and runs it while the row is in cache; splitting a row means a second launch
+// that recombines the slices first, and that launch costs more than the few workgroups of a small batch lose
+// (152064 columns, bf16: 64 rows 31 -> 26 us per call, 256 rows 62 -> 42 us, 512 rows 84 -> 71 us; one row 30 -> 27 us).
+// Sampling target: the draw is bound by the vector ALU (a Philox block per four elements), so few rows are cut
+// into enough slices to cover the chip several times over.
+static bool make_plan(const void* logits, int dtype, int64_t total_rows, int64_t vocab, bool sample, Plan* pl) {
   const int vec_full = dtype == SUBSPEC_F32 ? 4 : 8;
   const bool aligned = (vocab % vec_full == 0) && ((uintptr_t)logits % 16 == 0);
   pl->vec = aligned ? vec_full : 1;
   const int64_t quantum = (int64_t)kRowThreads * pl->vec;
-  int64_t splits = (2048 + total_rows - 1) / total_rows;
+  int64_t splits = sample ? (2048 + total_rows - 1) / total_rows : 1;
   splits = std::min<int64_t>(splits, std::max<int64_t>(1, vocab / 8192));
   splits = std::max<int64_t>(1, std::min<int64_t>(splits, kMaxSplits));
   int64_t chunk = (vocab + splits - 1) / splits;
@@ -804,7 +809,7 @@ static int tree_verify_impl(const void* logits, int dtype, int64_t batch, int64_
   if ((uintptr_t)logits % dtype_size(dtype) != 0) SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "tree_verify: logits misaligned");
 
   Plan pl;
-  if (!make_plan(logits, dtype, batch * rows, vocab, &pl))
+  if (!make_plan(logits, dtype, batch * rows, vocab, sa.sample != 0, &pl))
     SUBSPEC_FAIL(SUBSPEC_ERR_LIMIT, "tree_verify: vocab=%lld needs more than %d slices per row", (long long)vocab,
                  kMaxSplits);
   const size_t n = (size_t)batch * rows * kMaxSplits;
