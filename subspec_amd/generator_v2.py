@@ -210,7 +210,9 @@ class SubSpecSDGeneratorV2(SubSpecSDGenerator):
         log.update({"n_iter": n_iter, "n_tokens": n_tokens, "elapsed_time": elapsed,
                     "tput": n_tokens / elapsed if elapsed > 0 else 0.0,
                     "avg_sampled": sampled_count / n_iter if n_iter else 0.0,
-                    "post_verify_count": self.post_verify_count, "speculate_count": self.speculate_count})
+                    "post_verify_count": self.post_verify_count, "speculate_count": self.speculate_count,
+                    "post_verify_rate": (self.post_verify_count / (self.post_verify_count + self.speculate_count)
+                                         if self.post_verify_count + self.speculate_count else 0.0)})   # mixin.py:341-347
         if self.profiling:
             for name, pairs in phases.items():
                 log[f"avg_{name}_time"] = (sum(a.elapsed_time(b) for a, b in pairs) / len(pairs) / 1e3) if pairs else 0.0

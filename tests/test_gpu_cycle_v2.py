@@ -87,6 +87,7 @@ def test_v2_emits_what_v1_emits(agreeing, first_streamed):
         a, b = kv.cache.data[..., :L, :].float(), kv2.cache.data[..., :L, :].float()
         assert (a - b).abs().amax().item() <= 5e-2 * b.abs().amax().item()
         assert log["speculate_count"] + log["post_verify_count"] == log["n_iter"]
+        assert abs(log["post_verify_rate"] * log["n_iter"] - log["post_verify_count"]) < 1e-6
         if steps == 0:
             assert log["post_verify_count"] == 0 and log["n_iter"] == ref_log["n_iter"]
         if agreeing and steps == 4:
