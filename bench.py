@@ -20,8 +20,8 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 # HBM bytes per launch at the default workload, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs scaled
 # by a copy of known size (profiles/verify_cycle_config2_hbm_counters.md); None for other sizes.
 MEASURED_TRAFFIC = {
-    ("verify", 32, 152064): int(307238.1 * 1024 * 2.0 + 64.0 * 1024),
-    ("topk", 32, 152064): int(304269.5 * 1024 * 2.0 + 576.0 * 1024),
+    ("verify", 32, 152064): int(304836.5 * 1024 * 2.0 + 64.0 * 1024),
+    ("topk", 32, 152064): int(304339.5 * 1024 * 2.0 + 576.0 * 1024),
 }
 
 
