@@ -382,7 +382,9 @@ template <> struct RoundBound<SUBSPEC_BF16> { static constexpr float rel = 0x1p-
 // and p <= an upper bound from the hardware exponential give key <= bound / (1 - u), and an
 // element whose bound stays below the best key any lane of the wavefront has seen is skipped.
 // What is left per element is the Philox block, one exponential and a compare.
-template <int DT>
+// QUAD: the slice starts and ends on multiples of four elements and the rows are aligned for it, so the four logits
+// of a Philox block are one load (8 bytes of a 16-bit row, 16 of an fp32 row) and need no bounds.
+template <int DT, bool QUAD>
 __global__ __launch_bounds__(kRowThreads) void row_sample_kernel(
     const void* __restrict__ logits, VerifyParams vp, const Part1* __restrict__ part1, Part3* __restrict__ part3) {
   __shared__ float red_f[kRowThreads / kWave];
@@ -406,30 +408,54 @@ __global__ __launch_bounds__(kRowThreads) void row_sample_kernel(
   for (int64_t g0 = 0; g0 * 4 < n; g0 += kRowThreads) {   // same trip count for every lane: the votes below see whole wavefronts
     const int64_t g = g0 + threadIdx.x;
     float xs[4];
+    if constexpr (QUAD) {                              // one load, clamped to the last block of the slice
+      const int64_t q = min(g, n / 4 - 1);
+      if constexpr (DT == SUBSPEC_F32) {
+        const float4 v = *(const float4*)((const float*)logits + base + q * 4);
+        xs[0] = v.x; xs[1] = v.y; xs[2] = v.z; xs[3] = v.w;
+      } else {
+        const uint2 v = *(const uint2*)((const uint16_t*)logits + base + q * 4);
+        if constexpr (DT == SUBSPEC_BF16) {
+          xs[0] = __uint_as_float(v.x << 16); xs[1] = __uint_as_float(v.x & 0xffff0000u);
+          xs[2] = __uint_as_float(v.y << 16); xs[3] = __uint_as_float(v.y & 0xffff0000u);
+        } else {
+          xs[0] = f16_bits_to_float(v.x & 0xffffu); xs[1] = f16_bits_to_float(v.x >> 16);
+          xs[2] = f16_bits_to_float(v.y & 0xffffu); xs[3] = f16_bits_to_float(v.y >> 16);
+        }
+      }
+    } else {
 #pragma unroll
-    for (int e = 0; e < 4; ++e)                        // unconditional loads (clamped index), in flight during the Philox rounds
-      xs[e] = Elem<DT>::load(logits, base + min(g * 4 + e, n - 1));
+      for (int e = 0; e < 4; ++e)                      // unconditional loads (clamped index), in flight during the Philox rounds
+        xs[e] = Elem<DT>::load(logits, base + min(g * 4 + e, n - 1));
+    }
     uint32_t w[4];
     philox4x32_10((uint32_t)(c0 / 4 + g), (uint32_t)row, vp.offset[0], vp.offset[1], vp.key[0], vp.key[1], w);
+    bool cand[4];
+    bool any_cand = false;
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       const int64_t i = g * 4 + e;
-      const float x = xs[e];
-      const float xa = fmaxf(x * inv_t, -1e30f);                     // masked (-inf) logits stay finite below
+      const float xa = fmaxf(xs[e] * inv_t, -1e30f);                 // masked (-inf) logits stay finite below
       const float xu = fmaf(fabsf(xa), round_up, xa) + round_abs;
       const float bound = fmaf(__builtin_amdgcn_exp2f(fmaf(xu, kLog2e, mb)), p_scale, RoundBound<DT>::abs);
       const float one_minus_u = (float)((~w[e]) >> 9) + 0.5f;        // (1 - u) * 2^23, exact
-      const bool cand = i < n && !(bound < thr * one_minus_u);
-      if (__any(cand)) {                               // wavefront-uniform
-        if (cand) {
+      cand[e] = (QUAD ? g * 4 < n : i < n) && !(bound < thr * one_minus_u);
+      any_cand |= cand[e];
+    }
+    // one vote per block of four: the threshold only prunes, so refreshing it less often changes no result
+    if (__any(any_cand)) {                             // wavefront-uniform
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        if (cand[e]) {
+          const float x = xs[e];
           const float xw = warp ? Elem<DT>::round(div_rn(x, vp.temperature)) : x;
           const float p = rounded_prob<DT>(xw, rs.m, rs.S);
           const float u = ((float)(w[e] >> 9) + 0.5f) * 0x1p-23f;
           const float key = p / -logf(u);
-          if (key > best) { best = key; idx = (int)(c0 + i); }   // indices ascend: the first maximum stays
+          if (key > best) { best = key; idx = (int)(c0 + g * 4 + e); }   // indices ascend: the first maximum stays
         }
-        thr = fmaxf(wave_max(best), 0.f) * (0.9999f * 0x1p-23f);
       }
+      thr = fmaxf(wave_max(best), 0.f) * (0.9999f * 0x1p-23f);
     }
   }
   const float top = block_max<kRowThreads>(best, red_f);
@@ -744,7 +770,11 @@ static int run_verify(const void* logits, int64_t batch, int64_t rows, int64_t v
   if (pl.splits > 1) hipLaunchKernelGGL((row_exact_kernel<DT>), grid, dim3(kRowThreads), 0, st, logits, vp, p1, p2);
   if (vp.sample) {
     DominantKernelTimer timer(st);
-    hipLaunchKernelGGL((row_sample_kernel<DT>), grid, dim3(kRowThreads), 0, st, logits, vp, p1, p3);
+    // slices are whole numbers of 512-thread tiles of pl.vec elements: with pl.vec > 1 rows and slices are quad-aligned
+    if (pl.vec > 1 && vocab % 4 == 0)
+      hipLaunchKernelGGL((row_sample_kernel<DT, true>), grid, dim3(kRowThreads), 0, st, logits, vp, p1, p3);
+    else
+      hipLaunchKernelGGL((row_sample_kernel<DT, false>), grid, dim3(kRowThreads), 0, st, logits, vp, p1, p3);
   }
   const int64_t widest = std::max<int64_t>(rows, tp.n_nodes);
   const int slots = widest <= kWave ? 1 : widest <= 2 * kWave ? 2 : widest <= 4 * kWave ? 4 : 8;
