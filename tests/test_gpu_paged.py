@@ -133,8 +133,9 @@ def test_request_cache_cycle_matches_static_cache():
     assert len(req.kv_page_indices) == (prefix + 4 + page_len - 1) // page_len
 
 
+@pytest.mark.parametrize("depth,topk", [(5, 4), (20, 6)])          # 21-node trees; 121-node trees (two mask words, row windows)
 @pytest.mark.parametrize("driver", ["v1", "v2"])
-def test_speculative_cycle_over_the_paged_cache_equals_the_static_cache(driver):
+def test_speculative_cycle_over_the_paged_cache_equals_the_static_cache(driver, depth, topk):
     """The whole cycle (prefill, draft levels, target window, verification, compaction) over a page pool whose pages
     were handed out in scrambled order, against the same models over the contiguous cache.  Both runs go module by
     module (the one-call layers take contiguous caches only), so the cache layout is the only difference and
@@ -151,7 +152,7 @@ def test_speculative_cycle_over_the_paged_cache_equals_the_static_cache(driver):
     prompt = torch.randint(0, cfg.vocab_size, (1, 37), generator=torch.Generator().manual_seed(8)).to(DEV)
     runs = {}
     for impl in ("static", "paged"):
-        kv = create_kv_cache(impl, max_cache_len=512, config=cfg, device=DEV, dtype=torch.bfloat16)
+        kv = create_kv_cache(impl, max_cache_len=1024, config=cfg, device=DEV, dtype=torch.bfloat16)
         if impl == "paged":
             pool = kv.cache.pool
             held = pool.allocate(9)                               # scramble the order of the request's pages:
@@ -160,7 +161,7 @@ def test_speculative_cycle_over_the_paged_cache_equals_the_static_cache(driver):
         target, draft, _ = build_models(cfg, kv, device=DEV, weights=w)
         target.use_native_layers = draft.use_native_layers = False
         cls, extra = (SubSpecSDGenerator, {}) if driver == "v1" else (SubSpecSDGeneratorV2, dict(postspec_steps=2))
-        gen = cls(target, None, SubSpecSDDraftModel(draft), DraftParams(temperature=0.2, max_depth=5, topk_len=4),
+        gen = cls(target, None, SubSpecSDDraftModel(draft), DraftParams(temperature=0.2, max_depth=depth, topk_len=topk),
                   cache_implementation=impl, generator_kwargs=dict(verify_method="exact", **extra))
         out = gen.generate(prompt, max_new_tokens=40, do_sample=False, past_key_values=kv)[0].cpu()
         L = kv.get_seq_length()
