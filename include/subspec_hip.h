@@ -302,6 +302,23 @@ int subspec_int4_linear(const void* x, const uint32_t* wq, const uint32_t* sz, c
                         int64_t M, int64_t N, int64_t K, int64_t group_size, void* workspace, size_t workspace_bytes,
                         void* stream);
 
+/* The SwiGLU MLP's first projection and its activation in one launch:
+ *   act[m, f] = round(silu(round(gate[m, f]))) * round(up[m, f]),   gate | up = x * W^T (+ bias),
+ * W = the gate projection's F rows followed by the up projection's F rows (N = 2F, same tiled layout as
+ * subspec_int4_linear), every intermediate rounded to the activation dtype exactly where the separate
+ * projection and activation would round it.  A workgroup owns (gate tile, up tile) pairs, so the 2F
+ * projections never travel through memory.
+ *
+ * Replaces  act_fn(gate_proj(x)) * up_proj(x) of the decoder MLP (HuggingFace Qwen2MLP / LlamaMLP with
+ *           HQQLinear projections; the reference's patched form is LigerSwiGLUMLP.forward,
+ *           specdecodes/models/utils/flashinfer/rms_norm.py:43-78, with flashinfer.activation.silu_and_mul).
+ *
+ * x    device [M, K] bf16 / fp16, 1 <= M <= 64;  act  device [M, N / 2];  N % 32 == 0, K % 64 == 0;
+ * bias device [N] or NULL.  No workspace.
+ */
+int subspec_int4_gate_up_silu(const void* x, const uint32_t* wq, const uint32_t* sz, const void* bias, void* act,
+                              int dtype, int64_t M, int64_t N, int64_t K, void* stream);
+
 /* ------------------------------------------------------------------------------------------
  * One int4 decoder layer of the substitute draft over the rows of a tree level, issued as a fixed
  * sequence of launches from one host call (no per-module Python dispatch):

@@ -150,7 +150,11 @@ __device__ __forceinline__ i4_v4f i4_mfma32(i4_u4 a, i4_u4 b, i4_v4f c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(i4_v8h, a), __builtin_bit_cast(i4_v8h, b), c, 0, 0, 0);
 }
 
-template <int DT, int MT, int RT>
+// SILU (the gate|up projection of a SwiGLU MLP, N = 2F rows: gate rows first, up rows behind them): a workgroup
+// owns PAIRS of tiles, (gate tile p, up tile p + F/16), and its output stage writes act[m, f] =
+// round(silu(round(gate))) * round(up) to y[M, F] instead of the 2F projections -- the arithmetic of the separate
+// activation kernel on the values the plain projection would have stored, one launch and one round trip less.
+template <int DT, int MT, int RT, bool SILU = false>
 __global__ __launch_bounds__(kI4Threads) void int4_gemm_kernel(
     const uint16_t* __restrict__ x, const uint2* __restrict__ wq, const uint32_t* __restrict__ sz,
     const uint16_t* __restrict__ bias, const uint16_t* residual, uint16_t* y, float* __restrict__ partial, int M, int64_t N,
@@ -171,9 +175,13 @@ __global__ __launch_bounds__(kI4Threads) void int4_gemm_kernel(
   const int g_first = g_begin + wave;                            // this wavefront's groups: g_first + 4j
   const int nj = g_first < g_end ? (g_end - g_first + 3) / 4 : 0;
 
-  // tiles [tile0, tile0 + ntl) of this workgroup: an even split of all tiles over the grid
-  const int tile0 = (int)((int64_t)blockIdx.x * n_tiles / gridDim.x);
-  const int ntl = (int)((int64_t)(blockIdx.x + 1) * n_tiles / gridDim.x) - tile0;     // 1 .. RT
+  // tiles [tile0, tile0 + ntl) of this workgroup: an even split of all tiles (SILU: of all tile pairs) over the grid
+  const int n_units = SILU ? n_tiles / 2 : n_tiles;
+  const int unit0 = (int)((int64_t)blockIdx.x * n_units / gridDim.x);
+  const int n_own = (int)((int64_t)(blockIdx.x + 1) * n_units / gridDim.x) - unit0;
+  const int tile0 = unit0;                                                             // plain: first tile
+  const int ntl = SILU ? 2 * n_own : n_own;                                            // 1 .. RT
+  auto tile_of = [&](int t) { return SILU ? unit0 + (t >> 1) + (t & 1) * (n_tiles / 2) : tile0 + t; };
 
   i4_v4f acc[RT][MT];
 #pragma unroll
@@ -205,7 +213,7 @@ __global__ __launch_bounds__(kI4Threads) void int4_gemm_kernel(
   const int xl_read = ln * kXlStride + c * 16;
   int wofs[RT];                                                  // (tile, group 0) in units of groups
 #pragma unroll
-  for (int t = 0; t < RT; ++t) wofs[t] = (tile0 + min(t, ntl - 1)) * G;
+  for (int t = 0; t < RT; ++t) wofs[t] = tile_of(min(t, ntl - 1)) * G;
 
   i4_u4 xg[kXg];                                                 // block on its way from global memory to LDS
   i4_u2 wbuf[2][RT];
@@ -293,6 +301,8 @@ __global__ __launch_bounds__(kI4Threads) void int4_gemm_kernel(
   // round.  LDS holds two rounds, so a round needs one barrier; wavefront w finishes the activation
   // row blocks mt = w, w + 4, ... of the tile, so the sums and stores are spread over the workgroup.
   // accumulator layout: rows m = 16*mt + 4*c + rr, column n = 16*tile + ln
+  float gate_held[MT][4];                                        // SILU: the rounded gate values between two rounds
+  (void)gate_held;
 #pragma unroll
   for (int t = 0; t < RT; ++t) {
     if (t >= ntl) break;                                         // uniform
@@ -300,7 +310,7 @@ __global__ __launch_bounds__(kI4Threads) void int4_gemm_kernel(
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) *(i4_v4f*)(&stage[((wave * MT + mt) * 64 + lane) * 4]) = acc[t][mt];
     __syncthreads();                                             // round t written; round t - 1 fully read
-    const int64_t n = (int64_t)(tile0 + t) * 16 + ln;
+    const int64_t n = (int64_t)tile_of(t) * 16 + ln;
     const float bv = (splits == 1 && bias) ? I4<DT>::to_float(bias[n]) : 0.f;
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
@@ -312,12 +322,29 @@ __global__ __launch_bounds__(kI4Threads) void int4_gemm_kernel(
 #pragma unroll
         for (int rr = 0; rr < 4; ++rr) v[rr] += o[rr];
       }
+      if constexpr (SILU) {
+        // even round: the gate tile, kept in registers; odd round: its up tile, same wavefront, same lanes
+        if ((t & 1) == 0) {
 #pragma unroll
-      for (int rr = 0; rr < 4; ++rr) {
-        const int m = mt * 16 + c * 4 + rr;
-        if (m >= M) continue;
-        if (splits == 1) store_linear_out<DT>(y, (int64_t)m * N + n, v[rr] + bv, residual);
-        else partial[((int64_t)ks * M + m) * N + n] = v[rr];
+          for (int rr = 0; rr < 4; ++rr) gate_held[mt][rr] = Elem<DT>::round(v[rr] + bv);
+        } else {
+          const int64_t f = (int64_t)(unit0 + (t >> 1)) * 16 + ln;
+#pragma unroll
+          for (int rr = 0; rr < 4; ++rr) {
+            const int m = mt * 16 + c * 4 + rr;
+            if (m >= M) continue;
+            const float g = gate_held[mt][rr], u = Elem<DT>::round(v[rr] + bv);
+            Elem<DT>::store(y, (int64_t)m * (N / 2) + f, Elem<DT>::round(g / (1.f + __expf(-g))) * u);
+          }
+        }
+      } else {
+#pragma unroll
+        for (int rr = 0; rr < 4; ++rr) {
+          const int m = mt * 16 + c * 4 + rr;
+          if (m >= M) continue;
+          if (splits == 1) store_linear_out<DT>(y, (int64_t)m * N + n, v[rr] + bv, residual);
+          else partial[((int64_t)ks * M + m) * N + n] = v[rr];
+        }
       }
     }
   }
@@ -357,6 +384,30 @@ static I4Plan i4_plan(int64_t M, int64_t N, int64_t K) {
   gps = (gps + 3) / 4 * 4;
   splits = (G + gps - 1) / gps;
   return I4Plan{(int)wgs, row_tiles, splits, gps};
+}
+
+// gate|up projection with the SwiGLU output stage: x [M, K], weights of N = 2F rows (gate rows first), act [M, F]
+template <int DT>
+static int run_int4_silu(const void* x, const uint32_t* wq, const uint32_t* sz, const void* bias, void* act, int64_t M,
+                         int64_t N, int64_t K, hipStream_t st) {
+  const int64_t pairs = N / 32, slots = i4_slots(M);
+  // one or two (gate, up) pairs per workgroup; two only with few activation rows (the accumulators of four tiles
+  // times four row blocks would fill the register file)
+  const int rt = (pairs <= slots || M > 32) ? 2 : 4;
+  const int64_t wgs = (pairs + rt / 2 - 1) / (rt / 2);
+  const dim3 grid((unsigned)wgs, 1);
+  const int G = (int)(K / kGroup);
+#define SUBSPEC_I4_SILU(MT, RT)                                                                                    \
+  hipLaunchKernelGGL((int4_gemm_kernel<DT, MT, RT, true>), grid, dim3(kI4Threads), 0, st, (const uint16_t*)x,     \
+                     (const uint2*)wq, sz, (const uint16_t*)bias, (const uint16_t*)nullptr, (uint16_t*)act, (float*)nullptr,   \
+                     (int)M, N, (int)K, 1, (G + 3) / 4 * 4)
+  DominantKernelTimer timer(st);
+  if (M <= 16) { if (rt == 2) SUBSPEC_I4_SILU(1, 2); else SUBSPEC_I4_SILU(1, 4); }
+  else if (M <= 32) { if (rt == 2) SUBSPEC_I4_SILU(2, 2); else SUBSPEC_I4_SILU(2, 4); }
+  else { if (rt == 2) SUBSPEC_I4_SILU(4, 2); else SUBSPEC_I4_SILU(4, 4); }
+#undef SUBSPEC_I4_SILU
+  SUBSPEC_CHECK_HIP(hipGetLastError());
+  return SUBSPEC_OK;
 }
 
 template <int DT>
@@ -427,11 +478,32 @@ static size_t i4_workspace_one(int64_t M, int64_t N, int64_t K) {
   return (pl.splits > 1 ? align_up((size_t)pl.splits * M * N * sizeof(float), 256) : 0) + 256;
 }
 
+extern "C" int subspec_int4_gate_up_silu(const void* x, const uint32_t* wq, const uint32_t* sz, const void* bias, void* act,
+                                         int dtype, int64_t M, int64_t N, int64_t K, void* stream) {
+  return int4_gate_up_silu_ex(x, wq, sz, bias, act, dtype, M, N, K, stream);
+}
+
 extern "C" size_t subspec_int4_linear_workspace(int64_t M, int64_t N, int64_t K) {
   if (M <= 0 || N <= 0 || K <= 0) return 256;
   if (M <= 64) return i4_workspace_one(M, N, K);
   const size_t full = i4_workspace_one(64, N, K);
   return M % 64 ? std::max(full, i4_workspace_one(M % 64, N, K)) : full;
+}
+
+int subspec::int4_gate_up_silu_ex(const void* x, const uint32_t* wq, const uint32_t* sz, const void* bias, void* act, int dtype,
+                                  int64_t M, int64_t N, int64_t K, void* stream) {
+  if (dtype != SUBSPEC_BF16 && dtype != SUBSPEC_F16)
+    SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "int4_gate_up_silu: dtype %d not supported (bf16 / fp16 activations only)", dtype);
+  if (!x || !wq || !sz || !act) SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "int4_gate_up_silu: null pointer argument");
+  if (M <= 0 || M > 64 || N <= 0 || K <= 0 || N % 32 != 0 || K % kGroup != 0 || K > 65536)
+    SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "int4_gate_up_silu: M=%lld N=%lld K=%lld; 1 <= M <= 64, N a multiple of 32, K of 64",
+                 (long long)M, (long long)N, (long long)K);
+  if (N * K / 2 >= ((int64_t)1 << 31))
+    SUBSPEC_FAIL(SUBSPEC_ERR_LIMIT, "int4_gate_up_silu: N*K/2=%lld bytes of codes exceed the 2 GiB descriptor range", (long long)(N * K / 2));
+  if ((uintptr_t)x % 16 || (uintptr_t)wq % 16 || (uintptr_t)sz % 16 || (uintptr_t)act % 8)
+    SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "int4_gate_up_silu: x / wq / sz must be 16-byte aligned, act 8-byte aligned");
+  if (dtype == SUBSPEC_BF16) return run_int4_silu<SUBSPEC_BF16>(x, wq, sz, bias, act, M, N, K, (hipStream_t)stream);
+  return run_int4_silu<SUBSPEC_F16>(x, wq, sz, bias, act, M, N, K, (hipStream_t)stream);
 }
 
 int subspec::int4_linear_ex(const void* x, const uint32_t* wq, const uint32_t* sz, const void* bias, const void* residual,

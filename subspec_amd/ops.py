@@ -467,6 +467,31 @@ def int4_decoder_layer_(x: torch.Tensor, dims: "L.DecoderLayerDims", weights: "L
 decoder_layer_ = int4_decoder_layer_     # either weight storage: the pointer table's type selects the entry point
 
 
+def int4_gate_up_silu(x: torch.Tensor, wq: torch.Tensor, sz: torch.Tensor, intermediate_size: int,
+                      bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``silu(gate) * up`` of a SwiGLU MLP from the fused gate|up int4 weight (``2 * intermediate_size`` rows, gate rows
+    first) in one launch: ``x`` [..., K] (at most 64 rows) -> [..., intermediate_size]."""
+    dev = _require_gpu(x, wq, sz)
+    K = x.shape[-1]
+    M = x.numel() // K
+    N = 2 * int(intermediate_size)
+    if wq.dtype != torch.int32 or sz.dtype != torch.int32:
+        raise ValueError("int4_gate_up_silu: wq and sz must be int32 tensors in the tiled layout")
+    if wq.numel() * 8 != N * K or sz.numel() * 64 != N * K:
+        raise ValueError(f"int4_gate_up_silu: packed weight does not describe a [{N}, {K}] matrix")
+    x2 = x.reshape(M, K).contiguous()
+    if bias is not None:
+        if bias.dtype != x.dtype or bias.numel() != N:
+            raise ValueError("int4_gate_up_silu: bias must be [2 * intermediate_size] in the activation dtype")
+        bias = bias.contiguous()
+    act = torch.empty((M, N // 2), dtype=x.dtype, device=dev)
+    code = L.lib().subspec_int4_gate_up_silu(x2.data_ptr(), wq.data_ptr(), sz.data_ptr(),
+                                            None if bias is None else bias.data_ptr(), act.data_ptr(), _dtype_code(x2),
+                                            M, N, K, _stream(dev))
+    L.check(code, "subspec_int4_gate_up_silu")
+    return act.reshape(*x.shape[:-1], N // 2)
+
+
 def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
     """``weight * (x * rsqrt(mean(x^2) + eps)).to(x.dtype)`` over the last dimension in one launch
     (bf16 / fp16; hidden a multiple of 8, at most 16384)."""

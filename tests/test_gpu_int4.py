@@ -114,3 +114,34 @@ def test_quantizer_default_refines_zero_points():
         assert (y - ref).abs().amax() <= 1e-2 * ref.abs().amax()
         errs[optimize] = (y - want).pow(2).mean().item()
     assert errs[True] <= errs[False] * 1.02, errs
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_gate_up_projection_with_the_activation_in_its_output_stage(dtype):
+    """The fused launch against the plain projection followed by the activation on the values it stored: the same
+    accumulation per tile, the same roundings, so only the exponential (hardware exp against torch's) may differ --
+    nearly every element is identical, the rest within one unit in the last place.  Every activation-row tile
+    count, one and two tile pairs per workgroup, with and without bias."""
+    for seed, (F, K, M, bias) in enumerate([(16, 64, 1, False), (48, 192, 5, True), (512, 256, 16, False), (1184, 128, 17, True),
+                                            (18944, 3584, 8, False), (18944, 3584, 64, False), (2048, 512, 33, True),
+                                            (40000, 64, 3, False)]):
+        print("gate|up + silu", dtype, F, K, M, bias, flush=True)
+        g = torch.Generator().manual_seed(700 + seed)
+        W = torch.randn(2 * F, K, generator=g) * (2.0 / K ** 0.5)
+        codes, scale, zero = quant.quantize_int4_g64(W)
+        wq, sz = quant.pack_tiled(codes, scale, zero)
+        x = torch.randn(M, K, generator=g).to(dtype)
+        b = (torch.randn(2 * F, generator=g) * 0.1).to(dtype) if bias else None
+        bd = None if b is None else b.to(DEV)
+        got = ops.int4_gate_up_silu(x.to(DEV), wq.to(DEV), sz.to(DEV), F, bd)
+        gu = ops.int4_linear(x.to(DEV), wq.to(DEV), sz.to(DEV), 2 * F, bd)
+        gate, up = gu[:, :F].float(), gu[:, F:].float()
+        want = ((gate / (1 + torch.exp(-gate))).to(dtype).float() * up).to(dtype)
+        assert got.shape == (M, F) and got.dtype == dtype
+        differing = int((got != want).sum())
+        assert differing <= max(1, got.numel() // 1000), (F, K, M, differing)
+        ulp = 2.0 ** (-7 if dtype == torch.bfloat16 else -10)
+        assert ((got.float() - want.float()).abs() <= 2 * ulp * want.float().abs() + 1e-6).all()
+    with pytest.raises(ValueError):
+        ops.int4_gate_up_silu(torch.zeros(65, 64, dtype=dtype, device=DEV), torch.zeros(2 * 32 * 64 // 8, dtype=torch.int32, device=DEV),
+                              torch.zeros(2 * 32, dtype=torch.int32, device=DEV), 32)          # more than 64 rows
