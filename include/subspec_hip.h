@@ -319,6 +319,11 @@ int subspec_int4_linear(const void* x, const uint32_t* wq, const uint32_t* sz, c
 int subspec_int4_gate_up_silu(const void* x, const uint32_t* wq, const uint32_t* sz, const void* bias, void* act,
                               int dtype, int64_t M, int64_t N, int64_t K, void* stream);
 
+/* The same for a dense 16-bit gate|up weight W [2F, K] row-major (gate rows first), as the target's layers hold it;
+ * 2F * K * 2 bytes must stay below 2 GiB. */
+int subspec_dense_gate_up_silu(const void* x, const void* w, const void* bias, void* act, int dtype, int64_t M,
+                               int64_t N, int64_t K, void* stream);
+
 /* ------------------------------------------------------------------------------------------
  * One int4 decoder layer of the substitute draft over the rows of a tree level, issued as a fixed
  * sequence of launches from one host call (no per-module Python dispatch):

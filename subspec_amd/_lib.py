@@ -70,6 +70,7 @@ _SIGNATURES = {
     "subspec_int4_linear_workspace": (_sz, [_i64, _i64, _i64]),
     "subspec_int4_linear": (C.c_int, [_p, _p, _p, _p, _p, C.c_int, _i64, _i64, _i64, _i64, _p, _sz, _p]),
     "subspec_int4_gate_up_silu": (C.c_int, [_p, _p, _p, _p, _p, C.c_int, _i64, _i64, _i64, _p]),
+    "subspec_dense_gate_up_silu": (C.c_int, [_p, _p, _p, _p, C.c_int, _i64, _i64, _i64, _p]),
     "subspec_int4_decoder_layer_workspace": (_sz, [C.POINTER(DecoderLayerDims)]),
     "subspec_int4_decoder_layer": (C.c_int, [C.POINTER(DecoderLayerDims), C.POINTER(DecoderLayerWeights), _p, _p, _p, _p,
                                              _p, _p, _p, _sz, _p]),

@@ -181,6 +181,8 @@ int int4_linear_ex(const void* x, const uint32_t* wq, const uint32_t* sz, const 
 // the SwiGLU MLP's first projection and its activation in one launch
 int int4_gate_up_silu_ex(const void* x, const uint32_t* wq, const uint32_t* sz, const void* bias, void* act, int dtype,
                          int64_t M, int64_t N, int64_t K, void* stream);
+int dense_gate_up_silu_ex(const void* x, const void* w, const void* bias, void* act, int dtype, int64_t M, int64_t N,
+                          int64_t K, void* stream);
 int dense_linear_ex(const void* x, const void* w, const void* bias, const void* residual, void* y, int dtype, int64_t M,
                     int64_t N, int64_t K, void* workspace, size_t workspace_bytes, void* stream);
 

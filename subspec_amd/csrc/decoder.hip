@@ -243,11 +243,13 @@ static int run_layer(const subspec_decoder_layer_dims& s, const LayerWeights& w,
   if ((rc = project(w, w.o, a, nullptr, nullptr, o, DT, M, H, Q, sub, p.sub_bytes, st))) return rc;
   hipLaunchKernelGGL((add_rmsnorm_kernel<DT, true>), dim3(M), dim3(kNormThreads), 0, st, x, o, (const uint16_t*)w.post_norm, h, H,
                      s.rms_eps);
-  if (!w.dense && F % 16 == 0) {
-    // int4 weights: the activation sits in the output stage of the gate|up projection
+  if (!w.dense) {
+    // the activation sits in the output stage of the gate|up projection
     if ((rc = int4_gate_up_silu_ex(h, (const uint32_t*)w.gate_up.w, (const uint32_t*)w.gate_up.sz, nullptr, act, DT, M,
                                    2 * (int64_t)F, H, st)))
       return rc;
+  } else if (4 * (int64_t)F * H < ((int64_t)1 << 31)) {
+    if ((rc = dense_gate_up_silu_ex(h, w.gate_up.w, nullptr, act, DT, M, 2 * (int64_t)F, H, st))) return rc;
   } else {
     if ((rc = project(w, w.gate_up, h, nullptr, nullptr, gu, DT, M, 2 * (int64_t)F, H, sub, p.sub_bytes, st))) return rc;
     const int64_t act_pieces = (int64_t)M * F / 8;

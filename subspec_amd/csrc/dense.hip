@@ -38,7 +38,10 @@ __device__ __forceinline__ dn_v4f dn_mfma32(dn_u4 a, dn_u4 b, dn_v4f c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(dn_v8h, a), __builtin_bit_cast(dn_v8h, b), c, 0, 0, 0);
 }
 
-template <int DT, int MT, int RT>
+// SILU (the gate|up projection of a SwiGLU MLP, N = 2F rows: gate rows first, up rows behind them): a workgroup
+// owns PAIRS of tiles, (gate tile p, up tile p + F/16), and its output stage writes act[m, f] =
+// round(silu(round(gate))) * round(up) to y[M, F] instead of the 2F projections.
+template <int DT, int MT, int RT, bool SILU = false>
 __global__ __launch_bounds__(kDnThreads) void dense_gemm_kernel(
     const uint16_t* __restrict__ x, const uint16_t* __restrict__ w, const uint16_t* __restrict__ bias,
     const uint16_t* residual, uint16_t* y, float* __restrict__ partial, int M, int64_t N, int K, int splits,
@@ -58,9 +61,13 @@ __global__ __launch_bounds__(kDnThreads) void dense_gemm_kernel(
   const int g_first = g_begin + wave;                            // this wavefront's groups: g_first + 4j
   const int nj = g_first < g_end ? (g_end - g_first + 3) / 4 : 0;
 
-  // tiles [tile0, tile0 + ntl) of this workgroup: an even split of all tiles over the grid
-  const int tile0 = (int)((int64_t)blockIdx.x * n_tiles / gridDim.x);
-  const int ntl = (int)((int64_t)(blockIdx.x + 1) * n_tiles / gridDim.x) - tile0;     // 1 .. RT
+  // tiles [tile0, tile0 + ntl) of this workgroup: an even split of all tiles (SILU: of all tile pairs) over the grid
+  const int n_units = SILU ? n_tiles / 2 : n_tiles;
+  const int tile0 = (int)((int64_t)blockIdx.x * n_units / gridDim.x);                  // SILU: first pair = first gate tile
+  const int n_own = (int)((int64_t)(blockIdx.x + 1) * n_units / gridDim.x) - tile0;
+  const int ntl = SILU ? 2 * n_own : n_own;                                            // 1 .. RT
+  // tile t of this workgroup, counted from its first tile
+  auto tile_rel = [&](int t) { return SILU ? (t >> 1) + (t & 1) * (n_tiles / 2) : t; };
 
   dn_v4f acc[RT][MT];
 #pragma unroll
@@ -73,7 +80,7 @@ __global__ __launch_bounds__(kDnThreads) void dense_gemm_kernel(
   // return zeros outside the tensor.  The weight descriptor starts at this workgroup's first tile,
   // so its offsets stay far below the 2 GiB range whatever the size of the matrix.
   const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)x, 0, M * K * 2, 0x00027000);
-  const int64_t w_bytes = (int64_t)ntl * 16 * K * 2;
+  const int64_t w_bytes = (int64_t)(tile_rel(ntl - 1) + 1) * 16 * K * 2;            // up to the last tile it touches
   const __amdgpu_buffer_rsrc_t w_rsrc =
       __builtin_amdgcn_make_buffer_rsrc((void*)(w + (int64_t)tile0 * 16 * K), 0, (int)w_bytes, 0x00027000);
   constexpr int kXg = MT * 2;                                    // 16-byte pieces per lane of one group block
@@ -84,7 +91,7 @@ __global__ __launch_bounds__(kDnThreads) void dense_gemm_kernel(
   const int w_lane = (ln * K + c * 16) * 2;                      // byte offset of this lane's 32 bytes inside a tile
   int wofs[RT];                                                  // byte offset of (tile t, k = 0) from the first tile
 #pragma unroll
-  for (int t = 0; t < RT; ++t) wofs[t] = min(t, ntl - 1) * 16 * K * 2;
+  for (int t = 0; t < RT; ++t) wofs[t] = tile_rel(min(t, ntl - 1)) * 16 * K * 2;
 
   dn_u4 xg[kXg];                                                 // block on its way from global memory to LDS
   dn_u4 wbuf[2][RT][2];
@@ -154,6 +161,8 @@ __global__ __launch_bounds__(kDnThreads) void dense_gemm_kernel(
   // round.  LDS holds two rounds, so a round needs one barrier; wavefront w finishes the activation
   // row blocks mt = w, w + 4, ... of the tile.  Accumulator layout: rows m = 16*mt + 4*c + rr,
   // column n = 16*tile + ln.
+  float gate_held[MT][4];                                        // SILU: the rounded gate values between two rounds
+  (void)gate_held;
 #pragma unroll
   for (int t = 0; t < RT; ++t) {
     if (t >= ntl) break;                                         // uniform
@@ -161,7 +170,7 @@ __global__ __launch_bounds__(kDnThreads) void dense_gemm_kernel(
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) *(dn_v4f*)(&stage[((wave * MT + mt) * 64 + lane) * 4]) = acc[t][mt];
     __syncthreads();                                             // round t written; round t - 1 fully read
-    const int64_t n = (int64_t)(tile0 + t) * 16 + ln;
+    const int64_t n = (int64_t)(tile0 + tile_rel(t)) * 16 + ln;
     const float bv = (splits == 1 && bias) ? Elem<DT>::load(bias, n) : 0.f;
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
@@ -173,12 +182,29 @@ __global__ __launch_bounds__(kDnThreads) void dense_gemm_kernel(
 #pragma unroll
         for (int rr = 0; rr < 4; ++rr) v[rr] += o[rr];
       }
+      if constexpr (SILU) {
+        // even round: the gate tile, kept in registers; odd round: its up tile, same wavefront, same lanes
+        if ((t & 1) == 0) {
 #pragma unroll
-      for (int rr = 0; rr < 4; ++rr) {
-        const int m = mt * 16 + c * 4 + rr;
-        if (m >= M) continue;
-        if (splits == 1) store_linear_out<DT>(y, (int64_t)m * N + n, v[rr] + bv, residual);
-        else partial[((int64_t)ks * M + m) * N + n] = v[rr];
+          for (int rr = 0; rr < 4; ++rr) gate_held[mt][rr] = Elem<DT>::round(v[rr] + bv);
+        } else {
+          const int64_t f = (int64_t)(tile0 + (t >> 1)) * 16 + ln;
+#pragma unroll
+          for (int rr = 0; rr < 4; ++rr) {
+            const int m = mt * 16 + c * 4 + rr;
+            if (m >= M) continue;
+            const float g = gate_held[mt][rr], u = Elem<DT>::round(v[rr] + bv);
+            Elem<DT>::store(y, (int64_t)m * (N / 2) + f, Elem<DT>::round(g / (1.f + __expf(-g))) * u);
+          }
+        }
+      } else {
+#pragma unroll
+        for (int rr = 0; rr < 4; ++rr) {
+          const int m = mt * 16 + c * 4 + rr;
+          if (m >= M) continue;
+          if (splits == 1) store_linear_out<DT>(y, (int64_t)m * N + n, v[rr] + bv, residual);
+          else partial[((int64_t)ks * M + m) * N + n] = v[rr];
+        }
       }
     }
   }
@@ -214,6 +240,30 @@ static DnPlan dn_plan(int64_t M, int64_t N, int64_t K) {
   gps = (gps + 3) / 4 * 4;
   splits = (G + gps - 1) / gps;
   return DnPlan{(int)wgs, row_tiles, splits, gps};
+}
+
+// gate|up projection with the SwiGLU output stage: x [M, K], W [2F, K] (gate rows first), act [M, F]
+template <int DT>
+static int run_dense_silu(const void* x, const void* w, const void* bias, void* act, int64_t M, int64_t N, int64_t K,
+                          hipStream_t st) {
+  const int64_t pairs = N / 32;
+  // tile pairs per workgroup: one with few activation rows (more, smaller workgroups stream weights faster), two at
+  // 64 rows, where a workgroup's activation blocks are amortised over more tiles
+  const int rt = M <= 32 ? 2 : 4;
+  const int64_t wgs = (pairs + rt / 2 - 1) / (rt / 2);
+  const dim3 grid((unsigned)wgs, 1);
+  const int G = (int)(K / kDnGroup);
+#define SUBSPEC_DN_SILU(MT, RT)                                                                                    \
+  hipLaunchKernelGGL((dense_gemm_kernel<DT, MT, RT, true>), grid, dim3(kDnThreads), 0, st, (const uint16_t*)x,    \
+                     (const uint16_t*)w, (const uint16_t*)bias, (const uint16_t*)nullptr, (uint16_t*)act, (float*)nullptr,     \
+                     (int)M, N, (int)K, 1, (G + 3) / 4 * 4)
+  DominantKernelTimer timer(st);
+  if (M <= 16) SUBSPEC_DN_SILU(1, 2);
+  else if (M <= 32) SUBSPEC_DN_SILU(2, 2);
+  else SUBSPEC_DN_SILU(4, 4);
+#undef SUBSPEC_DN_SILU
+  SUBSPEC_CHECK_HIP(hipGetLastError());
+  return SUBSPEC_OK;
 }
 
 template <int DT>
@@ -260,6 +310,29 @@ extern "C" size_t subspec_dense_linear_workspace(int64_t M, int64_t N, int64_t K
 extern "C" int subspec_dense_linear(const void* x, const void* w, const void* bias, void* y, int dtype, int64_t M,
                                     int64_t N, int64_t K, void* workspace, size_t workspace_bytes, void* stream) {
   return dense_linear_ex(x, w, bias, nullptr, y, dtype, M, N, K, workspace, workspace_bytes, stream);
+}
+
+int subspec::dense_gate_up_silu_ex(const void* x, const void* w, const void* bias, void* act, int dtype, int64_t M, int64_t N,
+                                   int64_t K, void* stream) {
+  if (dtype != SUBSPEC_BF16 && dtype != SUBSPEC_F16)
+    SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "dense_gate_up_silu: dtype %d not supported (bf16 / fp16 only)", dtype);
+  if (!x || !w || !act) SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "dense_gate_up_silu: null pointer argument");
+  if (M <= 0 || M > 64 || N <= 0 || K <= 0 || N % 32 != 0 || K % kDnGroup != 0 || K > 65536)
+    SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "dense_gate_up_silu: M=%lld N=%lld K=%lld; 1 <= M <= 64, N a multiple of 32, K of 64",
+                 (long long)M, (long long)N, (long long)K);
+  // a workgroup's weight descriptor spans from its gate tiles to its up tiles: more than half the matrix
+  if (N * K * 2 >= ((int64_t)1 << 31))
+    SUBSPEC_FAIL(SUBSPEC_ERR_LIMIT, "dense_gate_up_silu: N*K*2=%lld bytes exceed the 2 GiB descriptor range", (long long)(N * K * 2));
+  if ((uintptr_t)x % 16 || (uintptr_t)w % 16 || (uintptr_t)act % 2)
+    SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "dense_gate_up_silu: x and w must be 16-byte aligned");
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == SUBSPEC_BF16) return run_dense_silu<SUBSPEC_BF16>(x, w, bias, act, M, N, K, st);
+  return run_dense_silu<SUBSPEC_F16>(x, w, bias, act, M, N, K, st);
+}
+
+extern "C" int subspec_dense_gate_up_silu(const void* x, const void* w, const void* bias, void* act, int dtype, int64_t M,
+                                          int64_t N, int64_t K, void* stream) {
+  return subspec::dense_gate_up_silu_ex(x, w, bias, act, dtype, M, N, K, stream);
 }
 
 int subspec::dense_linear_ex(const void* x, const void* w, const void* bias, const void* residual, void* y, int dtype, int64_t M,

@@ -492,6 +492,27 @@ def int4_gate_up_silu(x: torch.Tensor, wq: torch.Tensor, sz: torch.Tensor, inter
     return act.reshape(*x.shape[:-1], N // 2)
 
 
+def dense_gate_up_silu(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``silu(gate) * up`` from a dense fused weight [2F, K] (gate rows first) in one launch: x [..., K] (at most 64
+    rows) -> [..., F]."""
+    dev = _require_gpu(x, weight)
+    N, K = weight.shape
+    if x.shape[-1] != K or x.dtype != weight.dtype or N % 2:
+        raise ValueError("dense_gate_up_silu: x [..., K] and weight [2F, K] must agree in K and dtype")
+    M = x.numel() // K
+    x2 = x.reshape(M, K).contiguous()
+    weight = weight.contiguous()
+    if bias is not None:
+        if bias.dtype != x.dtype or bias.numel() != N:
+            raise ValueError("dense_gate_up_silu: bias must be [2F] in the activation dtype")
+        bias = bias.contiguous()
+    act = torch.empty((M, N // 2), dtype=x.dtype, device=dev)
+    code = L.lib().subspec_dense_gate_up_silu(x2.data_ptr(), weight.data_ptr(), None if bias is None else bias.data_ptr(),
+                                             act.data_ptr(), _dtype_code(x2), M, N, K, _stream(dev))
+    L.check(code, "subspec_dense_gate_up_silu")
+    return act.reshape(*x.shape[:-1], N // 2)
+
+
 def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
     """``weight * (x * rsqrt(mean(x^2) + eps)).to(x.dtype)`` over the last dimension in one launch
     (bf16 / fp16; hidden a multiple of 8, at most 16384)."""

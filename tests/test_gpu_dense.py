@@ -125,3 +125,25 @@ def test_single_dense_layer_against_float32_oracle():
     assert err <= 2e-2 * want.abs().amax().item(), (err, want.abs().amax().item())
     assert (kv.cache.k(0)[0].float().cpu() - kc).abs().amax().item() <= 2e-2 * kc.abs().amax().item()
     assert (kv.cache.v(0)[0].float().cpu() - vc).abs().amax().item() <= 2e-2 * vc.abs().amax().item()
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_dense_gate_up_projection_with_the_activation_in_its_output_stage(dtype):
+    """As for the int4 twin: the fused launch against the plain projection followed by the activation on the values
+    it stored; only the exponential may differ in its last place."""
+    for seed, (F, K, M, bias) in enumerate([(16, 64, 1, False), (48, 192, 5, True), (1184, 128, 17, True), (18944, 3584, 8, False),
+                                            (18944, 3584, 64, False), (2048, 512, 33, True), (40000, 64, 3, False)]):
+        print("dense gate|up + silu", dtype, F, K, M, bias, flush=True)
+        g = torch.Generator().manual_seed(800 + seed)
+        W = (torch.randn(2 * F, K, generator=g) * (2.0 / K ** 0.5)).to(dtype).to(DEV)
+        x = torch.randn(M, K, generator=g).to(dtype).to(DEV)
+        b = (torch.randn(2 * F, generator=g) * 0.1).to(dtype).to(DEV) if bias else None
+        got = ops.dense_gate_up_silu(x, W, b)
+        gu = ops.dense_linear(x, W, b)
+        gate, up = gu[:, :F].float(), gu[:, F:].float()
+        want = ((gate / (1 + torch.exp(-gate))).to(dtype).float() * up).to(dtype)
+        assert got.shape == (M, F) and got.dtype == dtype
+        differing = int((got != want).sum())
+        assert differing <= max(1, got.numel() // 1000), (F, K, M, differing)
+        ulp = 2.0 ** (-7 if dtype == torch.bfloat16 else -10)
+        assert ((got.float() - want.float()).abs() <= 2 * ulp * want.float().abs() + 1e-6).all()
