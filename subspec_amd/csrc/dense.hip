@@ -93,18 +93,25 @@ __global__ __launch_bounds__(kDnThreads) void dense_gemm_kernel(
 #pragma unroll
   for (int t = 0; t < RT; ++t) wofs[t] = tile_rel(min(t, ntl - 1)) * 16 * K * 2;
 
-  dn_u4 xg[kXg];                                                 // block on its way from global memory to LDS
-  dn_u4 wbuf[2][RT][2];
+  // Activation blocks on their way from global memory to LDS: requested kXSlots steps before they are parked (a
+  // block that is parked one step after its request makes every step wait for a whole round trip to L2).
+  constexpr int kXSlots = MT == 4 ? 1 : 2;   // 64 rows: one (with two the compiler waits for every request at the top of the loop body)
+  dn_u4 xg[kXSlots][kXg];
+  // Weights on their way, two groups ahead.  With one tile per workgroup they rotate through three register slots, so
+  // that a request never targets the slot the current step multiplies from (the compiler would issue it first, into
+  // other registers, and copy at the end of the loop body behind a wait for every request in flight).
+  constexpr int kWSlots = RT == 1 ? 3 : 2;
+  dn_u4 wbuf[kWSlots][RT][2];
 
-#define SUBSPEC_DN_FETCH_X(J)                                                                           \
+#define SUBSPEC_DN_FETCH_X(XS, J)                                                                       \
   {                                                                                                     \
     const int kc = min(g_first + 4 * (J), G - 1) * (kDnGroup * 2);                                      \
     _Pragma("unroll") for (int i = 0; i < kXg; ++i)                                                     \
-      xg[i] = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, xg_off + i * 16 * K, kc, 0);                \
+      xg[XS][i] = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, xg_off + i * 16 * K, kc, 0);            \
   }
 #define SUBSPEC_DN_PARK_X(SLOT)                                                                         \
   _Pragma("unroll") for (int i = 0; i < kXg; ++i)                                                       \
-    *(dn_u4*)(&xl[(SLOT) * (MT * 16 * kDnXlStride) + i * 8 * kDnXlStride + xl_write]) = xg[i];
+    *(dn_u4*)(&xl[(SLOT) * (MT * 16 * kDnXlStride) + i * 8 * kDnXlStride + xl_write]) = xg[(SLOT) % kXSlots][i];
 #define SUBSPEC_DN_FETCH_W(SLOT, J, T)                                                                  \
   {                                                                                                     \
     const int kc = wofs[T] + min(g_first + 4 * (J), G - 1) * (kDnGroup * 2);                            \
@@ -112,9 +119,9 @@ __global__ __launch_bounds__(kDnThreads) void dense_gemm_kernel(
     wbuf[SLOT][T][1] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, w_lane + 16, kc, 0);               \
   }
   // Step J works on LDS stage SLOT = J & 1.  Once its operands are in registers the stage is free:
-  // the block of group J + 2 (requested one step ago) is parked there and group J + 3 requested.
+  // the block of group J + 2 (requested kXSlots steps ago) is parked there and group J + 2 + kXSlots requested.
   // A step past the wavefront's last group multiplies activations that were replaced by zeros.
-#define SUBSPEC_DN_STEP(SLOT, J)                                                                        \
+#define SUBSPEC_DN_STEP(SLOT, WS, WNEXT, J)                                                             \
   {                                                                                                     \
     const bool step_live = (J) < nj;                                                                    \
     dn_u4 xa[MT][2];                                                                                    \
@@ -125,31 +132,49 @@ __global__ __launch_bounds__(kDnThreads) void dense_gemm_kernel(
       xa[mt][1] = step_live ? a1 : dn_u4{0u, 0u, 0u, 0u};                                               \
     }                                                                                                   \
     SUBSPEC_DN_PARK_X(SLOT);                                                                            \
-    SUBSPEC_DN_FETCH_X((J) + 3);                                                                        \
+    SUBSPEC_DN_FETCH_X((SLOT) % kXSlots, (J) + 2 + kXSlots);                                            \
     __builtin_amdgcn_sched_barrier(0);              /* keep the requests here: a full step ahead of their use */ \
+    /* The request for group J + 2 follows the last product of the tile whose registers it reuses: requested     */ \
+    /* earlier, the new weights get registers of their own and a copy at the end of the loop body, which waits   */ \
+    /* for EVERY request in flight.  (One tile per workgroup: a third slot instead, see wbuf.)                   */ \
     _Pragma("unroll") for (int t = 0; t < RT; ++t) {                                                    \
-      const dn_u4 b0 = wbuf[SLOT][t][0], b1 = wbuf[SLOT][t][1];                                         \
-      SUBSPEC_DN_FETCH_W(SLOT, (J) + 2, t);                                                             \
       _Pragma("unroll") for (int mt = 0; mt < MT; ++mt) {                                               \
-        acc[t][mt] = dn_mfma32<DT>(xa[mt][0], b0, acc[t][mt]);                                          \
-        acc[t][mt] = dn_mfma32<DT>(xa[mt][1], b1, acc[t][mt]);                                          \
+        acc[t][mt] = dn_mfma32<DT>(xa[mt][0], wbuf[WS][t][0], acc[t][mt]);                              \
+        acc[t][mt] = dn_mfma32<DT>(xa[mt][1], wbuf[WS][t][1], acc[t][mt]);                              \
       }                                                                                                 \
+      __builtin_amdgcn_sched_barrier(0);                                                                \
+      SUBSPEC_DN_FETCH_W(WNEXT, (J) + 2, t);                                                            \
     }                                                                                                   \
     __builtin_amdgcn_sched_barrier(0);                                                                  \
   }
 
-  SUBSPEC_DN_FETCH_X(0);
+  SUBSPEC_DN_FETCH_X(0, 0);
 #pragma unroll
   for (int t = 0; t < RT; ++t) SUBSPEC_DN_FETCH_W(0, 0, t);
   SUBSPEC_DN_PARK_X(0);
-  SUBSPEC_DN_FETCH_X(1);
+  SUBSPEC_DN_FETCH_X(1 % kXSlots, 1);
 #pragma unroll
   for (int t = 0; t < RT; ++t) SUBSPEC_DN_FETCH_W(1, 1, t);
   SUBSPEC_DN_PARK_X(1);
-  SUBSPEC_DN_FETCH_X(2);
-  for (int j = 0; j < nj; j += 2) {
-    SUBSPEC_DN_STEP(0, j);
-    SUBSPEC_DN_STEP(1, j + 1);
+  SUBSPEC_DN_FETCH_X(0, 2);
+  if constexpr (kXSlots == 2) SUBSPEC_DN_FETCH_X(1, 3);
+  if constexpr (RT == 1) {
+    // step J: LDS stage J % 2, weight slot J % 3, request for group J + 2 into slot (J + 2) % 3
+    for (int j = 0; j < nj; j += 6) {
+      SUBSPEC_DN_STEP(0, 0, 2, j);
+      SUBSPEC_DN_STEP(1, 1, 0, j + 1);
+      if (j + 2 >= nj) break;
+      SUBSPEC_DN_STEP(0, 2, 1, j + 2);
+      SUBSPEC_DN_STEP(1, 0, 2, j + 3);
+      if (j + 4 >= nj) break;
+      SUBSPEC_DN_STEP(0, 1, 0, j + 4);
+      SUBSPEC_DN_STEP(1, 2, 1, j + 5);
+    }
+  } else {
+    for (int j = 0; j < nj; j += 2) {
+      SUBSPEC_DN_STEP(0, 0, 0, j);
+      SUBSPEC_DN_STEP(1, 1, 1, j + 1);
+    }
   }
   __syncthreads();                                               // the stages are reused for the reduction below
 #undef SUBSPEC_DN_PARK_X
@@ -231,10 +256,16 @@ static DnPlan dn_plan(int64_t M, int64_t N, int64_t K) {
   const int G = (int)(K / kDnGroup);
   const int64_t tiles = N / 16, slots = M <= 16 ? 4096 : M <= 32 ? 1024 : 256;
   const int64_t want = (tiles + slots - 1) / slots;
-  const int row_tiles = want <= 1 ? 1 : want <= 2 ? 2 : 4;
+  int row_tiles = want <= 1 ? 1 : want <= 2 ? 2 : 4;
+  // More than 32 rows over a long K (the down projection, 3584 x 18944): one tile per workgroup fetches four bytes
+  // of activations for every byte of weights; four tiles and four K ranges keep as many workgroups with a quarter of
+  // that (M = 64: 46.7 us with the reduction against 61.5 us).
+  const bool long_k = M > 32 && G >= 224;
+  if (long_k) row_tiles = 4;
   const int64_t wgs = (tiles + row_tiles - 1) / row_tiles;
   int splits = (int)std::max<int64_t>(1, (slots + wgs / 2) / wgs);
   splits = std::min(splits, std::max(1, G / 112));             // a split costs a second launch: only for long K (two at K = 18944)
+  if (long_k) splits = 4;
   splits = std::min(splits, 16);
   int gps = (G + splits - 1) / splits;
   gps = (gps + 3) / 4 * 4;
@@ -247,9 +278,10 @@ template <int DT>
 static int run_dense_silu(const void* x, const void* w, const void* bias, void* act, int64_t M, int64_t N, int64_t K,
                           hipStream_t st) {
   const int64_t pairs = N / 32;
-  // tile pairs per workgroup: one with few activation rows (more, smaller workgroups stream weights faster), two at
-  // 64 rows, where a workgroup's activation blocks are amortised over more tiles
-  const int rt = M <= 32 ? 2 : 4;
+  // tile pairs per workgroup: one with few activation rows (more, smaller workgroups stream weights faster), three
+  // above 32 rows, where a workgroup's activation blocks are amortised over more tiles (37888 x 3584, M = 64: 79.9 us
+  // against 87.1 us at two pairs)
+  const int rt = M <= 32 ? 2 : 6;
   const int64_t wgs = (pairs + rt / 2 - 1) / (rt / 2);
   const dim3 grid((unsigned)wgs, 1);
   const int G = (int)(K / kDnGroup);
@@ -260,7 +292,7 @@ static int run_dense_silu(const void* x, const void* w, const void* bias, void* 
   DominantKernelTimer timer(st);
   if (M <= 16) SUBSPEC_DN_SILU(1, 2);
   else if (M <= 32) SUBSPEC_DN_SILU(2, 2);
-  else SUBSPEC_DN_SILU(4, 4);
+  else SUBSPEC_DN_SILU(4, 6);
 #undef SUBSPEC_DN_SILU
   SUBSPEC_CHECK_HIP(hipGetLastError());
   return SUBSPEC_OK;

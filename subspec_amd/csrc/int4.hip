@@ -215,9 +215,17 @@ __global__ __launch_bounds__(kI4Threads) void int4_gemm_kernel(
 #pragma unroll
   for (int t = 0; t < RT; ++t) wofs[t] = tile_of(min(t, ntl - 1)) * G;
 
-  i4_u4 xg[kXg];                                                 // block on its way from global memory to LDS
-  i4_u2 wbuf[2][RT];
-  uint32_t szbuf[2][RT];
+  // Activation blocks on their way from global memory to LDS: requested kXSlots steps before they are parked (a
+  // block that is parked one step after its request makes every step wait for a whole round trip to L2).
+  constexpr int kXSlots = MT == 4 ? 1 : 2;   // 64 rows: one (with two the compiler waits for every request at the top of the loop body)
+  i4_u4 xg[kXSlots][kXg];
+  // Weight words on their way: two groups ahead.  With one tile per workgroup they rotate through THREE register
+  // slots, so that a request never targets the slot the current step still reads: the compiler issues the request
+  // before those reads, gives it other registers and copies them at the end of the loop body, and that copy waits for
+  // EVERY request in flight, once per trip.  With more tiles it orders reads and requests so that two slots do.
+  constexpr int kWSlots = RT == 1 ? 3 : 2;
+  i4_u2 wbuf[kWSlots][RT];
+  uint32_t szbuf[kWSlots][RT];
   // Both constants of ((w >> s) & mask) | magic as run-time values (M >> 30 is zero): with two
   // literals the compiler emits v_and + v_or, with a scalar and a vector register operand one v_and_or_b32.
   // (xg_off >> 31 is zero too and lives in a vector register.)
@@ -225,15 +233,15 @@ __global__ __launch_bounds__(kI4Threads) void int4_gemm_kernel(
   const uint32_t one2 = DT == SUBSPEC_BF16 ? 0x3f803f80u : 0x3c003c00u;
   const i4_u4 ones = i4_u4{one2, one2, one2, one2};
 
-#define SUBSPEC_I4_FETCH_X(J)                                                                           \
+#define SUBSPEC_I4_FETCH_X(XS, J)                                                                       \
   {                                                                                                     \
     const int kc = min(g_first + 4 * (J), G - 1) * (kGroup * 2);                                        \
     _Pragma("unroll") for (int i = 0; i < kXg; ++i)                                                     \
-      xg[i] = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, xg_off + i * 16 * K, kc, 0);                \
+      xg[XS][i] = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, xg_off + i * 16 * K, kc, 0);            \
   }
 #define SUBSPEC_I4_PARK_X(SLOT)                                                                         \
   _Pragma("unroll") for (int i = 0; i < kXg; ++i)                                                       \
-    *(i4_u4*)(&xl[(SLOT) * (MT * 16 * kXlStride) + i * 8 * kXlStride + xl_write]) = xg[i];
+    *(i4_u4*)(&xl[(SLOT) * (MT * 16 * kXlStride) + i * 8 * kXlStride + xl_write]) = xg[(SLOT) % kXSlots][i];
 #define SUBSPEC_I4_FETCH_W(SLOT, J, T)                                                                  \
   {                                                                                                     \
     const int g = wofs[T] + min(g_first + 4 * (J), G - 1);                                              \
@@ -241,8 +249,8 @@ __global__ __launch_bounds__(kI4Threads) void int4_gemm_kernel(
     szbuf[SLOT][T] = __builtin_amdgcn_raw_buffer_load_b32(sz_rsrc, ln * 4, g * 64, 0);                  \
   }
   // Step J works on LDS stage SLOT = J & 1.  Once its operands are in registers the stage is free:
-  // the block of group J + 2 (requested one step ago) is parked there and group J + 3 requested.
-#define SUBSPEC_I4_STEP(SLOT, J)                                                                        \
+  // the block of group J + 2 (requested kXSlots steps ago) is parked there and group J + 2 + kXSlots requested.
+#define SUBSPEC_I4_STEP(SLOT, WS, WNEXT, J)                                                             \
   {                                                                                                     \
     const bool step_live = (J) < nj;                /* a dead step multiplies by a zero scale: no branch */ \
     i4_u4 xa[MT][2];                                                                                    \
@@ -252,7 +260,7 @@ __global__ __launch_bounds__(kI4Threads) void int4_gemm_kernel(
       xa[mt][1] = *(const i4_u4*)(xr + 8);                                                              \
     }                                                                                                   \
     SUBSPEC_I4_PARK_X(SLOT);                                                                            \
-    SUBSPEC_I4_FETCH_X((J) + 3);                                                                        \
+    SUBSPEC_I4_FETCH_X((SLOT) % kXSlots, (J) + 2 + kXSlots);                                            \
     __builtin_amdgcn_sched_barrier(0);              /* keep the requests here: a full step ahead of their use */ \
     i4_v4f xs[MT];                                  /* sum of the group's activations, rows 16mt + 4c + rr */ \
     _Pragma("unroll") for (int mt = 0; mt < MT; ++mt) {                                                 \
@@ -260,14 +268,14 @@ __global__ __launch_bounds__(kI4Threads) void int4_gemm_kernel(
       xs[mt] = i4_mfma32<DT>(xa[mt][1], ones, xs[mt]);                                                  \
     }                                                                                                   \
     _Pragma("unroll") for (int t = 0; t < RT; ++t) {                                                    \
-      const uint32_t w0 = wbuf[SLOT][t].x, w1 = wbuf[SLOT][t].y, szw = szbuf[SLOT][t];                  \
+      const uint32_t w0 = wbuf[WS][t].x, w1 = wbuf[WS][t].y, szw = szbuf[WS][t];                        \
       const i4_u4 b0 = i4_u4{code_pair(w0, 0, kmagic, kmask), code_pair(w0, 4, kmagic, kmask),          \
                              code_pair(w0, 8, kmagic, kmask), code_pair(w0, 12, kmagic, kmask)};        \
       const i4_u4 b1 = i4_u4{code_pair(w1, 0, kmagic, kmask), code_pair(w1, 4, kmagic, kmask),          \
                              code_pair(w1, 8, kmagic, kmask), code_pair(w1, 12, kmagic, kmask)};        \
       const float sc = (step_live && t < ntl) ? f16_bits_to_float(szw & 0xffffu) : 0.f;                 \
       const float szo = -sc * (f16_bits_to_float(szw >> 16) + I4<DT>::kOffset);                         \
-      SUBSPEC_I4_FETCH_W(SLOT, (J) + 2, t);                                                             \
+      SUBSPEC_I4_FETCH_W(WNEXT, (J) + 2, t);                                                            \
       _Pragma("unroll") for (int mt = 0; mt < MT; ++mt) {                                               \
         i4_v4f raw = i4_mfma32<DT>(xa[mt][0], b0, i4_v4f{0.f, 0.f, 0.f, 0.f});                          \
         raw = i4_mfma32<DT>(xa[mt][1], b1, raw);                                                        \
@@ -278,18 +286,33 @@ __global__ __launch_bounds__(kI4Threads) void int4_gemm_kernel(
     __builtin_amdgcn_sched_barrier(0);                                                                  \
   }
 
-  SUBSPEC_I4_FETCH_X(0);
+  SUBSPEC_I4_FETCH_X(0, 0);
 #pragma unroll
   for (int t = 0; t < RT; ++t) SUBSPEC_I4_FETCH_W(0, 0, t);
   SUBSPEC_I4_PARK_X(0);
-  SUBSPEC_I4_FETCH_X(1);
+  SUBSPEC_I4_FETCH_X(1 % kXSlots, 1);
 #pragma unroll
   for (int t = 0; t < RT; ++t) SUBSPEC_I4_FETCH_W(1, 1, t);
   SUBSPEC_I4_PARK_X(1);
-  SUBSPEC_I4_FETCH_X(2);
-  for (int j = 0; j < nj; j += 2) {
-    SUBSPEC_I4_STEP(0, j);
-    SUBSPEC_I4_STEP(1, j + 1);
+  SUBSPEC_I4_FETCH_X(0, 2);
+  if constexpr (kXSlots == 2) SUBSPEC_I4_FETCH_X(1, 3);
+  if constexpr (RT == 1) {
+    // step J: LDS stage J % 2, weight slot J % 3, request for group J + 2 into slot (J + 2) % 3
+    for (int j = 0; j < nj; j += 6) {
+      SUBSPEC_I4_STEP(0, 0, 2, j);
+      SUBSPEC_I4_STEP(1, 1, 0, j + 1);
+      if (j + 2 >= nj) break;
+      SUBSPEC_I4_STEP(0, 2, 1, j + 2);
+      SUBSPEC_I4_STEP(1, 0, 2, j + 3);
+      if (j + 4 >= nj) break;
+      SUBSPEC_I4_STEP(0, 1, 0, j + 4);
+      SUBSPEC_I4_STEP(1, 2, 1, j + 5);
+    }
+  } else {
+    for (int j = 0; j < nj; j += 2) {
+      SUBSPEC_I4_STEP(0, 0, 0, j);
+      SUBSPEC_I4_STEP(1, 1, 1, j + 1);
+    }
   }
   __syncthreads();                                               // the stages are reused for the reduction below
 #undef SUBSPEC_I4_PARK_X
