@@ -1,0 +1,69 @@
+"""The software pipelines of the linear kernels, checked in the compiler's assembly output.
+
+The int4 and dense GEMM kernels keep weight and activation requests several 64-k groups ahead of their use.
+That distance exists only while no instruction inside the main loop waits for EVERY outstanding request
+(``s_waitcnt vmcnt(0)``): one such wait per trip turns the prefetch back into load - wait - use.  The compiler
+inserts it whenever a loop-carried register slot is loaded while its old contents are still being read (the
+new value then lives in other registers and is copied into the slot at the end of the body, behind a full
+wait), which no test of results can see.  This test compiles the two sources to assembly with the build's own
+flags and looks at every loop of every GEMM kernel variant.
+"""
+import os
+import re
+import shutil
+import subprocess
+
+import pytest
+
+from subspec_amd import build as build_mod
+
+
+def _assembly(src: str, tmp_path) -> str:
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(hipcc):
+        pytest.skip("hipcc is not installed")
+    out = str(tmp_path / (os.path.basename(src) + ".s"))
+    flags = [f for f in build_mod.HIPCC_FLAGS if f != "-fPIC"]
+    subprocess.run([hipcc, *flags, "-S", "--cuda-device-only", "-w", src, "-o", out], check=True,
+                   stdout=subprocess.PIPE, stderr=subprocess.STDOUT, timeout=600)
+    with open(out) as f:
+        return f.read()
+
+
+def _loops_with_full_waits(asm: str, kernel_substring: str):
+    """[(kernel, loop length in lines, offsets of full waits)] for every loop of every matching kernel."""
+    found = []
+    kernel = None
+    open_loops = {}                                          # label -> (first line, offsets of full waits)
+    for i, line in enumerate(asm.split("\n")):
+        m = re.match(r"^(_Z\w+):", line)
+        if m:
+            kernel, open_loops = m.group(1), {}
+            continue
+        if kernel is None or kernel_substring not in kernel:
+            continue
+        m = re.match(r"^(\.LBB\d+_\d+):.*Loop Header", line)
+        if m:
+            open_loops[m.group(1)] = (i, [])
+        if "s_waitcnt" in line and re.search(r"vmcnt\(0\)", line):
+            for start, waits in open_loops.values():
+                waits.append(i - start)
+        m = re.search(r"\bs_cbranch_\w+\s+(\.LBB\d+_\d+)\b", line)
+        if m and m.group(1) in open_loops:
+            start, waits = open_loops.pop(m.group(1))
+            found.append((kernel, i - start, waits))
+    return found
+
+
+@pytest.mark.parametrize("source, kernel, min_kernels", [
+    ("int4.hip", "int4_gemm_kernel", 24),
+    ("dense.hip", "dense_gemm_kernel", 12),
+])
+def test_main_loops_never_wait_for_every_request(source, kernel, min_kernels, tmp_path):
+    asm = _assembly(os.path.join(build_mod.CSRC, source), tmp_path)
+    loops = _loops_with_full_waits(asm, kernel)
+    main_loops = [l for l in loops if l[1] >= 40]            # the pipelined loop; short loops are epilogue code
+    assert len({l[0] for l in main_loops}) >= min_kernels, "the parser found too few kernel variants"
+    stalled = [(k, n, w) for k, n, w in main_loops if w]
+    assert not stalled, "a full wait inside the pipelined loop of: " + ", ".join(
+        f"{k} (loop of {n} lines, at {w})" for k, n, w in stalled)
