@@ -1,4 +1,4 @@
-"""GPU: seeded random differential run of the verifier and the top-k expansion against the oracle.
+"""GPU: seeded random differential run of the verifier, the top-k expansion and the linear kernels against the oracle.
 
 Shapes, dtypes, tree forms and parameters are drawn at random (fixed seeds): trees of 1 to 300 nodes, vocabularies
 that are and are not multiples of the vector width, peaked / masked / heavily tied rows, an EOS token that may sit
@@ -146,3 +146,43 @@ def test_random_attention_and_compaction_cases(block):
         dev = cache.to(DEV)
         ops.kv_compact_(dev, torch.tensor(ctx, dtype=torch.int64, device=DEV), offset)
         assert torch.equal(dev.cpu(), okv.compact_static(cache, ctx, offset)), (tag, offset, count)
+
+
+@pytest.mark.parametrize("block", range(2))
+def test_random_linear_shapes_match_the_oracle(block):
+    """int4 g64 and dense projections (and the gate|up pair kernels with the SwiGLU stage) at random N, K, M: K from
+    one to 40 groups of 64 (every count of pipeline steps per wavefront, odd and even, shorter than the prefetch
+    distance and longer than one unrolled trip), 1 to 200 rows (one tile to several passes of 64)."""
+    from oracle import int4 as oi
+    from subspec_amd import quant
+    for case in range(20):
+        seed = 881000 + 100 * block + case
+        rng = random.Random(seed)
+        g = torch.Generator().manual_seed(seed)
+        dtype = rng.choice([torch.bfloat16, torch.float16])
+        N = 32 * rng.randrange(1, 48)
+        K = 64 * rng.randrange(1, 41)
+        M = rng.choice([1, 2, 7, 8, 16, 17, 32, 33, 64, 65, 200])
+        w = torch.randn(N, K, generator=g) * 0.02
+        x = torch.randn(M, K, generator=g).to(dtype)
+        b = (torch.randn(N, generator=g) * 0.1).to(dtype) if rng.random() < 0.5 else None
+        bd = None if b is None else b.to(DEV)
+        codes, scale, zero = quant.quantize_int4_g64(w)
+        wq, sz = quant.pack_tiled(codes, scale, zero)
+        tag = (seed, dtype, N, K, M, b is not None)
+
+        def silu_pairs(proj):                                    # float reference of the pair kernels' output
+            gate, up = proj[:, :N // 2].double(), proj[:, N // 2:].double()
+            return (gate / (1 + torch.exp(-gate)) * up).float()
+
+        def close(got, want):                                    # the fixed-shape tests hold the last-place checks
+            return (got - want).abs().amax().item() <= 1e-2 * max(want.abs().amax().item(), 1e-6)
+
+        want = oi.linear(x, codes, scale, zero, b)
+        assert close(ops.int4_linear(x.to(DEV), wq.to(DEV), sz.to(DEV), N, bd).float().cpu(), want), tag
+        if M <= 64:
+            assert close(ops.int4_gate_up_silu(x.to(DEV), wq.to(DEV), sz.to(DEV), N // 2, bd).float().cpu(), silu_pairs(want)), tag
+            wd = w.to(dtype)
+            want = x.float() @ wd.float().T + (0 if b is None else b.float())
+            assert close(ops.dense_linear(x.to(DEV), wd.to(DEV), bd).float().cpu(), want), tag
+            assert close(ops.dense_gate_up_silu(x.to(DEV), wd.to(DEV), bd).float().cpu(), silu_pairs(want)), tag
