@@ -48,7 +48,7 @@ def _loops_with_full_waits(asm: str, kernel_substring: str):
         if "s_waitcnt" in line and re.search(r"vmcnt\(0\)", line):
             for start, waits in open_loops.values():
                 waits.append(i - start)
-        m = re.search(r"\bs_cbranch_\w+\s+(\.LBB\d+_\d+)\b", line)
+        m = re.search(r"\bs_c?branch\w*\s+(\.LBB\d+_\d+)\b", line)
         if m and m.group(1) in open_loops:
             start, waits = open_loops.pop(m.group(1))
             found.append((kernel, i - start, waits))
