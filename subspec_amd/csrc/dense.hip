@@ -163,10 +163,8 @@ __global__ __launch_bounds__(kDnThreads) void dense_gemm_kernel(
     for (int j = 0; j < nj; j += 6) {
       SUBSPEC_DN_STEP(0, 0, 2, j);
       SUBSPEC_DN_STEP(1, 1, 0, j + 1);
-      if (j + 2 >= nj) break;
       SUBSPEC_DN_STEP(0, 2, 1, j + 2);
       SUBSPEC_DN_STEP(1, 0, 2, j + 3);
-      if (j + 4 >= nj) break;
       SUBSPEC_DN_STEP(0, 1, 0, j + 4);
       SUBSPEC_DN_STEP(1, 2, 1, j + 5);
     }
