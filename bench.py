@@ -17,12 +17,25 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0
-# HBM bytes per launch at the default workload, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs scaled
-# by a copy of known size (profiles/verify_cycle_config2_hbm_counters.md); None for other sizes.
-MEASURED_TRAFFIC = {
-    ("verify", 32, 152064): int(304836.5 * 1024 * 2.0 + 64.0 * 1024),
-    ("topk", 32, 152064): int(304339.5 * 1024 * 2.0 + 576.0 * 1024),
-}
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "verify_cycle_config2_hbm_counters.md")
+
+
+def measured_traffic(kernel, batch, vocab):
+    """HBM bytes per launch of `kernel` at the default workload, read from the committed counter summary (the rows
+    of its first table: FETCH_SIZE and WRITE_SIZE in KiB per dispatch from two `rocprofv3 --pmc` runs; FETCH_SIZE
+    counts the 16-byte-per-lane requests of these kernels at half their bytes, the calibration rows of the same
+    table show it, hence the factor 2).  None for any other size, or when the summary does not name the kernel: the
+    figure is a property of the profiled build, not of this run."""
+    import re
+    if (batch, vocab) != (32, 152064) or not os.path.exists(TRAFFIC_PROFILE):
+        return None
+    with open(TRAFFIC_PROFILE) as f:
+        for line in f:
+            m = re.match(r"\|\s*`subspec::" + re.escape(kernel) + r"[^|]*\|\s*([\d,\.]+)\s*\|\s*([\d,\.]+)\s*\|", line)
+            if m:
+                fetch_kib, write_kib = (float(g.replace(",", "")) for g in m.groups())
+                return int(fetch_kib * 1024 * 2.0 + write_kib * 1024)
+    return None
 
 
 def parse():
@@ -35,6 +48,8 @@ def parse():
     ap.add_argument("--cpu-trees", type=int, default=4, help="trees in the bounded CPU-baseline sample")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="lower bound of CPU-baseline work")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-e2e", action="store_true", help="default workload: leave out the bounded config-5 end-to-end block")
+    ap.add_argument("--e2e-tokens", type=int, default=32, help="default workload: new tokens of each config-5 run in the e2e block")
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="also run three plain copies of the logits tensor (known size) so that hardware byte counters "
                          "collected by rocprofv3 --pmc can be scaled")
@@ -209,10 +224,11 @@ def bench_dense(args):
         del wl
 
 
-def bench_e2e(args):
-    """BASELINE config 5: random-init Qwen2.5-7B-shaped decoder, target bf16 with layers 14-27 streamed
-    from pinned host memory every forward, substitute draft int4 g64 resident, depth-8 / k-8 tree
-    capped at 64 nodes, prompt 2048 random ids, 256 new tokens; exact and lossy verification."""
+def e2e_runs(args, runs, new_tokens, say=lambda *_: None):
+    """BASELINE config 5: random-init Qwen2.5-7B-shaped decoder, target bf16 with layers 14-27 streamed from pinned host
+    memory every forward, substitute draft int4 g64 resident, depth-8 / k-8 tree capped at 64 nodes, prompt 2048 random
+    ids; exact and lossy verification.  `runs`: (keep_layers, agreeing_draft) pairs, each generated with both
+    verification methods.  Returns one JSON-ready line per generation."""
     import torch
     from subspec_amd.cache import create_kv_cache
     from subspec_amd.draft import SubSpecSDDraftModel
@@ -223,57 +239,92 @@ def bench_e2e(args):
     from subspec_amd.utils import DraftParams
     from subspec_amd.wandb_logger import wandb_logger
     dev = "cuda:0"
-    t0 = time.perf_counter()
-    weights = None
-    if args.checkpoint:
-        cfg, weights = load_hf_checkpoint(args.checkpoint, device=dev)
-    else:
-        cfg = DecoderConfig()
-    if args.agreeing_draft:
-        weights = weights or init_weights(cfg, 0, dev)
-        for w in weights["layers"]:
-            for name in QUANTIZED:
-                t = w[name + ".weight"]
-                w[name + ".weight"] = quant.dequantize(*quant.quantize_int4_g64(t)).to(t.dtype)
-    kv = create_kv_cache("static", max_cache_len=2048 + args.new_tokens + 512 + 8, config=cfg, device=dev, dtype=torch.bfloat16)
-    target, draft, _ = build_models(cfg, kv, seed=0, device=dev, first_streamed=min(args.keep_layers, cfg.num_hidden_layers),
-                                    weights=weights, hqq_optimize=args.hqq_optimize)
-    print(f"# models built in {time.perf_counter() - t0:.1f} s", file=sys.stderr, flush=True)
-    prompt = torch.randint(0, cfg.vocab_size, (1, 2048), generator=torch.Generator().manual_seed(0)).to(dev)
-    for method, vk in (("exact", None), ("lossy", dict(threshold=0.3, window_size=6, threshold_method="entropy"))):
-        v2 = args.generator == "v2"
-        depth = args.tree_depth or (7 if v2 else 8)
-        cap = args.max_verify_tokens or None
-        gen = (SubSpecSDGeneratorV2 if v2 else SubSpecSDGenerator)(
-            target, None, SubSpecSDDraftModel(draft),
-            DraftParams(temperature=0.2, max_depth=depth, topk_len=args.tree_k, max_verify_tokens=cap),
-            generator_kwargs=dict(verify_method=method, verify_kwargs=vk,
-                                  **(dict(postspec_steps=args.postspec_steps) if v2 else {})))
-        kv.reset()
-        wandb_logger.clear_log_data()
-        if target.streamer is not None:
-            target.streamer.bytes_streamed = 0
-        out = gen.generate(prompt, max_new_tokens=args.new_tokens, do_sample=False, past_key_values=kv)
-        log = dict(wandb_logger.log_data)
-        line = {"metric": "accepted tokens/sec, end-to-end speculative cycle", "value": round(log["tput"], 2),
+    lines = []
+    base = None
+    for keep_layers, agreeing in runs:
+        t0 = time.perf_counter()
+        if args.checkpoint:
+            cfg, weights = load_hf_checkpoint(args.checkpoint, device=dev)
+        else:
+            cfg = DecoderConfig()
+            if base is None:
+                base = init_weights(cfg, 0, dev)
+            weights = {**base, "layers": [dict(w) for w in base["layers"]]}
+        if agreeing:
+            for w in weights["layers"]:
+                for name in QUANTIZED:
+                    t = w[name + ".weight"]
+                    w[name + ".weight"] = quant.dequantize(*quant.quantize_int4_g64(t)).to(t.dtype)
+        kv = create_kv_cache("static", max_cache_len=2048 + new_tokens + 512 + 8, config=cfg, device=dev, dtype=torch.bfloat16)
+        target, draft, _ = build_models(cfg, kv, seed=0, device=dev, first_streamed=min(keep_layers, cfg.num_hidden_layers),
+                                        weights=weights, hqq_optimize=args.hqq_optimize)
+        say(f"# models built in {time.perf_counter() - t0:.1f} s (resident target layers: {keep_layers}, agreeing draft: {agreeing})")
+        prompt = torch.randint(0, cfg.vocab_size, (1, 2048), generator=torch.Generator().manual_seed(0)).to(dev)
+        for method, vk in (("exact", None), ("lossy", dict(threshold=0.3, window_size=6, threshold_method="entropy"))):
+            v2 = args.generator == "v2"
+            depth = args.tree_depth or (7 if v2 else 8)
+            cap = args.max_verify_tokens or None
+            gen = (SubSpecSDGeneratorV2 if v2 else SubSpecSDGenerator)(
+                target, None, SubSpecSDDraftModel(draft),
+                DraftParams(temperature=0.2, max_depth=depth, topk_len=args.tree_k, max_verify_tokens=cap),
+                generator_kwargs=dict(verify_method=method, verify_kwargs=vk,
+                                      **(dict(postspec_steps=args.postspec_steps) if v2 else {})))
+            kv.reset()
+            wandb_logger.clear_log_data()
+            if target.streamer is not None:
+                target.streamer.bytes_streamed = 0
+            gen.generate(prompt, max_new_tokens=new_tokens, do_sample=False, past_key_values=kv)
+            log = dict(wandb_logger.log_data)
+            cycle_s = log.get("avg_draft_time", 0) + log.get("avg_target_time", 0) + log.get("avg_verify_time", 0)
+            h2d = target.streamer.bytes_streamed if target.streamer else 0
+            lines.append({
+                "metric": "accepted tokens/sec, end-to-end speculative cycle", "value": round(log["tput"], 2),
                 "unit": "tokens/s", "n_gpus": 1, "higher_is_better": True, "dtype": "bf16",
                 "data": ("synthetic prompt, weights from " + args.checkpoint if args.checkpoint else "synthetic")
-                        + (", target = the draft's dequantized int4 weights" if args.agreeing_draft else ""),
+                        + (", target = the draft's dequantized int4 weights" if agreeing else ""),
                 "config": {"workload": f"BASELINE config 5: {'checkpoint' if args.checkpoint else 'Qwen2.5-7B shape'}, "
-                                       + ("all layers resident" if args.keep_layers >= cfg.num_hidden_layers else
-                                          f"layers {args.keep_layers}-{cfg.num_hidden_layers - 1} streamed")
+                                       + ("all layers resident" if keep_layers >= cfg.num_hidden_layers else
+                                          f"layers {keep_layers}-{cfg.num_hidden_layers - 1} streamed")
                                        + f", int4 draft, depth {depth}, k {args.tree_k}, "
-                                       + (f"<={cap} nodes" if cap else f"{1 + depth * args.tree_k} nodes") + f", prompt 2048, {args.new_tokens} new tokens, verify {method}"
+                                       + (f"<={cap} nodes" if cap else f"{1 + depth * args.tree_k} nodes") + f", prompt 2048, {new_tokens} new tokens, verify {method}"
                                        + (", post-speculating driver" if v2 else ""),
-                           "verify_method": method, "generator": args.generator,
+                           "verify_method": method, "generator": args.generator, "resident_target_layers": min(keep_layers, cfg.num_hidden_layers),
+                           "agreeing_draft": bool(agreeing),
                            **({"post_verify_count": log["post_verify_count"], "speculate_count": log["speculate_count"]} if v2 else {}), "n_iter": log["n_iter"], "n_tokens": log["n_tokens"],
                            "tokens_per_cycle": round(log["avg_sampled"], 3),
                            "avg_draft_s": round(log.get("avg_draft_time", 0), 5),
                            "avg_target_s": round(log.get("avg_target_time", 0), 5),
                            "avg_verify_s": round(log.get("avg_verify_time", 0), 6),
+                           # tokens per second of the cycles alone (the prefill of the 2048-token prompt, which `value`
+                           # includes as the reference's tput does, weighs heavily on a short generation)
+                           "cycle_tokens_per_s": round(log["avg_sampled"] / cycle_s, 2) if cycle_s > 0 else None,
                            "elapsed_s": round(log["elapsed_time"], 3),
-                           "host_to_device_GB": round((target.streamer.bytes_streamed if target.streamer else 0) / 1e9, 2)}}
+                           "host_to_device_GB": round(h2d / 1e9, 2),
+                           "host_to_device_GB_per_s": round(h2d / 1e9 / log["elapsed_time"], 1) if h2d else 0.0}})
+        del target, draft, kv, weights
+        torch.cuda.empty_cache()
+    return lines
+
+
+def bench_e2e(args):
+    for line in e2e_runs(args, [(args.keep_layers, args.agreeing_draft)], args.new_tokens,
+                         say=lambda m: print(m, file=sys.stderr, flush=True)):
         print(json.dumps(line), flush=True)
+
+
+def e2e_block(args):
+    """The bounded config-5 runs the default line carries: `--e2e-tokens` new tokens after the 2048-token prompt, layers
+    14-27 streamed (the configuration BASELINE names) and all layers resident, random weights, exact and lossy; plus
+    the streamed cycle with a draft that agrees with its target (the high-acceptance end random weights cannot show)."""
+    keys = ("verify_method", "resident_target_layers", "agreeing_draft", "n_iter", "n_tokens", "tokens_per_cycle", "avg_draft_s",
+            "avg_target_s", "avg_verify_s", "cycle_tokens_per_s", "elapsed_s", "host_to_device_GB", "host_to_device_GB_per_s")
+    out = {"workload": f"BASELINE config 5, Qwen2.5-7B shape (28 layers, hidden 3584, 28/4 heads, FFN 18944, vocab 152064), int4 g64 "
+                       f"draft, depth 8, k 8, <=64 nodes, prompt 2048, {args.e2e_tokens} new tokens; tokens_per_s = new tokens / "
+                       "whole generate() including the prefill, cycle_tokens_per_s = tokens per cycle / (draft + target + verify)",
+           "runs": []}
+    for line in e2e_runs(args, [(14, False), (28, False), (14, True)], args.e2e_tokens):
+        out["runs"].append(dict({"tokens_per_s": line["value"]}, **{k: line["config"][k] for k in keys}))
+    return out
 
 
 def bench_greedy(args):
@@ -319,8 +370,17 @@ def cpu_baseline(cfg, probs_rows, parent_rows, n_trees, min_seconds):
     from oracle import topk as ot
     from oracle import verify as ov
 
-    cores = min(os.cpu_count() or 1, 16)
+    # threads: the CPUs this process may run on, capped by the thread limit the host sets for its jobs (OMP_NUM_THREADS)
+    cores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1)
+    if os.environ.get("OMP_NUM_THREADS", "").isdigit():
+        cores = max(1, min(cores, int(os.environ["OMP_NUM_THREADS"])))
     torch.set_num_threads(cores)
+    cpu_model = "unknown"
+    try:
+        with open("/proc/cpuinfo") as f:
+            cpu_model = next((l.split(":", 1)[1].strip() for l in f if l.startswith("model name")), "unknown")
+    except OSError:
+        pass
     vk = dict(threshold=cfg["threshold"], window_size=cfg["window_size"], threshold_method="entropy")
     logits = [cfg["logits"][b].cpu() for b in range(n_trees)]
     rows = probs_rows[: n_trees * 64].cpu()
@@ -345,7 +405,8 @@ def cpu_baseline(cfg, probs_rows, parent_rows, n_trees, min_seconds):
         if el >= min_seconds:
             break
     return {
-        "value": toks / el, "unit": "tokens/s", "cores": cores, "kind": "port",
+        "value": toks / el, "unit": "tokens/s", "cores": cores, "kind": "port", "cpu_model": cpu_model,
+        "host_logical_cpus": os.cpu_count(),
         "sample": f"{n_trees} of the batch's trees (64 rows x 152064 each: softmax, argmax, entr, DP) + "
                   f"top-16 of their {n_trees * 64} rows, {passes} passes in {el:.1f} s",
         "ms_per_tree": 1e3 * el / (passes * n_trees),
@@ -447,7 +508,9 @@ def main():
     def roof(nbytes, ms, which):
         gbs = nbytes / (ms * 1e-3) / 1e9
         return {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC.get((which, B, V))}
+                "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": measured_traffic(which, B, V),
+                "traffic_source": "profiles/verify_cycle_config2_hbm_counters.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of "
+                                  "the profiled build, not re-measured in this run)"}
 
     result = {
         "metric": "accepted tokens/sec + verify-cycle latency (Qwen2.5-7B shape); % HBM roofline",
@@ -462,16 +525,21 @@ def main():
                    "trees": B, "nodes": n, "vocab": V, "topk": k,
                    "tokens_per_step": tokens_per_step, "accepted_draft_tokens_per_step": accepted_per_step,
                    "verify_ms": round(verify_ms, 4), "topk_ms": round(topk_ms, 4)},
-        "roofline": dict(roof(bytes_verify, row_kernel_ms, "verify"), kernel="subspec::row_partial_kernel",
+        "roofline": dict(roof(bytes_verify, row_kernel_ms, "row_partial_kernel"), kernel="subspec::row_partial_kernel",
                          bytes_per_launch=bytes_verify, kernel_ms=round(row_kernel_ms, 4),
                          sequence_frac=round(bytes_verify / (verify_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)),
-        "roofline_topk": dict(roof(bytes_topk, topk_kernel_ms, "topk"), kernel="subspec::topk_slice_kernel",
+        "roofline_topk": dict(roof(bytes_topk, topk_kernel_ms, "topk_slice_kernel"), kernel="subspec::topk_slice_kernel",
                               bytes_per_launch=bytes_topk, kernel_ms=round(topk_kernel_ms, 4),
                               sequence_frac=round(bytes_topk / (topk_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)),
     }
+    cfg_cpu = None
     if not args.no_cpu_baseline:
         cfg_cpu = dict(cfg)
         result["cpu_baseline"] = cpu_baseline(cfg_cpu, draft, parent_probs, min(args.cpu_trees, B), args.cpu_seconds)
+    if not args.no_e2e:
+        cfg = cfg_cpu = draft = parent_probs = out = top = ws_v = ws_t = ev = None     # free the config-2 tensors
+        torch.cuda.empty_cache()
+        result["e2e_config5"] = e2e_block(args)
     print(json.dumps(result))
 
 

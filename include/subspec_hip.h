@@ -19,7 +19,7 @@
 extern "C" {
 #endif
 
-#define SUBSPEC_ABI_VERSION 1
+#define SUBSPEC_ABI_VERSION 2
 
 /* element types of logits / probabilities / KV / activations */
 #define SUBSPEC_F32 0
@@ -344,7 +344,8 @@ int subspec_dense_gate_up_silu(const void* x, const void* w, const void* bias, v
  *
  * x           device [n_rows, hidden], updated in place (the residual stream)
  * positions   device int32 [n_rows]   rotary position of each row (prefix_len + node depth)
- * cache_rows  device int32 [n_rows]   cache row each row's K / V is written to (prefix_len + slot)
+ * cache_rows  device int32 [n_rows]   cache row each row's K / V is written to (prefix_len + slot); a row outside
+ *             [0, kv_seq_stride) is not written (its K / V are dropped), so a bad tensor cannot leave the cache
  * anc_bits    device uint64 [n_rows, words]  as for subspec_tree_attention (words = ceil(n_tree_slots / 64))
  * k_cache, v_cache  device [n_kv_heads, kv_seq_stride, head_dim] of THIS layer (batch 1)
  * Limits: n_rows <= 64, n_tree_slots <= SUBSPEC_MAX_TREE_NODES, head_dim 128, hidden % 64 == 0 and <= 16384,
@@ -356,6 +357,10 @@ typedef struct subspec_decoder_layer_dims {
   int64_t n_rows, hidden, intermediate, n_q_heads, n_kv_heads, head_dim;
   int64_t kv_seq_stride, prefix_len, n_tree_slots;
   float rms_eps, rope_theta;
+  const float* rope_inv_freq; /* device float [head_dim / 2]: the inverse frequencies the caller's other code paths
+                                 use (HuggingFace: 1 / theta^(2i / head_dim), evaluated by torch), so that rows written
+                                 here and rows written by a prefill are rotated by identical angles; NULL: the kernel
+                                 evaluates rope_theta^(-2i / head_dim) itself */
 } subspec_decoder_layer_dims;
 
 typedef struct subspec_decoder_layer_weights {

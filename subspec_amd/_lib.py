@@ -29,7 +29,7 @@ class DecoderLayerDims(C.Structure):
     _fields_ = [("dtype", C.c_int32), ("reserved", C.c_int32),
                 ("n_rows", _i64), ("hidden", _i64), ("intermediate", _i64), ("n_q_heads", _i64), ("n_kv_heads", _i64),
                 ("head_dim", _i64), ("kv_seq_stride", _i64), ("prefix_len", _i64), ("n_tree_slots", _i64),
-                ("rms_eps", C.c_float), ("rope_theta", C.c_float)]
+                ("rms_eps", C.c_float), ("rope_theta", C.c_float), ("rope_inv_freq", C.c_void_p)]
 
 
 class DecoderLayerWeights(C.Structure):

@@ -125,6 +125,9 @@ class Tree:
             frontier = self.available_leaves
             first = self.current_size
             for j, (t, pr, lp) in enumerate(zip(lvl_tok, lvl_pr, lvl_par)):
+                if not 0 <= lp < len(frontier):
+                    raise ValueError(f"parent {lp} of a new node is not in the tree's frontier of {len(frontier)} nodes "
+                                     "(it was cut off by truncate())")
                 parent = frontier[lp]
                 self._token.append(int(t))
                 self._parent.append(parent)
@@ -177,7 +180,14 @@ class Tree:
         the tree at ``max_verify_tokens``; the dropped nodes are the least probable of the last level."""
         if n >= self.current_size:
             return torch.arange(self.current_size)
-        self._rebuild(list(range(max(1, int(n)))))
+        n = max(1, int(n))
+        frontier = [i for i in self.available_leaves if i < n]
+        self._rebuild(list(range(n)))
+        # The frontier stays what it was, minus the nodes cut off, IN ITS ORDER: a level added later names its parents
+        # by position in the previous level, and those positions must keep their meaning (a parent that was cut off
+        # is refused by add_nodes).  Shallower nodes that lost all their children do not become expandable.
+        if frontier:
+            self.available_leaves = frontier
         return torch.arange(self.current_size)
 
     # ------------------------------------------------------------------ export

@@ -128,22 +128,29 @@ template <int DT>
 __global__ __launch_bounds__(64) void rope_write_kernel(const uint16_t* __restrict__ qkv, const int32_t* __restrict__ positions,
                                                         const int32_t* __restrict__ cache_rows, uint16_t* __restrict__ q_out,
                                                         uint16_t* __restrict__ k_cache, uint16_t* __restrict__ v_cache,
-                                                        int M, int Hq, int Hkv, int D, int64_t seq_stride, float log2_theta) {
+                                                        int M, int Hq, int Hkv, int D, int64_t seq_stride, float log2_theta,
+                                                        const float* __restrict__ inv_freq_table) {
   const int m = blockIdx.x, hh = blockIdx.y, i = threadIdx.x;
   const int half = D / 2;
   if (i >= half) return;
   const uint16_t* src = qkv + ((int64_t)m * (Hq + 2 * Hkv) + hh) * D;
   const float lo = Elem<DT>::load(src, i), hi = Elem<DT>::load(src, i + half);
   uint16_t* dst;
-  if (hh < Hq) dst = q_out + ((int64_t)hh * M + m) * D;
-  else if (hh < Hq + Hkv) dst = k_cache + ((int64_t)(hh - Hq) * seq_stride + cache_rows[m]) * D;
-  else dst = v_cache + ((int64_t)(hh - Hq - Hkv) * seq_stride + cache_rows[m]) * D;
+  if (hh < Hq) {
+    dst = q_out + ((int64_t)hh * M + m) * D;
+  } else {
+    // a row outside the layer's cache is dropped: a bad rows tensor must not write beyond the cache
+    const int64_t row = cache_rows[m];
+    if (row < 0 || row >= seq_stride) return;
+    dst = (hh < Hq + Hkv ? k_cache + (int64_t)(hh - Hq) * seq_stride * D : v_cache + (int64_t)(hh - Hq - Hkv) * seq_stride * D) + row * D;
+  }
   if (hh >= Hq + Hkv) {                                 // value heads are copied
     Elem<DT>::store(dst, i, lo);
     Elem<DT>::store(dst, i + half, hi);
     return;
   }
-  const float inv_freq = exp2f(-(float)(2 * i) / (float)D * log2_theta);
+  // the caller's table (the values its other code paths use, so that both write identical rows), else theta^(-2i/D)
+  const float inv_freq = inv_freq_table ? inv_freq_table[i] : exp2f(-(float)(2 * i) / (float)D * log2_theta);
   float s, c;
   sincosf((float)positions[m] * inv_freq, &s, &c);
   c = Elem<DT>::round(c);
@@ -236,7 +243,7 @@ static int run_layer(const subspec_decoder_layer_dims& s, const LayerWeights& w,
                      (const uint16_t*)w.input_norm, h, H, s.rms_eps);
   if ((rc = project(w, w.qkv, h, w.qkv_bias, nullptr, qkv, DT, M, Q + 2 * KV, H, sub, p.sub_bytes, st))) return rc;
   hipLaunchKernelGGL((rope_write_kernel<DT>), dim3(M, Hq + 2 * Hkv), dim3(64), 0, st, qkv, positions, cache_rows, q, k_cache,
-                     v_cache, M, Hq, Hkv, D, s.kv_seq_stride, log2f(s.rope_theta));
+                     v_cache, M, Hq, Hkv, D, s.kv_seq_stride, log2f(s.rope_theta), s.rope_inv_freq);
   if ((rc = subspec_tree_attention(q, k_cache, v_cache, a, DT, 1, Hq, Hkv, M, s.n_tree_slots, D, s.kv_seq_stride, s.prefix_len,
                                    anc_bits, 0, 1.f / sqrtf((float)D), sub, p.sub_bytes, st)))
     return rc;

@@ -57,8 +57,10 @@ class SubSpecSDDraftModel:
 
     # ------------------------------------------------------------------ tree growth
     @torch.no_grad()
-    def speculate(self, input_ids: torch.Tensor, **kwargs) -> Tree:
-        """``input_ids`` [1, 1]: the root token; the cache already holds everything before it."""
+    def speculate(self, input_ids: torch.Tensor, cap: bool = True, **kwargs) -> Tree:
+        """``input_ids`` [1, 1]: the root token; the cache already holds everything before it.  ``cap``: cut the
+        tree to ``draft_params.max_verify_tokens`` nodes (the reference never cuts; a driver that goes on extending
+        the tree must not, because the draft's level state describes the uncut level)."""
         assert input_ids.shape == (1, 1), "the root of the tree is a single token"
         self.had_first_speculate = True
         p = self.draft_params
@@ -76,7 +78,7 @@ class SubSpecSDDraftModel:
         self._expand(self._probs(logits).unsqueeze(0), torch.ones((1, 1), device=dev, dtype=logits.dtype))
         for _ in range(p.max_depth - 1):
             self.speculate_once()
-        return self.update_tree(cap=True)
+        return self.update_tree(cap=cap)
 
     def _own_bits(self, device) -> torch.Tensor:
         """Row s: the mask words with only the bit of slot s set (word s // 64, bit s % 64; bit 63 is the sign bit of

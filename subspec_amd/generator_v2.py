@@ -54,6 +54,12 @@ class SubSpecSDGeneratorV2(SubSpecSDGenerator):
         self.speculate_count = 0
 
     # ------------------------------------------------------------------ pieces
+    def _speculate(self, input_ids):
+        # No cut to max_verify_tokens here (subspec_sd_v2.py never prunes the fresh tree): the draft keeps extending
+        # this tree from its deepest level, whose tokens, slots and masks describe the whole level.  A tree of more
+        # than 64 nodes is decoded by the target module by module instead of through the one-call layers.
+        return self.draft_model.speculate(input_ids, cap=False)
+
     def _window_forward(self, model, tree, position_offset: int, skip_nodes: int) -> torch.Tensor:
         """Forward of tree nodes ``skip_nodes ..`` (their cache rows are position_offset + node index)."""
         packed = tree.packed()

@@ -128,6 +128,13 @@ class Decoder:
         self._rope_len = 0
         self._rope_tables(kv.cache.max_cache_len + 8)
 
+    def bind_cache(self, kv: KVManager) -> None:
+        """Run over another cache from now on (the builder creates the cache after the models)."""
+        if kv is not self.kv:
+            self.kv = kv
+            self._native = None                      # whether the one-call layers apply depends on the cache layout
+        self._rope_tables(kv.cache.max_cache_len + 8)
+
     def _rope_tables(self, n: int) -> None:
         """cos / sin of positions 0 .. n - 1 (rebuilt when a growing cache passes their length)."""
         if n <= self._rope_len:
@@ -159,7 +166,7 @@ class Decoder:
         n = x.shape[0]
         dims = ops.decoder_layer_dims(self.dtype, n, cfg.hidden_size, cfg.intermediate_size, cfg.num_attention_heads,
                                       cfg.num_key_value_heads, cfg.head_dim, cache.max_cache_len, int(prefix_len),
-                                      int(slots), cfg.rms_norm_eps, cfg.rope_theta)
+                                      int(slots), cfg.rms_norm_eps, cfg.rope_theta, self._inv_freq)
         need = ops.decoder_layer_workspace(dims)
         ws = self._native_ws.get("ws")
         if ws is None or ws.numel() < need:

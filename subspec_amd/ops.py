@@ -100,9 +100,9 @@ def tree_verify(
             int(root), int(skip_nodes), -1 if eos_token_id is None else int(eos_token_id),
             method, gate, float(threshold), int(window_size),
             L.ENTROPY_ALWAYS if exact_entropy else L.ENTROPY_GUARD)
-    tail = (workspace.data_ptr(), workspace.numel() * workspace.element_size(),
-            out["tokens"].data_ptr(), out["contexts"].data_ptr(), out["counts"].data_ptr(),
+    outs = (out["tokens"].data_ptr(), out["contexts"].data_ptr(), out["counts"].data_ptr(),
             out["target"].data_ptr(), out["entropy"].data_ptr(), out["child_prob"].data_ptr(), _stream(dev))
+    tail = (workspace.data_ptr(), workspace.numel() * workspace.element_size(), *outs)
     if do_sample:
         mask = (1 << 64) - 1
         code = lib.subspec_tree_verify_sample(*head, float(temperature), int(seed) & mask, int(offset) & mask, *tail)
@@ -394,12 +394,20 @@ def temperature_warp(logits: torch.Tensor, temperature: float) -> torch.Tensor:
 
 def decoder_layer_dims(dtype: torch.dtype, n_rows: int, hidden: int, intermediate: int, n_q_heads: int, n_kv_heads: int,
                        head_dim: int, kv_seq_stride: int, prefix_len: int, n_tree_slots: int, rms_eps: float,
-                       rope_theta: float) -> "L.DecoderLayerDims":
+                       rope_theta: float, rope_inv_freq: Optional[torch.Tensor] = None) -> "L.DecoderLayerDims":
+    """``rope_inv_freq``: float32 device tensor [head_dim / 2] (kept alive by the caller) with the inverse frequencies
+    the caller's eager rotary uses; without it the kernel evaluates ``rope_theta ** (-2i / head_dim)`` itself."""
     code = {torch.bfloat16: L.BF16, torch.float16: L.F16}.get(dtype)
     if code is None:
         raise ValueError(f"decoder layer: dtype {dtype} not supported (bf16 / fp16 only)")
+    table = None
+    if rope_inv_freq is not None:
+        if rope_inv_freq.dtype != torch.float32 or rope_inv_freq.numel() != head_dim // 2 or not rope_inv_freq.is_cuda \
+                or not rope_inv_freq.is_contiguous():
+            raise ValueError("decoder layer: rope_inv_freq must be a contiguous float32 device tensor of head_dim / 2 elements")
+        table = rope_inv_freq.data_ptr()
     return L.DecoderLayerDims(code, 0, n_rows, hidden, intermediate, n_q_heads, n_kv_heads, head_dim, kv_seq_stride,
-                              prefix_len, n_tree_slots, rms_eps, rope_theta)
+                              prefix_len, n_tree_slots, rms_eps, rope_theta, table)
 
 
 def decoder_layer_weights(w: dict) -> "L.DecoderLayerWeights":

@@ -17,7 +17,7 @@ def test_library_exports_every_declared_symbol():
     for name in names:
         assert hasattr(lib, name), f"{name} declared in the header but not exported"
         assert name in L._SIGNATURES, f"{name} has no ctypes signature"
-    assert lib.subspec_abi_version() == 1
+    assert lib.subspec_abi_version() == 2
 
 
 def test_argument_errors_are_reported_without_a_gpu():

@@ -147,3 +147,31 @@ def test_v2_rejects_trees_beyond_the_slot_limit():
     gen = SubSpecSDGeneratorV2(target, None, SubSpecSDDraftModel(draft), DraftParams(max_depth=64, topk_len=8))
     with pytest.raises(ValueError):
         gen.generate(torch.zeros(1, 4, dtype=torch.long, device=DEV), max_new_tokens=4, do_sample=False, past_key_values=kv)
+
+
+@pytest.mark.parametrize("verify", ["exact", "lossy"])
+def test_v2_with_a_verify_cap_below_the_tree_size(verify):
+    """``max_verify_tokens`` smaller than ``1 + max_depth * topk_len`` (17 nodes, cap 12): the v1 driver cuts the
+    tree, the v2 driver must not (its draft keeps extending the uncut deepest level) -- the emitted tokens stay the
+    target's greedy continuation, the extension is still taken, and the cache holds the emitted sequence's rows."""
+    w = _weights(True)
+    kv = create_kv_cache("static", max_cache_len=512, config=CFG, device=DEV, dtype=torch.bfloat16)
+    target, draft, _ = build_models(CFG, kv, device=DEV, weights=w, first_streamed=2)
+    vk = dict(threshold=0.9, window_size=1, threshold_method="entropy") if verify == "lossy" else None
+    gen = SubSpecSDGeneratorV2(target, None, SubSpecSDDraftModel(draft),
+                               DraftParams(temperature=0.2, max_depth=4, topk_len=4, max_verify_tokens=12),
+                               generator_kwargs=dict(verify_method=verify, verify_kwargs=vk, postspec_steps=3))
+    prompt = torch.randint(0, CFG.vocab_size, (1, 32), generator=torch.Generator().manual_seed(4)).to(DEV)
+    wandb_logger.clear_log_data()
+    out = gen.generate(prompt, max_new_tokens=60, do_sample=False, past_key_values=kv)[0].cpu()
+    log = dict(wandb_logger.log_data)
+    print("v2 with cap", verify, log["n_iter"], log["avg_sampled"], log["post_verify_count"], flush=True)
+    assert out.numel() == 92 and kv.get_seq_length() == 91
+    if verify == "exact":
+        _assert_greedy_continuation(w, out, 32, "v2 cap")
+    assert log["post_verify_count"] >= 2 and log["avg_sampled"] > 2.5, log
+    kv2 = create_kv_cache("static", max_cache_len=512, config=CFG, device=DEV, dtype=torch.bfloat16)
+    t2, _, _ = build_models(CFG, kv2, device=DEV, weights=w)
+    t2.prefill(out[:-1].to(DEV), 0)
+    a, b = kv.cache.data[..., :91, :].float(), kv2.cache.data[..., :91, :].float()
+    assert (a - b).abs().amax().item() <= 5e-2 * b.abs().amax().item()

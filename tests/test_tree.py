@@ -114,3 +114,32 @@ def test_dynamic_cache_bookkeeping_on_the_host():
     static.cache.ensure(32)
     with pytest.raises(ValueError):
         static.cache.ensure(33)
+
+
+def _two_level_tree():
+    t = Tree(torch.tensor(7))
+    t.add_nodes(torch.tensor([[[10, 11, 12, 13], [20, 21, 22, 23]]]),
+                torch.tensor([[[.4, .3, .2, .1], [.2, .15, .1, .05]]]),
+                torch.tensor([[[0, 0, 0, 0], [0, 0, 1, 2]]]))
+    return t
+
+
+def test_truncate_keeps_the_frontier_positions_for_later_levels():
+    """A tree cut to its first n nodes and extended afterwards: the new level names its parents by position in the
+    level that was cut, so surviving positions must keep their nodes and cut positions must be refused -- not
+    re-mapped onto whatever childless nodes remain."""
+    t = _two_level_tree()                       # 9 nodes: root, level 1 = 1..4, level 2 = 5..8 (parents 1, 1, 2, 3)
+    t.truncate(7)                               # drops nodes 7 and 8 (positions 2 and 3 of the frontier)
+    assert t.size() == 7 and t.available_leaves == [5, 6]
+    t.add_nodes(torch.tensor([[[30, 31]]]), torch.tensor([[[.1, .05]]]), torch.tensor([[[1, 0]]]))
+    d = _data(t)
+    assert d["parent_indices"][7:] == [6, 5] and d["depths"][7:] == [3, 3]
+    # a parent position that was cut off is an error, not a silent re-parenting to a shallower node
+    t2 = _two_level_tree()
+    t2.truncate(7)
+    with pytest.raises(ValueError, match="truncate"):
+        t2.add_nodes(torch.tensor([[[30]]]), torch.tensor([[[.1]]]), torch.tensor([[[3]]]))
+    # cutting nothing changes nothing
+    t3 = _two_level_tree()
+    t3.truncate(9)
+    assert t3.available_leaves == [5, 6, 7, 8]
