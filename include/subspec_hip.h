@@ -106,6 +106,25 @@ int subspec_tree_verify(const void* logits, int dtype, int64_t batch, int64_t ro
                         int64_t* node_target, float* node_entropy, float* node_child_prob,
                         void* stream);
 
+/* subspec_tree_verify for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments,
+ * kernels and results as subspec_tree_verify (greedy target), minus the workspace: the per-slice partial
+ * records live in an array built into the library (SUBSPEC_TREE_VERIFY_STATIC_MAX_ROWS * 64 slices * 48
+ * bytes = 6 MiB of device memory per GPU, held until the process ends).  The call allocates nothing.
+ * batch * rows beyond SUBSPEC_TREE_VERIFY_STATIC_MAX_ROWS is rejected with SUBSPEC_ERR_LIMIT.  All calls
+ * on one GPU share that GPU's array: calls that overlap on one GPU (different streams or threads) race;
+ * calls in stream order do not.  Nothing in the array needs to start at zero. */
+#define SUBSPEC_TREE_VERIFY_STATIC_MAX_ROWS 2048
+
+int subspec_tree_verify_static(const void* logits, int dtype, int64_t batch, int64_t rows, int64_t vocab,
+                               const int32_t* token_ids, const int32_t* parents, int64_t n_nodes,
+                               int32_t root, int32_t skip_nodes, int64_t eos_token_id,
+                               int verify_method, int threshold_method, double threshold, int32_t window_size,
+                               int entropy_policy,
+                               int64_t* out_tokens, int64_t* out_ctx, int32_t* out_counts,
+                               int64_t* node_target, float* node_entropy, float* node_child_prob,
+                               void* stream);
+
 /* Tree verification with a SAMPLED target token (do_sample=True).
  *
  * Replaces the same call sites as subspec_tree_verify when the generator samples:

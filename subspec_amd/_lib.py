@@ -18,6 +18,7 @@ VERIFY_EXACT, VERIFY_LOSSY = 0, 1
 GATE_ENTROPY, GATE_PROB = 0, 1
 ENTROPY_GUARD, ENTROPY_ALWAYS = 0, 1
 MAX_TREE_NODES = 512
+TREE_VERIFY_STATIC_MAX_ROWS = 2048
 
 _lib = None
 
@@ -53,6 +54,9 @@ _SIGNATURES = {
     "subspec_tree_verify": (C.c_int, [_p, C.c_int, _i64, _i64, _i64, _p, _p, _i64, _i32, _i32, _i64,
                                       C.c_int, C.c_int, _f64, _i32, C.c_int, _p, _sz,
                                       _p, _p, _p, _p, _p, _p, _p]),
+    "subspec_tree_verify_static": (C.c_int, [_p, C.c_int, _i64, _i64, _i64, _p, _p, _i64, _i32, _i32, _i64,
+                                             C.c_int, C.c_int, _f64, _i32, C.c_int,
+                                             _p, _p, _p, _p, _p, _p, _p]),
     "subspec_tree_verify_sample": (C.c_int, [_p, C.c_int, _i64, _i64, _i64, _p, _p, _i64, _i32, _i32, _i64,
                                              C.c_int, C.c_int, _f64, _i32, C.c_int, C.c_float, C.c_uint64, C.c_uint64,
                                              _p, _sz, _p, _p, _p, _p, _p, _p, _p]),

@@ -28,6 +28,7 @@
 // row maximum; the normalized entropy of a 16-bit row is sum(entr(p)) with p, log p and p*log p
 // each rounded to that dtype, the sum rounded once, divided by float(ln V) and rounded again.
 #include "common.h"
+#include <mutex>
 #include <algorithm>
 
 namespace subspec {
@@ -916,4 +917,59 @@ extern "C" int subspec_tree_verify_sample(const void* logits, int dtype, int64_t
                           eos_token_id, verify_method, threshold_method, threshold, window_size, entropy_policy,
                           workspace, workspace_bytes, out_tokens, out_ctx, out_counts, node_target, node_entropy,
                           node_child_prob, drawn, stream);
+}
+
+// ------------------------------------------------------------------ allocation-free variant
+// The per-slice partial records (Part1 / Part2 / Part3) of the verifier in a file-scope device array instead of a
+// caller-supplied workspace, for callers that cannot allocate.  kStaticVerifyRows logits rows (batch * rows) is the
+// limit: 2048 rows x 64 slices x 48 bytes.  Every GPU holds its own copy of the array at its own address, looked up
+// once per device; all calls on a GPU share it and calls that overlap there race.  The kernels write every record
+// they later read, so the array needs no clearing between calls.
+namespace subspec {
+constexpr int64_t kStaticVerifyRows = SUBSPEC_TREE_VERIFY_STATIC_MAX_ROWS;
+constexpr size_t kStaticVerifyBytes =
+    (size_t)kStaticVerifyRows * kMaxSplits * (sizeof(Part1) + sizeof(Part2) + sizeof(Part3)) + 3 * 256;
+static __device__ __align__(256) unsigned char scratch[kStaticVerifyBytes];
+constexpr int kMaxDevices = 64;
+static void* g_scratch_ptr[kMaxDevices];            // device address of `scratch` on each GPU, 0 until looked up
+static std::mutex g_scratch_mutex;
+
+static int static_scratch(void** out) {
+  int dev = -1;
+  SUBSPEC_CHECK_HIP(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxDevices) SUBSPEC_FAIL(SUBSPEC_ERR_LIMIT, "tree_verify_static: device %d outside 0..%d", dev, kMaxDevices - 1);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* p = nullptr;
+    SUBSPEC_CHECK_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    if (!p) SUBSPEC_FAIL(SUBSPEC_ERR_HIP, "tree_verify_static: hipGetSymbolAddress returned a null address");
+    g_scratch_ptr[dev] = p;
+  }
+  *out = g_scratch_ptr[dev];
+  return SUBSPEC_OK;
+}
+}  // namespace subspec
+
+extern "C" int subspec_tree_verify_static(const void* logits, int dtype, int64_t batch, int64_t rows, int64_t vocab,
+                                          const int32_t* token_ids, const int32_t* parents, int64_t n_nodes,
+                                          int32_t root, int32_t skip_nodes, int64_t eos_token_id,
+                                          int verify_method, int threshold_method, double threshold, int32_t window_size,
+                                          int entropy_policy, int64_t* out_tokens, int64_t* out_ctx, int32_t* out_counts,
+                                          int64_t* node_target, float* node_entropy, float* node_child_prob,
+                                          void* stream) {
+  if (batch > 0 && rows > 0 && batch * rows > kStaticVerifyRows)
+    SUBSPEC_FAIL(SUBSPEC_ERR_LIMIT, "tree_verify_static: batch * rows = %lld exceeds the %lld rows the built-in scratch array holds "
+                 "(use subspec_tree_verify with a workspace)", (long long)(batch * rows), (long long)kStaticVerifyRows);
+  if (!dtype_ok(dtype)) SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "tree_verify_static: unknown dtype %d", dtype);
+  if (!logits || !token_ids || !parents || !out_tokens || !out_ctx || !out_counts || !node_target || !node_entropy ||
+      !node_child_prob)
+    SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "tree_verify_static: null pointer argument");
+  void* ws = nullptr;
+  const int rc = static_scratch(&ws);
+  if (rc != SUBSPEC_OK) return rc;
+  const SampleArgs greedy{0, 1.0f, 0, 0};
+  return tree_verify_impl(logits, dtype, batch, rows, vocab, token_ids, parents, n_nodes, root, skip_nodes,
+                          eos_token_id, verify_method, threshold_method, threshold, window_size, entropy_policy,
+                          ws, kStaticVerifyBytes, out_tokens, out_ctx, out_counts, node_target, node_entropy,
+                          node_child_prob, greedy, stream);
 }

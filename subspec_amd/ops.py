@@ -54,8 +54,14 @@ def tree_verify(
     temperature: float = 1.0,
     seed: int = 0,
     offset: int = 0,
+    out: Optional[Dict[str, torch.Tensor]] = None,
+    static_scratch: bool = False,
 ) -> Dict[str, torch.Tensor]:
     """Runs the fused verifier; everything stays on the device (no synchronisation here).
+
+    ``static_scratch=True`` calls ``subspec_tree_verify_static`` (greedy target only): the library's built-in scratch
+    array takes the place of the workspace; with ``out`` (the dictionary an earlier call returned, same shapes)
+    nothing at all is allocated.
 
     ``do_sample=True`` draws the target token of every row from ``softmax(logits / temperature)``
     (Philox stream ``seed`` / ``offset``) instead of taking the argmax.
@@ -85,10 +91,18 @@ def tree_verify(
     token_ids = token_ids.to(torch.int32).contiguous()
     parents = parents.to(torch.int32).contiguous()
     lib = L.lib()
-    need = lib.subspec_tree_verify_workspace(B, rows, V, _dtype_code(logits))
-    if workspace is None:
+    if static_scratch and do_sample:
+        raise ValueError("static_scratch serves the greedy verifier only")
+    if workspace is None and not static_scratch:
+        need = lib.subspec_tree_verify_workspace(B, rows, V, _dtype_code(logits))
         workspace = torch.empty(need, dtype=torch.uint8, device=dev)
-    out = {
+    if out is not None:
+        want = {"tokens": (B, n + 1), "contexts": (B, n + 1), "counts": (B, 4), "target": (B, rows),
+                "entropy": (B, rows), "child_prob": (B, rows)}
+        for key, shape in want.items():
+            if tuple(out[key].shape) != shape or out[key].device != dev or not out[key].is_contiguous():
+                raise ValueError(f"out[{key!r}] must be a contiguous {shape} tensor on {dev}")
+    out = out if out is not None else {
         "tokens": torch.empty((B, n + 1), dtype=torch.int64, device=dev),
         "contexts": torch.empty((B, n + 1), dtype=torch.int64, device=dev),
         "counts": torch.empty((B, 4), dtype=torch.int32, device=dev),
@@ -102,6 +116,9 @@ def tree_verify(
             L.ENTROPY_ALWAYS if exact_entropy else L.ENTROPY_GUARD)
     outs = (out["tokens"].data_ptr(), out["contexts"].data_ptr(), out["counts"].data_ptr(),
             out["target"].data_ptr(), out["entropy"].data_ptr(), out["child_prob"].data_ptr(), _stream(dev))
+    if static_scratch:
+        L.check(lib.subspec_tree_verify_static(*head, *outs), "subspec_tree_verify_static")
+        return out
     tail = (workspace.data_ptr(), workspace.numel() * workspace.element_size(), *outs)
     if do_sample:
         mask = (1 << 64) - 1
