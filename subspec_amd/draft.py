@@ -31,16 +31,48 @@ MASK_WORDS = MAX_SLOTS // 64
 
 
 class SubSpecSDDraftModel:
-    def __init__(self, decoder: Decoder, eos_token_id: Optional[int] = None):
+    def __init__(self, decoder, eos_token_id: Optional[int] = None):
+        # ``model``: a ``Decoder``, or the HuggingFace-shaped module the reference's builder quantizes in place through
+        # ``draft_model.model`` (run/core/builder.py:340-341); the latter becomes a ``Decoder`` once the cache is known
         self.model = decoder
+        self._decoder: Optional[Decoder] = decoder if isinstance(decoder, Decoder) else None
         self.eos_token_id = eos_token_id
         self.draft_params: Optional[DraftParams] = None
         self.past_key_values = None
         self.had_first_speculate = False
         self.postspec_count = 0
 
+    @classmethod
+    def from_pretrained(cls, pretrained_model_name_or_path=None, *model_args, target_model=None,
+                        torch_dtype=torch.float32, **model_kwargs) -> "SubSpecSDDraftModel":
+        """The reference's constructor for the substitute draft (draft_models/subspec_sd.py:29-45): no checkpoint of
+        its own, a second module tree over ``target_model``'s parameters (``hf_model.share_parameters``) that a
+        recipe's quantizer then converts; ``eos_token_id`` and ``device_map`` are taken from the keyword arguments
+        the builder passes (run/core/builder.py:119-131).  The target's dtype is kept: the shared parameters are the
+        target's own tensors, so there is nothing to convert."""
+        if target_model is None:
+            raise ValueError("SubSpecSDDraftModel.from_pretrained needs target_model (the draft shares its weights)")
+        if isinstance(target_model, Decoder):
+            raise TypeError("a Decoder target has its draft built by subspec_amd.model.build_models; from_pretrained "
+                            "takes the HuggingFace-shaped module the builder loads")
+        from .hf_model import share_parameters
+        return cls(share_parameters(target_model), eos_token_id=model_kwargs.pop("eos_token_id", None))
+
+    @property
+    def decoder(self) -> Decoder:
+        if self._decoder is None:
+            raise RuntimeError("the draft has no KV cache yet: call set_past_key_values(past_key_values) first "
+                               "(generate() does)")
+        return self._decoder
+
+    def eval(self) -> "SubSpecSDDraftModel":
+        return self
+
     def set_past_key_values(self, past_key_values) -> None:
         self.past_key_values = past_key_values
+        if past_key_values is not None:
+            from .hf_model import as_decoder
+            self._decoder = as_decoder(self.model, past_key_values)
 
     def get_tree(self) -> Tree:
         return self.tree
@@ -64,11 +96,11 @@ class SubSpecSDDraftModel:
         assert input_ids.shape == (1, 1), "the root of the tree is a single token"
         self.had_first_speculate = True
         p = self.draft_params
-        dev = self.model.device
+        dev = self.decoder.device
         self.prefix_len = int(self.past_key_values.get_seq_length())
-        logits = self.model.tree_forward(input_ids[0].to(dev), torch.zeros(1, dtype=torch.long, device=dev),
+        logits = self.decoder.tree_forward(input_ids[0].to(dev), torch.zeros(1, dtype=torch.long, device=dev),
                                          torch.ones(1, dtype=torch.int64, device=dev), self.prefix_len)
-        self.tree = Tree(input_ids[0, -1], self.model.dtype)
+        self.tree = Tree(input_ids[0, -1], self.decoder.dtype)
         self.levels = []
         self.level_state = {}                                                      # depth -> what speculate_once needs
         self.level_bits = torch.zeros((1, MASK_WORDS), dtype=torch.int64, device=dev)
@@ -108,14 +140,14 @@ class SubSpecSDDraftModel:
     @torch.no_grad()
     def speculate_once(self, **kwargs) -> None:
         """One more level: draft forward on the newest k nodes, then top-k over (k x vocab)."""
-        dev = self.model.device
+        dev = self.decoder.device
         n = self.token_ids.shape[1]
         total = self.first_slot + n
         if total > MAX_SLOTS:
             raise ValueError(f"draft tree exceeds the {MAX_SLOTS} tree slots of the attention mask")
         depths = torch.full((n,), self.depth, dtype=torch.long, device=dev)
         bits = self.level_bits[:, 0].contiguous() if total <= 64 else self.level_bits[:, :(total + 63) // 64].contiguous()
-        logits = self.model.tree_forward(self.token_ids[0], depths, bits, self.prefix_len,
+        logits = self.decoder.tree_forward(self.token_ids[0], depths, bits, self.prefix_len,
                                          first_slot=self.first_slot)
         self._expand(self._probs(logits).unsqueeze(0), self.parent_probs)
 
@@ -124,7 +156,7 @@ class SubSpecSDDraftModel:
         prob = torch.stack([lv[1][0] for lv in self.levels]).unsqueeze(0)
         par = torch.stack([lv[2][0] for lv in self.levels]).unsqueeze(0)
         packed = torch.stack([tok.double(), prob.double(), par.double()]).cpu()     # one device-to-host copy
-        self.tree.add_nodes(packed[0].long(), packed[1].to(self.model.dtype), packed[2].long())
+        self.tree.add_nodes(packed[0].long(), packed[1].to(self.decoder.dtype), packed[2].long())
         self.levels = []
         limit = self.draft_params.max_verify_tokens if cap else None
         if limit is not None and self.tree.size() > limit:
@@ -153,7 +185,7 @@ class SubSpecSDDraftModel:
         n = self.token_ids.shape[1]
         if self.first_slot + n > MAX_SLOTS or self.next_slot + n > MAX_SLOTS:
             return False
-        cache = self.model.kv.cache
+        cache = self.decoder.kv.cache
         return cache.growable or self.prefix_len + self.next_slot + n <= cache.max_cache_len
 
     @torch.no_grad()

@@ -46,6 +46,18 @@ class SubSpecSDGenerator:
         self.sample_stream = SampleStream(self.generator_kwargs.get("seed"))
         self._stop_strings = None                # HuggingFace StopStringCriteria of the current generate() call
 
+    def eval(self) -> "SubSpecSDGenerator":
+        """The reference's generators are ``nn.Module``s and the builder calls ``generator.eval()``
+        (run/core/builder.py:359); nothing here has a training mode."""
+        return self
+
+    def _bind(self, past_key_values: KVManager) -> None:
+        """Models handed over by the reference's builder are HuggingFace-shaped modules (quantized / offloaded by the
+        recipe); they become ``Decoder``s over the cache of this call.  ``Decoder``s are re-bound to it."""
+        from .hf_model import as_decoder
+        self.target_model = as_decoder(self.target_model, past_key_values)
+        self.draft_model.set_past_key_values(past_key_values)
+
     # ------------------------------------------------------------------ pieces of one cycle
     def _speculate(self, input_ids):
         return self.draft_model.speculate(input_ids)
@@ -128,9 +140,9 @@ class SubSpecSDGenerator:
 
     def _generate(self, input_ids, max_length: Optional[int], past_key_values: KVManager, stream_callback=None,
                   logits_processor=None, do_sample: bool = False):
+        self._bind(past_key_values)
         dev = self.target_model.device
         input_ids = input_ids.to(dev)
-        self.draft_model.set_past_key_values(past_key_values)
         p = self.draft_params
         ev = lambda: torch.cuda.Event(enable_timing=True)
         phases = {"draft": [], "target": [], "verify": []}

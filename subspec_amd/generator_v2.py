@@ -118,7 +118,7 @@ class SubSpecSDGeneratorV2(SubSpecSDGenerator):
         """subspec_sd_v2.py:32-55: the draft verifies the extension itself, the tree keeps the depth that walk reaches
         and is refilled."""
         draft = self.draft_model
-        logits = self._window_forward(draft.model, tree, position_offset, skip_nodes)
+        logits = self._window_forward(draft.decoder, tree, position_offset, skip_nodes)
         tokens, _, _ = self._verified(tree, root_ind, logits, None, False, skip_nodes)
         accepted_len = int(tokens.numel())
         tree.prune_to_depth(last_tree_depth + accepted_len)
@@ -141,9 +141,9 @@ class SubSpecSDGeneratorV2(SubSpecSDGenerator):
         p = self.draft_params
         if 1 + p.max_depth * p.topk_len > ops.L.MAX_TREE_NODES:
             raise ValueError(f"1 + max_depth * topk_len must not exceed the {ops.L.MAX_TREE_NODES} tree slots of the masks")
+        self._bind(past_key_values)
         dev = self.target_model.device
         input_ids = input_ids.to(dev)
-        self.draft_model.set_past_key_values(past_key_values)
         ev = lambda: torch.cuda.Event(enable_timing=True)
         phases = {"draft": [], "target": [], "verify": []}
         t_start = time.perf_counter()

@@ -182,18 +182,28 @@ class HqqQuantizer:
     per-layer config; every named ``nn.Linear`` is replaced in place.  A config may carry ``"optimize"``
     (default True, as hqq's ``Quantizer.quantize``): refine the zero points with hqq's proximal solver."""
 
+    @staticmethod
+    def _params(name: str, cfg) -> dict:
+        """nbits / group_size / axis / optimize of one entry: a plain dict, the nested dict hqq's ``BaseQuantizeConfig``
+        returns (``{"weight_quant_params": {...}}``), or an object with those attributes."""
+        if isinstance(cfg, dict) and isinstance(cfg.get("weight_quant_params"), dict):
+            cfg = dict(cfg["weight_quant_params"], **{k: v for k, v in cfg.items() if k == "optimize"})
+        get = cfg.get if isinstance(cfg, dict) else (lambda k, d=None: getattr(cfg, k, d))
+        p = {"nbits": int(get("nbits", 4)), "group_size": int(get("group_size", GROUP) or GROUP), "axis": int(get("axis", 1)),
+             "optimize": bool(get("optimize", True))}
+        if p["nbits"] != 4 or p["group_size"] != GROUP or p["axis"] != 1:
+            raise ValueError(f"{name}: only nbits=4, group_size={GROUP}, axis=1 is supported "
+                             f"(got {p['nbits']}, {p['group_size']}, {p['axis']})")
+        return p
+
     @classmethod
     def quantize_model(cls, model: nn.Module, quant_config: Dict[str, dict], compute_dtype: torch.dtype, device):
         for name, cfg in quant_config.items():
-            nbits = int(cfg.get("nbits", 4)) if isinstance(cfg, dict) else int(getattr(cfg, "nbits", 4))
-            gsize = int(cfg.get("group_size", GROUP)) if isinstance(cfg, dict) else int(getattr(cfg, "group_size", GROUP))
-            if nbits != 4 or gsize != GROUP:
-                raise ValueError(f"{name}: only nbits=4, group_size={GROUP} is supported (got {nbits}, {gsize})")
+            p = cls._params(name, cfg)
             parent_name, _, child = name.rpartition(".")
             parent = model.get_submodule(parent_name) if parent_name else model
             linear = getattr(parent, child)
             if not isinstance(linear, nn.Linear):
                 raise TypeError(f"{name} is {type(linear).__name__}, expected nn.Linear")
-            optimize = bool(cfg.get("optimize", True)) if isinstance(cfg, dict) else bool(getattr(cfg, "optimize", True))
-            setattr(parent, child, HqqInt4Linear.from_linear(linear, compute_dtype, device, optimize=optimize))
+            setattr(parent, child, HqqInt4Linear.from_linear(linear, compute_dtype, device, optimize=p["optimize"]))
         return model
