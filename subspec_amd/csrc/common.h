@@ -112,6 +112,40 @@ __device__ __forceinline__ void store_linear_out(void* y, int64_t i, float v, co
   Elem<DT>::store(y, i, v);
 }
 
+// ---------------------------------------------------------------- eight 16-bit elements in one 16-byte piece
+typedef uint32_t dec_u4 __attribute__((ext_vector_type(4)));
+
+template <int DT>
+__device__ __forceinline__ void unpack8(dec_u4 v, float* f) {
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    if constexpr (DT == SUBSPEC_BF16) {
+      f[2 * j] = bf16_bits_to_float(v[j] & 0xffffu);
+      f[2 * j + 1] = bf16_bits_to_float(v[j] >> 16);
+    } else {
+      f[2 * j] = f16_bits_to_float(v[j] & 0xffffu);
+      f[2 * j + 1] = f16_bits_to_float(v[j] >> 16);
+    }
+  }
+}
+template <int DT>
+__device__ __forceinline__ uint32_t to_bits(float v) {
+  if constexpr (DT == SUBSPEC_BF16) {
+    return __float_as_uint(round_bf16(v)) >> 16;
+  } else {
+    union { uint16_t u; _Float16 h; } c;
+    c.h = (_Float16)v;
+    return c.u;
+  }
+}
+template <int DT>
+__device__ __forceinline__ dec_u4 pack8(const float* f) {
+  dec_u4 v;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) v[j] = to_bits<DT>(f[2 * j]) | (to_bits<DT>(f[2 * j + 1]) << 16);
+  return v;
+}
+
 // ---------------------------------------------------------------- wave / block reductions
 __device__ __forceinline__ float wave_max(float v) {
 #pragma unroll
@@ -179,8 +213,15 @@ int int4_linear_ex(const void* x, const uint32_t* wq, const uint32_t* sz, const 
                    void* stream);
 // act[M, F] = round(silu(round(gate))) * round(up) with gate | up = x * W^T (+ bias), W of N = 2F rows (gate rows first):
 // the SwiGLU MLP's first projection and its activation in one launch
+// norm_gain != NULL: x is the un-normalized residual stream and RMSNorm (gain [K], eps) is the projection's prologue (M <= 32)
 int int4_gate_up_silu_ex(const void* x, const uint32_t* wq, const uint32_t* sz, const void* bias, void* act, int dtype,
-                         int64_t M, int64_t N, int64_t K, void* stream);
+                         int64_t M, int64_t N, int64_t K, const void* norm_gain, float norm_eps, void* stream);
+// q|k|v projection (N = (Hq + 2 Hkv) * 128 rows) with the rotary embedding and the cache write in its output stage:
+// q to q_out [Hq, M, 128], K / V rows to cache_rows[m] of the layer's [Hkv, seq_stride, 128] caches; optional RMSNorm prologue
+int int4_qkv_rope_ex(const void* x, const uint32_t* wq, const uint32_t* sz, const void* bias, int dtype, int64_t M, int64_t K,
+                     const void* norm_gain, float norm_eps, const int32_t* positions, const int32_t* cache_rows, void* q_out,
+                     void* k_cache, void* v_cache, int64_t n_q_heads, int64_t n_kv_heads, int64_t kv_seq_stride,
+                     float rope_theta, const float* inv_freq, void* stream);
 int dense_gate_up_silu_ex(const void* x, const void* w, const void* bias, void* act, int dtype, int64_t M, int64_t N,
                           int64_t K, void* stream);
 int dense_linear_ex(const void* x, const void* w, const void* bias, const void* residual, void* y, int dtype, int64_t M,

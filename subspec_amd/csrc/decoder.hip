@@ -26,39 +26,6 @@
 
 namespace subspec {
 
-typedef uint32_t dec_u4 __attribute__((ext_vector_type(4)));
-
-template <int DT>
-__device__ __forceinline__ void unpack8(dec_u4 v, float* f) {
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    if constexpr (DT == SUBSPEC_BF16) {
-      f[2 * j] = bf16_bits_to_float(v[j] & 0xffffu);
-      f[2 * j + 1] = bf16_bits_to_float(v[j] >> 16);
-    } else {
-      f[2 * j] = f16_bits_to_float(v[j] & 0xffffu);
-      f[2 * j + 1] = f16_bits_to_float(v[j] >> 16);
-    }
-  }
-}
-template <int DT>
-__device__ __forceinline__ uint32_t to_bits(float v) {
-  if constexpr (DT == SUBSPEC_BF16) {
-    return __float_as_uint(round_bf16(v)) >> 16;
-  } else {
-    union { uint16_t u; _Float16 h; } c;
-    c.h = (_Float16)v;
-    return c.u;
-  }
-}
-template <int DT>
-__device__ __forceinline__ dec_u4 pack8(const float* f) {
-  dec_u4 v;
-#pragma unroll
-  for (int j = 0; j < 4; ++j) v[j] = to_bits<DT>(f[2 * j]) | (to_bits<DT>(f[2 * j + 1]) << 16);
-  return v;
-}
-
 // x[m] (+= delta[m], rounded, written back) ; y[m] = w * round(x * rsqrt(mean(x^2) + eps))
 // One workgroup per row; H % 8 == 0.  kMaxPieces 16-byte pieces per thread cover H <= 256 * 8 * kMaxPieces.
 constexpr int kNormThreads = 256;
@@ -239,21 +206,38 @@ static int run_layer(const subspec_decoder_layer_dims& s, const LayerWeights& w,
            *o = (uint16_t*)(ws + p.o), *gu = (uint16_t*)(ws + p.gu), *act = (uint16_t*)(ws + p.act);
   void* sub = ws + p.sub;
   int rc;
-  hipLaunchKernelGGL((add_rmsnorm_kernel<DT, false>), dim3(M), dim3(kNormThreads), 0, st, x, (const uint16_t*)nullptr,
-                     (const uint16_t*)w.input_norm, h, H, s.rms_eps);
-  if ((rc = project(w, w.qkv, h, w.qkv_bias, nullptr, qkv, DT, M, Q + 2 * KV, H, sub, p.sub_bytes, st))) return rc;
-  hipLaunchKernelGGL((rope_write_kernel<DT>), dim3(M, Hq + 2 * Hkv), dim3(64), 0, st, qkv, positions, cache_rows, q, k_cache,
-                     v_cache, M, Hq, Hkv, D, s.kv_seq_stride, log2f(s.rope_theta), s.rope_inv_freq);
+  // int4 stack, a level of at most 32 rows: five launches per layer (six with a split-K down projection, seven when
+  // the keys are split) -- both norms are prologues of the projections that consume them, rotary + cache write is the
+  // output stage of q|k|v, the attention block's residual add the output stage of o_proj
+  const bool fused = !w.dense && M <= 32 && subspec_int4_linear_workspace(M, Q + 2 * KV, H) == 256;
+  if (fused) {
+    if ((rc = int4_qkv_rope_ex(x, (const uint32_t*)w.qkv.w, (const uint32_t*)w.qkv.sz, w.qkv_bias, DT, M, H, w.input_norm, s.rms_eps,
+                               positions, cache_rows, q, k_cache, v_cache, Hq, Hkv, s.kv_seq_stride, s.rope_theta, s.rope_inv_freq, st)))
+      return rc;
+  } else {
+    hipLaunchKernelGGL((add_rmsnorm_kernel<DT, false>), dim3(M), dim3(kNormThreads), 0, st, x, (const uint16_t*)nullptr,
+                       (const uint16_t*)w.input_norm, h, H, s.rms_eps);
+    if ((rc = project(w, w.qkv, h, w.qkv_bias, nullptr, qkv, DT, M, Q + 2 * KV, H, sub, p.sub_bytes, st))) return rc;
+    hipLaunchKernelGGL((rope_write_kernel<DT>), dim3(M, Hq + 2 * Hkv), dim3(64), 0, st, qkv, positions, cache_rows, q, k_cache,
+                       v_cache, M, Hq, Hkv, D, s.kv_seq_stride, log2f(s.rope_theta), s.rope_inv_freq);
+  }
   if ((rc = subspec_tree_attention(q, k_cache, v_cache, a, DT, 1, Hq, Hkv, M, s.n_tree_slots, D, s.kv_seq_stride, s.prefix_len,
                                    anc_bits, 0, 1.f / sqrtf((float)D), sub, p.sub_bytes, st)))
     return rc;
+  if (fused) {
+    // x = round(round(o_proj(a)) + x), then RMSNorm inside the gate|up projection
+    if ((rc = project(w, w.o, a, nullptr, x, x, DT, M, H, Q, sub, p.sub_bytes, st))) return rc;
+    if ((rc = int4_gate_up_silu_ex(x, (const uint32_t*)w.gate_up.w, (const uint32_t*)w.gate_up.sz, nullptr, act, DT, M,
+                                   2 * (int64_t)F, H, w.post_norm, s.rms_eps, st)))
+      return rc;
+  } else {
   if ((rc = project(w, w.o, a, nullptr, nullptr, o, DT, M, H, Q, sub, p.sub_bytes, st))) return rc;
   hipLaunchKernelGGL((add_rmsnorm_kernel<DT, true>), dim3(M), dim3(kNormThreads), 0, st, x, o, (const uint16_t*)w.post_norm, h, H,
                      s.rms_eps);
   if (!w.dense) {
     // the activation sits in the output stage of the gate|up projection
     if ((rc = int4_gate_up_silu_ex(h, (const uint32_t*)w.gate_up.w, (const uint32_t*)w.gate_up.sz, nullptr, act, DT, M,
-                                   2 * (int64_t)F, H, st)))
+                                   2 * (int64_t)F, H, nullptr, 0.f, st)))
       return rc;
   } else if (4 * (int64_t)F * H < ((int64_t)1 << 31)) {
     if ((rc = dense_gate_up_silu_ex(h, w.gate_up.w, nullptr, act, DT, M, 2 * (int64_t)F, H, st))) return rc;
@@ -261,6 +245,7 @@ static int run_layer(const subspec_decoder_layer_dims& s, const LayerWeights& w,
     if ((rc = project(w, w.gate_up, h, nullptr, nullptr, gu, DT, M, 2 * (int64_t)F, H, sub, p.sub_bytes, st))) return rc;
     const int64_t act_pieces = (int64_t)M * F / 8;
     hipLaunchKernelGGL((silu_mul_kernel<DT>), dim3((unsigned)((act_pieces + 255) / 256)), dim3(256), 0, st, gu, act, F, act_pieces);
+  }
   }
   // down projection with the residual add in its output stage: x = round(round(down(act)) + x)
   if ((rc = project(w, w.down, act, nullptr, x, x, DT, M, H, F, sub, p.sub_bytes, st))) return rc;

@@ -154,11 +154,42 @@ __device__ __forceinline__ i4_v4f i4_mfma32(i4_u4 a, i4_u4 b, i4_v4f c) {
 // owns PAIRS of tiles, (gate tile p, up tile p + F/16), and its output stage writes act[m, f] =
 // round(silu(round(gate))) * round(up) to y[M, F] instead of the 2F projections -- the arithmetic of the separate
 // activation kernel on the values the plain projection would have stored, one launch and one round trip less.
-template <int DT, int MT, int RT, bool SILU = false>
+//
+// ROPE (the fused q|k|v projection of an attention block): a workgroup owns the tile pair (j, j + 4) of one head (the
+// columns d and d + 64 that the rotate-half form combines), or two consecutive tiles of a value head, and its output
+// stage applies the rotary embedding and writes q to [Hq, M, 128] and the K / V rows into the layer's cache: the
+// [M, N] projection never travels through memory and the separate rotary launch is gone.
+//
+// NORM (RMSNorm as the prologue of the projection that consumes it): x is the residual stream itself.  The
+// per-element gain is applied where a block is parked in LDS (one rounding of x * gain), the squares are summed on
+// the way (every workgroup reads all of x anyway), and 1 / rms -- a per-row scalar -- multiplies the accumulators in
+// the output stage:  y = rstd[m] * sum_k round(x[m,k] g[k]) W[n,k].  Only without a K split across workgroups.
+constexpr int kEpiPlain = 0, kEpiSilu = 1, kEpiRope = 2;
+struct I4Fused {
+  const uint16_t* norm_gain;   // NORM: [K]
+  float norm_eps;
+  // ROPE
+  const int32_t* positions;    // [M]
+  const int32_t* cache_rows;   // [M]
+  uint16_t* q_out;             // [Hq, M, 128]
+  uint16_t* k_cache;           // [Hkv, seq_stride, 128]
+  uint16_t* v_cache;
+  const float* inv_freq;       // [64] or null
+  int hq, hkv;
+  int64_t seq_stride;
+  float log2_theta;
+};
+
+// XHALF (at most 8 activation rows, MT = 1): only rows 0..7 of a block are fetched, scaled and parked; rows 8..15 of the
+// LDS stages are cleared once.  Half the activation traffic and half the prologue arithmetic of a 16-row block.
+template <int DT, int MT, int RT, int EPI = kEpiPlain, bool NORM = false, bool XHALF = false>
 __global__ __launch_bounds__(kI4Threads) void int4_gemm_kernel(
     const uint16_t* __restrict__ x, const uint2* __restrict__ wq, const uint32_t* __restrict__ sz,
     const uint16_t* __restrict__ bias, const uint16_t* residual, uint16_t* y, float* __restrict__ partial, int M, int64_t N,
-    int K, int splits, int groups_per_split) {
+    int K, int splits, int groups_per_split, I4Fused fz) {
+  constexpr bool SILU = EPI == kEpiSilu, ROPE = EPI == kEpiRope, PAIRED = EPI != kEpiPlain;
+  __shared__ float sq_s[NORM ? 4 * MT * 16 : 1];                 // NORM: per wavefront, per row: sum of squares of its groups
+  __shared__ float rstd_s[NORM ? MT * 16 : 1];
   // 4 wavefronts x 2 stages of a [16*MT][64] activation block; reused for the final reduction
   // (two rounds of one accumulator tile set per wavefront)
   constexpr int kStageBytes = 4 * 2 * MT * 16 * kXlStride * 2, kRedBytes = 2 * 4 * MT * 256 * 4;
@@ -175,13 +206,21 @@ __global__ __launch_bounds__(kI4Threads) void int4_gemm_kernel(
   const int g_first = g_begin + wave;                            // this wavefront's groups: g_first + 4j
   const int nj = g_first < g_end ? (g_end - g_first + 3) / 4 : 0;
 
-  // tiles [tile0, tile0 + ntl) of this workgroup: an even split of all tiles (SILU: of all tile pairs) over the grid
-  const int n_units = SILU ? n_tiles / 2 : n_tiles;
+  // tiles [tile0, tile0 + ntl) of this workgroup: an even split of all tiles (SILU / ROPE: of all tile pairs) over the grid
+  const int n_units = PAIRED ? n_tiles / 2 : n_tiles;
   const int unit0 = (int)((int64_t)blockIdx.x * n_units / gridDim.x);
   const int n_own = (int)((int64_t)(blockIdx.x + 1) * n_units / gridDim.x) - unit0;
   const int tile0 = unit0;                                                             // plain: first tile
-  const int ntl = SILU ? 2 * n_own : n_own;                                            // 1 .. RT
-  auto tile_of = [&](int t) { return SILU ? unit0 + (t >> 1) + (t & 1) * (n_tiles / 2) : tile0 + t; };
+  const int ntl = PAIRED ? 2 * n_own : n_own;                                          // 1 .. RT
+  const int qk_units = ROPE ? (fz.hq + fz.hkv) * 4 : 0;                                // ROPE: pairs of the rotated heads
+  auto tile_of = [&](int t) {
+    if constexpr (SILU) return unit0 + (t >> 1) + (t & 1) * (n_tiles / 2);
+    if constexpr (ROPE) {
+      const int u = unit0 + (t >> 1);
+      return u < qk_units ? (u >> 2) * 8 + (u & 3) + (t & 1) * 4 : 2 * u + (t & 1);   // value heads: tiles 2u, 2u + 1
+    }
+    return tile0 + t;
+  };
 
   i4_v4f acc[RT][MT];
 #pragma unroll
@@ -206,7 +245,9 @@ __global__ __launch_bounds__(kI4Threads) void int4_gemm_kernel(
       __builtin_amdgcn_make_buffer_rsrc((void*)wq, 0, (int)(n_tiles * (int64_t)G * 512), 0x00027000);
   const __amdgpu_buffer_rsrc_t sz_rsrc =
       __builtin_amdgcn_make_buffer_rsrc((void*)sz, 0, (int)(n_tiles * (int64_t)G * 64), 0x00027000);
-  constexpr int kXg = MT * 2;                                    // 16-byte pieces per lane of one group block
+  const __amdgpu_buffer_rsrc_t g_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)(NORM ? fz.norm_gain : x), 0, K * 2, 0x00027000);
+  static_assert(!XHALF || MT == 1, "the 8-row block exists for one 16-row tile only");
+  constexpr int kXg = XHALF ? 1 : MT * 2;                        // 16-byte pieces per lane of one group block
   const int xg_off = ((lane >> 3) * K + (lane & 7) * 8) * 2;     // byte offset of piece 0; piece i is 8 rows further
   uint16_t* const xl = xstage + wave * (2 * MT * 16 * kXlStride);  // this wavefront's two stages
   const int xl_write = (lane >> 3) * kXlStride + (lane & 7) * 8;
@@ -219,6 +260,13 @@ __global__ __launch_bounds__(kI4Threads) void int4_gemm_kernel(
   // block that is parked one step after its request makes every step wait for a whole round trip to L2).
   constexpr int kXSlots = MT == 4 ? 1 : 2;   // 64 rows: one (with two the compiler waits for every request at the top of the loop body)
   i4_u4 xg[kXSlots][kXg];
+  i4_u4 gq[kXSlots];                                             // NORM: the gains of the lane's 8 k of the block on its way
+  float sq[kXg];                                                 // NORM: sum of squares of rows (lane >> 3) + 8 i over this wavefront's groups
+  (void)gq; (void)sq;
+  if constexpr (NORM) {
+#pragma unroll
+    for (int i = 0; i < kXg; ++i) sq[i] = 0.f;
+  }
   // Weight words on their way: two groups ahead.  With one tile per workgroup they rotate through THREE register
   // slots, so that a request never targets the slot the current step still reads: the compiler issues the request
   // before those reads, gives it other registers and copies them at the end of the loop body, and that copy waits for
@@ -238,10 +286,23 @@ __global__ __launch_bounds__(kI4Threads) void int4_gemm_kernel(
     const int kc = min(g_first + 4 * (J), G - 1) * (kGroup * 2);                                        \
     _Pragma("unroll") for (int i = 0; i < kXg; ++i)                                                     \
       xg[XS][i] = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, xg_off + i * 16 * K, kc, 0);            \
+    if constexpr (NORM) gq[XS] = __builtin_amdgcn_raw_buffer_load_b128(g_rsrc, (lane & 7) * 16, kc, 0); \
   }
-#define SUBSPEC_I4_PARK_X(SLOT)                                                                         \
-  _Pragma("unroll") for (int i = 0; i < kXg; ++i)                                                       \
-    *(i4_u4*)(&xl[(SLOT) * (MT * 16 * kXlStride) + i * 8 * kXlStride + xl_write]) = xg[(SLOT) % kXSlots][i];
+  // JP: index of the group being parked among this wavefront's groups (its squares count only if it exists)
+#define SUBSPEC_I4_PARK_X(SLOT, JP)                                                                     \
+  _Pragma("unroll") for (int i = 0; i < kXg; ++i) {                                                     \
+    i4_u4 piece = xg[(SLOT) % kXSlots][i];                                                              \
+    if constexpr (NORM) {                                                                               \
+      float f_[8], g_[8];                                                                               \
+      unpack8<DT>(piece, f_);                                                                           \
+      unpack8<DT>(gq[(SLOT) % kXSlots], g_);                                                            \
+      float ss_ = 0.f;                                                                                  \
+      _Pragma("unroll") for (int e = 0; e < 8; ++e) { ss_ = fmaf(f_[e], f_[e], ss_); f_[e] *= g_[e]; }  \
+      sq[i] += (JP) < nj ? ss_ : 0.f;                                                                   \
+      piece = pack8<DT>(f_);                                                                            \
+    }                                                                                                   \
+    *(i4_u4*)(&xl[(SLOT) * (MT * 16 * kXlStride) + i * 8 * kXlStride + xl_write]) = piece;              \
+  }
 #define SUBSPEC_I4_FETCH_W(SLOT, J, T)                                                                  \
   {                                                                                                     \
     const int g = wofs[T] + min(g_first + 4 * (J), G - 1);                                              \
@@ -259,7 +320,7 @@ __global__ __launch_bounds__(kI4Threads) void int4_gemm_kernel(
       xa[mt][0] = *(const i4_u4*)xr;                                                                    \
       xa[mt][1] = *(const i4_u4*)(xr + 8);                                                              \
     }                                                                                                   \
-    SUBSPEC_I4_PARK_X(SLOT);                                                                            \
+    SUBSPEC_I4_PARK_X(SLOT, (J) + 2);                                                                   \
     SUBSPEC_I4_FETCH_X((SLOT) % kXSlots, (J) + 2 + kXSlots);                                            \
     __builtin_amdgcn_sched_barrier(0);              /* keep the requests here: a full step ahead of their use */ \
     i4_v4f xs[MT];                                  /* sum of the group's activations, rows 16mt + 4c + rr */ \
@@ -286,14 +347,19 @@ __global__ __launch_bounds__(kI4Threads) void int4_gemm_kernel(
     __builtin_amdgcn_sched_barrier(0);                                                                  \
   }
 
+  if constexpr (XHALF) {
+    // rows 8..15 of both stages stay zero for the whole kernel
+    *(i4_u4*)(&xl[8 * kXlStride + xl_write]) = i4_u4{0u, 0u, 0u, 0u};
+    *(i4_u4*)(&xl[(MT * 16 * kXlStride) + 8 * kXlStride + xl_write]) = i4_u4{0u, 0u, 0u, 0u};
+  }
   SUBSPEC_I4_FETCH_X(0, 0);
 #pragma unroll
   for (int t = 0; t < RT; ++t) SUBSPEC_I4_FETCH_W(0, 0, t);
-  SUBSPEC_I4_PARK_X(0);
+  SUBSPEC_I4_PARK_X(0, 0);
   SUBSPEC_I4_FETCH_X(1 % kXSlots, 1);
 #pragma unroll
   for (int t = 0; t < RT; ++t) SUBSPEC_I4_FETCH_W(1, 1, t);
-  SUBSPEC_I4_PARK_X(1);
+  SUBSPEC_I4_PARK_X(1, 1);
   SUBSPEC_I4_FETCH_X(0, 2);
   if constexpr (kXSlots == 2) SUBSPEC_I4_FETCH_X(1, 3);
   if constexpr (RT == 1) {
@@ -314,7 +380,26 @@ __global__ __launch_bounds__(kI4Threads) void int4_gemm_kernel(
       SUBSPEC_I4_STEP(1, 1, 1, j + 1);
     }
   }
+  if constexpr (NORM) {
+    // the eight lanes that share a row hold its squares over different k; one value per (wavefront, row) goes to LDS
+#pragma unroll
+    for (int i = 0; i < kXg; ++i) {
+      float v = sq[i];
+      v += __shfl_xor(v, 1, kWave);
+      v += __shfl_xor(v, 2, kWave);
+      v += __shfl_xor(v, 4, kWave);
+      if ((lane & 7) == 0) sq_s[wave * (MT * 16) + (lane >> 3) + 8 * i] = v;
+    }
+    if constexpr (XHALF) {
+      if ((lane & 7) == 0) sq_s[wave * (MT * 16) + (lane >> 3) + 8] = 0.f;
+    }
+  }
   __syncthreads();                                               // the stages are reused for the reduction below
+  if constexpr (NORM) {
+    // ordered before its first use by the barrier of reduction round 0
+    if (tid < MT * 16)
+      rstd_s[tid] = rsqrtf((sq_s[tid] + sq_s[MT * 16 + tid] + sq_s[2 * MT * 16 + tid] + sq_s[3 * MT * 16 + tid]) / (float)K + fz.norm_eps);
+  }
 #undef SUBSPEC_I4_PARK_X
 #undef SUBSPEC_I4_FETCH_X
 #undef SUBSPEC_I4_FETCH_W
@@ -324,8 +409,8 @@ __global__ __launch_bounds__(kI4Threads) void int4_gemm_kernel(
   // round.  LDS holds two rounds, so a round needs one barrier; wavefront w finishes the activation
   // row blocks mt = w, w + 4, ... of the tile, so the sums and stores are spread over the workgroup.
   // accumulator layout: rows m = 16*mt + 4*c + rr, column n = 16*tile + ln
-  float gate_held[MT][4];                                        // SILU: the rounded gate values between two rounds
-  (void)gate_held;
+  float held[MT][4];                                             // SILU / ROPE: the rounded values of the even tile between two rounds
+  (void)held;
 #pragma unroll
   for (int t = 0; t < RT; ++t) {
     if (t >= ntl) break;                                         // uniform
@@ -345,19 +430,66 @@ __global__ __launch_bounds__(kI4Threads) void int4_gemm_kernel(
 #pragma unroll
         for (int rr = 0; rr < 4; ++rr) v[rr] += o[rr];
       }
-      if constexpr (SILU) {
-        // even round: the gate tile, kept in registers; odd round: its up tile, same wavefront, same lanes
+      if constexpr (NORM) {
+#pragma unroll
+        for (int rr = 0; rr < 4; ++rr) v[rr] *= rstd_s[mt * 16 + c * 4 + rr];
+      }
+      if constexpr (PAIRED) {
+        // even round: the first tile of the pair, kept in registers; odd round: its partner, same wavefront, same lanes
         if ((t & 1) == 0) {
 #pragma unroll
-          for (int rr = 0; rr < 4; ++rr) gate_held[mt][rr] = Elem<DT>::round(v[rr] + bv);
-        } else {
+          for (int rr = 0; rr < 4; ++rr) held[mt][rr] = Elem<DT>::round(v[rr] + bv);
+        } else if constexpr (SILU) {
           const int64_t f = (int64_t)(unit0 + (t >> 1)) * 16 + ln;
 #pragma unroll
           for (int rr = 0; rr < 4; ++rr) {
             const int m = mt * 16 + c * 4 + rr;
             if (m >= M) continue;
-            const float g = gate_held[mt][rr], u = Elem<DT>::round(v[rr] + bv);
+            const float g = held[mt][rr], u = Elem<DT>::round(v[rr] + bv);
             Elem<DT>::store(y, (int64_t)m * (N / 2) + f, Elem<DT>::round(g / (1.f + __expf(-g))) * u);
+          }
+        } else {
+          const int u = unit0 + (t >> 1);
+          if (u < qk_units) {
+            // rotary pair (d, d + 64) of head u / 4, d = 16 (u % 4) + ln; t * cos + rotate_half(t) * sin with each
+            // product and the sum rounded like the eager tensor ops
+            const int head = u >> 2, d = (u & 3) * 16 + ln;
+            const float inv_freq = fz.inv_freq ? fz.inv_freq[d] : exp2f(-(float)(2 * d) / 128.f * fz.log2_theta);
+#pragma unroll
+            for (int rr = 0; rr < 4; ++rr) {
+              const int m = mt * 16 + c * 4 + rr;
+              if (m >= M) continue;
+              float sn, cs;
+              sincosf((float)fz.positions[m] * inv_freq, &sn, &cs);
+              cs = Elem<DT>::round(cs);
+              sn = Elem<DT>::round(sn);
+              const float lo = held[mt][rr], hi = Elem<DT>::round(v[rr] + bv);
+              const float o_lo = Elem<DT>::round(lo * cs) + Elem<DT>::round(-hi * sn);
+              const float o_hi = Elem<DT>::round(hi * cs) + Elem<DT>::round(lo * sn);
+              uint16_t* dst;
+              if (head < fz.hq) {
+                dst = fz.q_out + ((int64_t)head * M + m) * 128;
+              } else {
+                const int64_t row = fz.cache_rows[m];
+                if (row < 0 || row >= fz.seq_stride) continue;   // a row outside the layer's cache is dropped
+                dst = fz.k_cache + ((int64_t)(head - fz.hq) * fz.seq_stride + row) * 128;
+              }
+              Elem<DT>::store(dst, d, o_lo);
+              Elem<DT>::store(dst, d + 64, o_hi);
+            }
+          } else {
+            // two consecutive tiles of a value head: copied
+            const int vt = 2 * (u - qk_units), kvh = vt >> 3, d = (vt & 7) * 16 + ln;
+#pragma unroll
+            for (int rr = 0; rr < 4; ++rr) {
+              const int m = mt * 16 + c * 4 + rr;
+              if (m >= M) continue;
+              const int64_t row = fz.cache_rows[m];
+              if (row < 0 || row >= fz.seq_stride) continue;
+              uint16_t* dst = fz.v_cache + ((int64_t)kvh * fz.seq_stride + row) * 128;
+              Elem<DT>::store(dst, d, held[mt][rr]);
+              Elem<DT>::store(dst, d + 16, v[rr] + bv);
+            }
           }
         }
       } else {
@@ -395,7 +527,11 @@ static I4Plan i4_plan(int64_t M, int64_t N, int64_t K) {
   const int64_t tiles = N / 16, slots = i4_slots(M);
   // row tiles per workgroup: the smallest compiled variant that covers all tiles in one resident wave of
   // workgroups; the grid then splits the tiles evenly, so every workgroup has row_tiles or row_tiles - 1
-  const int row_tiles = i4_row_tile_variant((tiles + slots - 1) / slots);
+  int row_tiles = i4_row_tile_variant((tiles + slots - 1) / slots);
+  // A long K over few tiles (the down projection) is split over workgroups, and every split re-reads its slice of the
+  // activations: two tiles per workgroup halve that traffic (3584x18944, 8 rows, five splits: 13.8 -> 12.7 us; three or
+  // five tiles per workgroup and fewer splits were slower: 14.1 to 15.7 us)
+  if (M <= 16 && row_tiles == 1 && tiles * 4 <= slots && G >= 112) row_tiles = 2;
   const int64_t wgs = (tiles + row_tiles - 1) / row_tiles;
   int splits = (int)std::max<int64_t>(1, (slots + wgs / 2) / wgs);
   // a split costs a second launch (the reduction) and fp32 partials: it pays from about 56 groups
@@ -409,26 +545,38 @@ static I4Plan i4_plan(int64_t M, int64_t N, int64_t K) {
   return I4Plan{(int)wgs, row_tiles, splits, gps};
 }
 
-// gate|up projection with the SwiGLU output stage: x [M, K], weights of N = 2F rows (gate rows first), act [M, F]
-template <int DT>
-static int run_int4_silu(const void* x, const uint32_t* wq, const uint32_t* sz, const void* bias, void* act, int64_t M,
-                         int64_t N, int64_t K, hipStream_t st) {
+// Paired-tile launches: the gate|up projection with the SwiGLU output stage (x [M, K], weights of N = 2F rows, gate rows
+// first, act [M, F]) and the q|k|v projection with the rotary / cache-write output stage; either with RMSNorm as prologue.
+template <int DT, int EPI>
+static int run_int4_paired(const void* x, const uint32_t* wq, const uint32_t* sz, const void* bias, void* out, int64_t M,
+                           int64_t N, int64_t K, const I4Fused& fz, hipStream_t st) {
   const int64_t pairs = N / 32, slots = i4_slots(M);
-  // one or two (gate, up) pairs per workgroup; two only with few activation rows (the accumulators of four tiles
+  // one or two pairs per workgroup; two only with few activation rows (the accumulators of four tiles
   // times four row blocks would fill the register file)
   const int rt = (pairs <= slots || M > 32) ? 2 : 4;
   const int64_t wgs = (pairs + rt / 2 - 1) / (rt / 2);
   const dim3 grid((unsigned)wgs, 1);
   const int G = (int)(K / kGroup);
-#define SUBSPEC_I4_SILU(MT, RT)                                                                                    \
-  hipLaunchKernelGGL((int4_gemm_kernel<DT, MT, RT, true>), grid, dim3(kI4Threads), 0, st, (const uint16_t*)x,     \
-                     (const uint2*)wq, sz, (const uint16_t*)bias, (const uint16_t*)nullptr, (uint16_t*)act, (float*)nullptr,   \
-                     (int)M, N, (int)K, 1, (G + 3) / 4 * 4)
+  const bool norm = fz.norm_gain != nullptr;
+#define SUBSPEC_I4_PAIRED(MT, RT, NORM)                                                                            \
+  if (MT == 1 && M <= 8)                                                                                           \
+    hipLaunchKernelGGL((int4_gemm_kernel<DT, 1, RT, EPI, NORM, true>), grid, dim3(kI4Threads), 0, st, (const uint16_t*)x, \
+                       (const uint2*)wq, sz, (const uint16_t*)bias, (const uint16_t*)nullptr, (uint16_t*)out, (float*)nullptr, \
+                       (int)M, N, (int)K, 1, (G + 3) / 4 * 4, fz);                                                 \
+  else                                                                                                             \
+  hipLaunchKernelGGL((int4_gemm_kernel<DT, MT, RT, EPI, NORM>), grid, dim3(kI4Threads), 0, st, (const uint16_t*)x, \
+                     (const uint2*)wq, sz, (const uint16_t*)bias, (const uint16_t*)nullptr, (uint16_t*)out, (float*)nullptr,   \
+                     (int)M, N, (int)K, 1, (G + 3) / 4 * 4, fz)
+#define SUBSPEC_I4_PAIRED_RT(MT, NORM) do { if (rt == 2) SUBSPEC_I4_PAIRED(MT, 2, NORM); else SUBSPEC_I4_PAIRED(MT, 4, NORM); } while (0)
   DominantKernelTimer timer(st);
-  if (M <= 16) { if (rt == 2) SUBSPEC_I4_SILU(1, 2); else SUBSPEC_I4_SILU(1, 4); }
-  else if (M <= 32) { if (rt == 2) SUBSPEC_I4_SILU(2, 2); else SUBSPEC_I4_SILU(2, 4); }
-  else { if (rt == 2) SUBSPEC_I4_SILU(4, 2); else SUBSPEC_I4_SILU(4, 4); }
-#undef SUBSPEC_I4_SILU
+  if (M <= 16) { if (norm) SUBSPEC_I4_PAIRED_RT(1, true); else SUBSPEC_I4_PAIRED_RT(1, false); }
+  else if (M <= 32) { if (norm) SUBSPEC_I4_PAIRED_RT(2, true); else SUBSPEC_I4_PAIRED_RT(2, false); }
+  else {
+    if (norm) SUBSPEC_FAIL(SUBSPEC_ERR_LIMIT, "int4 projection with the RMSNorm prologue: M=%lld exceeds 32 rows", (long long)M);
+    SUBSPEC_I4_PAIRED_RT(4, false);
+  }
+#undef SUBSPEC_I4_PAIRED_RT
+#undef SUBSPEC_I4_PAIRED
   SUBSPEC_CHECK_HIP(hipGetLastError());
   return SUBSPEC_OK;
 }
@@ -448,9 +596,14 @@ static int run_int4(const void* x, const uint32_t* wq, const uint32_t* sz, const
     float* partial = (float*)workspace;
     const dim3 grid((unsigned)pl.wgs, (unsigned)pl.splits);
 #define SUBSPEC_I4_LAUNCH(MT, RT)                                                                                  \
+  if (MT == 1 && M <= 8)                                                                                           \
+    hipLaunchKernelGGL((int4_gemm_kernel<DT, 1, RT, kEpiPlain, false, true>), grid, dim3(kI4Threads), 0, st, (const uint16_t*)x, \
+                       (const uint2*)wq, sz, (const uint16_t*)bias, (const uint16_t*)residual, (uint16_t*)y, partial, (int)M, N, (int)K, \
+                       pl.splits, pl.groups_per_split, I4Fused{});                                                 \
+  else                                                                                                             \
   hipLaunchKernelGGL((int4_gemm_kernel<DT, MT, RT>), grid, dim3(kI4Threads), 0, st, (const uint16_t*)x,            \
                      (const uint2*)wq, sz, (const uint16_t*)bias, (const uint16_t*)residual, (uint16_t*)y, partial, (int)M, N, (int)K, \
-                     pl.splits, pl.groups_per_split)
+                     pl.splits, pl.groups_per_split, I4Fused{})
 #define SUBSPEC_I4_LAUNCH_MT(MT)                                                                                   \
   do {                                                                                                             \
     if (pl.row_tiles == 1) SUBSPEC_I4_LAUNCH(MT, 1);                                                               \
@@ -503,7 +656,7 @@ static size_t i4_workspace_one(int64_t M, int64_t N, int64_t K) {
 
 extern "C" int subspec_int4_gate_up_silu(const void* x, const uint32_t* wq, const uint32_t* sz, const void* bias, void* act,
                                          int dtype, int64_t M, int64_t N, int64_t K, void* stream) {
-  return int4_gate_up_silu_ex(x, wq, sz, bias, act, dtype, M, N, K, stream);
+  return int4_gate_up_silu_ex(x, wq, sz, bias, act, dtype, M, N, K, nullptr, 0.f, stream);
 }
 
 extern "C" size_t subspec_int4_linear_workspace(int64_t M, int64_t N, int64_t K) {
@@ -513,20 +666,58 @@ extern "C" size_t subspec_int4_linear_workspace(int64_t M, int64_t N, int64_t K)
   return M % 64 ? std::max(full, i4_workspace_one(M % 64, N, K)) : full;
 }
 
-int subspec::int4_gate_up_silu_ex(const void* x, const uint32_t* wq, const uint32_t* sz, const void* bias, void* act, int dtype,
-                                  int64_t M, int64_t N, int64_t K, void* stream) {
+static int paired_args_ok(const char* what, const void* x, const uint32_t* wq, const uint32_t* sz, int dtype, int64_t M,
+                          int64_t N, int64_t K) {
   if (dtype != SUBSPEC_BF16 && dtype != SUBSPEC_F16)
-    SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "int4_gate_up_silu: dtype %d not supported (bf16 / fp16 activations only)", dtype);
-  if (!x || !wq || !sz || !act) SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "int4_gate_up_silu: null pointer argument");
+    SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "%s: dtype %d not supported (bf16 / fp16 activations only)", what, dtype);
+  if (!x || !wq || !sz) SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "%s: null pointer argument", what);
   if (M <= 0 || M > 64 || N <= 0 || K <= 0 || N % 32 != 0 || K % kGroup != 0 || K > 65536)
-    SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "int4_gate_up_silu: M=%lld N=%lld K=%lld; 1 <= M <= 64, N a multiple of 32, K of 64",
+    SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "%s: M=%lld N=%lld K=%lld; 1 <= M <= 64, N a multiple of 32, K of 64", what,
                  (long long)M, (long long)N, (long long)K);
   if (N * K / 2 >= ((int64_t)1 << 31))
-    SUBSPEC_FAIL(SUBSPEC_ERR_LIMIT, "int4_gate_up_silu: N*K/2=%lld bytes of codes exceed the 2 GiB descriptor range", (long long)(N * K / 2));
-  if ((uintptr_t)x % 16 || (uintptr_t)wq % 16 || (uintptr_t)sz % 16 || (uintptr_t)act % 8)
-    SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "int4_gate_up_silu: x / wq / sz must be 16-byte aligned, act 8-byte aligned");
-  if (dtype == SUBSPEC_BF16) return run_int4_silu<SUBSPEC_BF16>(x, wq, sz, bias, act, M, N, K, (hipStream_t)stream);
-  return run_int4_silu<SUBSPEC_F16>(x, wq, sz, bias, act, M, N, K, (hipStream_t)stream);
+    SUBSPEC_FAIL(SUBSPEC_ERR_LIMIT, "%s: N*K/2=%lld bytes of codes exceed the 2 GiB descriptor range", what, (long long)(N * K / 2));
+  if ((uintptr_t)x % 16 || (uintptr_t)wq % 16 || (uintptr_t)sz % 16)
+    SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "%s: x / wq / sz must be 16-byte aligned", what);
+  return SUBSPEC_OK;
+}
+
+int subspec::int4_gate_up_silu_ex(const void* x, const uint32_t* wq, const uint32_t* sz, const void* bias, void* act, int dtype,
+                                  int64_t M, int64_t N, int64_t K, const void* norm_gain, float norm_eps, void* stream) {
+  const int rc = paired_args_ok("int4_gate_up_silu", x, wq, sz, dtype, M, N, K);
+  if (rc) return rc;
+  if (!act || (uintptr_t)act % 8) SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "int4_gate_up_silu: act must be a non-null, 8-byte aligned pointer");
+  if (norm_gain && (uintptr_t)norm_gain % 16) SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "int4_gate_up_silu: the norm gain must be 16-byte aligned");
+  I4Fused fz{};
+  fz.norm_gain = (const uint16_t*)norm_gain;
+  fz.norm_eps = norm_eps;
+  if (dtype == SUBSPEC_BF16) return run_int4_paired<SUBSPEC_BF16, kEpiSilu>(x, wq, sz, bias, act, M, N, K, fz, (hipStream_t)stream);
+  return run_int4_paired<SUBSPEC_F16, kEpiSilu>(x, wq, sz, bias, act, M, N, K, fz, (hipStream_t)stream);
+}
+
+int subspec::int4_qkv_rope_ex(const void* x, const uint32_t* wq, const uint32_t* sz, const void* bias, int dtype, int64_t M,
+                              int64_t K, const void* norm_gain, float norm_eps, const int32_t* positions,
+                              const int32_t* cache_rows, void* q_out, void* k_cache, void* v_cache, int64_t n_q_heads,
+                              int64_t n_kv_heads, int64_t kv_seq_stride, float rope_theta, const float* inv_freq, void* stream) {
+  const int64_t N = (n_q_heads + 2 * n_kv_heads) * 128;
+  const int rc = paired_args_ok("int4_qkv_rope", x, wq, sz, dtype, M, N, K);
+  if (rc) return rc;
+  if (!positions || !cache_rows || !q_out || !k_cache || !v_cache) SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "int4_qkv_rope: null pointer argument");
+  if (norm_gain && (uintptr_t)norm_gain % 16) SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "int4_qkv_rope: the norm gain must be 16-byte aligned");
+  I4Fused fz{};
+  fz.norm_gain = (const uint16_t*)norm_gain;
+  fz.norm_eps = norm_eps;
+  fz.positions = positions;
+  fz.cache_rows = cache_rows;
+  fz.q_out = (uint16_t*)q_out;
+  fz.k_cache = (uint16_t*)k_cache;
+  fz.v_cache = (uint16_t*)v_cache;
+  fz.inv_freq = inv_freq;
+  fz.hq = (int)n_q_heads;
+  fz.hkv = (int)n_kv_heads;
+  fz.seq_stride = kv_seq_stride;
+  fz.log2_theta = log2f(rope_theta);
+  if (dtype == SUBSPEC_BF16) return run_int4_paired<SUBSPEC_BF16, kEpiRope>(x, wq, sz, bias, nullptr, M, N, K, fz, (hipStream_t)stream);
+  return run_int4_paired<SUBSPEC_F16, kEpiRope>(x, wq, sz, bias, nullptr, M, N, K, fz, (hipStream_t)stream);
 }
 
 int subspec::int4_linear_ex(const void* x, const uint32_t* wq, const uint32_t* sz, const void* bias, const void* residual,

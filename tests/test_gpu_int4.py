@@ -33,12 +33,12 @@ def _check(N, K, M, dtype, seed, bias=False):
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_small_shapes(dtype):
     for seed, (N, K, M) in enumerate([(16, 64, 1), (48, 192, 1), (64, 256, 2), (80, 512, 16), (128, 1024, 17),
-                                      (256, 2048, 33), (64, 3584, 64), (512, 128, 5)]):
+                                      (256, 2048, 33), (64, 3584, 64), (512, 128, 5), (96, 7168, 8), (32, 320, 3)]):
         _check(N, K, M, dtype, seed, bias=seed % 2 == 0)
 
 
 @pytest.mark.parametrize("N,K", [(4608, 3584), (3584, 3584), (37888, 3584), (3584, 18944)])
-@pytest.mark.parametrize("M", [1, 16, 64])
+@pytest.mark.parametrize("M", [1, 8, 16, 64])                 # 8: one draft level (top-k 8), the 8-row activation block
 def test_config4_qwen_shapes(N, K, M):
     _check(N, K, M, torch.bfloat16, 100 + M)
 
