@@ -352,16 +352,21 @@ __global__ __launch_bounds__(kI4Threads) void int4_gemm_kernel(
     *(i4_u4*)(&xl[8 * kXlStride + xl_write]) = i4_u4{0u, 0u, 0u, 0u};
     *(i4_u4*)(&xl[(MT * 16 * kXlStride) + 8 * kXlStride + xl_write]) = i4_u4{0u, 0u, 0u, 0u};
   }
+  // The requests before the loop are issued in the order the loop issues them (activation block, then the weights of
+  // the group two steps back), so that the first trip finds the same queue of outstanding requests as every later
+  // one: the compiler gives each wait ONE count that must hold on every path into the loop, and a prologue that ends
+  // with the activation requests makes that count "nothing may be outstanding but the newest block" on every trip --
+  // the weights would be waited for one step after their request, whatever the distance in the source.
   SUBSPEC_I4_FETCH_X(0, 0);
+  if constexpr (kXSlots == 2) SUBSPEC_I4_FETCH_X(1, 1);
+  SUBSPEC_I4_PARK_X(0, 0);
+  if constexpr (kXSlots == 2) { SUBSPEC_I4_FETCH_X(0, 2); } else { SUBSPEC_I4_FETCH_X(0, 1); }
 #pragma unroll
   for (int t = 0; t < RT; ++t) SUBSPEC_I4_FETCH_W(0, 0, t);
-  SUBSPEC_I4_PARK_X(0, 0);
-  SUBSPEC_I4_FETCH_X(1 % kXSlots, 1);
+  SUBSPEC_I4_PARK_X(1, 1);
+  if constexpr (kXSlots == 2) { SUBSPEC_I4_FETCH_X(1, 3); } else { SUBSPEC_I4_FETCH_X(0, 2); }
 #pragma unroll
   for (int t = 0; t < RT; ++t) SUBSPEC_I4_FETCH_W(1, 1, t);
-  SUBSPEC_I4_PARK_X(1, 1);
-  SUBSPEC_I4_FETCH_X(0, 2);
-  if constexpr (kXSlots == 2) SUBSPEC_I4_FETCH_X(1, 3);
   if constexpr (RT == 1) {
     // step J: LDS stage J % 2, weight slot J % 3, request for group J + 2 into slot (J + 2) % 3
     for (int j = 0; j < nj; j += 6) {
