@@ -380,6 +380,20 @@ typedef struct subspec_decoder_layer_dims {
                                  use (HuggingFace: 1 / theta^(2i / head_dim), evaluated by torch), so that rows written
                                  here and rows written by a prefill are rotated by identical angles; NULL: the kernel
                                  evaluates rope_theta^(-2i / head_dim) itself */
+  const int64_t* prefix_len_dev; /* device int64 or NULL.  Not NULL: attention reads the prefix length here when the kernels
+                                 run, and prefix_len above is the upper bound the launches are laid out for -- a sequence
+                                 of layer calls captured into a HIP graph is replayed while the prefix grows (the
+                                 reference captures its draft step the same way, with device-side positions:
+                                 specdecodes/models/draft_models/subspec_sd_fi.py:65-179); positions / cache_rows are
+                                 device arrays already */
+  const int32_t* page_indices; /* NULL: k_cache / v_cache are the layer's contiguous [n_kv_heads, kv_seq_stride, head_dim]
+                                 caches.  Not NULL: a paged cache -- k_cache is ONE LAYER of a page pool
+                                 [max_pages][2 (K, V)][page_len][n_kv_heads][head_dim], v_cache is ignored, cache row p lives
+                                 in page page_indices[p / page_len] at token p % page_len (see subspec_tree_attention_paged),
+                                 and kv_seq_stride must be n_pages * page_len (rotary rows are written and attention reads
+                                 through the table: flashinfer append_paged_kv_cache + the paged wrapper's run,
+                                 specdecodes/models/utils/flashinfer/attention_wrapper.py:244-253,288-316) */
+  int64_t n_pages, max_pages, page_len;
 } subspec_decoder_layer_dims;
 
 typedef struct subspec_decoder_layer_weights {

@@ -30,7 +30,9 @@ class DecoderLayerDims(C.Structure):
     _fields_ = [("dtype", C.c_int32), ("reserved", C.c_int32),
                 ("n_rows", _i64), ("hidden", _i64), ("intermediate", _i64), ("n_q_heads", _i64), ("n_kv_heads", _i64),
                 ("head_dim", _i64), ("kv_seq_stride", _i64), ("prefix_len", _i64), ("n_tree_slots", _i64),
-                ("rms_eps", C.c_float), ("rope_theta", C.c_float), ("rope_inv_freq", C.c_void_p)]
+                ("rms_eps", C.c_float), ("rope_theta", C.c_float), ("rope_inv_freq", C.c_void_p),
+                ("prefix_len_dev", C.c_void_p), ("page_indices", C.c_void_p), ("n_pages", _i64), ("max_pages", _i64),
+                ("page_len", _i64)]
 
 
 class DecoderLayerWeights(C.Structure):

@@ -93,6 +93,9 @@ struct AttnParams {
   float scale_log2;            // softmax scale * log2(e)
   // paged cache (one request): row p of K lives at page_table[p >> page_shift], token p & (page_len - 1) of
   // a pool layer [max_pages][2 (K, V)][page_len][hkv][128]; V is v_delta elements behind K
+  // when not null, the prefix length is read here by the kernel and `prefix` above is only the upper bound the grid
+  // and the key chunks were laid out for (a captured launch replayed while the prefix grows)
+  const int64_t* prefix_dev;
   const int32_t* page_table;
   int page_shift, max_pages;
   int64_t page_stride, tok_stride, v_delta;   // elements
@@ -127,7 +130,8 @@ __global__ __launch_bounds__(kAttnThreads) __attribute__((amdgpu_waves_per_eu(2,
   const int qh = kvh * group + (head_ok ? head_in_group : 0);
   const int bh = b * (int)ap.hq + qh;
   const int n = (int)ap.n_rows;
-  const int64_t kv_len = ap.prefix + ap.n_slots;
+  const int64_t prefix = ap.prefix_dev ? min(max(*ap.prefix_dev, (int64_t)0), ap.prefix) : ap.prefix;
+  const int64_t kv_len = prefix + ap.n_slots;
 
   // ---- Q^T operands of the wave's two 16-row tiles: Q[row][32*ks + 8*lg .. +7]
   int row[ROWT];
@@ -204,7 +208,7 @@ __global__ __launch_bounds__(kAttnThreads) __attribute__((amdgpu_waves_per_eu(2,
       bits[nt][1] = (row_ok[nt] && w + 1 < ap.mask_words) ? row_bits[nt][w + 1] : 0ull;
     }
   };
-  int held_word = (int)(max(max(key0, ap.prefix / kKeyBlock * kKeyBlock) - ap.prefix, (int64_t)0) >> 6);
+  int held_word = (int)(max(max(key0, prefix / kKeyBlock * kKeyBlock) - prefix, (int64_t)0) >> 6);
   load_bits(held_word);
 
   SUBSPEC_ATTN_FETCH(key0);
@@ -228,10 +232,10 @@ __global__ __launch_bounds__(kAttnThreads) __attribute__((amdgpu_waves_per_eu(2,
     float mloc[ROWT];
 #pragma unroll
     for (int nt = 0; nt < ROWT; ++nt) mloc[nt] = -INFINITY;
-    const bool plain = kb + kKeyBlock <= ap.prefix;    // block lies entirely in the prefix: no mask (uniform)
+    const bool plain = kb + kKeyBlock <= prefix;    // block lies entirely in the prefix: no mask (uniform)
     // a 64-key block touches at most two consecutive words of the bitsets: word0 and word0 + 1.  They were
     // fetched before the loop for the first masked block; trees beyond 128 slots fetch again as the blocks move on.
-    const int word0 = (int)(max(kb - ap.prefix, (int64_t)0) >> 6);
+    const int word0 = (int)(max(kb - prefix, (int64_t)0) >> 6);
     if (!plain && word0 != held_word) {                // uniform
       held_word = word0;
       load_bits(word0);
@@ -267,8 +271,8 @@ __global__ __launch_bounds__(kAttnThreads) __attribute__((amdgpu_waves_per_eu(2,
         for (int r = 0; r < 4; ++r) {
           const int64_t pos = kb + kt * 16 + lg * 4 + r;
           const bool in_range = pos < kv_len;
-          const bool tree = pos >= ap.prefix;
-          const int rel = tree ? (int)(pos - ap.prefix) : 0;   // tree slot, < 64 * mask_words when in range
+          const bool tree = pos >= prefix;
+          const int rel = tree ? (int)(pos - prefix) : 0;   // tree slot, < 64 * mask_words when in range
           const int sh = rel & 63;
           const bool first_word = (rel >> 6) == word0;
 #pragma unroll
@@ -414,13 +418,11 @@ extern "C" size_t subspec_tree_attention_workspace(int64_t batch, int64_t n_q_he
   return align_up(slots * kAttnD * sizeof(float), 256) + align_up(slots * 2 * sizeof(float), 256);
 }
 
-struct PagedArgs { const int32_t* page_table; int64_t n_pages, max_pages, page_len; };
-
 static int tree_attention_impl(const char* what, const void* q, const void* k_cache, const void* v_cache, void* out, int dtype,
                                int64_t batch, int64_t n_q_heads, int64_t n_kv_heads, int64_t n_rows, int64_t n_tree_slots,
                                int64_t head_dim, int64_t kv_seq_stride, int64_t prefix_len, const uint64_t* anc_bits,
-                               int64_t anc_batch_stride, float scale, const PagedArgs* paged, void* workspace,
-                               size_t workspace_bytes, void* stream) {
+                               int64_t anc_batch_stride, float scale, const KvPages* paged, const int64_t* prefix_dev,
+                               void* workspace, size_t workspace_bytes, void* stream) {
   if (dtype != SUBSPEC_BF16 && dtype != SUBSPEC_F16)
     SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "%s: dtype %d not supported (bf16 / fp16 only)", what, dtype);
   if (!q || !k_cache || !v_cache || !out || !anc_bits) SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "%s: null pointer argument", what);
@@ -445,11 +447,12 @@ static int tree_attention_impl(const char* what, const void* q, const void* k_ca
   ap.prefix = prefix_len; ap.anc_batch_stride = anc_batch_stride;
   ap.mask_words = (int)((n_tree_slots + 63) / 64);
   ap.row0 = 0; ap.win_rows = (int)std::min<int64_t>(n_rows, kAttnRows);
+  ap.prefix_dev = prefix_dev;
   ap.page_table = nullptr; ap.page_shift = 0; ap.max_pages = 0; ap.page_stride = ap.tok_stride = ap.v_delta = 0;
   if (paged) {
     int shift = 0;
     while ((1ll << shift) < paged->page_len) ++shift;
-    ap.page_table = paged->page_table;
+    ap.page_table = paged->table;
     ap.page_shift = shift;
     ap.max_pages = (int)paged->max_pages;
     ap.tok_stride = n_kv_heads * kAttnD;
@@ -520,7 +523,7 @@ extern "C" int subspec_tree_attention(const void* q, const void* k_cache, const 
                                       void* workspace, size_t workspace_bytes, void* stream) {
   return tree_attention_impl("tree_attention", q, k_cache, v_cache, out, dtype, batch, n_q_heads, n_kv_heads, n_rows,
                              n_tree_slots, head_dim, kv_seq_stride, prefix_len, anc_bits, anc_batch_stride, scale, nullptr,
-                             workspace, workspace_bytes, stream);
+                             nullptr, workspace, workspace_bytes, stream);
 }
 
 extern "C" int subspec_tree_attention_paged(const void* q, const void* kv_pool_layer, const int32_t* page_indices,
@@ -533,9 +536,27 @@ extern "C" int subspec_tree_attention_paged(const void* q, const void* kv_pool_l
     SUBSPEC_FAIL(SUBSPEC_ERR_LIMIT, "tree_attention_paged: page_len=%lld must be a power of two up to 4096", (long long)page_len);
   if (n_pages <= 0 || max_pages < n_pages || max_pages > 0x7fffffff)
     SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "tree_attention_paged: n_pages=%lld max_pages=%lld", (long long)n_pages, (long long)max_pages);
-  const PagedArgs pg{page_indices, n_pages, max_pages, page_len};
+  const KvPages pg{page_indices, n_pages, max_pages, page_len};
   // the request's pages play the part of the cache length: rows beyond them do not exist
   return tree_attention_impl("tree_attention_paged", q, kv_pool_layer, kv_pool_layer, out, dtype, 1, n_q_heads, n_kv_heads,
-                             n_rows, n_tree_slots, head_dim, n_pages * page_len, prefix_len, anc_bits, 0, scale, &pg, workspace,
-                             workspace_bytes, stream);
+                             n_rows, n_tree_slots, head_dim, n_pages * page_len, prefix_len, anc_bits, 0, scale, &pg, nullptr,
+                             workspace, workspace_bytes, stream);
+}
+
+int subspec::tree_attention_ex(const void* q, const void* k_cache, const void* v_cache, void* out, int dtype, int64_t n_q_heads,
+                               int64_t n_kv_heads, int64_t n_rows, int64_t n_tree_slots, int64_t kv_seq_stride, int64_t prefix_len,
+                               const int64_t* prefix_dev, const KvPages* pages, const uint64_t* anc_bits, float scale,
+                               void* workspace, size_t workspace_bytes, void* stream) {
+  if (pages) {
+    if (!pages->table) SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "tree_attention: null page table");
+    if (pages->page_len <= 0 || (pages->page_len & (pages->page_len - 1)) != 0 || pages->page_len > 4096)
+      SUBSPEC_FAIL(SUBSPEC_ERR_LIMIT, "tree_attention: page_len=%lld must be a power of two up to 4096", (long long)pages->page_len);
+    if (pages->n_pages <= 0 || pages->max_pages < pages->n_pages || pages->max_pages > 0x7fffffff)
+      SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "tree_attention: n_pages=%lld max_pages=%lld", (long long)pages->n_pages, (long long)pages->max_pages);
+    return tree_attention_impl("tree_attention", q, k_cache, k_cache, out, dtype, 1, n_q_heads, n_kv_heads, n_rows, n_tree_slots, kAttnD,
+                               pages->n_pages * pages->page_len, prefix_len, anc_bits, 0, scale, pages, prefix_dev, workspace,
+                               workspace_bytes, stream);
+  }
+  return tree_attention_impl("tree_attention", q, k_cache, v_cache, out, dtype, 1, n_q_heads, n_kv_heads, n_rows, n_tree_slots, kAttnD,
+                             kv_seq_stride, prefix_len, anc_bits, 0, scale, nullptr, prefix_dev, workspace, workspace_bytes, stream);
 }

@@ -206,6 +206,59 @@ __device__ __forceinline__ int block_min_i(int v, int* scratch) {
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 
+// A request's page table over one layer of a page pool [max_pages][2 (K, V)][page_len][n_kv_heads][128]
+struct KvPages { const int32_t* table; int64_t n_pages, max_pages, page_len; };
+
+// Where the K / V row of (kv head, cache row) lives, for kernels that write rows: contiguous [Hkv, seq_stride, 128]
+// caches, or one layer of a page pool (then v_cache is unused and a row outside the request's pages does not exist).
+struct KvRowMap {
+  uint16_t* k_cache;
+  uint16_t* v_cache;
+  int64_t seq_stride;            // rows a head holds (contiguous), or pages * page_len (paged)
+  const int32_t* page_table;     // null: contiguous
+  int page_shift, max_pages, hkv;
+  int64_t page_elems;            // paged: elements of one page of K (page_len * hkv * 128); V follows K inside a page
+};
+// element offset pointers of row `row` of head `kvh`, or false when the row is outside the cache
+__device__ __forceinline__ bool kv_row_ptrs(const KvRowMap& m, int kvh, int64_t row, uint16_t** k, uint16_t** v) {
+  if (row < 0 || row >= m.seq_stride) return false;
+  if (m.page_table) {
+    const int page = min(max(m.page_table[row >> m.page_shift], 0), m.max_pages - 1);     // a bad table must not leave the pool
+    const int64_t off = (int64_t)page * 2 * m.page_elems + ((row & ((1 << m.page_shift) - 1)) * m.hkv + kvh) * 128;
+    *k = m.k_cache + off;
+    *v = m.k_cache + off + m.page_elems;
+  } else {
+    const int64_t off = ((int64_t)kvh * m.seq_stride + row) * 128;
+    *k = m.k_cache + off;
+    *v = m.v_cache + off;
+  }
+  return true;
+}
+inline KvRowMap make_kv_row_map(void* k_cache, void* v_cache, int64_t seq_stride, int64_t hkv, const KvPages* pages) {
+  KvRowMap m{};
+  m.k_cache = (uint16_t*)k_cache;
+  m.v_cache = (uint16_t*)v_cache;
+  m.seq_stride = seq_stride;
+  m.hkv = (int)hkv;
+  if (pages) {
+    int shift = 0;
+    while ((1ll << shift) < pages->page_len) ++shift;
+    m.page_table = pages->table;
+    m.page_shift = shift;
+    m.max_pages = (int)pages->max_pages;
+    m.page_elems = pages->page_len * hkv * 128;
+    m.seq_stride = pages->n_pages * pages->page_len;
+  }
+  return m;
+}
+// subspec_tree_attention (batch 1, head_dim 128) with two options of the decoder-layer entry points: prefix_dev (the
+// kernel reads the prefix length from device memory, prefix_len is its upper bound) and pages (k_cache = one layer of
+// a page pool, v_cache unused)
+int tree_attention_ex(const void* q, const void* k_cache, const void* v_cache, void* out, int dtype, int64_t n_q_heads,
+                      int64_t n_kv_heads, int64_t n_rows, int64_t n_tree_slots, int64_t kv_seq_stride, int64_t prefix_len,
+                      const int64_t* prefix_dev, const KvPages* pages, const uint64_t* anc_bits, float scale, void* workspace,
+                      size_t workspace_bytes, void* stream);
+
 // Linear layers with a fused residual add (y = x W^T + bias + residual; residual may alias y); the C entry points
 // are these with residual = NULL.  Used by the decoder-layer sequence.
 int int4_linear_ex(const void* x, const uint32_t* wq, const uint32_t* sz, const void* bias, const void* residual, void* y,
@@ -220,8 +273,7 @@ int int4_gate_up_silu_ex(const void* x, const uint32_t* wq, const uint32_t* sz, 
 // q to q_out [Hq, M, 128], K / V rows to cache_rows[m] of the layer's [Hkv, seq_stride, 128] caches; optional RMSNorm prologue
 int int4_qkv_rope_ex(const void* x, const uint32_t* wq, const uint32_t* sz, const void* bias, int dtype, int64_t M, int64_t K,
                      const void* norm_gain, float norm_eps, const int32_t* positions, const int32_t* cache_rows, void* q_out,
-                     void* k_cache, void* v_cache, int64_t n_q_heads, int64_t n_kv_heads, int64_t kv_seq_stride,
-                     float rope_theta, const float* inv_freq, void* stream);
+                     const KvRowMap& kv, int64_t n_q_heads, float rope_theta, const float* inv_freq, void* stream);
 int dense_gate_up_silu_ex(const void* x, const void* w, const void* bias, void* act, int dtype, int64_t M, int64_t N,
                           int64_t K, void* stream);
 int dense_linear_ex(const void* x, const void* w, const void* bias, const void* residual, void* y, int dtype, int64_t M,

@@ -94,8 +94,7 @@ __global__ __launch_bounds__(256) void silu_mul_kernel(const uint16_t* __restric
 template <int DT>
 __global__ __launch_bounds__(64) void rope_write_kernel(const uint16_t* __restrict__ qkv, const int32_t* __restrict__ positions,
                                                         const int32_t* __restrict__ cache_rows, uint16_t* __restrict__ q_out,
-                                                        uint16_t* __restrict__ k_cache, uint16_t* __restrict__ v_cache,
-                                                        int M, int Hq, int Hkv, int D, int64_t seq_stride, float log2_theta,
+                                                        KvRowMap kv, int M, int Hq, int Hkv, int D, float log2_theta,
                                                         const float* __restrict__ inv_freq_table) {
   const int m = blockIdx.x, hh = blockIdx.y, i = threadIdx.x;
   const int half = D / 2;
@@ -107,9 +106,9 @@ __global__ __launch_bounds__(64) void rope_write_kernel(const uint16_t* __restri
     dst = q_out + ((int64_t)hh * M + m) * D;
   } else {
     // a row outside the layer's cache is dropped: a bad rows tensor must not write beyond the cache
-    const int64_t row = cache_rows[m];
-    if (row < 0 || row >= seq_stride) return;
-    dst = (hh < Hq + Hkv ? k_cache + (int64_t)(hh - Hq) * seq_stride * D : v_cache + (int64_t)(hh - Hq - Hkv) * seq_stride * D) + row * D;
+    uint16_t *kp, *vp;
+    if (!kv_row_ptrs(kv, (hh - Hq) % Hkv, cache_rows[m], &kp, &vp)) return;
+    dst = hh < Hq + Hkv ? kp : vp;
   }
   if (hh >= Hq + Hkv) {                                 // value heads are copied
     Elem<DT>::store(dst, i, lo);
@@ -177,6 +176,15 @@ static int check_dims(const subspec_decoder_layer_dims* s) {
     SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "decoder_layer: prefix_len=%lld, n_tree_slots=%lld do not fit a cache of %lld rows",
                  (long long)s->prefix_len, (long long)s->n_tree_slots, (long long)s->kv_seq_stride);
   if (!(s->rope_theta > 1.f) || !(s->rms_eps > 0.f)) SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "decoder_layer: rope_theta / rms_eps out of range");
+  if (s->page_indices) {
+    if (s->page_len <= 0 || (s->page_len & (s->page_len - 1)) != 0 || s->page_len > 4096)
+      SUBSPEC_FAIL(SUBSPEC_ERR_LIMIT, "decoder_layer: page_len=%lld must be a power of two up to 4096", (long long)s->page_len);
+    if (s->n_pages <= 0 || s->max_pages < s->n_pages || s->max_pages > 0x7fffffff)
+      SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "decoder_layer: n_pages=%lld max_pages=%lld", (long long)s->n_pages, (long long)s->max_pages);
+    if (s->kv_seq_stride != s->n_pages * s->page_len)
+      SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "decoder_layer: kv_seq_stride=%lld must equal n_pages * page_len = %lld for a paged cache",
+                   (long long)s->kv_seq_stride, (long long)(s->n_pages * s->page_len));
+  }
   return SUBSPEC_OK;
 }
 
@@ -205,6 +213,9 @@ static int run_layer(const subspec_decoder_layer_dims& s, const LayerWeights& w,
   uint16_t *h = (uint16_t*)(ws + p.h), *qkv = (uint16_t*)(ws + p.qkv), *q = (uint16_t*)(ws + p.q), *a = (uint16_t*)(ws + p.a),
            *o = (uint16_t*)(ws + p.o), *gu = (uint16_t*)(ws + p.gu), *act = (uint16_t*)(ws + p.act);
   void* sub = ws + p.sub;
+  const KvPages pages{s.page_indices, s.n_pages, s.max_pages, s.page_len};
+  const KvPages* pg = s.page_indices ? &pages : nullptr;
+  const KvRowMap kv = make_kv_row_map(k_cache, v_cache, s.kv_seq_stride, Hkv, pg);
   int rc;
   // int4 stack, a level of at most 32 rows: five launches per layer (six with a split-K down projection, seven when
   // the keys are split) -- both norms are prologues of the projections that consume them, rotary + cache write is the
@@ -212,17 +223,17 @@ static int run_layer(const subspec_decoder_layer_dims& s, const LayerWeights& w,
   const bool fused = !w.dense && M <= 32 && subspec_int4_linear_workspace(M, Q + 2 * KV, H) == 256;
   if (fused) {
     if ((rc = int4_qkv_rope_ex(x, (const uint32_t*)w.qkv.w, (const uint32_t*)w.qkv.sz, w.qkv_bias, DT, M, H, w.input_norm, s.rms_eps,
-                               positions, cache_rows, q, k_cache, v_cache, Hq, Hkv, s.kv_seq_stride, s.rope_theta, s.rope_inv_freq, st)))
+                               positions, cache_rows, q, kv, Hq, s.rope_theta, s.rope_inv_freq, st)))
       return rc;
   } else {
     hipLaunchKernelGGL((add_rmsnorm_kernel<DT, false>), dim3(M), dim3(kNormThreads), 0, st, x, (const uint16_t*)nullptr,
                        (const uint16_t*)w.input_norm, h, H, s.rms_eps);
     if ((rc = project(w, w.qkv, h, w.qkv_bias, nullptr, qkv, DT, M, Q + 2 * KV, H, sub, p.sub_bytes, st))) return rc;
-    hipLaunchKernelGGL((rope_write_kernel<DT>), dim3(M, Hq + 2 * Hkv), dim3(64), 0, st, qkv, positions, cache_rows, q, k_cache,
-                       v_cache, M, Hq, Hkv, D, s.kv_seq_stride, log2f(s.rope_theta), s.rope_inv_freq);
+    hipLaunchKernelGGL((rope_write_kernel<DT>), dim3(M, Hq + 2 * Hkv), dim3(64), 0, st, qkv, positions, cache_rows, q, kv,
+                       M, Hq, Hkv, D, log2f(s.rope_theta), s.rope_inv_freq);
   }
-  if ((rc = subspec_tree_attention(q, k_cache, v_cache, a, DT, 1, Hq, Hkv, M, s.n_tree_slots, D, s.kv_seq_stride, s.prefix_len,
-                                   anc_bits, 0, 1.f / sqrtf((float)D), sub, p.sub_bytes, st)))
+  if ((rc = tree_attention_ex(q, k_cache, v_cache, a, DT, Hq, Hkv, M, s.n_tree_slots, s.kv_seq_stride, s.prefix_len,
+                              s.prefix_len_dev, pg, anc_bits, 1.f / sqrtf((float)D), sub, p.sub_bytes, st)))
     return rc;
   if (fused) {
     // x = round(round(o_proj(a)) + x), then RMSNorm inside the gate|up projection
@@ -289,7 +300,7 @@ static int decoder_layer_entry(const subspec_decoder_layer_dims* dims, const Lay
                                void* workspace, size_t workspace_bytes, void* stream) {
   const int rc = check_dims(dims);
   if (rc != SUBSPEC_OK) return rc;
-  if (!x || !positions || !cache_rows || !anc_bits || !k_cache || !v_cache)
+  if (!x || !positions || !cache_rows || !anc_bits || !k_cache || (!v_cache && !dims->page_indices))
     SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "decoder_layer: null pointer argument");
   if (!w.input_norm || !w.post_norm || !w.qkv.w || !w.o.w || !w.gate_up.w || !w.down.w ||
       (!w.dense && (!w.qkv.sz || !w.o.sz || !w.gate_up.sz || !w.down.sz)))

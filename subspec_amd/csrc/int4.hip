@@ -172,11 +172,9 @@ struct I4Fused {
   const int32_t* positions;    // [M]
   const int32_t* cache_rows;   // [M]
   uint16_t* q_out;             // [Hq, M, 128]
-  uint16_t* k_cache;           // [Hkv, seq_stride, 128]
-  uint16_t* v_cache;
+  KvRowMap kv;                 // where the K / V rows go (contiguous caches or a page pool)
   const float* inv_freq;       // [64] or null
   int hq, hkv;
-  int64_t seq_stride;
   float log2_theta;
 };
 
@@ -471,13 +469,11 @@ __global__ __launch_bounds__(kI4Threads) void int4_gemm_kernel(
               const float lo = held[mt][rr], hi = Elem<DT>::round(v[rr] + bv);
               const float o_lo = Elem<DT>::round(lo * cs) + Elem<DT>::round(-hi * sn);
               const float o_hi = Elem<DT>::round(hi * cs) + Elem<DT>::round(lo * sn);
-              uint16_t* dst;
+              uint16_t *dst, *unused;
               if (head < fz.hq) {
                 dst = fz.q_out + ((int64_t)head * M + m) * 128;
-              } else {
-                const int64_t row = fz.cache_rows[m];
-                if (row < 0 || row >= fz.seq_stride) continue;   // a row outside the layer's cache is dropped
-                dst = fz.k_cache + ((int64_t)(head - fz.hq) * fz.seq_stride + row) * 128;
+              } else if (!kv_row_ptrs(fz.kv, head - fz.hq, fz.cache_rows[m], &dst, &unused)) {
+                continue;                                        // a row outside the layer's cache is dropped
               }
               Elem<DT>::store(dst, d, o_lo);
               Elem<DT>::store(dst, d + 64, o_hi);
@@ -489,9 +485,8 @@ __global__ __launch_bounds__(kI4Threads) void int4_gemm_kernel(
             for (int rr = 0; rr < 4; ++rr) {
               const int m = mt * 16 + c * 4 + rr;
               if (m >= M) continue;
-              const int64_t row = fz.cache_rows[m];
-              if (row < 0 || row >= fz.seq_stride) continue;
-              uint16_t* dst = fz.v_cache + ((int64_t)kvh * fz.seq_stride + row) * 128;
+              uint16_t *dst, *unused;
+              if (!kv_row_ptrs(fz.kv, kvh, fz.cache_rows[m], &unused, &dst)) continue;
               Elem<DT>::store(dst, d, held[mt][rr]);
               Elem<DT>::store(dst, d + 16, v[rr] + bv);
             }
@@ -701,12 +696,14 @@ int subspec::int4_gate_up_silu_ex(const void* x, const uint32_t* wq, const uint3
 
 int subspec::int4_qkv_rope_ex(const void* x, const uint32_t* wq, const uint32_t* sz, const void* bias, int dtype, int64_t M,
                               int64_t K, const void* norm_gain, float norm_eps, const int32_t* positions,
-                              const int32_t* cache_rows, void* q_out, void* k_cache, void* v_cache, int64_t n_q_heads,
-                              int64_t n_kv_heads, int64_t kv_seq_stride, float rope_theta, const float* inv_freq, void* stream) {
+                              const int32_t* cache_rows, void* q_out, const KvRowMap& kv, int64_t n_q_heads,
+                              float rope_theta, const float* inv_freq, void* stream) {
+  const int64_t n_kv_heads = kv.hkv;
   const int64_t N = (n_q_heads + 2 * n_kv_heads) * 128;
   const int rc = paired_args_ok("int4_qkv_rope", x, wq, sz, dtype, M, N, K);
   if (rc) return rc;
-  if (!positions || !cache_rows || !q_out || !k_cache || !v_cache) SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "int4_qkv_rope: null pointer argument");
+  if (!positions || !cache_rows || !q_out || !kv.k_cache || (!kv.page_table && !kv.v_cache))
+    SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "int4_qkv_rope: null pointer argument");
   if (norm_gain && (uintptr_t)norm_gain % 16) SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "int4_qkv_rope: the norm gain must be 16-byte aligned");
   I4Fused fz{};
   fz.norm_gain = (const uint16_t*)norm_gain;
@@ -714,12 +711,10 @@ int subspec::int4_qkv_rope_ex(const void* x, const uint32_t* wq, const uint32_t*
   fz.positions = positions;
   fz.cache_rows = cache_rows;
   fz.q_out = (uint16_t*)q_out;
-  fz.k_cache = (uint16_t*)k_cache;
-  fz.v_cache = (uint16_t*)v_cache;
+  fz.kv = kv;
   fz.inv_freq = inv_freq;
   fz.hq = (int)n_q_heads;
   fz.hkv = (int)n_kv_heads;
-  fz.seq_stride = kv_seq_stride;
   fz.log2_theta = log2f(rope_theta);
   if (dtype == SUBSPEC_BF16) return run_int4_paired<SUBSPEC_BF16, kEpiRope>(x, wq, sz, bias, nullptr, M, N, K, fz, (hipStream_t)stream);
   return run_int4_paired<SUBSPEC_F16, kEpiRope>(x, wq, sz, bias, nullptr, M, N, K, fz, (hipStream_t)stream);

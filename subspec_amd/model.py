@@ -151,8 +151,9 @@ class Decoder:
         per layer instead of one per module): every layer int4-packed, or every layer dense 16-bit."""
         if self._native is None:
             packed = [("qkv_proj.wq" in w) for w in self.layers]
+            # either cache layout: contiguous per-layer caches, or the page pool (rows written and read through the table)
             self._native = (bool(self.layers) and (all(packed) or not any(packed)) and self.dtype != torch.float32
-                            and self.kv.cache.contiguous)
+                            and (self.kv.cache.contiguous or hasattr(self.kv.cache, "pool")))
             if self._native:
                 make = ops.decoder_layer_weights if packed[0] else ops.dense_layer_weights
                 self._native_make = make
@@ -161,12 +162,23 @@ class Decoder:
                 self._native_ws = {}
         return self._native
 
-    def _run_native_layers(self, x, positions, rows, anc_bits, prefix_len: int, slots: int) -> torch.Tensor:
+    def _run_native_layers(self, x, positions, rows, anc_bits, prefix_len: int, slots: int,
+                           prefix_len_dev: Optional[torch.Tensor] = None) -> torch.Tensor:
         cfg, cache = self.cfg, self.kv.cache
         n = x.shape[0]
+        paged = not cache.contiguous
+        if paged:
+            table = cache.table()
+            paging = dict(page_indices=table, max_pages=cache.pool.max_pages, page_len=cache.page_len)
+            stride = table.numel() * cache.page_len
+            layer_kv = lambda i: (cache.pool.cache_data[i], cache.pool.cache_data[i])
+        else:
+            paging, stride = {}, cache.max_cache_len
+            layer_kv = lambda i: (cache.k(i), cache.v(i))
         dims = ops.decoder_layer_dims(self.dtype, n, cfg.hidden_size, cfg.intermediate_size, cfg.num_attention_heads,
-                                      cfg.num_key_value_heads, cfg.head_dim, cache.max_cache_len, int(prefix_len),
-                                      int(slots), cfg.rms_norm_eps, cfg.rope_theta, self._inv_freq)
+                                      cfg.num_key_value_heads, cfg.head_dim, stride, int(prefix_len),
+                                      int(slots), cfg.rms_norm_eps, cfg.rope_theta, self._inv_freq,
+                                      prefix_len_dev=prefix_len_dev, **paging)
         need = ops.decoder_layer_workspace(dims)
         ws = self._native_ws.get("ws")
         if ws is None or ws.numel() < need:
@@ -175,12 +187,12 @@ class Decoder:
         pos32, rows32 = positions.to(torch.int32), rows.to(torch.int32)
         bits = anc_bits.to(torch.int64).contiguous()
         for i, w in enumerate(self._native_weights):
-            ops.decoder_layer_(x, dims, w, pos32, rows32, bits, cache.k(i), cache.v(i), ws)
+            ops.decoder_layer_(x, dims, w, pos32, rows32, bits, *layer_kv(i), ws)
         if self.streamer is not None and self.streamer.n:
             base = self.first_streamed
 
             def step(j, w):                       # w: views into the device slab that holds layer base + j right now
-                ops.decoder_layer_(x, dims, self._native_make(w), pos32, rows32, bits, cache.k(base + j), cache.v(base + j), ws)
+                ops.decoder_layer_(x, dims, self._native_make(w), pos32, rows32, bits, *layer_kv(base + j), ws)
 
             self.streamer.run(step)
         return x

@@ -411,9 +411,14 @@ def temperature_warp(logits: torch.Tensor, temperature: float) -> torch.Tensor:
 
 def decoder_layer_dims(dtype: torch.dtype, n_rows: int, hidden: int, intermediate: int, n_q_heads: int, n_kv_heads: int,
                        head_dim: int, kv_seq_stride: int, prefix_len: int, n_tree_slots: int, rms_eps: float,
-                       rope_theta: float, rope_inv_freq: Optional[torch.Tensor] = None) -> "L.DecoderLayerDims":
+                       rope_theta: float, rope_inv_freq: Optional[torch.Tensor] = None,
+                       prefix_len_dev: Optional[torch.Tensor] = None, page_indices: Optional[torch.Tensor] = None,
+                       max_pages: int = 0, page_len: int = 0) -> "L.DecoderLayerDims":
     """``rope_inv_freq``: float32 device tensor [head_dim / 2] (kept alive by the caller) with the inverse frequencies
-    the caller's eager rotary uses; without it the kernel evaluates ``rope_theta ** (-2i / head_dim)`` itself."""
+    the caller's eager rotary uses; without it the kernel evaluates ``rope_theta ** (-2i / head_dim)`` itself.
+    ``prefix_len_dev``: int64 device tensor of one element that holds the prefix length when the kernels run
+    (``prefix_len`` is then its upper bound): layer calls captured into a graph.  ``page_indices``: int32 device page
+    table of a paged cache (``k_cache`` of the layer call = one layer of the pool, ``kv_seq_stride`` = pages * page_len)."""
     code = {torch.bfloat16: L.BF16, torch.float16: L.F16}.get(dtype)
     if code is None:
         raise ValueError(f"decoder layer: dtype {dtype} not supported (bf16 / fp16 only)")
@@ -423,8 +428,19 @@ def decoder_layer_dims(dtype: torch.dtype, n_rows: int, hidden: int, intermediat
                 or not rope_inv_freq.is_contiguous():
             raise ValueError("decoder layer: rope_inv_freq must be a contiguous float32 device tensor of head_dim / 2 elements")
         table = rope_inv_freq.data_ptr()
+    dyn = None
+    if prefix_len_dev is not None:
+        if prefix_len_dev.dtype != torch.int64 or prefix_len_dev.numel() != 1 or not prefix_len_dev.is_cuda:
+            raise ValueError("decoder layer: prefix_len_dev must be an int64 device tensor of one element")
+        dyn = prefix_len_dev.data_ptr()
+    pages, n_pages = None, 0
+    if page_indices is not None:
+        if page_indices.dtype != torch.int32 or not page_indices.is_cuda or not page_indices.is_contiguous():
+            raise ValueError("decoder layer: page_indices must be a contiguous int32 device tensor")
+        pages, n_pages = page_indices.data_ptr(), page_indices.numel()
     return L.DecoderLayerDims(code, 0, n_rows, hidden, intermediate, n_q_heads, n_kv_heads, head_dim, kv_seq_stride,
-                              prefix_len, n_tree_slots, rms_eps, rope_theta, table)
+                              prefix_len, n_tree_slots, rms_eps, rope_theta, table, dyn, pages, n_pages, int(max_pages),
+                              int(page_len))
 
 
 def decoder_layer_weights(w: dict) -> "L.DecoderLayerWeights":

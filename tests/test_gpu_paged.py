@@ -135,11 +135,13 @@ def test_request_cache_cycle_matches_static_cache():
 
 @pytest.mark.parametrize("depth,topk", [(5, 4), (20, 6)])          # 21-node trees; 121-node trees (two mask words, row windows)
 @pytest.mark.parametrize("driver", ["v1", "v2"])
-def test_speculative_cycle_over_the_paged_cache_equals_the_static_cache(driver, depth, topk):
+@pytest.mark.parametrize("native", [False, True])
+def test_speculative_cycle_over_the_paged_cache_equals_the_static_cache(driver, depth, topk, native):
     """The whole cycle (prefill, draft levels, target window, verification, compaction) over a page pool whose pages
-    were handed out in scrambled order, against the same models over the contiguous cache.  Both runs go module by
-    module (the one-call layers take contiguous caches only), so the cache layout is the only difference and
-    tokens and cached K / V must agree bit for bit."""
+    were handed out in scrambled order, against the same models over the contiguous cache.  Both runs go the same way
+    -- module by module, or through the one-call decoder layers, which write the rotated rows and read the keys
+    through the page table --, so the cache layout is the only difference and tokens and cached K / V must agree bit
+    for bit."""
     from subspec_amd.cache import create_kv_cache
     from subspec_amd.draft import SubSpecSDDraftModel
     from subspec_amd.generator import SubSpecSDGenerator
@@ -159,7 +161,8 @@ def test_speculative_cycle_over_the_paged_cache_equals_the_static_cache(driver, 
             pool.deallocate(held[::2])                            # gaps in what the pool hands out later, and the
             kv.cache.request.kv_page_indices.extend(reversed(pool.allocate(3)))   # first three logical pages backwards
         target, draft, _ = build_models(cfg, kv, device=DEV, weights=w)
-        target.use_native_layers = draft.use_native_layers = False
+        target.use_native_layers = draft.use_native_layers = native
+        assert target.native_layers and draft.native_layers       # both layouts qualify for the one-call layers
         cls, extra = (SubSpecSDGenerator, {}) if driver == "v1" else (SubSpecSDGeneratorV2, dict(postspec_steps=2))
         gen = cls(target, None, SubSpecSDDraftModel(draft), DraftParams(temperature=0.2, max_depth=depth, topk_len=topk),
                   cache_implementation=impl, generator_kwargs=dict(verify_method="exact", **extra))
