@@ -75,6 +75,8 @@ def parse():
     ap.add_argument("--hqq-optimize", action="store_true",
                     help="e2e workload: refine the draft's zero points with hqq's proximal solver (what the reference's "
                          "quantizer does by default; worth it for real weights, --checkpoint)")
+    ap.add_argument("--draft-graph", action="store_true",
+                    help="e2e workload: replay each speculation (all draft levels) from a captured HIP graph")
     ap.add_argument("--keep-layers", type=int, default=14, help="e2e workload: target layers kept resident; the rest stream")
     ap.add_argument("--workload", default="verify-cycle", choices=["verify-cycle", "attention", "int4", "dense", "greedy", "sampling", "e2e"],
                     help="verify-cycle (default, BASELINE config 2) is the benchmark line; the others time one "
@@ -267,7 +269,7 @@ def e2e_runs(args, runs, new_tokens, say=lambda *_: None):
             gen = (SubSpecSDGeneratorV2 if v2 else SubSpecSDGenerator)(
                 target, None, SubSpecSDDraftModel(draft),
                 DraftParams(temperature=0.2, max_depth=depth, topk_len=args.tree_k, max_verify_tokens=cap),
-                generator_kwargs=dict(verify_method=method, verify_kwargs=vk,
+                generator_kwargs=dict(verify_method=method, verify_kwargs=vk, draft_graph=bool(getattr(args, "draft_graph", False)),
                                       **(dict(postspec_steps=args.postspec_steps) if v2 else {})))
             kv.reset()
             wandb_logger.clear_log_data()
@@ -288,7 +290,8 @@ def e2e_runs(args, runs, new_tokens, say=lambda *_: None):
                                        + f", int4 draft, depth {depth}, k {args.tree_k}, "
                                        + (f"<={cap} nodes" if cap else f"{1 + depth * args.tree_k} nodes") + f", prompt 2048, {new_tokens} new tokens, verify {method}"
                                        + (", post-speculating driver" if v2 else ""),
-                           "verify_method": method, "generator": args.generator, "resident_target_layers": min(keep_layers, cfg.num_hidden_layers),
+                           "verify_method": method, "generator": args.generator,
+                           "draft_graph_replays": gen.draft_model.graph_replays, "resident_target_layers": min(keep_layers, cfg.num_hidden_layers),
                            "agreeing_draft": bool(agreeing),
                            **({"post_verify_count": log["post_verify_count"], "speculate_count": log["speculate_count"]} if v2 else {}), "n_iter": log["n_iter"], "n_tokens": log["n_tokens"],
                            "tokens_per_cycle": round(log["avg_sampled"], 3),

@@ -41,6 +41,15 @@ class SubSpecSDDraftModel:
         self.past_key_values = None
         self.had_first_speculate = False
         self.postspec_count = 0
+        # Graph replay of speculate(): the reference captures its draft step into a CUDA graph with device-side
+        # positions (draft_models/subspec_sd_fi.py:65-179); here ALL levels of one speculation are one captured graph
+        # per prefix bucket, replayed with the prefix length in device memory.  Off unless asked for.
+        self.capture_graphs = False
+        self.graph_bucket = 256                   # a graph serves prefixes up to the next multiple of this
+        self.graph_warmup = 2                     # eager speculations before the first capture (library handles, tables)
+        self._graphs = {}
+        self._eager_speculations = 0
+        self.graph_replays = 0
 
     @classmethod
     def from_pretrained(cls, pretrained_model_name_or_path=None, *model_args, target_model=None,
@@ -95,22 +104,75 @@ class SubSpecSDDraftModel:
         the tree must not, because the draft's level state describes the uncut level)."""
         assert input_ids.shape == (1, 1), "the root of the tree is a single token"
         self.had_first_speculate = True
-        p = self.draft_params
         dev = self.decoder.device
         self.prefix_len = int(self.past_key_values.get_seq_length())
-        logits = self.decoder.tree_forward(input_ids[0].to(dev), torch.zeros(1, dtype=torch.long, device=dev),
-                                         torch.ones(1, dtype=torch.int64, device=dev), self.prefix_len)
         self.tree = Tree(input_ids[0, -1], self.decoder.dtype)
+        bound = self._graph_bound() if self.capture_graphs else None
+        if bound is None or self._eager_speculations < self.graph_warmup:
+            self._eager_speculations += 1
+            self._grow_levels(input_ids[0].to(dev), self.prefix_len, None)
+        else:
+            self._replay_levels(input_ids[0].to(dev), bound)
+        return self.update_tree(cap=cap)
+
+    def _grow_levels(self, root: torch.Tensor, prefix_len: int, prefix_len_dev: Optional[torch.Tensor]) -> None:
+        """All levels of one speculation, device work only (nothing is read back): the root's forward, then
+        ``max_depth - 1`` tree steps.  With ``prefix_len_dev`` no launch depends on the actual prefix length."""
+        dev = self.decoder.device
+        self._prefix_len_dev, self._prefix_bound = prefix_len_dev, prefix_len
+        logits = self.decoder.tree_forward(root, torch.zeros(1, dtype=torch.long, device=dev),
+                                           torch.ones(1, dtype=torch.int64, device=dev), prefix_len,
+                                           prefix_len_dev=prefix_len_dev)
         self.levels = []
         self.level_state = {}                                                      # depth -> what speculate_once needs
-        self.level_bits = torch.zeros((1, MASK_WORDS), dtype=torch.int64, device=dev)
-        self.level_bits[0, 0] = 1                                                  # root: slot 0
+        self.level_bits = self._own_bits(dev)[0:1].clone()                         # root: slot 0 (no host value involved)
         self.next_slot = 1
         self.depth = 0
         self._expand(self._probs(logits).unsqueeze(0), torch.ones((1, 1), device=dev, dtype=logits.dtype))
-        for _ in range(p.max_depth - 1):
+        for _ in range(self.draft_params.max_depth - 1):
             self.speculate_once()
-        return self.update_tree(cap=cap)
+        self._prefix_len_dev = None
+
+    # ------------------------------------------------------------------ graph replay
+    _STATE = ("levels", "level_state", "level_bits", "next_slot", "first_slot", "depth", "token_ids", "parent_probs")
+
+    def _graph_bound(self) -> Optional[int]:
+        """Upper bound of the prefix length the graph for the current prefix is laid out for, or None when this
+        speculation cannot be replayed from a graph (cache that may move or is paged, layers not one-call, tree wider
+        than a launch window, no room left in the cache)."""
+        dec, p = self.decoder, self.draft_params
+        cache = dec.kv.cache
+        slots = 1 + (p.max_depth - 1) * p.topk_len
+        if cache.growable or not cache.contiguous or not (dec.use_native_layers and dec.native_layers):
+            return None
+        if p.topk_len > 64 or slots > MAX_SLOTS:
+            return None
+        bound = (self.prefix_len // self.graph_bucket + 1) * self.graph_bucket
+        bound = min(bound, cache.max_cache_len - slots)
+        return bound if bound >= self.prefix_len else None
+
+    def _replay_levels(self, root: torch.Tensor, bound: int) -> None:
+        key = (bound, self.draft_params.max_depth, self.draft_params.topk_len, float(self.draft_params.temperature))
+        entry = self._graphs.get(key)
+        if entry is None:
+            dev = self.decoder.device
+            self._own_bits(dev)                                                    # tables are built outside the capture
+            self.decoder.kv.cache.ensure(bound + 1 + (self.draft_params.max_depth - 1) * self.draft_params.topk_len)
+            entry = {"root": torch.zeros(1, dtype=torch.long, device=dev),
+                     "prefix": torch.zeros(1, dtype=torch.int64, device=dev), "graph": torch.cuda.CUDAGraph()}
+            entry["root"].copy_(root)
+            entry["prefix"].fill_(self.prefix_len)
+            torch.cuda.synchronize()
+            with torch.cuda.graph(entry["graph"]):
+                self._grow_levels(entry["root"], bound, entry["prefix"])
+            entry["state"] = {name: getattr(self, name) for name in self._STATE}
+            self._graphs[key] = entry
+        entry["root"].copy_(root)
+        entry["prefix"].fill_(self.prefix_len)
+        entry["graph"].replay()
+        self.graph_replays += 1
+        for name, value in entry["state"].items():                                 # what the eager code leaves on the host
+            setattr(self, name, dict(value) if isinstance(value, dict) else list(value) if isinstance(value, list) else value)
 
     def _own_bits(self, device) -> torch.Tensor:
         """Row s: the mask words with only the bit of slot s set (word s // 64, bit s % 64; bit 63 is the sign bit of
@@ -147,8 +209,11 @@ class SubSpecSDDraftModel:
             raise ValueError(f"draft tree exceeds the {MAX_SLOTS} tree slots of the attention mask")
         depths = torch.full((n,), self.depth, dtype=torch.long, device=dev)
         bits = self.level_bits[:, 0].contiguous() if total <= 64 else self.level_bits[:, :(total + 63) // 64].contiguous()
-        logits = self.decoder.tree_forward(self.token_ids[0], depths, bits, self.prefix_len,
-                                         first_slot=self.first_slot)
+        dyn = getattr(self, "_prefix_len_dev", None)
+        # inside _grow_levels the prefix length may live on the device; prefix_len is then the bound the launches use
+        logits = self.decoder.tree_forward(self.token_ids[0], depths, bits,
+                                           self._prefix_bound if dyn is not None else self.prefix_len,
+                                           first_slot=self.first_slot, prefix_len_dev=dyn)
         self._expand(self._probs(logits).unsqueeze(0), self.parent_probs)
 
     def update_tree(self, cap: bool = False) -> Tree:

@@ -42,6 +42,8 @@ class SubSpecSDGenerator:
         self.prefill_chunk_size = self.generator_kwargs.get("prefill_chunk_size", None)
         self.eos_token_id = eos_token_id if eos_token_id is not None else getattr(tokenizer, "eos_token_id", None)
         self.draft_model.eos_token_id = self.eos_token_id
+        if "draft_graph" in self.generator_kwargs:       # replay each speculation from a captured graph (static cache)
+            self.draft_model.capture_graphs = bool(self.generator_kwargs["draft_graph"])
         # Philox stream of the sampling target; generator_kwargs["seed"] fixes it, else torch's seed
         self.sample_stream = SampleStream(self.generator_kwargs.get("seed"))
         self._stop_strings = None                # HuggingFace StopStringCriteria of the current generate() call

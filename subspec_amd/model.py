@@ -261,21 +261,34 @@ class Decoder:
         return self.logits(x if all_logits else x[-1:])
 
     def tree_forward(self, token_ids: torch.Tensor, depths: torch.Tensor, anc_bits: torch.Tensor, prefix_len: int,
-                     first_slot: int = 0, n_tree_slots: Optional[int] = None) -> torch.Tensor:
+                     first_slot: int = 0, n_tree_slots: Optional[int] = None,
+                     prefix_len_dev: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Forward of tree nodes occupying cache rows prefix_len+first_slot.. ; ``depths`` are the node
         depths (rotary position = prefix_len + depth), ``anc_bits`` int64 [n] bitsets over tree
         slots ([n, ceil(slots / 64)] words above 64 slots).  Up to 64 rows go through the one-call layers; a larger
         window (a whole large tree in the target) runs module by module, so that every weight matrix is read once
-        for all rows (library GEMMs) and only attention is split into launches of 64 rows.  Returns logits [n, V]."""
+        for all rows (library GEMMs) and only attention is split into launches of 64 rows.  Returns logits [n, V].
+
+        ``prefix_len_dev`` (int64 device tensor of one element): the prefix length is taken from the device when the
+        kernels run and ``prefix_len`` is only its upper bound -- nothing on the host side depends on the actual
+        value, so the call can be captured into a graph and replayed as the sequence grows (one-call layers only)."""
         n = token_ids.numel()
         slots = first_slot + n if n_tree_slots is None else n_tree_slots
         self.kv.cache.ensure(prefix_len + max(slots, first_slot + n))
         self._rope_tables(prefix_len + max(slots, first_slot + n) + 8)
-        positions = depths.to(self.device) + prefix_len
-        rows = torch.arange(prefix_len + first_slot, prefix_len + first_slot + n, device=self.device)
         cfg = self.cfg
-        if self.use_native_layers and self.native_layers and n <= 64 and slots <= ops.L.MAX_TREE_NODES:
-            return self.logits(self._run_native_layers(self.embed[token_ids], positions, rows, anc_bits, prefix_len, slots))
+        native = self.use_native_layers and self.native_layers and n <= 64 and slots <= ops.L.MAX_TREE_NODES
+        if prefix_len_dev is not None:
+            if not native:
+                raise ValueError("a device-side prefix length needs the one-call decoder layers (at most 64 rows)")
+            positions = depths.to(self.device) + prefix_len_dev
+            rows = torch.arange(first_slot, first_slot + n, device=self.device) + prefix_len_dev
+        else:
+            positions = depths.to(self.device) + prefix_len
+            rows = torch.arange(prefix_len + first_slot, prefix_len + first_slot + n, device=self.device)
+        if native:
+            return self.logits(self._run_native_layers(self.embed[token_ids], positions, rows, anc_bits, prefix_len, slots,
+                                                       prefix_len_dev=prefix_len_dev))
 
         def attn(i, q):
             return self.kv.cache.tree_attention(i, q, anc_bits, prefix_len, slots).reshape(n, cfg.q_size)
