@@ -156,7 +156,7 @@ def bench_attention(args):
         copies = max(2, COLD_BYTES // (2 * B * 4 * 4160 * 128 * 2) + 1)
         ks = [torch.randn(B, 4, 4160, 128, device=dev).to(torch.bfloat16) for _ in range(copies)]
         vs = [torch.randn(B, 4, 4160, 128, device=dev).to(torch.bfloat16) for _ in range(copies)]
-        need = ops.L.lib().subspec_tree_attention_workspace(B, 28, 4096, 64)
+        need = ops.L.lib().subspec_tree_attention_workspace(B, 28, 4, 64, 4096, 64)
         ws = torch.empty(max(need, 256), dtype=torch.uint8, device=dev)
         call_us, kernel_us = _time_us(_rotating(lambda i: ops.tree_attention(q, ks[i], vs[i], anc, 4096, workspace=ws), copies),
                                       max(args.steps, copies), args.warmup)
@@ -172,7 +172,7 @@ def bench_attention(args):
     layer = torch.randn(max_pages, 2, page_len, 4, 128, device=dev).to(torch.bfloat16)
     pages = torch.randperm(max_pages, device=dev)[:n_pages].to(torch.int32)
     q = torch.randn(1, 28, 64, 128, device=dev).to(torch.bfloat16)
-    need = ops.L.lib().subspec_tree_attention_workspace(1, 28, 4096, 64)
+    need = ops.L.lib().subspec_tree_attention_workspace(1, 28, 4, 64, 4096, 64)
     ws = torch.empty(max(need, 256), dtype=torch.uint8, device=dev)
     call_us, kernel_us = _time_us(lambda: ops.tree_attention_paged(q, layer, pages, anc, 4096, workspace=ws), args.steps, args.warmup)
     _kernel_line("tree-masked GQA attention latency, paged KV", "config 3 shape, B=1, KV pool [300,2,16,4,128] bf16, shuffled pages",

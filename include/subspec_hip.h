@@ -222,7 +222,8 @@ int subspec_topk_expand(const void* probs, const void* parent_probs, int dtype, 
  *            j % 64 of word j / 64); batch element b uses rows from b * anc_batch_stride (0: shared tree)
  * workspace  partial results when the keys are split over workgroups (may be NULL if the size is 256)
  */
-size_t subspec_tree_attention_workspace(int64_t batch, int64_t n_q_heads, int64_t prefix_len, int64_t n_tree_slots);
+size_t subspec_tree_attention_workspace(int64_t batch, int64_t n_q_heads, int64_t n_kv_heads, int64_t n_rows,
+                                        int64_t prefix_len, int64_t n_tree_slots);
 
 int subspec_tree_attention(const void* q, const void* k_cache, const void* v_cache, void* out, int dtype,
                            int64_t batch, int64_t n_q_heads, int64_t n_kv_heads, int64_t n_rows,
@@ -247,7 +248,7 @@ int subspec_tree_attention(const void* q, const void* k_cache, const void* v_cac
  *   flashinfer.BatchPrefillWithPagedKVCacheWrapper.run with custom_mask (mode "tree")
  *           specdecodes/models/utils/flashinfer/attention_wrapper.py:104-137 and its forward call
  * kv_pool_layer = one layer of the pool; every other argument as in subspec_tree_attention (batch 1,
- * workspace = subspec_tree_attention_workspace(1, n_q_heads, prefix_len, n_tree_slots)).
+ * workspace = subspec_tree_attention_workspace(1, n_q_heads, n_kv_heads, n_rows, prefix_len, n_tree_slots)).
  *
  * subspec_kv_compact_paged replaces
  *   KvCachePool.reorder_cache_with_offset (clone of every layer, index_select / index_copy_, copy back)

@@ -64,7 +64,7 @@ _SIGNATURES = {
                                              _p, _sz, _p, _p, _p, _p, _p, _p, _p]),
     "subspec_topk_expand_workspace": (_sz, [_i64, _i64, _i64, _i32]),
     "subspec_topk_expand": (C.c_int, [_p, _p, C.c_int, _i64, _i64, _i64, _i32, _p, _sz, _p, _p, _p, _p]),
-    "subspec_tree_attention_workspace": (_sz, [_i64, _i64, _i64, _i64]),
+    "subspec_tree_attention_workspace": (_sz, [_i64, _i64, _i64, _i64, _i64, _i64]),
     "subspec_tree_attention": (C.c_int, [_p, _p, _p, _p, C.c_int, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _p, _i64,
                                          C.c_float, _p, _sz, _p]),
     "subspec_tree_attention_paged": (C.c_int, [_p, _p, _p, _i64, _i64, _i64, _p, C.c_int, _i64, _i64, _i64, _i64, _i64, _i64, _p,

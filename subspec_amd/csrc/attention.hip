@@ -37,7 +37,7 @@
 
 namespace subspec {
 
-constexpr int kAttnThreads = 512;
+constexpr int kAttnThreads = 512;         // 256 for the one-head shape
 constexpr int kAttnRows = 64;          // query rows per head
 constexpr int kAttnD = 128;
 constexpr int kKeyBlock = 64;
@@ -101,8 +101,11 @@ struct AttnParams {
   int64_t page_stride, tok_stride, v_delta;   // elements
 };
 
-template <int DT, bool PAGED, int ROWT, int WPH>
-__global__ __launch_bounds__(kAttnThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void tree_attention_kernel(
+// THREADS = 512: eight wavefronts; 256: four wavefronts, each 16 rows of ONE head (ROWT = 1, WPH = 4) -- with 33 to 64
+// query rows and few sequences this shape gets its workgroups from the heads instead of from key chunks, so the
+// split-KV partials (fp32, rows x 128 per head and chunk) stay below the K / V bytes themselves.
+template <int DT, bool PAGED, int ROWT, int WPH, int THREADS = kAttnThreads>
+__global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2))) void tree_attention_kernel(
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ kc, const uint16_t* __restrict__ vc,
     const uint64_t* __restrict__ anc, AttnParams ap, uint16_t* __restrict__ out, float* __restrict__ part_o,
     float* __restrict__ part_ml) {
@@ -124,7 +127,7 @@ __global__ __launch_bounds__(kAttnThreads) __attribute__((amdgpu_waves_per_eu(2,
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int lq = lane & 15, lg = lane >> 4;            // query column of the lane, lane group
-  constexpr int kHeadsPerWG = 8 / WPH;                 // heads of one KV head that share a workgroup's K / V stages
+  constexpr int kHeadsPerWG = (THREADS / 64) / WPH;    // heads of one KV head that share a workgroup's K / V stages
   const int head_in_group = pair * kHeadsPerWG + wave / WPH;
   const bool head_ok = head_in_group < group;
   const int qh = kvh * group + (head_ok ? head_in_group : 0);
@@ -178,25 +181,42 @@ __global__ __launch_bounds__(kAttnThreads) __attribute__((amdgpu_waves_per_eu(2,
   // block; the next block is requested as soon as the current one sits in LDS, so the request
   // travels while the current block is multiplied.  Plain scalars on purpose: arrays captured by
   // a lambda end up in memory and every prefetch would be waited for at once.
-  uint4 k0, k1, v0, v1;
-  const int skey = tid >> 4, sdc = tid & 15;           // this thread stages keys skey, skey + 32, d-chunk sdc
+  constexpr int KPT = 1024 / THREADS;                  // keys of a block per thread: 2 (512 threads) or 4 (256)
+  constexpr int KSTEP = 64 / KPT;
+  uint4 k0, k1, k2, k3, v0, v1, v2, v3;
+  (void)k2; (void)k3; (void)v2; (void)v3;
+  const int skey = tid >> 4, sdc = tid & 15;           // this thread stages keys skey + KSTEP * i, d-chunk sdc
 #define SUBSPEC_ATTN_FETCH(KB)                                                                   \
   do {                                                                                           \
     const int64_t p0_ = row_offset(min((KB) + skey, kv_len - 1));                                \
-    const int64_t p1_ = row_offset(min((KB) + 32 + skey, kv_len - 1));                           \
+    const int64_t p1_ = row_offset(min((KB) + KSTEP + skey, kv_len - 1));                        \
     k0 = *(const uint4*)(kbase + p0_ + sdc * 8);                                                 \
     k1 = *(const uint4*)(kbase + p1_ + sdc * 8);                                                 \
     v0 = *(const uint4*)(vbase + p0_ + sdc * 8);                                                 \
     v1 = *(const uint4*)(vbase + p1_ + sdc * 8);                                                 \
+    if constexpr (KPT == 4) {                                                                    \
+      const int64_t p2_ = row_offset(min((KB) + 2 * KSTEP + skey, kv_len - 1));                  \
+      const int64_t p3_ = row_offset(min((KB) + 3 * KSTEP + skey, kv_len - 1));                  \
+      k2 = *(const uint4*)(kbase + p2_ + sdc * 8);                                               \
+      k3 = *(const uint4*)(kbase + p3_ + sdc * 8);                                               \
+      v2 = *(const uint4*)(vbase + p2_ + sdc * 8);                                               \
+      v3 = *(const uint4*)(vbase + p3_ + sdc * 8);                                               \
+    }                                                                                            \
   } while (0)
 #define SUBSPEC_ATTN_STAGE(BUF)                                                                  \
   do {                                                                                           \
     uint16_t* ksw_ = Ks2[BUF];                                                                   \
     uint16_t* vsw_ = Vs2[BUF];                                                                   \
     *(uint4*)(ksw_ + skey * kKStride + sdc * 8) = k0;                                            \
-    *(uint4*)(ksw_ + (skey + 32) * kKStride + sdc * 8) = k1;                                     \
+    *(uint4*)(ksw_ + (skey + KSTEP) * kKStride + sdc * 8) = k1;                                  \
     *(uint4*)(vsw_ + skey * kVStride + sdc * 8) = v0;                                            \
-    *(uint4*)(vsw_ + (skey + 32) * kVStride + sdc * 8) = v1;                                     \
+    *(uint4*)(vsw_ + (skey + KSTEP) * kVStride + sdc * 8) = v1;                                  \
+    if constexpr (KPT == 4) {                                                                    \
+      *(uint4*)(ksw_ + (skey + 2 * KSTEP) * kKStride + sdc * 8) = k2;                            \
+      *(uint4*)(ksw_ + (skey + 3 * KSTEP) * kKStride + sdc * 8) = k3;                            \
+      *(uint4*)(vsw_ + (skey + 2 * KSTEP) * kVStride + sdc * 8) = v2;                            \
+      *(uint4*)(vsw_ + (skey + 3 * KSTEP) * kVStride + sdc * 8) = v3;                            \
+    }                                                                                            \
   } while (0)
 
   // mask words of the first block of this chunk that reaches into the tree (none does: the loads are harmless)
@@ -398,24 +418,66 @@ __global__ __launch_bounds__(256) void tree_attention_merge_kernel(
   *(uint2*)(out + (((int64_t)b * ap.n_rows + ap.row0 + row) * ap.hq + qh) * kAttnD + d4 * 4) = packed;
 }
 
-static int attn_chunks(int64_t batch, int64_t hq, int64_t kv_len) {
+// Launch shape of one window of query rows.
+struct AttnPlan { int threads, rowt, wph, heads_per_wg, chunks; };
+static AttnPlan attn_plan(int64_t batch, int64_t hq, int64_t hkv, int64_t win_rows, int64_t kv_len) {
+  AttnPlan pl;
+  const int group = (int)(hq / hkv);
   const int64_t blocks = (kv_len + kKeyBlock - 1) / kKeyBlock;
-  // aim at roughly one workgroup per compute unit
-  int64_t chunks = std::max<int64_t>(1, 1024 / std::max<int64_t>(1, batch * hq));
-  chunks = std::min<int64_t>(chunks, std::max<int64_t>(1, blocks / 2));   // at least 128 keys per chunk
-  return (int)std::min<int64_t>(chunks, 64);
+  if (win_rows <= 32) {
+    // a draft level: a wavefront is a whole head, eight heads share the staged keys
+    pl.threads = 512; pl.rowt = win_rows <= 16 ? 1 : 2; pl.wph = 1;
+  } else if (batch * hq >= 128) {
+    // 33 to 64 rows, many (sequence, head) pairs: four heads share the staged keys (two wavefronts of 32 rows per head);
+    // the LDS traffic per head is less than half that of the one-head shape, which is what bounds this case
+    pl.threads = 512; pl.rowt = 2; pl.wph = 2;
+  } else {
+    // 33 to 64 rows, few sequences: one head per 256-thread workgroup, so that the workgroups come from the heads
+    // and not from key chunks whose partial results would outweigh the keys
+    pl.threads = 256; pl.rowt = 1; pl.wph = 4;
+  }
+  pl.heads_per_wg = (pl.threads / 64) / pl.wph;
+  const int64_t wgs_per_chunk = batch * hkv * ((group + pl.heads_per_wg - 1) / pl.heads_per_wg);
+  // enough workgroups to cover the chip once, at least two key blocks per chunk ...
+  // enough workgroups to cover the chip once (three times with the small one-head workgroups, two or three of which
+  // share a compute unit), at least two key blocks per chunk ...
+  const int64_t target_wgs = pl.threads == 256 ? 768 : 256;
+  int64_t chunks = std::max<int64_t>(1, (target_wgs + wgs_per_chunk - 1) / wgs_per_chunk);
+  if (win_rows <= 32) chunks = std::max<int64_t>(chunks, 1024 / std::max<int64_t>(1, batch * hq));   // few rows: short chunks, latency first
+  chunks = std::min<int64_t>(chunks, std::max<int64_t>(1, blocks / 2));
+  // ... and the partial results (fp32 rows x 128 per head and chunk) are priced against the K / V bytes (16-bit,
+  // 2 x kv_len x 128 per KV head): at most twice as many (config 3, one sequence: 29 MB of partials for 8.5 MB of keys
+  // before, 16.6 MB now; the same bytes again are read by the merge)
+  const int64_t by_bytes = std::max<int64_t>(1, 2 * (kv_len * hkv) / std::max<int64_t>(1, hq * win_rows));
+  chunks = std::min<int64_t>(chunks, by_bytes);
+  pl.chunks = (int)std::min<int64_t>(chunks, 64);
+  return pl;
+}
+// the most partial slots any window of a call can need (the first window is the largest)
+static int attn_chunks_bound(int64_t batch, int64_t hq, int64_t hkv, int64_t n_rows, int64_t kv_len) {
+  int c = 1;
+  for (int64_t rows : {std::min<int64_t>(n_rows, kAttnRows), (int64_t)(n_rows % kAttnRows ? n_rows % kAttnRows : kAttnRows)})
+    c = std::max(c, attn_plan(batch, hq, hkv, rows, kv_len).chunks);
+  return c;
 }
 
 }  // namespace subspec
 
 using namespace subspec;
 
-extern "C" size_t subspec_tree_attention_workspace(int64_t batch, int64_t n_q_heads, int64_t prefix_len, int64_t n_tree_slots) {
-  if (batch <= 0 || n_q_heads <= 0) return 256;
-  const int chunks = attn_chunks(batch, n_q_heads, prefix_len + n_tree_slots);
+static size_t attn_partial_bytes(int64_t batch, int64_t hq, int chunks, size_t* o_bytes) {
+  const size_t slots = (size_t)batch * hq * chunks * kAttnRows;
+  *o_bytes = align_up(slots * kAttnD * sizeof(float), 256);
+  return *o_bytes + align_up(slots * 2 * sizeof(float), 256);
+}
+
+extern "C" size_t subspec_tree_attention_workspace(int64_t batch, int64_t n_q_heads, int64_t n_kv_heads, int64_t n_rows,
+                                                   int64_t prefix_len, int64_t n_tree_slots) {
+  if (batch <= 0 || n_q_heads <= 0 || n_kv_heads <= 0 || n_q_heads % n_kv_heads != 0 || n_rows <= 0) return 256;
+  const int chunks = attn_chunks_bound(batch, n_q_heads, n_kv_heads, n_rows, prefix_len + n_tree_slots);
   if (chunks == 1) return 256;
-  const size_t slots = (size_t)batch * n_q_heads * chunks * kAttnRows;
-  return align_up(slots * kAttnD * sizeof(float), 256) + align_up(slots * 2 * sizeof(float), 256);
+  size_t o_bytes;
+  return attn_partial_bytes(batch, n_q_heads, chunks, &o_bytes);
 }
 
 static int tree_attention_impl(const char* what, const void* q, const void* k_cache, const void* v_cache, void* out, int dtype,
@@ -460,55 +522,53 @@ static int tree_attention_impl(const char* what, const void* q, const void* k_ca
     ap.page_stride = 2 * ap.v_delta;
   }
   const int64_t kv_len = prefix_len + n_tree_slots;
-  ap.chunks = attn_chunks(batch, n_q_heads, kv_len);
   const int64_t blocks = (kv_len + kKeyBlock - 1) / kKeyBlock;
-  ap.chunk_keys = (blocks + ap.chunks - 1) / ap.chunks * kKeyBlock;
-  ap.chunks = (int)((kv_len + ap.chunk_keys - 1) / ap.chunk_keys);
   ap.scale_log2 = scale * kLog2e;
   const int group = (int)(n_q_heads / n_kv_heads);
-  // wavefront = ROWT 16-row tiles of one head; WPH wavefronts per head; 8 / WPH heads share a workgroup's K / V stages:
-  // up to 16 rows (a draft level): 1 tile, 8 heads; up to 32 rows: 2 tiles, 8 heads; up to 64 rows: 2 tiles x 2 wavefronts, 4 heads
-  ap.units = batch * n_kv_heads * ap.chunks;
   float* part_o = nullptr;
   float* part_ml = nullptr;
-  if (ap.chunks > 1) {
-    const size_t slots = (size_t)batch * n_q_heads * ap.chunks * kAttnRows;
-    const size_t need = align_up(slots * kAttnD * sizeof(float), 256) + align_up(slots * 2 * sizeof(float), 256);
+  const int chunks_bound = attn_chunks_bound(batch, n_q_heads, n_kv_heads, n_rows, kv_len);
+  if (chunks_bound > 1) {
+    size_t o_bytes;
+    const size_t need = attn_partial_bytes(batch, n_q_heads, chunks_bound, &o_bytes);
     if (!workspace || workspace_bytes < need)
       SUBSPEC_FAIL(SUBSPEC_ERR_WORKSPACE, "%s: workspace of %zu bytes is smaller than the %zu required", what,
                    workspace_bytes, need);
     if ((uintptr_t)workspace % 16) SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "%s: workspace must be 16-byte aligned", what);
     part_o = (float*)workspace;
-    part_ml = (float*)((char*)workspace + align_up(slots * kAttnD * sizeof(float), 256));
+    part_ml = (float*)((char*)workspace + o_bytes);
   }
   hipStream_t st = (hipStream_t)stream;
   // more than 64 query rows: one launch (pair) per window of 64, in stream order, sharing the partial buffers
   for (int64_t row0 = 0; row0 < n_rows; row0 += kAttnRows) {
-  ap.row0 = (int)row0;
-  ap.win_rows = (int)std::min<int64_t>(n_rows - row0, kAttnRows);
-  const int wph = ap.win_rows <= 32 ? 1 : 2, rowt = ap.win_rows <= 16 ? 1 : 2;
-  const int heads_per_wg = 8 / wph;
-  ap.pairs_per_kv = (group + heads_per_wg - 1) / heads_per_wg;
-  const dim3 grid((unsigned)((ap.units + kXcds - 1) / kXcds * kXcds * ap.pairs_per_kv));
-  const int64_t merge_rows = batch * n_q_heads * ap.win_rows / 8 >= 1024 ? 8 : 2;   // rows per merge workgroup
-  const dim3 merge_grid((unsigned)((ap.win_rows + merge_rows - 1) / merge_rows), (unsigned)(batch * n_q_heads));
-#define SUBSPEC_ATTN_KERNEL(DT, PAGED, ROWT, WPH)                                                                  \
-  hipLaunchKernelGGL((tree_attention_kernel<DT, PAGED, ROWT, WPH>), grid, dim3(kAttnThreads), 0, st, (const uint16_t*)q, \
+    ap.row0 = (int)row0;
+    ap.win_rows = (int)std::min<int64_t>(n_rows - row0, kAttnRows);
+    const AttnPlan pl = attn_plan(batch, n_q_heads, n_kv_heads, ap.win_rows, kv_len);
+    ap.chunk_keys = (blocks + pl.chunks - 1) / pl.chunks * kKeyBlock;
+    ap.chunks = (int)((kv_len + ap.chunk_keys - 1) / ap.chunk_keys);
+    ap.units = batch * n_kv_heads * ap.chunks;
+    ap.pairs_per_kv = (group + pl.heads_per_wg - 1) / pl.heads_per_wg;
+    const dim3 grid((unsigned)((ap.units + kXcds - 1) / kXcds * kXcds * ap.pairs_per_kv));
+    const int64_t merge_rows = batch * n_q_heads * ap.win_rows / 8 >= 1024 ? 8 : 2;   // rows per merge workgroup
+    const dim3 merge_grid((unsigned)((ap.win_rows + merge_rows - 1) / merge_rows), (unsigned)(batch * n_q_heads));
+#define SUBSPEC_ATTN_KERNEL(DT, PAGED, ROWT, WPH, THREADS)                                                          \
+  hipLaunchKernelGGL((tree_attention_kernel<DT, PAGED, ROWT, WPH, THREADS>), grid, dim3(THREADS), 0, st, (const uint16_t*)q, \
                      (const uint16_t*)k_cache, (const uint16_t*)v_cache, anc_bits, ap, (uint16_t*)out, part_o, part_ml)
 #define SUBSPEC_ATTN_LAUNCH(DT, PAGED)                                                                             \
   do {                                                                                                             \
     {                                                                                                              \
       DominantKernelTimer timer(st);                                                                               \
-      if (rowt == 1) SUBSPEC_ATTN_KERNEL(DT, PAGED, 1, 1);                                                         \
-      else if (wph == 1) SUBSPEC_ATTN_KERNEL(DT, PAGED, 2, 1);                                                     \
-      else SUBSPEC_ATTN_KERNEL(DT, PAGED, 2, 2);                                                                   \
+      if (pl.threads == 256) SUBSPEC_ATTN_KERNEL(DT, PAGED, 1, 4, 256);                                            \
+      else if (pl.wph == 2) SUBSPEC_ATTN_KERNEL(DT, PAGED, 2, 2, 512);                                             \
+      else if (pl.rowt == 1) SUBSPEC_ATTN_KERNEL(DT, PAGED, 1, 1, 512);                                            \
+      else SUBSPEC_ATTN_KERNEL(DT, PAGED, 2, 1, 512);                                                              \
     }                                                                                                              \
     if (ap.chunks > 1)                                                                                             \
       hipLaunchKernelGGL((tree_attention_merge_kernel<DT>), merge_grid, dim3(merge_rows * 32), 0, st, part_o, part_ml, ap, \
                          (uint16_t*)out);                                                                          \
   } while (0)
-  if (dtype == SUBSPEC_BF16) { if (paged) SUBSPEC_ATTN_LAUNCH(SUBSPEC_BF16, true); else SUBSPEC_ATTN_LAUNCH(SUBSPEC_BF16, false); }
-  else { if (paged) SUBSPEC_ATTN_LAUNCH(SUBSPEC_F16, true); else SUBSPEC_ATTN_LAUNCH(SUBSPEC_F16, false); }
+    if (dtype == SUBSPEC_BF16) { if (paged) SUBSPEC_ATTN_LAUNCH(SUBSPEC_BF16, true); else SUBSPEC_ATTN_LAUNCH(SUBSPEC_BF16, false); }
+    else { if (paged) SUBSPEC_ATTN_LAUNCH(SUBSPEC_F16, true); else SUBSPEC_ATTN_LAUNCH(SUBSPEC_F16, false); }
 #undef SUBSPEC_ATTN_LAUNCH
 #undef SUBSPEC_ATTN_KERNEL
   }

@@ -152,7 +152,7 @@ static LayerPlan layer_plan(const subspec_decoder_layer_dims& s) {
   sub = std::max(sub, subspec_dense_linear_workspace(s.n_rows, H, Q));
   sub = std::max(sub, subspec_dense_linear_workspace(s.n_rows, 2 * F, H));
   sub = std::max(sub, subspec_dense_linear_workspace(s.n_rows, H, F));
-  sub = std::max(sub, subspec_tree_attention_workspace(1, s.n_q_heads, s.prefix_len, s.n_tree_slots));
+  sub = std::max(sub, subspec_tree_attention_workspace(1, s.n_q_heads, s.n_kv_heads, s.n_rows, s.prefix_len, s.n_tree_slots));
   p.sub_bytes = align_up(sub, 256);
   p.sub = take(p.sub_bytes);
   p.total = off;

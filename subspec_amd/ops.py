@@ -267,7 +267,7 @@ def tree_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
         raise ValueError("anc_bits batch dimension must be 1 or B")
     stride = n if (len(rows_shape) == 2 and rows_shape[0] == B and B > 1) else 0
     lib = L.lib()
-    need = lib.subspec_tree_attention_workspace(B, Hq, int(prefix_len), slots)
+    need = lib.subspec_tree_attention_workspace(B, Hq, Hkv, n, int(prefix_len), slots)
     if workspace is None and need > 256:
         workspace = torch.empty(need, dtype=torch.uint8, device=dev)
     out = torch.empty((B, n, Hq * D), dtype=q.dtype, device=dev)
@@ -307,7 +307,7 @@ def tree_attention_paged(q: torch.Tensor, pool_layer: torch.Tensor, page_indices
         raise ValueError("anc_bits must be int64 [n] ([n, ceil(slots / 64)] above 64 tree slots)")
     q, anc_bits = q.contiguous(), anc_bits.contiguous()
     lib = L.lib()
-    need = lib.subspec_tree_attention_workspace(1, Hq, int(prefix_len), slots)
+    need = lib.subspec_tree_attention_workspace(1, Hq, Hkv, n, int(prefix_len), slots)
     if workspace is None and need > 256:
         workspace = torch.empty(need, dtype=torch.uint8, device=dev)
     out = torch.empty((1, n, Hq * D), dtype=q.dtype, device=dev)
