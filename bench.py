@@ -78,7 +78,7 @@ def parse():
     ap.add_argument("--draft-graph", action="store_true",
                     help="e2e workload: replay each speculation (all draft levels) from a captured HIP graph")
     ap.add_argument("--keep-layers", type=int, default=14, help="e2e workload: target layers kept resident; the rest stream")
-    ap.add_argument("--workload", default="verify-cycle", choices=["verify-cycle", "attention", "int4", "dense", "greedy", "sampling", "e2e"],
+    ap.add_argument("--workload", default="verify-cycle", choices=["verify-cycle", "attention", "int4", "dense", "greedy", "sampling", "topk", "e2e"],
                     help="verify-cycle (default, BASELINE config 2) is the benchmark line; the others time one "
                          "kernel family of configs 1, 3 and 4 and print one JSON line per shape")
     return ap.parse_args()
@@ -190,7 +190,7 @@ def bench_int4(args):
         del W_
         copies = max(2, COLD_BYTES // (wq.numel() * 4) + 1)
         wqs, szs = [wq.clone() for _ in range(copies)], [sz.clone() for _ in range(copies)]
-        for M in (1, 16, 64):
+        for M in (1, 8, 16, 64):                          # 8: one draft level at top-k 8
             x = torch.randn(M, K, device=dev).to(torch.bfloat16)
             ws = torch.empty(max(ops.L.lib().subspec_int4_linear_workspace(M, N, K), 256), dtype=torch.uint8, device=dev)
             warm_us, warm_kernel_us = _time_us(lambda: ops.int4_linear(x, wq, sz, N, workspace=ws), args.steps, args.warmup)
@@ -330,6 +330,32 @@ def e2e_block(args):
     return out
 
 
+def bench_topk(args):
+    """Top-16 expansion of 2048 x 152064 bf16 rows on three kinds of rows: the default workload's (softmax of scaled
+    Gaussians), near-uniform rows (every probability within 0.1 % of 1 / V: in bf16 almost all entries of a row are
+    EQUAL, the ballot threshold of the slice kernel rejects nothing and its prune steps do the work), and one-hot
+    rows.  The second is the worst case for the screening."""
+    import torch
+    from subspec_amd import ops
+    dev = torch.device("cuda:0")
+    rows, V, k = 2048, 152064, 16
+    g = torch.Generator(device=dev).manual_seed(5)
+    kinds = {}
+    z = torch.randn(rows, 1, V, generator=g, device=dev) * (torch.rand(rows, 1, 1, generator=g, device=dev) * 2.5 + 0.5)
+    kinds["softmax of scaled Gaussians (the default workload's rows)"] = torch.softmax(z.to(torch.bfloat16), -1)
+    del z
+    kinds["near-uniform rows (1 / V within 0.1 %)"] = ((1.0 + 1e-3 * torch.rand(rows, 1, V, generator=g, device=dev)) / V).to(torch.bfloat16)
+    hot = torch.zeros(rows, 1, V, device=dev, dtype=torch.bfloat16)
+    hot[torch.arange(rows, device=dev), 0, torch.randint(0, V, (rows,), generator=g, device=dev)] = 1
+    kinds["one-hot rows"] = hot
+    parent = torch.rand(rows, 1, generator=g, device=dev).to(torch.bfloat16)
+    ws = torch.empty(ops.L.lib().subspec_topk_expand_workspace(rows, 1, V, k), dtype=torch.uint8, device=dev)
+    for name, probs in kinds.items():
+        call_us, kernel_us = _time_us(lambda: ops.topk_expand(probs, parent, k, workspace=ws), args.steps, args.warmup)
+        _kernel_line("top-k expansion latency", f"top-16 of 2048 x 152064 bf16 rows, {name}", call_us, kernel_us, rows * V * 2, 0,
+                     "subspec::topk_slice_kernel", extra={"rows": name})
+
+
 def bench_greedy(args):
     import torch
     from subspec_amd import ops, workloads as W
@@ -432,7 +458,7 @@ def main():
         sys.exit(1)
     L.lib()                                            # fail loudly when the HIP library is missing
     if args.workload != "verify-cycle":
-        {"attention": bench_attention, "int4": bench_int4, "dense": bench_dense, "greedy": bench_greedy, "sampling": bench_sampling,
+        {"attention": bench_attention, "int4": bench_int4, "dense": bench_dense, "greedy": bench_greedy, "sampling": bench_sampling, "topk": bench_topk,
          "e2e": bench_e2e}[args.workload](args)
         return
     dev = torch.device("cuda:0")

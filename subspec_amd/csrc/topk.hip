@@ -52,15 +52,44 @@ __device__ __forceinline__ uint32_t pk_max_u16(uint32_t a, uint32_t b) {
 // grow with u for q > 0, so "key >= tau_key" can be tested on the raw bits with an unsigned
 // compare; patterns with the sign bit set compare high and are sorted out by the precise test.
 template <int DT>
-__device__ __forceinline__ uint32_t min_pattern_reaching(float q, float tau_key) {
-  if (!(q > 0.f)) return 0;
+__device__ __forceinline__ bool pattern_reaches(uint32_t u, float q, float tau_key) {
+  const float v = DT == SUBSPEC_BF16 ? bf16_bits_to_float(u) : f16_bits_to_float(u);
+  return Elem<DT>::round(v * q) >= tau_key;
+}
+template <int DT>
+__device__ __forceinline__ uint32_t min_pattern_reaching_search(float q, float tau_key) {
   uint32_t lo = 0, hi = DT == SUBSPEC_BF16 ? 0x7f80u : 0x7c00u;     // +inf
   while (lo < hi) {
     const uint32_t mid = (lo + hi) >> 1;
-    const float v = DT == SUBSPEC_BF16 ? bf16_bits_to_float(mid) : f16_bits_to_float(mid);
-    if (Elem<DT>::round(v * q) >= tau_key) hi = mid; else lo = mid + 1;
+    if (pattern_reaches<DT>(mid, q, tau_key)) hi = mid; else lo = mid + 1;
   }
   return lo;
+}
+// The answer lies next to the pattern of tau_key / q: start just above it and walk down while the pattern below still
+// reaches (a few dependent steps instead of the fifteen of a bisection, which every workgroup would pay three times
+// on its critical path).  Whatever the walk returns satisfies "reaches, and the pattern below does not", which
+// with monotone keys IS the minimum; anything unexpected falls back to the bisection.
+template <int DT>
+__device__ __forceinline__ uint32_t min_pattern_reaching(float q, float tau_key) {
+  if (!(q > 0.f)) return 0;
+  if (!(tau_key > 0.f)) return 0;                      // every non-negative pattern reaches
+  constexpr uint32_t kInf = DT == SUBSPEC_BF16 ? 0x7f80u : 0x7c00u;
+  const float x = tau_key / q;
+  uint32_t u;
+  if constexpr (DT == SUBSPEC_BF16) {
+    u = (__float_as_uint(x) + 0xffffu) >> 16;          // smallest pattern whose value is >= x (x > 0 or NaN)
+  } else {
+    union { uint16_t b; _Float16 h; } c;
+    c.h = (_Float16)fminf(x, 65504.f);
+    u = (uint32_t)c.b + 1;
+  }
+  u = min(u + 1, kInf);
+  if (!pattern_reaches<DT>(u, q, tau_key)) return min_pattern_reaching_search<DT>(q, tau_key);
+  for (int step = 0; step < 6; ++step) {
+    if (u == 0 || !pattern_reaches<DT>(u - 1, q, tau_key)) return u;
+    --u;
+  }
+  return min_pattern_reaching_search<DT>(q, tau_key);
 }
 
 template <int DT, int VEC> struct PTile;
@@ -135,14 +164,14 @@ __device__ int prune_list(uint64_t* list, int count, uint64_t cut, int* counter)
 }
 
 template <int DT, int VEC, int U>
-__global__ __launch_bounds__(kTopkThreads) void topk_slice_kernel(
+__global__ __launch_bounds__(kTopkThreads) __attribute__((amdgpu_waves_per_eu(8, 8))) void topk_slice_kernel(
     const void* __restrict__ probs, const void* __restrict__ parent_probs, int64_t vocab, int leaves, int splits,
     int64_t chunk, int k, uint64_t* __restrict__ cand, int32_t* __restrict__ cand_count,
     int64_t* __restrict__ token_ids, void* __restrict__ topk_probs, int64_t* __restrict__ parent_indices) {
   __shared__ uint64_t list[kTopkCap];
   __shared__ uint64_t kth_slot;
   __shared__ uint32_t wave_prefix[kTopkThreads / kWave];
-  __shared__ int count, overflow;
+  __shared__ int count, overflow, tie_total;
 
   const int64_t row = blockIdx.y;                      // b * leaves + l
   const int c = blockIdx.x;
@@ -182,7 +211,7 @@ __global__ __launch_bounds__(kTopkThreads) void topk_slice_kernel(
       }
     }
   }
-  if (tid == 0) { count = 0; overflow = 0; }
+  if (tid == 0) { count = 0; overflow = 0; tie_total = 0; }
   {
     const int m = (k + 3) / 4;
     const uint32_t prefix = sany ? (uint32_t)(pack_candidate(smax, 0) >> 48) : 0u;
@@ -209,12 +238,28 @@ __global__ __launch_bounds__(kTopkThreads) void topk_slice_kernel(
   float tau_key = tau ? candidate_key(tau) : -INFINITY;
 
   // ---- stream the slice; survivors go to the LDS list
+  // Ties.  The bound is reached by at least k elements of the SAMPLE (the first U tiles of every thread, i.e. the
+  // lowest indices of the slice).  An element of a later group whose key only EQUALS the bound has a higher index than
+  // all of them and can never be among the best k, so later groups are screened strictly.  Inside the sample, when
+  // more than kTieLimit elements equal the bound (rows that are mostly one value: zeros under a low temperature,
+  // uniform rows), only the k of them with the lowest indices are taken, in index order; appending them all would
+  // overflow the list and send the workgroup through the slow one-element-per-step path.
+  constexpr int kTieLimit = 256;
   const int64_t ngroups = (ntiles + kTopkThreads - 1) / kTopkThreads;
-  auto scan_tile = [&](const PTile<DT, VEC>& t, int64_t j) {
+  // Flood test: in how many threads does the sample's maximum merely EQUAL the bound?  In a row that is mostly one
+  // value that is nearly all of them; a wrong "yes" only costs speed (the plain loop below is exact for any row).
+  if (tau != 0) {
+    const int n_eq = __popcll(__ballot(sany && smax == tau_key));
+    if ((tid & (kWave - 1)) == 0 && n_eq) atomicAdd(&tie_total, n_eq);
+    __syncthreads();
+  }
+  const bool tie_flood = tau != 0 && tie_total > kTieLimit;       // uniform
+  const float tie_key = tau_key;                       // the first bound: the ties pass after the loop is about this one
+  auto scan_tile = [&](const PTile<DT, VEC>& t, int64_t j, float bound) {    // bound: tau_key, or the next float up
 #pragma unroll
     for (int e = 0; e < VEC; ++e) {
       const float key = Elem<DT>::round(t.get(e) * q);
-      if (key >= tau_key) {
+      if (key >= bound) {
         const uint64_t pc = pack_candidate(key, flat0 + (uint32_t)(j * VEC + e));
         if (pc >= tau) {
           const int slot = atomicAdd(&count, 1);
@@ -226,11 +271,26 @@ __global__ __launch_bounds__(kTopkThreads) void topk_slice_kernel(
   // fast path: U tiles per thread in flight, no bookkeeping between groups.  For 16-bit rows a
   // tile is first screened with packed unsigned maxima against the bit pattern of the threshold
   // (five instructions for eight elements); only tiles that may hold a survivor are unpacked.
-  uint32_t screen = 0;                                 // (pattern - 1) in both halves; 0: screen nothing out
-  if constexpr (VEC == 8) {
-    const uint32_t thr = min_pattern_reaching<DT>(q, tau_key);
-    screen = thr ? (thr - 1) * 0x10001u : 0;
-  }
+  uint32_t screen = 0, screen_strict = 0;              // (pattern - 1) in both halves; 0: screen nothing out
+  float tau_key_up = tau_key;                          // the next float above the bound: "key > bound" as "key >= this"
+  auto set_screens = [&]() {
+    tau_key_up = tau ? nextafterf(tau_key, INFINITY) : tau_key;
+    if constexpr (VEC == 8) {
+      const uint32_t thr = min_pattern_reaching<DT>(q, tau_key);
+      screen = thr ? (thr - 1) * 0x10001u : 0;
+      const uint32_t thr2 = tau ? min_pattern_reaching<DT>(q, tau_key_up) : 0;
+      screen_strict = thr2 ? (thr2 - 1) * 0x10001u : 0;
+    }
+  };
+  set_screens();
+  auto tile_may_reach = [&](const PTile<DT, VEC>& t, uint32_t scr) {
+    if constexpr (VEC == 8) {
+      const uint32_t mm = pk_max_u16(pk_max_u16(t.r.x, t.r.y), pk_max_u16(t.r.z, t.r.w));
+      return scr == 0 || pk_max_u16(mm, scr) != scr;
+    } else {
+      return true;
+    }
+  };
   for (int64_t g0 = 0; g0 < ngroups; g0 += U) {
     if (g0 > 0) {                                      // group 0 is already in registers (the sample)
 #pragma unroll
@@ -239,17 +299,13 @@ __global__ __launch_bounds__(kTopkThreads) void topk_slice_kernel(
         t[i].load(probs, base + j * VEC);
       }
     }
+    const bool strict = tau != 0 && (g0 > 0 || tie_flood);        // uniform
+    const uint32_t scr = strict ? screen_strict : screen;
+    const float bound = strict ? tau_key_up : tau_key;
 #pragma unroll
     for (int i = 0; i < U; ++i) {
       const int64_t j = (g0 + i) * kTopkThreads + tid;
-      if (j < ntiles) {
-        if constexpr (VEC == 8) {
-          const uint32_t mm = pk_max_u16(pk_max_u16(t[i].r.x, t[i].r.y), pk_max_u16(t[i].r.z, t[i].r.w));
-          if (screen == 0 || pk_max_u16(mm, screen) != screen) scan_tile(t[i], j);
-        } else {
-          scan_tile(t[i], j);
-        }
-      }
+      if (j < ntiles && tile_may_reach(t[i], scr)) scan_tile(t[i], j, bound);
     }
     // two checkpoints tighten the threshold to the exact k-th best of what has been seen, so that
     // few later elements survive and the final selection stays small
@@ -262,11 +318,54 @@ __global__ __launch_bounds__(kTopkThreads) void topk_slice_kernel(
         tau = kth_best<kTopkThreads>(list, cnt, k, &kth_slot);
         tau_key = candidate_key(tau);
         prune_list<kTopkThreads>(list, cnt, tau, &count);
-        if constexpr (VEC == 8) {
-          const uint32_t thr = min_pattern_reaching<DT>(q, tau_key);
-          screen = thr ? (thr - 1) * 0x10001u : 0;
+        set_screens();
+      }
+    }
+  }
+  if (tie_flood) {                                     // workgroup-uniform
+    // The sample was screened strictly; now the k lowest-index elements of it that EQUAL the first bound, tile row by
+    // tile row (ranks from a prefix sum over the workgroup).  The tiles are loaded again, one at a time (they are in
+    // L2), so that the streaming loop above keeps its registers.  If the bound has been tightened since, these are
+    // below the cut and the final selection drops them.
+    int taken = 0;                                     // uniform
+#pragma unroll 1
+    for (int i = 0; i < U && taken < k; ++i) {
+      const int64_t j = tid + (int64_t)i * kTopkThreads;
+      PTile<DT, VEC> tt;
+      tt.load(probs, base + min(j, ntiles - 1) * VEC);
+      int eq = 0;
+      if (j < ntiles) {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) eq += Elem<DT>::round(tt.get(e) * q) == tie_key;
+      }
+      int incl = eq;                                   // inclusive prefix inside the wavefront
+#pragma unroll
+      for (int o = 1; o < kWave; o <<= 1) {
+        const int up = __shfl_up(incl, o, kWave);
+        if ((tid & (kWave - 1)) >= o) incl += up;
+      }
+      __syncthreads();                                 // wave_prefix is free (the bound has been read)
+      if ((tid & (kWave - 1)) == kWave - 1) wave_prefix[tid / kWave] = (uint32_t)incl;
+      __syncthreads();
+      int before = 0, total = 0;
+      for (int w = 0; w < kTopkThreads / kWave; ++w) {
+        if (w < tid / kWave) before += (int)wave_prefix[w];
+        total += (int)wave_prefix[w];
+      }
+      int rank = taken + before + incl - eq;           // rank of this thread's first equal element
+      if (eq && rank < k) {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+          if (Elem<DT>::round(tt.get(e) * q) == tie_key) {
+            if (rank < k) {
+              const int slot = atomicAdd(&count, 1);
+              if (slot < kTopkCap) list[slot] = pack_candidate(tie_key, flat0 + (uint32_t)(j * VEC + e)); else overflow = 1;
+            }
+            ++rank;
+          }
         }
       }
+      taken += total;
     }
   }
   __syncthreads();

@@ -52,6 +52,38 @@ def test_heavy_ties_and_adversarial_order(dtype):
     _check(asc.flip(-1).contiguous(), torch.ones(1, 1, dtype=dtype), 16)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("batch", [1, 24])
+def test_rows_that_are_mostly_one_value(dtype, batch):
+    """Rows in which most elements share one value, so the bound the kernel takes from its sample is that value and
+    thousands of elements tie with it: the k best are whatever lies above, then the ties of lowest index."""
+    g = torch.Generator().manual_seed(11)
+    V, k = 152064, 16
+    print("ties", dtype, batch, flush=True)
+    base = torch.full((batch, 1, V), 1.0 / V)
+    rows = []
+    for b in range(batch):
+        r = base[b, 0].clone()
+        kind = b % 6
+        if kind == 1:                                   # a handful above the plateau, fewer than k
+            r[torch.randint(0, V, (5,), generator=g)] = 0.01
+        elif kind == 2:                                 # more than k above it, late in the row
+            r[V - 4000 + torch.randperm(3000, generator=g)[:40]] = torch.rand(40, generator=g) * 0.01 + 1e-4
+        elif kind == 3:                                 # one-hot: the plateau is zero
+            r.zero_()
+            r[int(torch.randint(0, V, (1,), generator=g))] = 1.0
+        elif kind == 4:                                 # plateau only in the first part, smaller values after it
+            r[20000:] = 1e-7
+        elif kind == 5:                                 # every thread's sample holds one larger value among ties
+            r[::64] = 2.0 / V
+        rows.append(r)
+    probs = torch.stack(rows).view(batch, 1, V).to(dtype)
+    parent = (torch.rand(batch, 1, generator=g) * 0.9 + 0.1).to(dtype)
+    _check(probs, parent, k)
+    # several leaves per tree: the flat index order across leaves decides among ties
+    _check(probs[:1].expand(1, 4, V).contiguous(), torch.full((1, 4), 0.5, dtype=dtype), k)
+
+
 def test_config2_rows_bf16_full_vocab():
     g = torch.Generator().manual_seed(2)
     V = 152064
