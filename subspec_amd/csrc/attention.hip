@@ -62,16 +62,6 @@ typedef __bf16 v2bf_t __attribute__((ext_vector_type(2)));
 typedef _Float16 v2h_t __attribute__((ext_vector_type(2)));
 typedef float v2f_t __attribute__((ext_vector_type(2)));
 
-// two floats -> one packed pair of 16-bit floats (round to nearest even), one conversion instruction
-template <int DT>
-__device__ __forceinline__ uint32_t pack2(float lo, float hi) {
-  const v2f_t v = {lo, hi};
-  if constexpr (DT == SUBSPEC_BF16) {
-    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, v2bf_t));
-  } else {
-    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, v2h_t));
-  }
-}
 
 // Transposing LDS read of 16-bit elements (ds_read_b64_tr_b16): within each group of 16 lanes,
 // lane i receives element i%4 of the four 8-byte rows addressed by lanes i/4, i/4 + 4, i/4 + 8,

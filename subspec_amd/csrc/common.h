@@ -138,11 +138,20 @@ __device__ __forceinline__ uint32_t to_bits(float v) {
     return c.u;
   }
 }
+typedef float dec_f2 __attribute__((ext_vector_type(2)));
+typedef __bf16 dec_bf2 __attribute__((ext_vector_type(2)));
+typedef _Float16 dec_h2 __attribute__((ext_vector_type(2)));
+// two values rounded to nearest even and packed, low half first (one packed conversion per pair)
+template <int DT>
+__device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+  if constexpr (DT == SUBSPEC_BF16) return __builtin_bit_cast(uint32_t, __builtin_convertvector(dec_f2{lo, hi}, dec_bf2));
+  else return __builtin_bit_cast(uint32_t, __builtin_convertvector(dec_f2{lo, hi}, dec_h2));
+}
 template <int DT>
 __device__ __forceinline__ dec_u4 pack8(const float* f) {
   dec_u4 v;
 #pragma unroll
-  for (int j = 0; j < 4; ++j) v[j] = to_bits<DT>(f[2 * j]) | (to_bits<DT>(f[2 * j + 1]) << 16);
+  for (int j = 0; j < 4; ++j) v[j] = pack2<DT>(f[2 * j], f[2 * j + 1]);
   return v;
 }
 

@@ -180,17 +180,27 @@ struct I4Fused {
 
 // XHALF (at most 8 activation rows, MT = 1): only rows 0..7 of a block are fetched, scaled and parked; rows 8..15 of the
 // LDS stages are cleared once.  Half the activation traffic and half the prologue arithmetic of a 16-row block.
-template <int DT, int MT, int RT, int EPI = kEpiPlain, bool NORM = false, bool XHALF = false>
-__global__ __launch_bounds__(kI4Threads) void int4_gemm_kernel(
+//
+// PRE > 0 (with XHALF; a wavefront has at most PRE groups): nothing is pipelined.  Every request of the wavefront --
+// its gains, its PRE activation blocks, then all its weight words -- goes out before the first wait, the activation
+// blocks (L2 hits, requested first, so their waits do not include the weights) are parked in PRE private LDS stages while
+// the weights are on their way from HBM, and the steps then run against registers.  With one workgroup per compute unit
+// (the q|k|v and o projections of a draft level: 288 and 224 workgroups) a two-group pipeline has nothing to hide a round
+// trip behind and pays one per two steps; here the wavefront pays one.  A stage holds 8 rows of 128 bytes, 16-byte piece p
+// of row r at position p ^ r; MFMA rows 8..15 read a block of zeros.
+template <int DT, int MT, int RT, int EPI = kEpiPlain, bool NORM = false, bool XHALF = false, int PRE = 0>
+__global__ __launch_bounds__(PRE > 0 ? 2 * kI4Threads : kI4Threads) void int4_gemm_kernel(
     const uint16_t* __restrict__ x, const uint2* __restrict__ wq, const uint32_t* __restrict__ sz,
     const uint16_t* __restrict__ bias, const uint16_t* residual, uint16_t* y, float* __restrict__ partial, int M, int64_t N,
     int K, int splits, int groups_per_split, I4Fused fz) {
   constexpr bool SILU = EPI == kEpiSilu, ROPE = EPI == kEpiRope, PAIRED = EPI != kEpiPlain;
-  __shared__ float sq_s[NORM ? 4 * MT * 16 : 1];                 // NORM: per wavefront, per row: sum of squares of its groups
+  constexpr int NW = PRE > 0 ? 8 : 4;                            // wavefronts of the workgroup; wavefront w takes groups w, w + NW, ...
+  __shared__ float sq_s[NORM ? NW * MT * 16 : 1];                 // NORM: per wavefront, per row: sum of squares of its groups
   __shared__ float rstd_s[NORM ? MT * 16 : 1];
   // 4 wavefronts x 2 stages of a [16*MT][64] activation block; reused for the final reduction
   // (two rounds of one accumulator tile set per wavefront)
-  constexpr int kStageBytes = 4 * 2 * MT * 16 * kXlStride * 2, kRedBytes = 2 * 4 * MT * 256 * 4;
+  constexpr int kPreBytes = PRE > 0 ? NW * PRE * (1024 + 128) + NW * 16 : 0;   // stages, gains, one block of zeros per wavefront
+  constexpr int kStageBytes = PRE > 0 ? kPreBytes : 4 * 2 * MT * 16 * kXlStride * 2, kRedBytes = 2 * NW * MT * 256 * 4;
   __shared__ __attribute__((aligned(16))) unsigned char lds_raw[kStageBytes > kRedBytes ? kStageBytes : kRedBytes];
   uint16_t* const xstage = (uint16_t*)lds_raw;
   float* const red = (float*)lds_raw;
@@ -202,12 +212,14 @@ __global__ __launch_bounds__(kI4Threads) void int4_gemm_kernel(
   const int ks = blockIdx.y;
   const int g_begin = ks * groups_per_split, g_end = min(G, g_begin + groups_per_split);
   const int g_first = g_begin + wave;                            // this wavefront's groups: g_first + 4j
-  const int nj = g_first < g_end ? (g_end - g_first + 3) / 4 : 0;
+  const int nj = g_first < g_end ? (g_end - g_first + NW - 1) / NW : 0;
 
   // tiles [tile0, tile0 + ntl) of this workgroup: an even split of all tiles (SILU / ROPE: of all tile pairs) over the grid
   const int n_units = PAIRED ? n_tiles / 2 : n_tiles;
-  const int unit0 = (int)((int64_t)blockIdx.x * n_units / gridDim.x);
-  const int n_own = (int)((int64_t)(blockIdx.x + 1) * n_units / gridDim.x) - unit0;
+  // (32-bit unsigned quotients: the host refuses N / 16 >= 65536, so the products fit; a 64-bit division would be a
+  // few hundred instructions on every wavefront's way to its first request)
+  const int unit0 = (int)((uint32_t)blockIdx.x * (uint32_t)n_units / gridDim.x);
+  const int n_own = (int)(((uint32_t)blockIdx.x + 1u) * (uint32_t)n_units / gridDim.x) - unit0;
   const int tile0 = unit0;                                                             // plain: first tile
   const int ntl = PAIRED ? 2 * n_own : n_own;                                          // 1 .. RT
   const int qk_units = ROPE ? (fz.hq + fz.hkv) * 4 : 0;                                // ROPE: pairs of the rotated heads
@@ -345,11 +357,92 @@ __global__ __launch_bounds__(kI4Threads) void int4_gemm_kernel(
     __builtin_amdgcn_sched_barrier(0);                                                                  \
   }
 
-  if constexpr (XHALF) {
+  if constexpr (XHALF && PRE == 0) {
     // rows 8..15 of both stages stay zero for the whole kernel
     *(i4_u4*)(&xl[8 * kXlStride + xl_write]) = i4_u4{0u, 0u, 0u, 0u};
     *(i4_u4*)(&xl[(MT * 16 * kXlStride) + 8 * kXlStride + xl_write]) = i4_u4{0u, 0u, 0u, 0u};
   }
+  if constexpr (PRE > 0) {
+    static_assert(PRE == 0 || (XHALF && MT == 1), "the preloading variant exists for 8-row blocks only");
+    unsigned char* const stages = lds_raw + wave * (PRE * 1024);
+    unsigned char* const gains = lds_raw + NW * PRE * 1024 + wave * (PRE * 128);
+    unsigned char* const zeros = lds_raw + NW * PRE * (1024 + 128) + wave * 16;
+    static_assert(PRE * 8 <= 64, "one gain piece per lane");
+    i4_u4 gpiece;
+    (void)gpiece;
+    if constexpr (NORM) {                                        // piece q = 8 J + p of the wavefront's gains: lane q
+      const int q = min(lane, PRE * 8 - 1);
+      gpiece = __builtin_amdgcn_raw_buffer_load_b128(g_rsrc, (q & 7) * 16, min(g_first + NW * (q >> 3), G - 1) * (kGroup * 2), 0);
+    }
+    i4_u4 xall[PRE];
+#pragma unroll
+    for (int J = 0; J < PRE; ++J)
+      xall[J] = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, xg_off, min(g_first + NW * J, G - 1) * (kGroup * 2), 0);
+    // (scale, zero) words: a group's 16 words are 64 bytes, and one request per (group, tile) would be half of all
+    // requests for a ninth of the bytes.  Lane group c fetches the words of steps c and 4 + c instead, two requests
+    // per tile, and a step picks its word up from lane group J % 4 with a cross-lane read.
+    static_assert(PRE <= 8, "two (scale, zero) requests per tile cover eight steps");
+    uint32_t szq[RT][2];
+#pragma unroll
+    for (int t = 0; t < RT; ++t)
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const int g = wofs[t] + min(g_first + NW * min(4 * h + c, PRE - 1), G - 1);
+        szq[t][h] = __builtin_amdgcn_raw_buffer_load_b32(sz_rsrc, ln * 4 + g * 64, 0, 0);
+      }
+    i4_u2 wall[PRE][RT];
+#pragma unroll
+    for (int J = 0; J < PRE; ++J)
+#pragma unroll
+      for (int t = 0; t < RT; ++t) {
+        const int g = wofs[t] + min(g_first + NW * J, G - 1);
+        wall[J][t] = __builtin_amdgcn_raw_buffer_load_b64(w_rsrc, lane * 8, g * 512, 0);
+      }
+    if (lane == 0) *(i4_u4*)zeros = i4_u4{0u, 0u, 0u, 0u};
+    if constexpr (NORM) {
+      if (lane < PRE * 8) *(i4_u4*)(gains + lane * 16) = gpiece;
+    }
+    const int prow = lane >> 3, ppiece = lane & 7;
+#pragma unroll
+    for (int J = 0; J < PRE; ++J) {
+      i4_u4 piece = xall[J];
+      if constexpr (NORM) {
+        float f_[8], g_[8];
+        unpack8<DT>(piece, f_);
+        unpack8<DT>(*(const i4_u4*)(gains + (J * 8 + ppiece) * 16), g_);
+        float ss_ = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) { ss_ = fmaf(f_[e], f_[e], ss_); f_[e] *= g_[e]; }
+        sq[0] += J < nj ? ss_ : 0.f;
+        piece = pack8<DT>(f_);
+      }
+      *(i4_u4*)(stages + J * 1024 + prow * 128 + ((ppiece ^ prow) << 4)) = piece;
+    }
+    const int rd0 = ln * 128 + (((2 * c) ^ ln) << 4), rd1 = ln * 128 + (((2 * c + 1) ^ ln) << 4);
+#pragma unroll
+    for (int J = 0; J < PRE; ++J) {
+      const bool step_live = J < nj;
+      const i4_u4 xa0 = *(const i4_u4*)(ln < 8 ? stages + J * 1024 + rd0 : zeros);
+      const i4_u4 xa1 = *(const i4_u4*)(ln < 8 ? stages + J * 1024 + rd1 : zeros);
+      i4_v4f xs = i4_mfma32<DT>(xa0, ones, i4_v4f{0.f, 0.f, 0.f, 0.f});
+      xs = i4_mfma32<DT>(xa1, ones, xs);
+#pragma unroll
+      for (int t = 0; t < RT; ++t) {
+        const uint32_t w0 = wall[J][t].x, w1 = wall[J][t].y;
+        const uint32_t szw = (uint32_t)__shfl((int)szq[t][J >> 2], (J & 3) * 16 + ln, kWave);
+        const i4_u4 b0 = i4_u4{code_pair(w0, 0, kmagic, kmask), code_pair(w0, 4, kmagic, kmask),
+                               code_pair(w0, 8, kmagic, kmask), code_pair(w0, 12, kmagic, kmask)};
+        const i4_u4 b1 = i4_u4{code_pair(w1, 0, kmagic, kmask), code_pair(w1, 4, kmagic, kmask),
+                               code_pair(w1, 8, kmagic, kmask), code_pair(w1, 12, kmagic, kmask)};
+        const float sc = (step_live && t < ntl) ? f16_bits_to_float(szw & 0xffffu) : 0.f;
+        const float szo = -sc * (f16_bits_to_float(szw >> 16) + I4<DT>::kOffset);
+        i4_v4f raw = i4_mfma32<DT>(xa0, b0, i4_v4f{0.f, 0.f, 0.f, 0.f});
+        raw = i4_mfma32<DT>(xa1, b1, raw);
+#pragma unroll
+        for (int rr = 0; rr < 4; ++rr) acc[t][0][rr] = fmaf(sc, raw[rr], fmaf(szo, xs[rr], acc[t][0][rr]));
+      }
+    }
+  } else {
   // The requests before the loop are issued in the order the loop issues them (activation block, then the weights of
   // the group two steps back), so that the first trip finds the same queue of outstanding requests as every later
   // one: the compiler gives each wait ONE count that must hold on every path into the loop, and a prologue that ends
@@ -383,6 +476,7 @@ __global__ __launch_bounds__(kI4Threads) void int4_gemm_kernel(
       SUBSPEC_I4_STEP(1, 1, 1, j + 1);
     }
   }
+  }
   if constexpr (NORM) {
     // the eight lanes that share a row hold its squares over different k; one value per (wavefront, row) goes to LDS
 #pragma unroll
@@ -401,13 +495,77 @@ __global__ __launch_bounds__(kI4Threads) void int4_gemm_kernel(
   if constexpr (NORM) {
     // ordered before its first use by the barrier of reduction round 0
     if (tid < MT * 16)
-      rstd_s[tid] = rsqrtf((sq_s[tid] + sq_s[MT * 16 + tid] + sq_s[2 * MT * 16 + tid] + sq_s[3 * MT * 16 + tid]) / (float)K + fz.norm_eps);
+    {
+      float ss = 0.f;
+#pragma unroll
+      for (int w = 0; w < NW; ++w) ss += sq_s[w * MT * 16 + tid];
+      rstd_s[tid] = rsqrtf(ss / (float)K + fz.norm_eps);
+    }
   }
 #undef SUBSPEC_I4_PARK_X
 #undef SUBSPEC_I4_FETCH_X
 #undef SUBSPEC_I4_FETCH_W
 #undef SUBSPEC_I4_STEP
 
+  if constexpr (PRE > 0) {
+    // ---- 8-row output stage: every wavefront leaves its accumulators of all tiles in LDS, and after ONE barrier
+    // wavefront m finishes row m: lane (pair or tile, column) sums the eight partials in wavefront order and runs the
+    // output stage of its element, so the rotary arithmetic of a row pair is one evaluation per thread, in parallel
+    // over rows, instead of four in a row on one wavefront.
+#pragma unroll
+    for (int t = 0; t < RT; ++t) *(i4_v4f*)(&red[((t * NW + wave) * 64 + lane) * 4]) = acc[t][0];
+    __syncthreads();
+    const int m = wave;                                          // row of this wavefront (NW == 8 rows)
+    const int item = lane >> 4;                                  // plain: tile; paired: pair of tiles
+    if (m >= M || item >= (PAIRED ? RT / 2 : RT)) return;
+    const int t0 = PAIRED ? 2 * item : item;
+    if (t0 >= ntl) return;
+    auto summed = [&](int t) {
+      float v = 0.f;
+#pragma unroll
+      for (int w = 0; w < NW; ++w) v += red[((t * NW + w) * 64 + (m >> 2) * 16 + ln) * 4 + (m & 3)];
+      if constexpr (NORM) v *= rstd_s[m];
+      return v;
+    };
+    const int64_t n0 = (int64_t)tile_of(t0) * 16 + ln;
+    const float b0v = (splits == 1 && bias) ? I4<DT>::to_float(bias[n0]) : 0.f;
+    const float v0 = summed(t0);
+    if constexpr (!PAIRED) {
+      if (splits == 1) store_linear_out<DT>(y, (int64_t)m * N + n0, v0 + b0v, residual);
+      else partial[((int64_t)ks * M + m) * N + n0] = v0;
+    } else {
+      const int64_t n1 = (int64_t)tile_of(t0 + 1) * 16 + ln;
+      const float b1v = bias ? I4<DT>::to_float(bias[n1]) : 0.f;
+      const float first = Elem<DT>::round(v0 + b0v), second_raw = summed(t0 + 1) + b1v;
+      const int u = unit0 + item;
+      if constexpr (SILU) {
+        const float up = Elem<DT>::round(second_raw);
+        Elem<DT>::store(y, (int64_t)m * (N / 2) + (int64_t)u * 16 + ln, Elem<DT>::round(first / (1.f + __expf(-first))) * up);
+      } else if (u < qk_units) {
+        const int head = u >> 2, d = (u & 3) * 16 + ln;
+        const float inv_freq = fz.inv_freq ? fz.inv_freq[d] : exp2f(-(float)(2 * d) / 128.f * fz.log2_theta);
+        float sn, cs;
+        sincosf((float)fz.positions[m] * inv_freq, &sn, &cs);
+        cs = Elem<DT>::round(cs);
+        sn = Elem<DT>::round(sn);
+        const float lo = first, hi = Elem<DT>::round(second_raw);
+        const float o_lo = Elem<DT>::round(lo * cs) + Elem<DT>::round(-hi * sn);
+        const float o_hi = Elem<DT>::round(hi * cs) + Elem<DT>::round(lo * sn);
+        uint16_t *dst, *unused;
+        if (head < fz.hq) dst = fz.q_out + ((int64_t)head * M + m) * 128;
+        else if (!kv_row_ptrs(fz.kv, head - fz.hq, fz.cache_rows[m], &dst, &unused)) return;   // a row outside the layer's cache is dropped
+        Elem<DT>::store(dst, d, o_lo);
+        Elem<DT>::store(dst, d + 64, o_hi);
+      } else {
+        const int vt = 2 * (u - qk_units), kvh = vt >> 3, d = (vt & 7) * 16 + ln;
+        uint16_t *dst, *unused;
+        if (!kv_row_ptrs(fz.kv, kvh, fz.cache_rows[m], &unused, &dst)) return;
+        Elem<DT>::store(dst, d, first);
+        Elem<DT>::store(dst, d + 16, second_raw);
+      }
+    }
+    return;
+  }
   // ---- sum the four wavefronts' partial accumulators in wavefront order (0, 1, 2, 3), one tile per
   // round.  LDS holds two rounds, so a round needs one barrier; wavefront w finishes the activation
   // row blocks mt = w, w + 4, ... of the tile, so the sums and stores are spread over the workgroup.
@@ -417,7 +575,7 @@ __global__ __launch_bounds__(kI4Threads) void int4_gemm_kernel(
 #pragma unroll
   for (int t = 0; t < RT; ++t) {
     if (t >= ntl) break;                                         // uniform
-    float* stage = red + (t & 1) * (4 * MT * 256);
+    float* stage = red + (t & 1) * (NW * MT * 256);
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) *(i4_v4f*)(&stage[((wave * MT + mt) * 64 + lane) * 4]) = acc[t][mt];
     __syncthreads();                                             // round t written; round t - 1 fully read
@@ -428,7 +586,7 @@ __global__ __launch_bounds__(kI4Threads) void int4_gemm_kernel(
       if ((mt & 3) != wave) continue;                            // uniform
       i4_v4f v = *(const i4_v4f*)(&stage[((0 * MT + mt) * 64 + lane) * 4]);
 #pragma unroll
-      for (int w = 1; w < 4; ++w) {
+      for (int w = 1; w < NW; ++w) {
         const i4_v4f o = *(const i4_v4f*)(&stage[((w * MT + mt) * 64 + lane) * 4]);
 #pragma unroll
         for (int rr = 0; rr < 4; ++rr) v[rr] += o[rr];
@@ -518,6 +676,14 @@ __global__ __launch_bounds__(256) void int4_reduce_kernel(const float* __restric
 }
 
 struct I4Plan { int wgs, row_tiles, splits, groups_per_split; };
+// Groups per wavefront that the preloading variant is compiled for, and the K ranges (in groups per workgroup) it takes:
+// long enough that the pipelined loop would pay several round trips, short enough for the registers and the LDS stages.
+constexpr int kI4Pre = 7;
+// Its workgroups hold 63 KB of LDS, two per compute unit: launches of more than 512 stay with the pipelined variant.
+static bool i4_preload_fits(int groups_per_workgroup, int64_t workgroups) {
+  return groups_per_workgroup > 32 && groups_per_workgroup <= 8 * kI4Pre && workgroups <= 512;
+}
+
 constexpr int kI4MaxRowTiles = 5;
 static int i4_row_tile_variant(int64_t need) { return need <= 1 ? 1 : need <= 2 ? 2 : need <= 3 ? 3 : kI4MaxRowTiles; }
 // Resident workgroups the launch is balanced for (register use allows 2 per SIMD row for M > 32).
@@ -532,6 +698,16 @@ static I4Plan i4_plan(int64_t M, int64_t N, int64_t K) {
   // activations: two tiles per workgroup halve that traffic (3584x18944, 8 rows, five splits: 13.8 -> 12.7 us; three or
   // five tiles per workgroup and fewer splits were slower: 14.1 to 15.7 us)
   if (M <= 16 && row_tiles == 1 && tiles * 4 <= slots && G >= 112) row_tiles = 2;
+  if (M <= 8 && G >= 112) {
+    // At most 8 rows and a long K: ranges of at most 56 groups, which the preloading variant takes (all of a
+    // workgroup's weights requested at once), over as many tiles per workgroup (at most 3) as keeps the launch within
+    // the 512 workgroups that are resident at its LDS use (3584x18944: 12.2 -> ? us)
+    const int splits = (G + 8 * kI4Pre - 1) / (8 * kI4Pre);
+    const int gps = ((G + splits - 1) / splits + 3) / 4 * 4;
+    int rt = 1;
+    while (rt < 3 && (tiles + rt - 1) / rt * splits > 512) ++rt;
+    return I4Plan{(int)((tiles + rt - 1) / rt), rt, (G + gps - 1) / gps, gps};
+  }
   const int64_t wgs = (tiles + row_tiles - 1) / row_tiles;
   int splits = (int)std::max<int64_t>(1, (slots + wgs / 2) / wgs);
   // a split costs a second launch (the reduction) and fp32 partials: it pays from about 56 groups
@@ -559,7 +735,11 @@ static int run_int4_paired(const void* x, const uint32_t* wq, const uint32_t* sz
   const int G = (int)(K / kGroup);
   const bool norm = fz.norm_gain != nullptr;
 #define SUBSPEC_I4_PAIRED(MT, RT, NORM)                                                                            \
-  if (MT == 1 && M <= 8)                                                                                           \
+  if (MT == 1 && M <= 8 && RT <= 2 && i4_preload_fits(G, wgs))                                                          \
+    hipLaunchKernelGGL((int4_gemm_kernel<DT, 1, RT, EPI, NORM, true, (RT <= 2 ? kI4Pre : 0)>), grid, dim3(2 * kI4Threads), 0, st, \
+                       (const uint16_t*)x, (const uint2*)wq, sz, (const uint16_t*)bias, (const uint16_t*)nullptr, (uint16_t*)out, \
+                       (float*)nullptr, (int)M, N, (int)K, 1, (G + 3) / 4 * 4, fz);                                \
+  else if (MT == 1 && M <= 8)                                                                                      \
     hipLaunchKernelGGL((int4_gemm_kernel<DT, 1, RT, EPI, NORM, true>), grid, dim3(kI4Threads), 0, st, (const uint16_t*)x, \
                        (const uint2*)wq, sz, (const uint16_t*)bias, (const uint16_t*)nullptr, (uint16_t*)out, (float*)nullptr, \
                        (int)M, N, (int)K, 1, (G + 3) / 4 * 4, fz);                                                 \
@@ -596,7 +776,11 @@ static int run_int4(const void* x, const uint32_t* wq, const uint32_t* sz, const
     float* partial = (float*)workspace;
     const dim3 grid((unsigned)pl.wgs, (unsigned)pl.splits);
 #define SUBSPEC_I4_LAUNCH(MT, RT)                                                                                  \
-  if (MT == 1 && M <= 8)                                                                                           \
+  if (MT == 1 && M <= 8 && RT <= 3 && i4_preload_fits(pl.groups_per_split, (int64_t)pl.wgs * pl.splits))                                        \
+    hipLaunchKernelGGL((int4_gemm_kernel<DT, 1, RT, kEpiPlain, false, true, (RT <= 3 ? kI4Pre : 0)>), grid, dim3(2 * kI4Threads), 0, st, \
+                       (const uint16_t*)x, (const uint2*)wq, sz, (const uint16_t*)bias, (const uint16_t*)residual, (uint16_t*)y, partial, \
+                       (int)M, N, (int)K, pl.splits, pl.groups_per_split, I4Fused{});                              \
+  else if (MT == 1 && M <= 8)                                                                                      \
     hipLaunchKernelGGL((int4_gemm_kernel<DT, 1, RT, kEpiPlain, false, true>), grid, dim3(kI4Threads), 0, st, (const uint16_t*)x, \
                        (const uint2*)wq, sz, (const uint16_t*)bias, (const uint16_t*)residual, (uint16_t*)y, partial, (int)M, N, (int)K, \
                        pl.splits, pl.groups_per_split, I4Fused{});                                                 \
@@ -676,6 +860,7 @@ static int paired_args_ok(const char* what, const void* x, const uint32_t* wq, c
                  (long long)M, (long long)N, (long long)K);
   if (N * K / 2 >= ((int64_t)1 << 31))
     SUBSPEC_FAIL(SUBSPEC_ERR_LIMIT, "%s: N*K/2=%lld bytes of codes exceed the 2 GiB descriptor range", what, (long long)(N * K / 2));
+  if (N >= (int64_t)1 << 20) SUBSPEC_FAIL(SUBSPEC_ERR_LIMIT, "%s: N=%lld exceeds the limit of 2^20 - 16 output features", what, (long long)N);
   if ((uintptr_t)x % 16 || (uintptr_t)wq % 16 || (uintptr_t)sz % 16)
     SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "%s: x / wq / sz must be 16-byte aligned", what);
   return SUBSPEC_OK;
@@ -734,6 +919,7 @@ int subspec::int4_linear_ex(const void* x, const uint32_t* wq, const uint32_t* s
   if (K > 65536) SUBSPEC_FAIL(SUBSPEC_ERR_LIMIT, "int4_linear: K=%lld too large", (long long)K);
   if (N * K / 2 >= ((int64_t)1 << 31))
     SUBSPEC_FAIL(SUBSPEC_ERR_LIMIT, "int4_linear: N*K/2=%lld bytes of codes exceed the 2 GiB descriptor range", (long long)(N * K / 2));
+  if (N >= (int64_t)1 << 20) SUBSPEC_FAIL(SUBSPEC_ERR_LIMIT, "int4_linear: N=%lld exceeds the limit of 2^20 - 16 output features", (long long)N);
   if ((uintptr_t)x % 16 || (uintptr_t)wq % 16 || (uintptr_t)sz % 16 || (uintptr_t)y % 8)
     SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "int4_linear: x / wq / sz must be 16-byte aligned, y 8-byte aligned");
   {
