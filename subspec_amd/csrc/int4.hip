@@ -20,7 +20,10 @@
 // one v_and_or_b32 per two weights and the products accumulate in fp32:
 //   sum_k (q_k - z) s x_k = s * (sum_k (off + q_k) x_k - (z + off) * sum_k x_k)    per group.
 // M = 1   : int4_gemv_kernel, v_dot2_f32 on (weight pair, activation pair); HBM-bound,
-//           algorithmic bytes = N*K/2 + N*(K/64)*4 (+ activations).
+//           algorithmic bytes = N*K/2 + N*(K/64)*4 (+ activations).  (K of at most 2048 only; longer K: next line.)
+// M = 1-8, K > 2048: int4_rows8_kernel, the same MFMA arithmetic with nothing pipelined: every request of a
+//           wavefront is issued before its first wait.  This is the shape of a draft level (8 rows, one workgroup per
+//           compute unit), where a pipeline of a few groups is bound by round trips, not by bytes.
 // M = 2-64: int4_gemm_kernel, v_mfma_f32_16x16x32 with the activations as A and the weight tile as
 //           B operand; the 32 k of one MFMA step all come from one quantization group, so the raw
 //           accumulator of a group is scaled once.  The wavefronts of a workgroup split K, their
@@ -180,27 +183,18 @@ struct I4Fused {
 
 // XHALF (at most 8 activation rows, MT = 1): only rows 0..7 of a block are fetched, scaled and parked; rows 8..15 of the
 // LDS stages are cleared once.  Half the activation traffic and half the prologue arithmetic of a 16-row block.
-//
-// PRE > 0 (with XHALF; a wavefront has at most PRE groups): nothing is pipelined.  Every request of the wavefront --
-// its gains, its PRE activation blocks, then all its weight words -- goes out before the first wait, the activation
-// blocks (L2 hits, requested first, so their waits do not include the weights) are parked in PRE private LDS stages while
-// the weights are on their way from HBM, and the steps then run against registers.  With one workgroup per compute unit
-// (the q|k|v and o projections of a draft level: 288 and 224 workgroups) a two-group pipeline has nothing to hide a round
-// trip behind and pays one per two steps; here the wavefront pays one.  A stage holds 8 rows of 128 bytes, 16-byte piece p
-// of row r at position p ^ r; MFMA rows 8..15 read a block of zeros.
-template <int DT, int MT, int RT, int EPI = kEpiPlain, bool NORM = false, bool XHALF = false, int PRE = 0>
-__global__ __launch_bounds__(PRE > 0 ? 2 * kI4Threads : kI4Threads) void int4_gemm_kernel(
+template <int DT, int MT, int RT, int EPI = kEpiPlain, bool NORM = false, bool XHALF = false>
+__global__ __launch_bounds__(kI4Threads) void int4_gemm_kernel(
     const uint16_t* __restrict__ x, const uint2* __restrict__ wq, const uint32_t* __restrict__ sz,
     const uint16_t* __restrict__ bias, const uint16_t* residual, uint16_t* y, float* __restrict__ partial, int M, int64_t N,
     int K, int splits, int groups_per_split, I4Fused fz) {
   constexpr bool SILU = EPI == kEpiSilu, ROPE = EPI == kEpiRope, PAIRED = EPI != kEpiPlain;
-  constexpr int NW = PRE > 0 ? 8 : 4;                            // wavefronts of the workgroup; wavefront w takes groups w, w + NW, ...
+  constexpr int NW = 4;                                          // wavefronts of the workgroup; wavefront w takes groups w, w + 4, ...
   __shared__ float sq_s[NORM ? NW * MT * 16 : 1];                 // NORM: per wavefront, per row: sum of squares of its groups
   __shared__ float rstd_s[NORM ? MT * 16 : 1];
   // 4 wavefronts x 2 stages of a [16*MT][64] activation block; reused for the final reduction
   // (two rounds of one accumulator tile set per wavefront)
-  constexpr int kPreBytes = PRE > 0 ? NW * PRE * (1024 + 128) + NW * 16 : 0;   // stages, gains, one block of zeros per wavefront
-  constexpr int kStageBytes = PRE > 0 ? kPreBytes : 4 * 2 * MT * 16 * kXlStride * 2, kRedBytes = 2 * NW * MT * 256 * 4;
+  constexpr int kStageBytes = 4 * 2 * MT * 16 * kXlStride * 2, kRedBytes = 2 * NW * MT * 256 * 4;
   __shared__ __attribute__((aligned(16))) unsigned char lds_raw[kStageBytes > kRedBytes ? kStageBytes : kRedBytes];
   uint16_t* const xstage = (uint16_t*)lds_raw;
   float* const red = (float*)lds_raw;
@@ -357,92 +351,11 @@ __global__ __launch_bounds__(PRE > 0 ? 2 * kI4Threads : kI4Threads) void int4_ge
     __builtin_amdgcn_sched_barrier(0);                                                                  \
   }
 
-  if constexpr (XHALF && PRE == 0) {
+  if constexpr (XHALF) {
     // rows 8..15 of both stages stay zero for the whole kernel
     *(i4_u4*)(&xl[8 * kXlStride + xl_write]) = i4_u4{0u, 0u, 0u, 0u};
     *(i4_u4*)(&xl[(MT * 16 * kXlStride) + 8 * kXlStride + xl_write]) = i4_u4{0u, 0u, 0u, 0u};
   }
-  if constexpr (PRE > 0) {
-    static_assert(PRE == 0 || (XHALF && MT == 1), "the preloading variant exists for 8-row blocks only");
-    unsigned char* const stages = lds_raw + wave * (PRE * 1024);
-    unsigned char* const gains = lds_raw + NW * PRE * 1024 + wave * (PRE * 128);
-    unsigned char* const zeros = lds_raw + NW * PRE * (1024 + 128) + wave * 16;
-    static_assert(PRE * 8 <= 64, "one gain piece per lane");
-    i4_u4 gpiece;
-    (void)gpiece;
-    if constexpr (NORM) {                                        // piece q = 8 J + p of the wavefront's gains: lane q
-      const int q = min(lane, PRE * 8 - 1);
-      gpiece = __builtin_amdgcn_raw_buffer_load_b128(g_rsrc, (q & 7) * 16, min(g_first + NW * (q >> 3), G - 1) * (kGroup * 2), 0);
-    }
-    i4_u4 xall[PRE];
-#pragma unroll
-    for (int J = 0; J < PRE; ++J)
-      xall[J] = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, xg_off, min(g_first + NW * J, G - 1) * (kGroup * 2), 0);
-    // (scale, zero) words: a group's 16 words are 64 bytes, and one request per (group, tile) would be half of all
-    // requests for a ninth of the bytes.  Lane group c fetches the words of steps c and 4 + c instead, two requests
-    // per tile, and a step picks its word up from lane group J % 4 with a cross-lane read.
-    static_assert(PRE <= 8, "two (scale, zero) requests per tile cover eight steps");
-    uint32_t szq[RT][2];
-#pragma unroll
-    for (int t = 0; t < RT; ++t)
-#pragma unroll
-      for (int h = 0; h < 2; ++h) {
-        const int g = wofs[t] + min(g_first + NW * min(4 * h + c, PRE - 1), G - 1);
-        szq[t][h] = __builtin_amdgcn_raw_buffer_load_b32(sz_rsrc, ln * 4 + g * 64, 0, 0);
-      }
-    i4_u2 wall[PRE][RT];
-#pragma unroll
-    for (int J = 0; J < PRE; ++J)
-#pragma unroll
-      for (int t = 0; t < RT; ++t) {
-        const int g = wofs[t] + min(g_first + NW * J, G - 1);
-        wall[J][t] = __builtin_amdgcn_raw_buffer_load_b64(w_rsrc, lane * 8, g * 512, 0);
-      }
-    if (lane == 0) *(i4_u4*)zeros = i4_u4{0u, 0u, 0u, 0u};
-    if constexpr (NORM) {
-      if (lane < PRE * 8) *(i4_u4*)(gains + lane * 16) = gpiece;
-    }
-    const int prow = lane >> 3, ppiece = lane & 7;
-#pragma unroll
-    for (int J = 0; J < PRE; ++J) {
-      i4_u4 piece = xall[J];
-      if constexpr (NORM) {
-        float f_[8], g_[8];
-        unpack8<DT>(piece, f_);
-        unpack8<DT>(*(const i4_u4*)(gains + (J * 8 + ppiece) * 16), g_);
-        float ss_ = 0.f;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) { ss_ = fmaf(f_[e], f_[e], ss_); f_[e] *= g_[e]; }
-        sq[0] += J < nj ? ss_ : 0.f;
-        piece = pack8<DT>(f_);
-      }
-      *(i4_u4*)(stages + J * 1024 + prow * 128 + ((ppiece ^ prow) << 4)) = piece;
-    }
-    const int rd0 = ln * 128 + (((2 * c) ^ ln) << 4), rd1 = ln * 128 + (((2 * c + 1) ^ ln) << 4);
-#pragma unroll
-    for (int J = 0; J < PRE; ++J) {
-      const bool step_live = J < nj;
-      const i4_u4 xa0 = *(const i4_u4*)(ln < 8 ? stages + J * 1024 + rd0 : zeros);
-      const i4_u4 xa1 = *(const i4_u4*)(ln < 8 ? stages + J * 1024 + rd1 : zeros);
-      i4_v4f xs = i4_mfma32<DT>(xa0, ones, i4_v4f{0.f, 0.f, 0.f, 0.f});
-      xs = i4_mfma32<DT>(xa1, ones, xs);
-#pragma unroll
-      for (int t = 0; t < RT; ++t) {
-        const uint32_t w0 = wall[J][t].x, w1 = wall[J][t].y;
-        const uint32_t szw = (uint32_t)__shfl((int)szq[t][J >> 2], (J & 3) * 16 + ln, kWave);
-        const i4_u4 b0 = i4_u4{code_pair(w0, 0, kmagic, kmask), code_pair(w0, 4, kmagic, kmask),
-                               code_pair(w0, 8, kmagic, kmask), code_pair(w0, 12, kmagic, kmask)};
-        const i4_u4 b1 = i4_u4{code_pair(w1, 0, kmagic, kmask), code_pair(w1, 4, kmagic, kmask),
-                               code_pair(w1, 8, kmagic, kmask), code_pair(w1, 12, kmagic, kmask)};
-        const float sc = (step_live && t < ntl) ? f16_bits_to_float(szw & 0xffffu) : 0.f;
-        const float szo = -sc * (f16_bits_to_float(szw >> 16) + I4<DT>::kOffset);
-        i4_v4f raw = i4_mfma32<DT>(xa0, b0, i4_v4f{0.f, 0.f, 0.f, 0.f});
-        raw = i4_mfma32<DT>(xa1, b1, raw);
-#pragma unroll
-        for (int rr = 0; rr < 4; ++rr) acc[t][0][rr] = fmaf(sc, raw[rr], fmaf(szo, xs[rr], acc[t][0][rr]));
-      }
-    }
-  } else {
   // The requests before the loop are issued in the order the loop issues them (activation block, then the weights of
   // the group two steps back), so that the first trip finds the same queue of outstanding requests as every later
   // one: the compiler gives each wait ONE count that must hold on every path into the loop, and a prologue that ends
@@ -476,7 +389,6 @@ __global__ __launch_bounds__(PRE > 0 ? 2 * kI4Threads : kI4Threads) void int4_ge
       SUBSPEC_I4_STEP(1, 1, 1, j + 1);
     }
   }
-  }
   if constexpr (NORM) {
     // the eight lanes that share a row hold its squares over different k; one value per (wavefront, row) goes to LDS
 #pragma unroll
@@ -507,65 +419,6 @@ __global__ __launch_bounds__(PRE > 0 ? 2 * kI4Threads : kI4Threads) void int4_ge
 #undef SUBSPEC_I4_FETCH_W
 #undef SUBSPEC_I4_STEP
 
-  if constexpr (PRE > 0) {
-    // ---- 8-row output stage: every wavefront leaves its accumulators of all tiles in LDS, and after ONE barrier
-    // wavefront m finishes row m: lane (pair or tile, column) sums the eight partials in wavefront order and runs the
-    // output stage of its element, so the rotary arithmetic of a row pair is one evaluation per thread, in parallel
-    // over rows, instead of four in a row on one wavefront.
-#pragma unroll
-    for (int t = 0; t < RT; ++t) *(i4_v4f*)(&red[((t * NW + wave) * 64 + lane) * 4]) = acc[t][0];
-    __syncthreads();
-    const int m = wave;                                          // row of this wavefront (NW == 8 rows)
-    const int item = lane >> 4;                                  // plain: tile; paired: pair of tiles
-    if (m >= M || item >= (PAIRED ? RT / 2 : RT)) return;
-    const int t0 = PAIRED ? 2 * item : item;
-    if (t0 >= ntl) return;
-    auto summed = [&](int t) {
-      float v = 0.f;
-#pragma unroll
-      for (int w = 0; w < NW; ++w) v += red[((t * NW + w) * 64 + (m >> 2) * 16 + ln) * 4 + (m & 3)];
-      if constexpr (NORM) v *= rstd_s[m];
-      return v;
-    };
-    const int64_t n0 = (int64_t)tile_of(t0) * 16 + ln;
-    const float b0v = (splits == 1 && bias) ? I4<DT>::to_float(bias[n0]) : 0.f;
-    const float v0 = summed(t0);
-    if constexpr (!PAIRED) {
-      if (splits == 1) store_linear_out<DT>(y, (int64_t)m * N + n0, v0 + b0v, residual);
-      else partial[((int64_t)ks * M + m) * N + n0] = v0;
-    } else {
-      const int64_t n1 = (int64_t)tile_of(t0 + 1) * 16 + ln;
-      const float b1v = bias ? I4<DT>::to_float(bias[n1]) : 0.f;
-      const float first = Elem<DT>::round(v0 + b0v), second_raw = summed(t0 + 1) + b1v;
-      const int u = unit0 + item;
-      if constexpr (SILU) {
-        const float up = Elem<DT>::round(second_raw);
-        Elem<DT>::store(y, (int64_t)m * (N / 2) + (int64_t)u * 16 + ln, Elem<DT>::round(first / (1.f + __expf(-first))) * up);
-      } else if (u < qk_units) {
-        const int head = u >> 2, d = (u & 3) * 16 + ln;
-        const float inv_freq = fz.inv_freq ? fz.inv_freq[d] : exp2f(-(float)(2 * d) / 128.f * fz.log2_theta);
-        float sn, cs;
-        sincosf((float)fz.positions[m] * inv_freq, &sn, &cs);
-        cs = Elem<DT>::round(cs);
-        sn = Elem<DT>::round(sn);
-        const float lo = first, hi = Elem<DT>::round(second_raw);
-        const float o_lo = Elem<DT>::round(lo * cs) + Elem<DT>::round(-hi * sn);
-        const float o_hi = Elem<DT>::round(hi * cs) + Elem<DT>::round(lo * sn);
-        uint16_t *dst, *unused;
-        if (head < fz.hq) dst = fz.q_out + ((int64_t)head * M + m) * 128;
-        else if (!kv_row_ptrs(fz.kv, head - fz.hq, fz.cache_rows[m], &dst, &unused)) return;   // a row outside the layer's cache is dropped
-        Elem<DT>::store(dst, d, o_lo);
-        Elem<DT>::store(dst, d + 64, o_hi);
-      } else {
-        const int vt = 2 * (u - qk_units), kvh = vt >> 3, d = (vt & 7) * 16 + ln;
-        uint16_t *dst, *unused;
-        if (!kv_row_ptrs(fz.kv, kvh, fz.cache_rows[m], &unused, &dst)) return;
-        Elem<DT>::store(dst, d, first);
-        Elem<DT>::store(dst, d + 16, second_raw);
-      }
-    }
-    return;
-  }
   // ---- sum the four wavefronts' partial accumulators in wavefront order (0, 1, 2, 3), one tile per
   // round.  LDS holds two rounds, so a round needs one barrier; wavefront w finishes the activation
   // row blocks mt = w, w + 4, ... of the tile, so the sums and stores are spread over the workgroup.
@@ -663,6 +516,261 @@ __global__ __launch_bounds__(PRE > 0 ? 2 * kI4Threads : kI4Threads) void int4_ge
   }
 }
 
+// ------------------------------------------------------------------ 1 <= M <= 8, at most 56 groups per workgroup
+// Nothing is pipelined.  Eight wavefronts split the workgroup's K range by group (wavefront w: groups w, w + 8, ..., at
+// most kR8Groups of them); each issues EVERY request it will need before its first wait -- its gains, its activation
+// blocks, the (scale, zero) words of all its tiles, the weight words of its first RTR tiles -- parks the activation blocks
+// (L2 hits, requested first, so waiting for them does not wait for the weights) in private LDS stages while the weights
+// are on their way from HBM, and then runs its steps against registers.  With about one workgroup per compute unit
+// (the projections of a draft level) a short pipeline has nothing to hide a round trip behind and pays one per two
+// steps; here the wavefront pays one.  The workgroup's tiles are taken in NR rounds of RTR: a step of round r hands its
+// weight registers to the same step of round r + 1, so the wavefront keeps kR8Groups * RTR requests in flight until the
+// last round, and the parked activations serve all rounds.
+//
+// LDS: a stage holds the 8 rows x 128 bytes of one group, 16-byte piece p of row r at position p ^ r (conflict-free
+// reads without padding); MFMA rows 8..15 read a block of zeros.  (scale, zero): a group's 16 words are 64 bytes, and one
+// request per (group, tile) would be half of all requests for a ninth of the bytes, so lane group c fetches the words
+// of steps c and 4 + c, two requests per tile, and a step picks its word up from lane group J % 4 with a cross-lane read.
+//
+// Output stage: every wavefront leaves rows 0..7 of its accumulators in LDS, and after one barrier wavefront m finishes
+// row m: a lane sums the eight partials of its element in wavefront order and runs the output stage (plain / SwiGLU /
+// rotary, as in int4_gemm_kernel) once.
+constexpr int kR8Waves = 8, kR8Groups = 7, kR8Threads = kR8Waves * 64;
+template <int DT, int RTR, int NR, int EPI, bool NORM>
+__global__ __launch_bounds__(kR8Threads) void int4_rows8_kernel(
+    const uint16_t* __restrict__ x, const uint2* __restrict__ wq, const uint32_t* __restrict__ sz,
+    const uint16_t* __restrict__ bias, const uint16_t* residual, uint16_t* y, float* __restrict__ partial, int M, int64_t N,
+    int K, int splits, int groups_per_split, I4Fused fz) {
+  constexpr bool SILU = EPI == kEpiSilu, ROPE = EPI == kEpiRope, PAIRED = EPI != kEpiPlain;
+  constexpr int RT = RTR * NR, NW = kR8Waves, NG = kR8Groups;
+  static_assert(NG <= 8, "two (scale, zero) requests per tile cover eight steps");
+  static_assert(NG * 8 <= 64, "one gain piece per lane");
+  constexpr int kStageBytes = NW * NG * (1024 + 128) + NW * 16;   // stages, gains, one block of zeros per wavefront
+  constexpr int kRedBytes = RT * NW * 32 * 16;                     // rows 0..7 of every wavefront's accumulators
+  __shared__ __attribute__((aligned(16))) unsigned char lds_raw[kStageBytes > kRedBytes ? kStageBytes : kRedBytes];
+  __shared__ float sq_s[NORM ? NW * 8 : 1];                      // NORM: per wavefront, per row: sum of squares over its groups
+  __shared__ float rstd_s[NORM ? 8 : 1];
+  float* const red = (float*)lds_raw;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int ln = lane & 15, c = lane >> 4;
+  const int G = K / kGroup;
+  const int n_tiles = (int)(N / 16);
+  const int ks = blockIdx.y;
+  const int g_begin = ks * groups_per_split, g_end = min(G, g_begin + groups_per_split);
+  const int g_first = g_begin + wave;
+  const int nj = g_first < g_end ? (g_end - g_first + NW - 1) / NW : 0;      // <= NG (the host's plan)
+
+  // tiles of this workgroup: an even split of all tiles (SILU / ROPE: of all tile pairs) over the grid; 32-bit unsigned
+  // quotients (the host refuses N / 16 >= 65536, so the products fit)
+  const int n_units = PAIRED ? n_tiles / 2 : n_tiles;
+  const int unit0 = (int)((uint32_t)blockIdx.x * (uint32_t)n_units / gridDim.x);
+  const int n_own = (int)(((uint32_t)blockIdx.x + 1u) * (uint32_t)n_units / gridDim.x) - unit0;
+  const int ntl = PAIRED ? 2 * n_own : n_own;                    // 1 .. RT
+  const int qk_units = ROPE ? (fz.hq + fz.hkv) * 4 : 0;
+  auto tile_of = [&](int t) {
+    if constexpr (SILU) return unit0 + (t >> 1) + (t & 1) * (n_tiles / 2);
+    if constexpr (ROPE) {
+      const int u = unit0 + (t >> 1);
+      return u < qk_units ? (u >> 2) * 8 + (u & 3) + (t & 1) * 4 : 2 * u + (t & 1);
+    }
+    return unit0 + t;
+  };
+
+  const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)x, 0, M * K * 2, 0x00027000);
+  const __amdgpu_buffer_rsrc_t w_rsrc =
+      __builtin_amdgcn_make_buffer_rsrc((void*)wq, 0, (int)(n_tiles * (int64_t)G * 512), 0x00027000);
+  const __amdgpu_buffer_rsrc_t sz_rsrc =
+      __builtin_amdgcn_make_buffer_rsrc((void*)sz, 0, (int)(n_tiles * (int64_t)G * 64), 0x00027000);
+  const __amdgpu_buffer_rsrc_t g_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)(NORM ? fz.norm_gain : x), 0, K * 2, 0x00027000);
+  const int prow = lane >> 3, ppiece = lane & 7;                 // the lane's row and 16-byte piece of an activation block
+  const int xg_off = (prow * K + ppiece * 8) * 2;                // rows past M read zeros (outside the descriptor)
+  int wofs[RT];                                                  // (tile, group 0) in units of groups; tiles past ntl repeat the last
+#pragma unroll
+  for (int t = 0; t < RT; ++t) wofs[t] = tile_of(min(t, ntl - 1)) * G;
+  // both constants of ((w >> s) & mask) | magic as run-time values, so that the compiler emits one v_and_or_b32
+  const uint32_t kmask = 0x000f000fu | (uint32_t)(M >> 30), kmagic = I4<DT>::kMagic | ((uint32_t)xg_off >> 31);
+  const uint32_t one2 = DT == SUBSPEC_BF16 ? 0x3f803f80u : 0x3c003c00u;
+  const i4_u4 ones = i4_u4{one2, one2, one2, one2};
+
+  unsigned char* const stages = lds_raw + wave * (NG * 1024);
+  unsigned char* const gains = lds_raw + NW * NG * 1024 + wave * (NG * 128);
+  unsigned char* const zeros = lds_raw + NW * NG * (1024 + 128) + wave * 16;
+
+  // ---- every request
+  i4_u4 gpiece;
+  (void)gpiece;
+  if constexpr (NORM) {                                          // piece q = 8 J + p of the wavefront's gains: lane q
+    const int q = min(lane, NG * 8 - 1);
+    gpiece = __builtin_amdgcn_raw_buffer_load_b128(g_rsrc, (q & 7) * 16, min(g_first + NW * (q >> 3), G - 1) * (kGroup * 2), 0);
+  }
+  i4_u4 xall[NG];
+#pragma unroll
+  for (int J = 0; J < NG; ++J)
+    xall[J] = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, xg_off, min(g_first + NW * J, G - 1) * (kGroup * 2), 0);
+  // the activation requests stay ahead of all others: a wait for a block that was requested after the weights would
+  // be a wait for the weights
+  __builtin_amdgcn_sched_barrier(0);
+  uint32_t szq[RT][2];
+#pragma unroll
+  for (int t = 0; t < RT; ++t)
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int g = wofs[t] + min(g_first + NW * min(4 * h + c, NG - 1), G - 1);
+      szq[t][h] = __builtin_amdgcn_raw_buffer_load_b32(sz_rsrc, ln * 4 + g * 64, 0, 0);
+    }
+  i4_u2 wall[NG][RTR];
+#pragma unroll
+  for (int J = 0; J < NG; ++J)
+#pragma unroll
+    for (int tt = 0; tt < RTR; ++tt)
+      wall[J][tt] = __builtin_amdgcn_raw_buffer_load_b64(w_rsrc, lane * 8, (wofs[tt] + min(g_first + NW * J, G - 1)) * 512, 0);
+
+  __builtin_amdgcn_sched_barrier(0);
+  // ---- park the activation blocks
+  if (lane == 0) *(i4_u4*)zeros = i4_u4{0u, 0u, 0u, 0u};
+  if constexpr (NORM) {
+    if (lane < NG * 8) *(i4_u4*)(gains + lane * 16) = gpiece;
+  }
+  float sq = 0.f;                                                // NORM: squares of row prow over this wavefront's groups
+  (void)sq;
+#pragma unroll
+  for (int J = 0; J < NG; ++J) {
+    i4_u4 piece = xall[J];
+    if constexpr (NORM) {
+      float f_[8], g_[8];
+      unpack8<DT>(piece, f_);
+      unpack8<DT>(*(const i4_u4*)(gains + (J * 8 + ppiece) * 16), g_);
+      float ss_ = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) { ss_ = fmaf(f_[e], f_[e], ss_); f_[e] *= g_[e]; }
+      sq += J < nj ? ss_ : 0.f;
+      piece = pack8<DT>(f_);
+    }
+    *(i4_u4*)(stages + J * 1024 + prow * 128 + ((ppiece ^ prow) << 4)) = piece;
+  }
+
+  // ---- the steps: round r takes tiles r RTR .. r RTR + RTR - 1; a dead step or tile multiplies by a zero scale
+  i4_v4f acc[RT];
+#pragma unroll
+  for (int t = 0; t < RT; ++t) acc[t] = i4_v4f{0.f, 0.f, 0.f, 0.f};
+  const int rd0 = ln * 128 + (((2 * c) ^ ln) << 4), rd1 = ln * 128 + (((2 * c + 1) ^ ln) << 4);
+#pragma unroll
+  for (int r = 0; r < NR; ++r) {
+#pragma unroll
+    for (int J = 0; J < NG; ++J) {
+      const bool step_live = J < nj;
+      const i4_u4 xa0 = *(const i4_u4*)(ln < 8 ? stages + J * 1024 + rd0 : zeros);
+      const i4_u4 xa1 = *(const i4_u4*)(ln < 8 ? stages + J * 1024 + rd1 : zeros);
+      i4_v4f xs = i4_mfma32<DT>(xa0, ones, i4_v4f{0.f, 0.f, 0.f, 0.f});     // the group's activation sums, rows 4c + rr
+      xs = i4_mfma32<DT>(xa1, ones, xs);
+#pragma unroll
+      for (int tt = 0; tt < RTR; ++tt) {
+        const int t = r * RTR + tt;
+        const uint32_t w0 = wall[J][tt].x, w1 = wall[J][tt].y;
+        if (r + 1 < NR)                                          // the same step of the next round inherits the registers
+          wall[J][tt] = __builtin_amdgcn_raw_buffer_load_b64(w_rsrc, lane * 8, (wofs[min(t + RTR, RT - 1)] + min(g_first + NW * J, G - 1)) * 512, 0);
+        const uint32_t szw = (uint32_t)__shfl((int)szq[t][J >> 2], (J & 3) * 16 + ln, kWave);
+        const i4_u4 b0 = i4_u4{code_pair(w0, 0, kmagic, kmask), code_pair(w0, 4, kmagic, kmask),
+                               code_pair(w0, 8, kmagic, kmask), code_pair(w0, 12, kmagic, kmask)};
+        const i4_u4 b1 = i4_u4{code_pair(w1, 0, kmagic, kmask), code_pair(w1, 4, kmagic, kmask),
+                               code_pair(w1, 8, kmagic, kmask), code_pair(w1, 12, kmagic, kmask)};
+        const float sc = (step_live && t < ntl) ? f16_bits_to_float(szw & 0xffffu) : 0.f;
+        const float szo = -sc * (f16_bits_to_float(szw >> 16) + I4<DT>::kOffset);
+        i4_v4f raw = i4_mfma32<DT>(xa0, b0, i4_v4f{0.f, 0.f, 0.f, 0.f});
+        raw = i4_mfma32<DT>(xa1, b1, raw);
+#pragma unroll
+        for (int rr = 0; rr < 4; ++rr) acc[t][rr] = fmaf(sc, raw[rr], fmaf(szo, xs[rr], acc[t][rr]));
+        // With two rounds the compiler otherwise sinks all these updates below the last MFMA (they are needed only at
+        // the end) and keeps every raw product and scale word alive until then, in scratch memory: the empty statement
+        // makes the accumulator observable here, so the update is evaluated in its step.
+        if constexpr (NR > 1) asm volatile("" : "+v"(acc[t][0]), "+v"(acc[t][1]), "+v"(acc[t][2]), "+v"(acc[t][3]));
+      }
+    }
+  }
+
+  // ---- output stage
+  if constexpr (NORM) {
+    // the eight lanes that share a row hold its squares over different k; one value per (wavefront, row) goes to LDS
+    float v = sq;
+    v += __shfl_xor(v, 1, kWave);
+    v += __shfl_xor(v, 2, kWave);
+    v += __shfl_xor(v, 4, kWave);
+    if (ppiece == 0) sq_s[wave * 8 + prow] = v;
+  }
+  __syncthreads();                                               // every wavefront is done with its stages
+  if constexpr (NORM) {
+    if (tid < 8) {
+      float ss = 0.f;
+#pragma unroll
+      for (int w = 0; w < NW; ++w) ss += sq_s[w * 8 + tid];
+      rstd_s[tid] = rsqrtf(ss / (float)K + fz.norm_eps);
+    }
+  }
+  if (lane < 32) {                                               // accumulator rows 4c + rr: lane groups 0 and 1 hold rows 0..7
+#pragma unroll
+    for (int t = 0; t < RT; ++t) *(i4_v4f*)(&red[((t * NW + wave) * 32 + lane) * 4]) = acc[t];
+  }
+  __syncthreads();
+  const int m = wave;                                            // this wavefront's row
+  if (m >= M) return;
+  auto summed = [&](int t) {
+    float v = 0.f;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) v += red[((t * NW + w) * 32 + (m >> 2) * 16 + ln) * 4 + (m & 3)];
+    if constexpr (NORM) v *= rstd_s[m];
+    return v;
+  };
+  constexpr int kItems = PAIRED ? RT / 2 : RT;                   // lane group c takes items c, c + 4, ...
+#pragma unroll
+  for (int i0 = 0; i0 < kItems; i0 += 4) {
+    const int item = i0 + c;
+    const int t0 = PAIRED ? 2 * item : item;
+    if (item >= kItems || t0 >= ntl) continue;
+    const int64_t n0 = (int64_t)tile_of(t0) * 16 + ln;
+    const float b0v = (splits == 1 && bias) ? I4<DT>::to_float(bias[n0]) : 0.f;
+    const float v0 = summed(t0);
+    if constexpr (!PAIRED) {
+      if (splits == 1) store_linear_out<DT>(y, (int64_t)m * N + n0, v0 + b0v, residual);
+      else partial[((int64_t)ks * M + m) * N + n0] = v0;
+    } else {
+      const int64_t n1 = (int64_t)tile_of(t0 + 1) * 16 + ln;
+      const float b1v = bias ? I4<DT>::to_float(bias[n1]) : 0.f;
+      const float first = Elem<DT>::round(v0 + b0v), second_raw = summed(t0 + 1) + b1v;
+      const int u = unit0 + item;
+      if constexpr (SILU) {
+        // act[m, f] = round(silu(round(gate))) * round(up): the arithmetic of the separate activation kernel
+        const float up = Elem<DT>::round(second_raw);
+        Elem<DT>::store(y, (int64_t)m * (N / 2) + (int64_t)u * 16 + ln, Elem<DT>::round(first / (1.f + __expf(-first))) * up);
+      } else if (u < qk_units) {
+        // rotary pair (d, d + 64) of head u / 4, d = 16 (u % 4) + ln; t * cos + rotate_half(t) * sin with each
+        // product and the sum rounded like the eager tensor ops
+        const int head = u >> 2, d = (u & 3) * 16 + ln;
+        const float inv_freq = fz.inv_freq ? fz.inv_freq[d] : exp2f(-(float)(2 * d) / 128.f * fz.log2_theta);
+        float sn, cs;
+        sincosf((float)fz.positions[m] * inv_freq, &sn, &cs);
+        cs = Elem<DT>::round(cs);
+        sn = Elem<DT>::round(sn);
+        const float lo = first, hi = Elem<DT>::round(second_raw);
+        const float o_lo = Elem<DT>::round(lo * cs) + Elem<DT>::round(-hi * sn);
+        const float o_hi = Elem<DT>::round(hi * cs) + Elem<DT>::round(lo * sn);
+        uint16_t *dst, *unused;
+        if (head < fz.hq) dst = fz.q_out + ((int64_t)head * M + m) * 128;
+        else if (!kv_row_ptrs(fz.kv, head - fz.hq, fz.cache_rows[m], &dst, &unused)) continue;   // a row outside the layer's cache is dropped
+        Elem<DT>::store(dst, d, o_lo);
+        Elem<DT>::store(dst, d + 64, o_hi);
+      } else {
+        // two consecutive tiles of a value head: copied
+        const int vt = 2 * (u - qk_units), kvh = vt >> 3, d = (vt & 7) * 16 + ln;
+        uint16_t *dst, *unused;
+        if (!kv_row_ptrs(fz.kv, kvh, fz.cache_rows[m], &unused, &dst)) continue;
+        Elem<DT>::store(dst, d, first);
+        Elem<DT>::store(dst, d + 16, second_raw);
+      }
+    }
+  }
+}
+
 template <int DT>
 __global__ __launch_bounds__(256) void int4_reduce_kernel(const float* __restrict__ partial,
                                                           const uint16_t* __restrict__ bias, const uint16_t* residual,
@@ -676,12 +784,18 @@ __global__ __launch_bounds__(256) void int4_reduce_kernel(const float* __restric
 }
 
 struct I4Plan { int wgs, row_tiles, splits, groups_per_split; };
-// Groups per wavefront that the preloading variant is compiled for, and the K ranges (in groups per workgroup) it takes:
-// long enough that the pipelined loop would pay several round trips, short enough for the registers and the LDS stages.
-constexpr int kI4Pre = 7;
-// Its workgroups hold 63 KB of LDS, two per compute unit: launches of more than 512 stay with the pipelined variant.
-static bool i4_preload_fits(int groups_per_workgroup, int64_t workgroups) {
-  return groups_per_workgroup > 32 && groups_per_workgroup <= 8 * kI4Pre && workgroups <= 512;
+// The 8-row kernel takes K ranges (groups per workgroup) long enough that the pipelined loop would pay several round
+// trips and short enough for its registers and LDS stages.  Its workgroups hold 63 KB of LDS, two per compute unit.
+constexpr int kR8Range = kR8Waves * kR8Groups;
+static bool i4_rows8_plain(int64_t M, int G) { return M <= 8 && G > 32; }
+// Tile pairs per workgroup of a paired 8-row launch, 0 if it should not be one: one pair while that fits the 512
+// resident workgroups; beyond that whole compute units' worth -- ceil(pairs / 256) pairs each, 3 to 5, in two rounds,
+// so that no compute unit gets a second workgroup while others have one.
+static int i4_rows8_pairs(int64_t M, int G, int64_t pairs) {
+  if (!(M <= 8 && G > 32 && G <= kR8Range)) return 0;
+  if (pairs <= 512) return 1;
+  const int64_t p = (pairs + 255) / 256;
+  return p <= 5 ? (int)std::max<int64_t>(p, 3) : 0;
 }
 
 constexpr int kI4MaxRowTiles = 5;
@@ -691,23 +805,23 @@ static int i4_slots(int64_t M) { return M > 32 ? 512 : 1024; }
 static I4Plan i4_plan(int64_t M, int64_t N, int64_t K) {
   const int G = (int)(K / kGroup);
   const int64_t tiles = N / 16, slots = i4_slots(M);
+  if (i4_rows8_plain(M, G)) {
+    // The 8-row kernel: K ranges of at most 56 groups, and as many tiles per workgroup (1, 2, 3 in one round; 4, 6, 8, 10
+    // in two) as brings the launch down to one workgroup per compute unit.  (Qwen2.5-7B shapes inside the resident
+    // cycle, planned for 256, 400 or 512 resident workgroups: 43.6, 42.9, 42.7 tokens/s.)
+    const int splits = (G + kR8Range - 1) / kR8Range;
+    const int gps = ((G + splits - 1) / splits + 3) / 4 * 4;
+    const int64_t need = (tiles * splits + 255) / 256;
+    const int rt = need <= 3 ? (int)std::max<int64_t>(need, 1) : need <= 4 ? 4 : need <= 6 ? 6 : need <= 8 ? 8 : 10;
+    return I4Plan{(int)((tiles + rt - 1) / rt), rt, (G + gps - 1) / gps, gps};
+  }
   // row tiles per workgroup: the smallest compiled variant that covers all tiles in one resident wave of
   // workgroups; the grid then splits the tiles evenly, so every workgroup has row_tiles or row_tiles - 1
   int row_tiles = i4_row_tile_variant((tiles + slots - 1) / slots);
   // A long K over few tiles (the down projection) is split over workgroups, and every split re-reads its slice of the
-  // activations: two tiles per workgroup halve that traffic (3584x18944, 8 rows, five splits: 13.8 -> 12.7 us; three or
-  // five tiles per workgroup and fewer splits were slower: 14.1 to 15.7 us)
+  // activations: two tiles per workgroup halve that traffic (3584x18944, 16 rows, five splits; three or
+  // five tiles per workgroup and fewer splits were slower)
   if (M <= 16 && row_tiles == 1 && tiles * 4 <= slots && G >= 112) row_tiles = 2;
-  if (M <= 8 && G >= 112) {
-    // At most 8 rows and a long K: ranges of at most 56 groups, which the preloading variant takes (all of a
-    // workgroup's weights requested at once), over as many tiles per workgroup (at most 3) as keeps the launch within
-    // the 512 workgroups that are resident at its LDS use (3584x18944: 12.2 -> ? us)
-    const int splits = (G + 8 * kI4Pre - 1) / (8 * kI4Pre);
-    const int gps = ((G + splits - 1) / splits + 3) / 4 * 4;
-    int rt = 1;
-    while (rt < 3 && (tiles + rt - 1) / rt * splits > 512) ++rt;
-    return I4Plan{(int)((tiles + rt - 1) / rt), rt, (G + gps - 1) / gps, gps};
-  }
   const int64_t wgs = (tiles + row_tiles - 1) / row_tiles;
   int splits = (int)std::max<int64_t>(1, (slots + wgs / 2) / wgs);
   // a split costs a second launch (the reduction) and fp32 partials: it pays from about 56 groups
@@ -735,11 +849,7 @@ static int run_int4_paired(const void* x, const uint32_t* wq, const uint32_t* sz
   const int G = (int)(K / kGroup);
   const bool norm = fz.norm_gain != nullptr;
 #define SUBSPEC_I4_PAIRED(MT, RT, NORM)                                                                            \
-  if (MT == 1 && M <= 8 && RT <= 2 && i4_preload_fits(G, wgs))                                                          \
-    hipLaunchKernelGGL((int4_gemm_kernel<DT, 1, RT, EPI, NORM, true, (RT <= 2 ? kI4Pre : 0)>), grid, dim3(2 * kI4Threads), 0, st, \
-                       (const uint16_t*)x, (const uint2*)wq, sz, (const uint16_t*)bias, (const uint16_t*)nullptr, (uint16_t*)out, \
-                       (float*)nullptr, (int)M, N, (int)K, 1, (G + 3) / 4 * 4, fz);                                \
-  else if (MT == 1 && M <= 8)                                                                                      \
+  if (MT == 1 && M <= 8)                                                                                           \
     hipLaunchKernelGGL((int4_gemm_kernel<DT, 1, RT, EPI, NORM, true>), grid, dim3(kI4Threads), 0, st, (const uint16_t*)x, \
                        (const uint2*)wq, sz, (const uint16_t*)bias, (const uint16_t*)nullptr, (uint16_t*)out, (float*)nullptr, \
                        (int)M, N, (int)K, 1, (G + 3) / 4 * 4, fz);                                                 \
@@ -749,6 +859,25 @@ static int run_int4_paired(const void* x, const uint32_t* wq, const uint32_t* sz
                      (int)M, N, (int)K, 1, (G + 3) / 4 * 4, fz)
 #define SUBSPEC_I4_PAIRED_RT(MT, NORM) do { if (rt == 2) SUBSPEC_I4_PAIRED(MT, 2, NORM); else SUBSPEC_I4_PAIRED(MT, 4, NORM); } while (0)
   DominantKernelTimer timer(st);
+  const int p8_plan = i4_rows8_pairs(M, G, pairs);
+  if (const int p8 = (EPI == kEpiRope && p8_plan > 1) ? 0 : p8_plan) {
+    const dim3 grid8((unsigned)((pairs + p8 - 1) / p8), 1);
+#define SUBSPEC_I4_ROWS8(RTR, NR, NORM)                                                                            \
+  hipLaunchKernelGGL((int4_rows8_kernel<DT, RTR, NR, EPI, NORM>), grid8, dim3(kR8Threads), 0, st, (const uint16_t*)x, \
+                     (const uint2*)wq, sz, (const uint16_t*)bias, (const uint16_t*)nullptr, (uint16_t*)out, (float*)nullptr,   \
+                     (int)M, N, (int)K, 1, kR8Range, fz)
+#define SUBSPEC_I4_ROWS8_P(NORM)                                                                                   \
+  do {                                                                                                             \
+    if (p8 == 1) SUBSPEC_I4_ROWS8(2, 1, NORM);                                                                     \
+    else if constexpr (EPI == kEpiRope) return SUBSPEC_ERR_LIMIT;                                                  \
+    else if (p8 == 3) SUBSPEC_I4_ROWS8(3, 2, NORM);                                                                \
+    else if (p8 == 4) SUBSPEC_I4_ROWS8(4, 2, NORM);                                                                \
+    else SUBSPEC_I4_ROWS8(5, 2, NORM);                                                                             \
+  } while (0)
+    if (norm) SUBSPEC_I4_ROWS8_P(true); else SUBSPEC_I4_ROWS8_P(false);
+#undef SUBSPEC_I4_ROWS8_P
+#undef SUBSPEC_I4_ROWS8
+  } else
   if (M <= 16) { if (norm) SUBSPEC_I4_PAIRED_RT(1, true); else SUBSPEC_I4_PAIRED_RT(1, false); }
   else if (M <= 32) { if (norm) SUBSPEC_I4_PAIRED_RT(2, true); else SUBSPEC_I4_PAIRED_RT(2, false); }
   else {
@@ -766,7 +895,7 @@ static int run_int4(const void* x, const uint32_t* wq, const uint32_t* sz, const
                     int64_t M, int64_t N, int64_t K, void* workspace, hipStream_t st) {
   // One row: the GEMV kernel, unless the matrix has few rows and a long K (down projection): then its one workgroup
   // per 16-row tile leaves most of the chip idle and the split-K GEMM path is faster (3584x18944 from HBM: 22 against 32 us).
-  if (M == 1 && i4_plan(M, N, K).splits == 1) {
+  if (M == 1 && !i4_rows8_plain(M, (int)(K / kGroup)) && i4_plan(M, N, K).splits == 1) {
     const size_t smem = (size_t)K * 2 + (size_t)(K / 16) * 4 + 64 * 4;
     DominantKernelTimer timer(st);
     hipLaunchKernelGGL((int4_gemv_kernel<DT>), dim3((unsigned)(N / 16)), dim3(kI4Threads), smem, st, (const uint16_t*)x,
@@ -776,16 +905,16 @@ static int run_int4(const void* x, const uint32_t* wq, const uint32_t* sz, const
     float* partial = (float*)workspace;
     const dim3 grid((unsigned)pl.wgs, (unsigned)pl.splits);
 #define SUBSPEC_I4_LAUNCH(MT, RT)                                                                                  \
-  if (MT == 1 && M <= 8 && RT <= 3 && i4_preload_fits(pl.groups_per_split, (int64_t)pl.wgs * pl.splits))                                        \
-    hipLaunchKernelGGL((int4_gemm_kernel<DT, 1, RT, kEpiPlain, false, true, (RT <= 3 ? kI4Pre : 0)>), grid, dim3(2 * kI4Threads), 0, st, \
-                       (const uint16_t*)x, (const uint2*)wq, sz, (const uint16_t*)bias, (const uint16_t*)residual, (uint16_t*)y, partial, \
-                       (int)M, N, (int)K, pl.splits, pl.groups_per_split, I4Fused{});                              \
-  else if (MT == 1 && M <= 8)                                                                                      \
+  if (MT == 1 && M <= 8)                                                                                           \
     hipLaunchKernelGGL((int4_gemm_kernel<DT, 1, RT, kEpiPlain, false, true>), grid, dim3(kI4Threads), 0, st, (const uint16_t*)x, \
                        (const uint2*)wq, sz, (const uint16_t*)bias, (const uint16_t*)residual, (uint16_t*)y, partial, (int)M, N, (int)K, \
                        pl.splits, pl.groups_per_split, I4Fused{});                                                 \
   else                                                                                                             \
   hipLaunchKernelGGL((int4_gemm_kernel<DT, MT, RT>), grid, dim3(kI4Threads), 0, st, (const uint16_t*)x,            \
+                     (const uint2*)wq, sz, (const uint16_t*)bias, (const uint16_t*)residual, (uint16_t*)y, partial, (int)M, N, (int)K, \
+                     pl.splits, pl.groups_per_split, I4Fused{})
+#define SUBSPEC_I4_ROWS8(RTR, NR)                                                                                  \
+  hipLaunchKernelGGL((int4_rows8_kernel<DT, RTR, NR, kEpiPlain, false>), grid, dim3(kR8Threads), 0, st, (const uint16_t*)x, \
                      (const uint2*)wq, sz, (const uint16_t*)bias, (const uint16_t*)residual, (uint16_t*)y, partial, (int)M, N, (int)K, \
                      pl.splits, pl.groups_per_split, I4Fused{})
 #define SUBSPEC_I4_LAUNCH_MT(MT)                                                                                   \
@@ -797,10 +926,22 @@ static int run_int4(const void* x, const uint32_t* wq, const uint32_t* sz, const
   } while (0)
     {
       DominantKernelTimer timer(st);
+      if (i4_rows8_plain(M, (int)(K / kGroup))) {
+        switch (pl.row_tiles) {
+          case 1: SUBSPEC_I4_ROWS8(1, 1); break;
+          case 2: SUBSPEC_I4_ROWS8(2, 1); break;
+          case 3: SUBSPEC_I4_ROWS8(3, 1); break;
+          case 4: SUBSPEC_I4_ROWS8(2, 2); break;
+          case 6: SUBSPEC_I4_ROWS8(3, 2); break;
+          case 8: SUBSPEC_I4_ROWS8(4, 2); break;
+          default: SUBSPEC_I4_ROWS8(5, 2); break;
+        }
+      } else
       if (M <= 16) SUBSPEC_I4_LAUNCH_MT(1);
       else if (M <= 32) SUBSPEC_I4_LAUNCH_MT(2);
       else SUBSPEC_I4_LAUNCH_MT(4);
     }
+#undef SUBSPEC_I4_ROWS8
 #undef SUBSPEC_I4_LAUNCH_MT
 #undef SUBSPEC_I4_LAUNCH
     if (pl.splits > 1)
