@@ -90,6 +90,19 @@ def test_random_shape_sweep():
         _check(N, K, M, torch.bfloat16 if i % 2 == 0 else torch.float16, 950 + i, bias=bool(i % 2))
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_rows_up_to_8_long_k(dtype):
+    """At most 8 rows and K > 2048 take the kernel that issues every request up front: every tile count per
+    workgroup it is compiled for (1, 2, 3 in one round; 4, 6, 8, 10 in two), launches beyond one workgroup per
+    compute unit, K ranges that are not multiples of 8 groups (dead steps), several K ranges, ragged last
+    workgroups, with and without bias."""
+    cases = [(16 * 7, 64 * 33, 3), (16 * 300, 64 * 40, 8), (16 * 601, 64 * 56, 5), (16 * 1000, 64 * 35, 2),
+             (16 * 1501, 64 * 34, 8), (16 * 1900, 64 * 33, 1), (16 * 2400, 64 * 34, 7), (16 * 3001, 64 * 33, 8),
+             (16 * 9, 64 * 57, 8), (16 * 130, 64 * 120, 4), (16 * 224, 64 * 296, 6), (16 * 40, 64 * 1000, 8)]
+    for i, (N, K, M) in enumerate(cases):
+        _check(N, K, M, dtype, 1200 + i, bias=bool(i % 2))
+
+
 def test_quantizer_default_refines_zero_points():
     """HqqQuantizer.quantize_model refines the zero points unless told not to (as hqq does); the module then
     computes the affine dequantization of those tensors, and its output is at least as close to the unquantized
@@ -124,7 +137,10 @@ def test_gate_up_projection_with_the_activation_in_its_output_stage(dtype):
     count, one and two tile pairs per workgroup, with and without bias."""
     for seed, (F, K, M, bias) in enumerate([(16, 64, 1, False), (48, 192, 5, True), (512, 256, 16, False), (1184, 128, 17, True),
                                             (18944, 3584, 8, False), (18944, 3584, 64, False), (2048, 512, 33, True),
-                                            (40000, 64, 3, False)]):
+                                            (40000, 64, 3, False),
+                                            # 8 rows, K > 2048: one, three, four and five tile pairs per workgroup
+                                            (16 * 500, 2112, 8, True), (9728, 2112, 8, False), (14336, 2240, 5, True),
+                                            (16 * 1190, 2176, 1, False), (16 * 1500, 2112, 8, False)]):
         print("gate|up + silu", dtype, F, K, M, bias, flush=True)
         g = torch.Generator().manual_seed(700 + seed)
         W = torch.randn(2 * F, K, generator=g) * (2.0 / K ** 0.5)
@@ -139,9 +155,16 @@ def test_gate_up_projection_with_the_activation_in_its_output_stage(dtype):
         want = ((gate / (1 + torch.exp(-gate))).to(dtype).float() * up).to(dtype)
         assert got.shape == (M, F) and got.dtype == dtype
         differing = int((got != want).sum())
-        assert differing <= max(1, got.numel() // 1000), (F, K, M, differing)
+        # more than five tile pairs per compute unit: the fused launch stays on the four-wavefront kernel while the
+        # plain projection of 8 rows takes the eight-wavefront one, so the partial sums are grouped differently
+        same_grouping = not (M <= 8 and K > 2048 and F // 16 > 1280)
+        if same_grouping:
+            assert differing <= max(1, got.numel() // 1000), (F, K, M, differing)
         ulp = 2.0 ** (-7 if dtype == torch.bfloat16 else -10)
-        assert ((got.float() - want.float()).abs() <= 2 * ulp * want.float().abs() + 1e-6).all()
+        # (with another grouping a projection that nearly cancels differs by its absolute rounding, not by a unit in
+        # the last place: the bound is then absolute, against the largest output)
+        atol = 1e-6 if same_grouping else 2e-3 * want.float().abs().amax().item()
+        assert ((got.float() - want.float()).abs() <= (2 if same_grouping else 4) * ulp * want.float().abs() + atol).all()
     with pytest.raises(ValueError):
         ops.int4_gate_up_silu(torch.zeros(65, 64, dtype=dtype, device=DEV), torch.zeros(2 * 32 * 64 // 8, dtype=torch.int32, device=DEV),
                               torch.zeros(2 * 32, dtype=torch.int32, device=DEV), 32)          # more than 64 rows
