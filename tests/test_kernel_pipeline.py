@@ -18,7 +18,16 @@ import pytest
 from subspec_amd import build as build_mod
 
 
+_ASSEMBLY = {}                                               # source path -> assembly text (one compilation per run)
+
+
 def _assembly(src: str, tmp_path) -> str:
+    if src not in _ASSEMBLY:
+        _ASSEMBLY[src] = _compile_to_assembly(src, tmp_path)
+    return _ASSEMBLY[src]
+
+
+def _compile_to_assembly(src: str, tmp_path) -> str:
     hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
     if not os.path.exists(hipcc):
         pytest.skip("hipcc is not installed")
@@ -67,3 +76,42 @@ def test_main_loops_never_wait_for_every_request(source, kernel, min_kernels, tm
     stalled = [(k, n, w) for k, n, w in main_loops if w]
     assert not stalled, "a full wait inside the pipelined loop of: " + ", ".join(
         f"{k} (loop of {n} lines, at {w})" for k, n, w in stalled)
+
+
+def _kernel_bodies(asm: str, kernel_substring: str):
+    """{kernel: lines of its body} for every matching kernel."""
+    bodies, kernel = {}, None
+    for line in asm.split("\n"):
+        m = re.match(r"^(_Z\w+):", line)
+        if m:
+            kernel = m.group(1) if kernel_substring in m.group(1) else None
+            if kernel:
+                bodies[kernel] = []
+            continue
+        if kernel:
+            bodies[kernel].append(line)
+            if "s_endpgm" in line:
+                kernel = None
+    return bodies
+
+
+def test_the_8_row_kernel_keeps_its_requests_in_order_and_its_registers(tmp_path):
+    """int4_rows8_kernel issues every request before its first wait and relies on three things no result can show:
+    the activation blocks are requested before any weight word (vector memory returns in order, so a block requested
+    after the weights could only be waited for together with them), the steps stream (their waits leave later requests
+    outstanding), and nothing lives in scratch memory (without a pin the compiler sinks the accumulator updates of the
+    two-round variants below the last MFMA and spills every raw product)."""
+    asm = _assembly(os.path.join(build_mod.CSRC, "int4.hip"), tmp_path)
+    bodies = _kernel_bodies(asm, "int4_rows8_kernel")
+    assert len(bodies) >= 20, "the parser found too few kernel variants"
+    for kernel, lines in bodies.items():
+        assert not any("scratch_" in l for l in lines), f"{kernel} uses scratch memory"
+        loads = [(i, l) for i, l in enumerate(lines) if re.search(r"\bbuffer_load_dword", l)]
+        x_loads = [i for i, l in loads if "dwordx4" in l]                # activation blocks (and the gain piece)
+        w_loads = [i for i, l in loads if "dwordx2" in l]                # weight words
+        assert x_loads and w_loads, kernel
+        assert max(x_loads) < min(w_loads), f"{kernel}: an activation block is requested after a weight word"
+        first_mfma = next(i for i, l in enumerate(lines) if "v_mfma" in l)
+        waits = [int(m.group(1)) for l in lines[:first_mfma + 40] for m in [re.search(r"vmcnt\((\d+)\)", l)] if m]
+        # the wait in front of the first product leaves the weight words of the later steps on their way
+        assert waits and min(waits) >= 4, f"{kernel}: the first step waits for (nearly) every request: {sorted(set(waits))}"
