@@ -78,6 +78,8 @@ def parse():
     ap.add_argument("--draft-graph", action="store_true",
                     help="e2e workload: replay each speculation (all draft levels) from a captured HIP graph")
     ap.add_argument("--keep-layers", type=int, default=14, help="e2e workload: target layers kept resident; the rest stream")
+    ap.add_argument("--ring-slabs", type=int, default=4,
+                    help="e2e workload: device slabs of the streaming ring (layers the copies may run ahead of compute)")
     ap.add_argument("--workload", default="verify-cycle", choices=["verify-cycle", "attention", "int4", "dense", "greedy", "sampling", "topk", "e2e"],
                     help="verify-cycle (default, BASELINE config 2) is the benchmark line; the others time one "
                          "kernel family of configs 1, 3 and 4 and print one JSON line per shape")
@@ -260,7 +262,8 @@ def e2e_runs(args, runs, new_tokens, say=lambda *_: None):
                     w[name + ".weight"] = quant.dequantize(*quant.quantize_int4_g64(t)).to(t.dtype)
         kv = create_kv_cache("static", max_cache_len=2048 + new_tokens + 512 + 8, config=cfg, device=dev, dtype=torch.bfloat16)
         target, draft, _ = build_models(cfg, kv, seed=0, device=dev, first_streamed=min(keep_layers, cfg.num_hidden_layers),
-                                        weights=weights, hqq_optimize=args.hqq_optimize)
+                                        weights=weights, hqq_optimize=args.hqq_optimize,
+                                        n_slabs=getattr(args, "ring_slabs", 4))
         say(f"# models built in {time.perf_counter() - t0:.1f} s (resident target layers: {keep_layers}, agreeing draft: {agreeing})")
         prompt = torch.randint(0, cfg.vocab_size, (1, 2048), generator=torch.Generator().manual_seed(0)).to(dev)
         for method, vk in (("exact", None), ("lossy", dict(threshold=0.3, window_size=6, threshold_method="entropy"))):
@@ -293,6 +296,7 @@ def e2e_runs(args, runs, new_tokens, say=lambda *_: None):
                                        + (", post-speculating driver" if v2 else ""),
                            "verify_method": method, "generator": args.generator,
                            "draft_graph_replays": gen.draft_model.graph_replays, "resident_target_layers": min(keep_layers, cfg.num_hidden_layers),
+                           "ring_slabs": (target.streamer.n_slabs if target.streamer is not None else 0),
                            "agreeing_draft": bool(agreeing),
                            **({"post_verify_count": log["post_verify_count"], "speculate_count": log["speculate_count"]} if v2 else {}), "n_iter": log["n_iter"], "n_tokens": log["n_tokens"],
                            "tokens_per_cycle": round(log["avg_sampled"], 3),

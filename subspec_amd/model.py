@@ -384,9 +384,11 @@ def weights_from_tensors(cfg: DecoderConfig, tensors: Dict[str, torch.Tensor], d
 
 
 def build_models(cfg: DecoderConfig, kv: KVManager, seed: int = 0, device="cuda:0", dtype=torch.bfloat16,
-                 first_streamed: Optional[int] = None, weights: Optional[dict] = None, hqq_optimize: bool = False):
+                 first_streamed: Optional[int] = None, weights: Optional[dict] = None, hqq_optimize: bool = False,
+                 n_slabs: int = 4):
     """Target (bf16, layers >= first_streamed in pinned host memory) and substitute draft (same
-    weights, int4 g64, resident) over one shared KV cache."""
+    weights, int4 g64, resident) over one shared KV cache.  ``n_slabs``: device slabs of the streaming ring, i.e.
+    how many layers the copies may run ahead of the compute stream (``LayerStreamer``)."""
     w = init_weights(cfg, seed, device, dtype) if weights is None else weights     # e.g. from load_hf_checkpoint
     draft_layers = quantize_layers(w["layers"], optimize=hqq_optimize)
     streamer = None
@@ -394,7 +396,7 @@ def build_models(cfg: DecoderConfig, kv: KVManager, seed: int = 0, device="cuda:
     if first_streamed is not None and first_streamed < cfg.num_hidden_layers:
         layout = LayerSlabLayout(layer_shapes(cfg), dtype)
         host = [{k: v.cpu() for k, v in layers[i].items()} for i in range(first_streamed, cfg.num_hidden_layers)]
-        streamer = LayerStreamer(layout, host, device)
+        streamer = LayerStreamer(layout, host, device, n_slabs=n_slabs)
         layers = layers[:first_streamed]
     target = Decoder(cfg, w["embed"], layers, w["norm"], w["lm_head"], kv, streamer, first_streamed)
     draft = Decoder(cfg, w["embed"], draft_layers, w["norm"], w["lm_head"], kv)

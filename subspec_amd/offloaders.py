@@ -46,7 +46,10 @@ class OffloadState:
 class PrefetchOffloader:
     n_slabs = 4
 
-    def __init__(self, model: nn.Module, device_map: Dict[str, object], draft_model=None, **_unused):
+    def __init__(self, model: nn.Module, device_map: Dict[str, object], draft_model=None, n_slabs: Optional[int] = None,
+                 **_unused):
+        if n_slabs is not None:
+            self.n_slabs = int(n_slabs)                  # ring depth: layers the copies may run ahead (default of the class)
         missing = _uncovered(model, device_map)
         if missing:
             raise ValueError("The device_map provided does not give any device for the following parameters: "

@@ -68,12 +68,23 @@ class Recipe(QuantOffloadRecipe):
     host memory and streamed (recipes/subspec/hqq_4bit_postspec.py:10-58 offloads every quantized layer, i.e.
     ``keep_first_n_layers_on_gpu = 0``, the default here too)."""
 
-    def __init__(self, keep_first_n_layers_on_gpu: int = 0, nbits: int = 4, group_size: int = 64):
+    def __init__(self, keep_first_n_layers_on_gpu: int = 0, nbits: int = 4, group_size: int = 64,
+                 prefetch_slabs: Optional[int] = None):
         super().__init__()
         self.quantizer = HqqQuantizer
         self.offloader = PrefetchOffloader
         self.keep_first_n_layers_on_gpu = int(keep_first_n_layers_on_gpu)
         self.nbits, self.group_size = int(nbits), int(group_size)
+        # Device slabs of the streaming ring (None: the offloader's default of 4).  The copies of the next forward run
+        # that many layers ahead, through verification and speculation; with a deep draft tree (the reference's
+        # depth 48: 100 ms of speculation per cycle) a deeper ring keeps the link busy for all of it, at 466 MB of HBM
+        # per slab at the Qwen2.5-7B shape.
+        self.prefetch_slabs = prefetch_slabs
+
+    def apply_offloading(self, model, device_map, draft_model=None):
+        if self.prefetch_slabs is None:
+            return super().apply_offloading(model, device_map, draft_model=draft_model)
+        return self.offloader(model, device_map=device_map, draft_model=draft_model, n_slabs=self.prefetch_slabs)
 
     def generate_configurations(self, target_model, draft_model, max_length, cpu_offload_gb, dtype, device):
         layer_cnt = len(target_model.model.layers)

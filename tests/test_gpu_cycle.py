@@ -28,27 +28,31 @@ CFG = DecoderConfig(num_hidden_layers=4, hidden_size=256, num_attention_heads=2,
                     head_dim=128, intermediate_size=512, vocab_size=2048)
 
 
-def _models(first_streamed=None, max_len=256, seed=3):
+def _models(first_streamed=None, max_len=256, seed=3, n_slabs=4):
     kv = create_kv_cache("static", max_cache_len=max_len, config=CFG, device=DEV, dtype=torch.bfloat16)
-    target, draft, w = build_models(CFG, kv, seed=seed, device=DEV, first_streamed=first_streamed)
+    target, draft, w = build_models(CFG, kv, seed=seed, device=DEV, first_streamed=first_streamed, n_slabs=n_slabs)
     return kv, target, draft, w
 
 
-def test_streamed_forward_is_bit_identical_to_resident():
+@pytest.mark.parametrize("first_streamed,n_slabs,ring", [(2, 4, 2), (1, 2, 2), (0, 3, 3), (0, 9, 4)])
+def test_streamed_forward_is_bit_identical_to_resident(first_streamed, n_slabs, ring):
+    """Every ring depth: fewer slabs than streamed layers (slabs are reused inside one forward), as many, and a
+    request for more than there are layers (clamped)."""
     prompt = torch.randint(0, CFG.vocab_size, (40,), generator=torch.Generator().manual_seed(1)).to(DEV)
     kv_a, tgt_a, _, _ = _models(first_streamed=None)
-    kv_b, tgt_b, _, _ = _models(first_streamed=2)
+    kv_b, tgt_b, _, _ = _models(first_streamed=first_streamed, n_slabs=n_slabs)
     la = tgt_a.prefill(prompt, 0)
     lb = tgt_b.prefill(prompt, 0)
-    assert tgt_b.streamer is not None and tgt_b.streamer.n == 2
+    n = CFG.num_hidden_layers - first_streamed
+    assert tgt_b.streamer is not None and tgt_b.streamer.n == n and tgt_b.streamer.n_slabs == ring
     assert torch.equal(la, lb)
     assert torch.equal(kv_a.cache.data, kv_b.cache.data)
     # several forwards in a row reuse the two slabs; still identical
     for _ in range(3):
         assert torch.equal(tgt_a.prefill(prompt[:7], 40), tgt_b.prefill(prompt[:7], 40))
-    # 4 forwards x 2 streamed layers, plus the prefetch of the next forward's first layers that the ring keeps in flight
+    # 4 forwards x n streamed layers, plus the prefetch of the next forward's first layers that the ring keeps in flight
     st = tgt_b.streamer
-    assert 4 * 2 * st.layout.nbytes <= st.bytes_streamed <= (4 * 2 + st.n_slabs - 1) * st.layout.nbytes
+    assert 4 * n * st.layout.nbytes <= st.bytes_streamed <= (4 * n + st.n_slabs - 1) * st.layout.nbytes
 
 
 def test_draft_tree_levels_are_canonical_topk():

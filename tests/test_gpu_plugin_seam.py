@@ -41,7 +41,10 @@ def _greedy_continuation(path, seq, start, tag):
 def test_builder_sequence_runs_the_cycle(tmp_path, method):
     path = str(tmp_path)
     write_checkpoint(path, hf=HF, seed=3)
-    recipe = resolve("subspec_amd.recipes:Recipe")(keep_first_n_layers_on_gpu=2)
+    v2 = method.endswith("v2")
+    # v2: three streamed layers through a ring of two slabs (the recipe's prefetch_slabs), v1: two through the default
+    recipe = resolve("subspec_amd.recipes:Recipe")(**(dict(keep_first_n_layers_on_gpu=1, prefetch_slabs=2) if v2
+                                                      else dict(keep_first_n_layers_on_gpu=2)))
     b = builder_stub(recipe, device=DEV)
     b.max_length = 160
     StubRegistry.entries.clear()
@@ -54,7 +57,7 @@ def test_builder_sequence_runs_the_cycle(tmp_path, method):
                                                                  cpu_offload_gb=None, dtype=b.dtype, device=DEV)
     recipe.apply_quantization(draft.model, draft_config["quant_config"], b.dtype, DEV)
     off = recipe.apply_offloading(model, target_config["device_map"], draft_model=draft)
-    assert off.first_streamed == 2 and off.streamer.n == 2
+    assert (off.first_streamed, off.streamer.n, off.streamer.n_slabs) == ((1, 3, 2) if v2 else (2, 2, 2))
     # placement: resident layers and the draft's int4 tiles on the GPU, streamed layers alias their pinned slabs
     assert model.model.layers[0].mlp.up_proj.weight.device.type == "cuda" and model.lm_head.weight.device.type == "cuda"
     assert model.model.layers[3].mlp.up_proj.weight.device.type == "cpu" and model.model.layers[3].mlp.up_proj.weight.is_pinned()
