@@ -525,7 +525,10 @@ __global__ __launch_bounds__(kI4Threads) void int4_gemm_kernel(
 // (the projections of a draft level) a short pipeline has nothing to hide a round trip behind and pays one per two
 // steps; here the wavefront pays one.  The workgroup's tiles are taken in NR rounds of RTR: a step of round r hands its
 // weight registers to the same step of round r + 1, so the wavefront keeps kR8Groups * RTR requests in flight until the
-// last round, and the parked activations serve all rounds.
+// last round, and the parked activations serve all rounds.  Many tiles go in rounds of two: nothing can be multiplied
+// before the first round's words are there, so a first round of five tiles (half of the SwiGLU projection's ten) is
+// 6.8 us of pure transfer in front of 9.7 us of steps, a first round of two 3 us (37888 x 3584: 22.9 -> 20.2 us per
+// call); rounds of one tile gain nothing more (14 requests per wavefront in flight cover the latency, 7 just do).
 //
 // LDS: a stage holds the 8 rows x 128 bytes of one group, 16-byte piece p of row r at position p ^ r (conflict-free
 // reads without padding); MFMA rows 8..15 read a block of zeros.  (scale, zero): a group's 16 words are 64 bytes, and one
@@ -681,7 +684,7 @@ __global__ __launch_bounds__(kR8Threads) void int4_rows8_kernel(
         raw = i4_mfma32<DT>(xa1, b1, raw);
 #pragma unroll
         for (int rr = 0; rr < 4; ++rr) acc[t][rr] = fmaf(sc, raw[rr], fmaf(szo, xs[rr], acc[t][rr]));
-        // With two rounds the compiler otherwise sinks all these updates below the last MFMA (they are needed only at
+        // With several rounds the compiler otherwise sinks all these updates below the last MFMA (they are needed only at
         // the end) and keeps every raw product and scale word alive until then, in scratch memory: the empty statement
         // makes the accumulator observable here, so the update is evaluated in its step.
         if constexpr (NR > 1) asm volatile("" : "+v"(acc[t][0]), "+v"(acc[t][1]), "+v"(acc[t][2]), "+v"(acc[t][3]));
@@ -789,8 +792,8 @@ struct I4Plan { int wgs, row_tiles, splits, groups_per_split; };
 constexpr int kR8Range = kR8Waves * kR8Groups;
 static bool i4_rows8_plain(int64_t M, int G) { return M <= 8 && G > 32; }
 // Tile pairs per workgroup of a paired 8-row launch, 0 if it should not be one: one pair while that fits the 512
-// resident workgroups; beyond that whole compute units' worth -- ceil(pairs / 256) pairs each, 3 to 5, in two rounds,
-// so that no compute unit gets a second workgroup while others have one.
+// resident workgroups; beyond that whole compute units' worth -- ceil(pairs / 256) pairs each, 3 to 5, in rounds of
+// one pair, so that no compute unit gets a second workgroup while others have one.
 static int i4_rows8_pairs(int64_t M, int G, int64_t pairs) {
   if (!(M <= 8 && G > 32 && G <= kR8Range)) return 0;
   if (pairs <= 512) return 1;
@@ -807,7 +810,7 @@ static I4Plan i4_plan(int64_t M, int64_t N, int64_t K) {
   const int64_t tiles = N / 16, slots = i4_slots(M);
   if (i4_rows8_plain(M, G)) {
     // The 8-row kernel: K ranges of at most 56 groups, and as many tiles per workgroup (1, 2, 3 in one round; 4, 6, 8, 10
-    // in two) as brings the launch down to one workgroup per compute unit.  (Qwen2.5-7B shapes inside the resident
+    // in rounds of two) as brings the launch down to one workgroup per compute unit.  (Qwen2.5-7B shapes inside the resident
     // cycle, planned for 256, 400 or 512 resident workgroups: 43.6, 42.9, 42.7 tokens/s.)
     const int splits = (G + kR8Range - 1) / kR8Range;
     const int gps = ((G + splits - 1) / splits + 3) / 4 * 4;
@@ -870,9 +873,9 @@ static int run_int4_paired(const void* x, const uint32_t* wq, const uint32_t* sz
   do {                                                                                                             \
     if (p8 == 1) SUBSPEC_I4_ROWS8(2, 1, NORM);                                                                     \
     else if constexpr (EPI == kEpiRope) return SUBSPEC_ERR_LIMIT;                                                  \
-    else if (p8 == 3) SUBSPEC_I4_ROWS8(3, 2, NORM);                                                                \
-    else if (p8 == 4) SUBSPEC_I4_ROWS8(4, 2, NORM);                                                                \
-    else SUBSPEC_I4_ROWS8(5, 2, NORM);                                                                             \
+    else if (p8 == 3) SUBSPEC_I4_ROWS8(2, 3, NORM);                                                                \
+    else if (p8 == 4) SUBSPEC_I4_ROWS8(2, 4, NORM);                                                                \
+    else SUBSPEC_I4_ROWS8(2, 5, NORM);                                                                             \
   } while (0)
     if (norm) SUBSPEC_I4_ROWS8_P(true); else SUBSPEC_I4_ROWS8_P(false);
 #undef SUBSPEC_I4_ROWS8_P
@@ -932,9 +935,9 @@ static int run_int4(const void* x, const uint32_t* wq, const uint32_t* sz, const
           case 2: SUBSPEC_I4_ROWS8(2, 1); break;
           case 3: SUBSPEC_I4_ROWS8(3, 1); break;
           case 4: SUBSPEC_I4_ROWS8(2, 2); break;
-          case 6: SUBSPEC_I4_ROWS8(3, 2); break;
-          case 8: SUBSPEC_I4_ROWS8(4, 2); break;
-          default: SUBSPEC_I4_ROWS8(5, 2); break;
+          case 6: SUBSPEC_I4_ROWS8(2, 3); break;
+          case 8: SUBSPEC_I4_ROWS8(2, 4); break;
+          default: SUBSPEC_I4_ROWS8(2, 5); break;
         }
       } else
       if (M <= 16) SUBSPEC_I4_LAUNCH_MT(1);
