@@ -104,16 +104,24 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
   __shared__ __attribute__((aligned(16))) uint16_t Vs2[2][kKeyBlock * kVStride];
 
   // workgroups of one (batch, kv head, chunk) unit sit in consecutive slots of one XCD
-  const int64_t lin = blockIdx.x;
-  const int xcd = (int)(lin % kXcds);
-  const int64_t slot = lin / kXcds;
-  const int pair = (int)(slot % ap.pairs_per_kv);
-  const int64_t unit = (slot / ap.pairs_per_kv) * kXcds + xcd;
-  if (unit >= ap.units) return;
-  const int chunk = (int)(unit % ap.chunks);
-  const int64_t bkv = unit / ap.chunks;
-  const int kvh = (int)(bkv % ap.hkv), b = (int)(bkv / ap.hkv);
-  const int group = (int)(ap.hq / ap.hkv);
+  // Every kernel argument is wanted in a scalar register HERE: left alone, the compiler fetches the fields of the
+  // parameter block where they are first used, in six batches with a wait each -- six dependent round trips to the
+  // scalar cache (cold at every launch) before the first key is requested.
+  asm volatile("" ::"s"(ap.batch), "s"(ap.hq), "s"(ap.hkv), "s"(ap.n_rows), "s"(ap.n_slots), "s"(ap.seq_stride), "s"(ap.prefix),
+               "s"(ap.anc_batch_stride), "s"(ap.mask_words), "s"(ap.row0), "s"(ap.win_rows), "s"(ap.chunks), "s"(ap.chunk_keys),
+               "s"(ap.pairs_per_kv), "s"(ap.units), "s"(ap.scale_log2), "s"(ap.prefix_dev), "s"(ap.page_table),
+               "s"(ap.page_shift), "s"(ap.max_pages), "s"(ap.page_stride), "s"(ap.tok_stride), "s"(ap.v_delta));
+  asm volatile("" ::"s"(q), "s"(kc), "s"(vc), "s"(anc), "s"(out), "s"(part_o), "s"(part_ml));
+  const uint32_t lin = blockIdx.x;
+  const int xcd = (int)(lin % (uint32_t)kXcds);
+  const uint32_t slot = lin / (uint32_t)kXcds;
+  const int pair = (int)(slot % (uint32_t)ap.pairs_per_kv);
+  const uint32_t unit = (slot / (uint32_t)ap.pairs_per_kv) * (uint32_t)kXcds + (uint32_t)xcd;
+  if ((int64_t)unit >= ap.units) return;
+  const int chunk = (int)(unit % (uint32_t)ap.chunks);
+  const uint32_t bkv = unit / (uint32_t)ap.chunks;
+  const int kvh = (int)(bkv % (uint32_t)ap.hkv), b = (int)(bkv / (uint32_t)ap.hkv);
+  const int group = (int)((uint32_t)ap.hq / (uint32_t)ap.hkv);
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int lq = lane & 15, lg = lane >> 4;            // query column of the lane, lane group

@@ -544,6 +544,16 @@ __global__ __launch_bounds__(kR8Threads) void int4_rows8_kernel(
     const uint16_t* __restrict__ x, const uint2* __restrict__ wq, const uint32_t* __restrict__ sz,
     const uint16_t* __restrict__ bias, const uint16_t* residual, uint16_t* y, float* __restrict__ partial, int M, int64_t N,
     int K, int splits, int groups_per_split, I4Fused fz) {
+  // Every argument is wanted in a scalar register HERE: left alone, the compiler fetches the fields of the parameter
+  // block where they are first used -- several batches with a wait each before the first request, and more in the
+  // output stage (positions, cache rows, the cache map), each a round trip to the scalar cache that is cold at every launch.
+  asm volatile("" ::"s"(x), "s"(wq), "s"(sz), "s"(bias), "s"(residual), "s"(y), "s"(partial), "s"(M), "s"(N), "s"(K), "s"(splits),
+               "s"(groups_per_split));
+  if constexpr (NORM) asm volatile("" ::"s"(fz.norm_gain), "s"(fz.norm_eps));
+  if constexpr (EPI == kEpiRope)
+    asm volatile("" ::"s"(fz.positions), "s"(fz.cache_rows), "s"(fz.q_out), "s"(fz.kv.k_cache), "s"(fz.kv.v_cache),
+                 "s"(fz.kv.seq_stride), "s"(fz.kv.page_table), "s"(fz.kv.page_shift), "s"(fz.kv.max_pages), "s"(fz.kv.hkv),
+                 "s"(fz.kv.page_elems), "s"(fz.inv_freq), "s"(fz.hq), "s"(fz.hkv), "s"(fz.log2_theta));
   constexpr bool SILU = EPI == kEpiSilu, ROPE = EPI == kEpiRope, PAIRED = EPI != kEpiPlain;
   constexpr int RT = RTR * NR, NW = kR8Waves, NG = kR8Groups;
   static_assert(NG <= 8, "two (scale, zero) requests per tile cover eight steps");
