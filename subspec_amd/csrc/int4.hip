@@ -405,7 +405,7 @@ __global__ __launch_bounds__(kI4Threads) void int4_gemm_kernel(
   }
   __syncthreads();                                               // the stages are reused for the reduction below
   if constexpr (NORM) {
-    // ordered before its first use by the barrier of reduction round 0
+    // ordered before its first use by the barrier of the first reduction round
     if (tid < MT * 16)
     {
       float ss = 0.f;
