@@ -668,6 +668,7 @@ __global__ __launch_bounds__(kR8Threads) void int4_rows8_kernel(
 #pragma unroll
   for (int t = 0; t < RT; ++t) acc[t] = i4_v4f{0.f, 0.f, 0.f, 0.f};
   const int rd0 = ln * 128 + (((2 * c) ^ ln) << 4), rd1 = ln * 128 + (((2 * c + 1) ^ ln) << 4);
+  i4_v4f xsum[NG];
 #pragma unroll
   for (int r = 0; r < NR; ++r) {
 #pragma unroll
@@ -675,8 +676,11 @@ __global__ __launch_bounds__(kR8Threads) void int4_rows8_kernel(
       const bool step_live = J < nj;
       const i4_u4 xa0 = *(const i4_u4*)(ln < 8 ? stages + J * 1024 + rd0 : zeros);
       const i4_u4 xa1 = *(const i4_u4*)(ln < 8 ? stages + J * 1024 + rd1 : zeros);
-      i4_v4f xs = i4_mfma32<DT>(xa0, ones, i4_v4f{0.f, 0.f, 0.f, 0.f});     // the group's activation sums, rows 4c + rr
-      xs = i4_mfma32<DT>(xa1, ones, xs);
+      if (r == 0) {                                              // the group's activation sums, rows 4c + rr: kept for all rounds
+        xsum[J] = i4_mfma32<DT>(xa0, ones, i4_v4f{0.f, 0.f, 0.f, 0.f});
+        xsum[J] = i4_mfma32<DT>(xa1, ones, xsum[J]);
+      }
+      const i4_v4f xs = xsum[J];
 #pragma unroll
       for (int tt = 0; tt < RTR; ++tt) {
         const int t = r * RTR + tt;
