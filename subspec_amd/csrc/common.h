@@ -113,6 +113,7 @@ __device__ __forceinline__ void store_linear_out(void* y, int64_t i, float v, co
 }
 
 // ---------------------------------------------------------------- eight 16-bit elements in one 16-byte piece
+
 typedef uint32_t dec_u4 __attribute__((ext_vector_type(4)));
 
 template <int DT>

@@ -47,7 +47,11 @@ struct Part3 { float key; int32_t idx; };             // best race key of a slic
 template <int DT, int VEC> struct Tile;
 template <> struct Tile<SUBSPEC_F32, 4> {
   float4 r;
-  __device__ __forceinline__ void load(const void* p, int64_t i) { r = *(const float4*)((const float*)p + i); }
+  __device__ __forceinline__ void load(const void* p, int64_t i) {
+    typedef float f4v __attribute__((ext_vector_type(4)));
+    const f4v v = __builtin_nontemporal_load((const f4v*)((const float*)p + i));
+    r = make_float4(v.x, v.y, v.z, v.w);
+  }
   __device__ __forceinline__ void fill_neg_inf() { r = make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY); }
   __device__ __forceinline__ float get(int k) const { return k == 0 ? r.x : k == 1 ? r.y : k == 2 ? r.z : r.w; }
   __device__ __forceinline__ void fence() { asm volatile("" : "+v"(r.x), "+v"(r.y), "+v"(r.z), "+v"(r.w)); }
@@ -61,7 +65,13 @@ template <> struct Tile<SUBSPEC_F32, 1> {
 };
 template <int DT> struct Tile16x8 {
   uint4 r;
-  __device__ __forceinline__ void load(const void* p, int64_t i) { r = *(const uint4*)((const uint16_t*)p + i); }
+  // streaming (non-temporal) load: every element of the rows is read once, and fetched that way the rows do not
+  // displace each other in the L2 on their way through (2048 x 152064 bf16: 109 -> 105 us, 112 -> 103 us)
+  __device__ __forceinline__ void load(const void* p, int64_t i) {
+    typedef uint32_t u4v __attribute__((ext_vector_type(4)));
+    const u4v v = __builtin_nontemporal_load((const u4v*)((const uint16_t*)p + i));
+    r = make_uint4(v.x, v.y, v.z, v.w);
+  }
   __device__ __forceinline__ void fill_neg_inf() {
     const uint32_t w = DT == SUBSPEC_BF16 ? 0xff80ff80u : 0xfc00fc00u;
     r = make_uint4(w, w, w, w);
