@@ -542,7 +542,9 @@ constexpr int kR8Waves = 8, kR8Groups = 7, kR8Threads = kR8Waves * 64;
 // Cache policy of this kernel's weight requests (the auxiliary operand of the buffer-load builtins, bit 1 =
 // non-temporal): every weight byte is read once per launch, so it is fetched as streaming data that does not displace
 // the activations and the other launches' lines in the L2 (37888 x 3584, 8 rows, from HBM: 20.1 -> 18.7 us per call).
-// The same hint changes nothing in the pipelined kernel at 16 or 64 rows and costs the dense kernels 15 to 20 %.
+// The same hint changes nothing in the pipelined kernel at 16 or 64 rows and costs the dense kernels 15 to 25 %: their
+// wavefronts fetch each 128-byte line with two requests (a lane's 32 bytes are two 16-byte loads), and a streamed line
+// does not wait in the first-level cache for the second one.  A request of this kernel covers whole lines.
 constexpr int kStream = 2;
 template <int DT, int RTR, int NR, int EPI, bool NORM>
 __global__ __launch_bounds__(kR8Threads) void int4_rows8_kernel(
