@@ -52,6 +52,7 @@ template <> struct Tile<SUBSPEC_F32, 4> {
     const f4v v = __builtin_nontemporal_load((const f4v*)((const float*)p + i));
     r = make_float4(v.x, v.y, v.z, v.w);
   }
+  __device__ __forceinline__ void load_cached(const void* p, int64_t i) { r = *(const float4*)((const float*)p + i); }
   __device__ __forceinline__ void fill_neg_inf() { r = make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY); }
   __device__ __forceinline__ float get(int k) const { return k == 0 ? r.x : k == 1 ? r.y : k == 2 ? r.z : r.w; }
   __device__ __forceinline__ void fence() { asm volatile("" : "+v"(r.x), "+v"(r.y), "+v"(r.z), "+v"(r.w)); }
@@ -59,6 +60,7 @@ template <> struct Tile<SUBSPEC_F32, 4> {
 template <> struct Tile<SUBSPEC_F32, 1> {
   float r;
   __device__ __forceinline__ void load(const void* p, int64_t i) { r = ((const float*)p)[i]; }
+  __device__ __forceinline__ void load_cached(const void* p, int64_t i) { load(p, i); }
   __device__ __forceinline__ void fill_neg_inf() { r = -INFINITY; }
   __device__ __forceinline__ float get(int) const { return r; }
   __device__ __forceinline__ void fence() { asm volatile("" : "+v"(r)); }
@@ -72,6 +74,8 @@ template <int DT> struct Tile16x8 {
     const u4v v = __builtin_nontemporal_load((const u4v*)((const uint16_t*)p + i));
     r = make_uint4(v.x, v.y, v.z, v.w);
   }
+  // ordinary load, for a tile that is read again soon (the reference tile of a slice)
+  __device__ __forceinline__ void load_cached(const void* p, int64_t i) { r = *(const uint4*)((const uint16_t*)p + i); }
   __device__ __forceinline__ void fill_neg_inf() {
     const uint32_t w = DT == SUBSPEC_BF16 ? 0xff80ff80u : 0xfc00fc00u;
     r = make_uint4(w, w, w, w);
@@ -103,6 +107,7 @@ template <> struct Tile<SUBSPEC_F16, 8> : Tile16x8<SUBSPEC_F16> {};
 template <int DT> struct Tile16x1 {
   uint16_t r;
   __device__ __forceinline__ void load(const void* p, int64_t i) { r = ((const uint16_t*)p)[i]; }
+  __device__ __forceinline__ void load_cached(const void* p, int64_t i) { load(p, i); }
   __device__ __forceinline__ void fill_neg_inf() { r = DT == SUBSPEC_BF16 ? 0xff80 : 0xfc00; }
   __device__ __forceinline__ float get(int) const {
     return DT == SUBSPEC_BF16 ? bf16_bits_to_float(r) : f16_bits_to_float(r);
@@ -288,7 +293,7 @@ __global__ __launch_bounds__(kRowThreads) void row_partial_kernel(
   float ref;
   {
     Tile<DT, VEC> t0;
-    if (tid < ntiles) t0.load(logits, base + (int64_t)tid * VEC); else t0.fill_neg_inf();
+    if (tid < ntiles) t0.load_cached(logits, base + (int64_t)tid * VEC); else t0.fill_neg_inf();   // the loop reads it again
     float r = warped<DT, WARP>(t0.get(0), vp.temperature);
 #pragma unroll
     for (int k = 1; k < VEC; ++k) r = fmaxf(r, warped<DT, WARP>(t0.get(k), vp.temperature));
