@@ -115,3 +115,26 @@ def test_the_8_row_kernel_keeps_its_requests_in_order_and_its_registers(tmp_path
         waits = [int(m.group(1)) for l in lines[:first_mfma + 40] for m in [re.search(r"vmcnt\((\d+)\)", l)] if m]
         # the wait in front of the first product leaves the weight words of the later steps on their way
         assert waits and min(waits) >= 4, f"{kernel}: the first step waits for (nearly) every request: {sorted(set(waits))}"
+
+
+def test_no_hand_written_instruction_sits_next_to_an_mfma():
+    """With MFMA results kept in ordinary vector registers (-amdgpu-mfma-vgpr-form=1) the compiler inserts the wait
+    states between an MFMA and the vector ALU instruction that reads its result, but only for instructions it emitted
+    itself: a vector ALU instruction written as inline assembly is opaque to that pass and has read half-written
+    accumulators.  The kernels therefore contain no assembly TEXT at all -- every asm statement is an empty one that
+    only pins a value to a register class (the constants of v_and_or_b32 are made opaque by arithmetic on run-time
+    values instead) -- and this test keeps it that way."""
+    pattern = re.compile(r"\basm\s*(?:volatile)?\s*\(\s*\"([^\"]*)\"")
+    seen = 0
+    for name in sorted(os.listdir(build_mod.CSRC)):
+        if not name.endswith((".hip", ".h")):
+            continue
+        with open(os.path.join(build_mod.CSRC, name)) as f:
+            text = f.read()
+        for m in pattern.finditer(text):
+            seen += 1
+            line = text.count("\n", 0, m.start()) + 1
+            assert m.group(1).strip() == "", f"{name}:{line}: inline assembly with instruction text: {m.group(1)!r}"
+        assert "__asm__" not in text, f"{name}: __asm__ spelling is not covered by this check"
+    assert seen >= 8, "the pattern no longer finds the register pins it is meant to inspect"
+    assert "-amdgpu-mfma-vgpr-form=1" in build_mod.HIPCC_FLAGS
