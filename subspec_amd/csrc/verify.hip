@@ -748,10 +748,12 @@ __global__ __launch_bounds__(kTailThreads) void tree_accept_kernel(
 struct Plan { int vec, splits; int64_t chunk; };
 
 // Slices per row; a slice is a whole number of 512-thread tiles.
-// Greedy target: one slice, whatever the number of rows.  The workgroup that holds a whole row decides by itself
-// whether the row needs the exact pass and runs it while the row is in cache; splitting a row means a second launch
-// that recombines the slices first, and that launch costs more than the few workgroups of a small batch lose
-// (152064 columns, bf16: 64 rows 31 -> 26 us per call, 256 rows 62 -> 42 us, 512 rows 84 -> 71 us; one row 30 -> 27 us).
+// Greedy target: one slice from 256 rows on.  The workgroup that holds a whole row decides by itself whether the row
+// needs the exact pass and runs it while the row is in cache.  Fewer rows are cut into up to 8 slices, about 256
+// workgroups in all, although that costs a second launch (row_exact_kernel, which recombines the slices and returns at
+// once for a row that needs nothing): a compute unit streams at a fixed rate, and 64 workgroups leave three quarters
+// of the chip idle (64 x 152064 fp32: statistics pass 15.7 -> 6 us, a call with reused output tensors 20.7 -> 17.9 us;
+// calls that allocate their outputs are bound by the host at 26 us either way).
 // Sampling target: the draw is bound by the vector ALU (a Philox block per four elements), so few rows are cut
 // into enough slices to cover the chip several times over.
 static bool make_plan(const void* logits, int dtype, int64_t total_rows, int64_t vocab, bool sample, Plan* pl) {
@@ -759,7 +761,7 @@ static bool make_plan(const void* logits, int dtype, int64_t total_rows, int64_t
   const bool aligned = (vocab % vec_full == 0) && ((uintptr_t)logits % 16 == 0);
   pl->vec = aligned ? vec_full : 1;
   const int64_t quantum = (int64_t)kRowThreads * pl->vec;
-  int64_t splits = sample ? (2048 + total_rows - 1) / total_rows : 1;
+  int64_t splits = sample ? (2048 + total_rows - 1) / total_rows : std::min<int64_t>(8, std::max<int64_t>(1, 256 / total_rows));
   splits = std::min<int64_t>(splits, std::max<int64_t>(1, vocab / 8192));
   splits = std::max<int64_t>(1, std::min<int64_t>(splits, kMaxSplits));
   int64_t chunk = (vocab + splits - 1) / splits;
