@@ -135,6 +135,7 @@ struct VerifyParams {
   float theta;
   float ln_vocab;       // float(ln V), or 1 when V == 1 (lossy_tree_verify.py:68)
   int sample;           // 1: the target token of a row is drawn from its distribution
+  int ties_in_accept;   // 1: sliced rows without the exact pass (no entropy gate): the acceptance kernel resolves ties
   Divisor temperature;  // rows are divided by .t (and rounded to their dtype) when .t != 1
   uint32_t key[2];      // Philox key: the caller's 64-bit seed
   uint32_t offset[2];   // Philox counter words 2, 3: the caller's 64-bit stream offset
@@ -550,15 +551,22 @@ __global__ __launch_bounds__(kTailThreads) void tree_accept_kernel(
   int status = 0;
 
   // ---- per scored row: max, sum, argmax token, entropy
+  bool tie_rows[kSlots];
+  float tie_pmax[kSlots];
 #pragma unroll
   for (int s = 0; s < kSlots; ++s) {
     const int r = s * kWave + lane;
+    tie_rows[s] = false;
+    tie_pmax[s] = 0.f;
     if (r < rows) {
       const int64_t grow = (int64_t)b * rows + r;
       const RowStat rs = combine_row<DT>(part1 + grow * vp.splits, vp);
       int tgt = rs.first_idx;
       float h = rs.h;
-      if (rs.need_emu || rs.need_tie) {
+      if (vp.ties_in_accept) {
+        tie_rows[s] = rs.need_tie;                     // resolved below, by the whole wavefront
+        tie_pmax[s] = rs.pmax;
+      } else if (rs.need_emu || rs.need_tie) {
         float H = 0.f;
         int tie = 0x7fffffff;
         for (int c = 0; c < vp.splits; ++c) {
@@ -586,6 +594,32 @@ __global__ __launch_bounds__(kTailThreads) void tree_accept_kernel(
     }
   }
   __syncthreads();
+  // Sliced rows of a run without the entropy gate come without the exact pass.  A row whose rounded probabilities
+  // may tie with the maximum (a maximum below 2 in magnitude, or a subnormal rounded maximum: not what a language
+  // model's logits look like) is scanned here by the whole wavefront: first index whose rounded probability equals
+  // the rounded maximum, as row_exact_body finds it.  Slow (a row per pass), and next to never taken.
+  if (vp.ties_in_accept) {
+#pragma unroll
+    for (int s = 0; s < kSlots; ++s) {
+      uint64_t pending = __ballot(tie_rows[s]);
+      while (pending) {                                // uniform
+        const int src = __builtin_ctzll(pending);
+        pending &= pending - 1;
+        const int r = s * kWave + src;
+        const float m = sm_m[r], S = sm_S[r], pmax = __shfl(tie_pmax[s], src, kWave);
+        const int64_t base = ((int64_t)b * rows + r) * vp.vocab;
+        int tie = 0x7fffffff;
+        for (int64_t i = lane; i < vp.vocab && tie == 0x7fffffff; i += kWave)
+          if (rounded_prob<DT>(load_warped<DT>(logits, base + i, vp), m, S) == pmax) tie = (int)i;
+        tie = wave_min_i(tie);
+        if (lane == src && tie != 0x7fffffff) {
+          sm_tgt[r] = tie;
+          node_target[(int64_t)b * rows + r] = tie;
+        }
+      }
+    }
+    __syncthreads();
+  }
 
   // ---- per node: token, parent, p[parent(i), token(i)]
   int tok[kSlots], par[kSlots];
@@ -750,10 +784,12 @@ struct Plan { int vec, splits; int64_t chunk; };
 // Slices per row; a slice is a whole number of 512-thread tiles.
 // Greedy target: one slice from 256 rows on.  The workgroup that holds a whole row decides by itself whether the row
 // needs the exact pass and runs it while the row is in cache.  Fewer rows are cut into up to 8 slices, about 256
-// workgroups in all, although that costs a second launch (row_exact_kernel, which recombines the slices and returns at
-// once for a row that needs nothing): a compute unit streams at a fixed rate, and 64 workgroups leave three quarters
-// of the chip idle (64 x 152064 fp32: statistics pass 15.7 -> 6 us, a call with reused output tensors 20.7 -> 17.9 us;
-// calls that allocate their outputs are bound by the host at 26 us either way).
+// workgroups in all: a compute unit streams at a fixed rate, and 64 workgroups leave three quarters of the chip idle
+// (64 x 152064 fp32: statistics pass 15.7 -> 6 us).  With the entropy gate that costs a second launch (row_exact_kernel,
+// which recombines the slices and returns at once for a row that needs nothing); without it the only thing the exact
+// pass could find is a tie of rounded probabilities with the maximum, and the acceptance kernel looks for that itself
+// in the rows that can have one.  A prepared call: 20.7 us with one workgroup per row, 15.1 with slices and the second
+// launch, 12.6 without it; calls that allocate their outputs are bound by the host at 26 us either way.
 // Sampling target: the draw is bound by the vector ALU (a Philox block per four elements), so few rows are cut
 // into enough slices to cover the chip several times over.
 static bool make_plan(const void* logits, int dtype, int64_t total_rows, int64_t vocab, bool sample, Plan* pl) {
@@ -799,7 +835,8 @@ static int run_verify(const void* logits, int64_t batch, int64_t rows, int64_t v
   };
   // the timed kernel is the longest one: the statistics pass, or the draw when sampling
   if (vp.sample) partial(); else { DominantKernelTimer timer(st); partial(); }
-  if (pl.splits > 1) hipLaunchKernelGGL((row_exact_kernel<DT>), grid, dim3(kRowThreads), 0, st, logits, vp, p1, p2);
+  if (pl.splits > 1 && !vp.ties_in_accept)
+    hipLaunchKernelGGL((row_exact_kernel<DT>), grid, dim3(kRowThreads), 0, st, logits, vp, p1, p2);
   if (vp.sample) {
     DominantKernelTimer timer(st);
     // slices are whole numbers of 512-thread tiles of pl.vec elements: with pl.vec > 1 rows and slices are quad-aligned
@@ -888,6 +925,7 @@ static int tree_verify_impl(const void* logits, int dtype, int64_t batch, int64_
   vp.theta = (float)threshold;
   vp.ln_vocab = vocab > 1 ? (float)log((double)vocab) : 1.0f;
   vp.sample = sa.sample;
+  vp.ties_in_accept = (pl.splits > 1 && !vp.gate_entropy && !sa.sample) ? 1 : 0;
   vp.temperature = make_divisor(sa.temperature);
   vp.key[0] = (uint32_t)sa.seed;
   vp.key[1] = (uint32_t)(sa.seed >> 32);

@@ -118,6 +118,33 @@ def test_config1_greedy_fp32_full_vocab(seed):
     assert out["target"][0].tolist() == torch.softmax(cfg["logits"], -1).argmax(-1).tolist()
 
 
+def test_prepared_call_follows_its_tensors():
+    """A prepared call launches on the tensors it was made with: new inputs are written INTO them, the outputs are
+    the same dictionary every time, and every call agrees with the oracle and with a plain tree_verify call."""
+    cfgs = [W.greedy_config(seed) for seed in (3, 4)]
+    logits = cfgs[0]["logits"].to(DEV).clone()
+    tok = torch.tensor(cfgs[0]["tokens"], dtype=torch.int32, device=DEV)
+    par = torch.tensor(cfgs[0]["parents"], dtype=torch.int32, device=DEV)
+    prepared = ops.PreparedTreeVerify(logits, tok, par)
+    for cfg in cfgs + cfgs[:1]:
+        logits.copy_(cfg["logits"])
+        tok.copy_(torch.tensor(cfg["tokens"], dtype=torch.int32))
+        par.copy_(torch.tensor(cfg["parents"], dtype=torch.int32))
+        out = prepared()
+        assert out is prepared.out
+        torch.cuda.synchronize()
+        got = {k: v.cpu() for k, v in out.items()}
+        assert _unpack(got) == ov.verify_logits(cfg["logits"], cfg["tokens"], cfg["parents"])
+        plain = _run(cfg["logits"], cfg["tokens"], cfg["parents"])
+        for key in ("tokens", "contexts"):
+            n = got["counts"][0, 0].item()
+            assert torch.equal(got[key][0, :n], plain[key][0, :n]), key
+        for key in ("counts", "target", "entropy", "child_prob"):
+            assert torch.equal(got[key], plain[key]), key
+    with pytest.raises(ValueError):
+        ops.PreparedTreeVerify(logits, tok.to(torch.int64), par)
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_config2_lossy_entropy_full_vocab(dtype):
     cfg = W.lossy_config(seed=3, batch=5, dtype=dtype)
@@ -163,7 +190,10 @@ def test_near_threshold_rows_take_the_rounded_path():
     assert torch.equal(out["entropy"][0][near], ref_h[near])
 
 
-@pytest.mark.parametrize("dtype,vocab", [(torch.float16, 1001), (torch.float32, 777), (torch.bfloat16, 50257)])
+# the long vocabularies are cut into slices (few rows): without the entropy gate the acceptance kernel then looks for
+# ties of the rounded probabilities itself, with it the exact pass is a launch of its own
+@pytest.mark.parametrize("dtype,vocab", [(torch.float16, 1001), (torch.float32, 777), (torch.bfloat16, 50257),
+                                         (torch.bfloat16, 65536), (torch.float16, 40000), (torch.float32, 32768)])
 def test_ragged_vocab_and_ties(dtype, vocab):
     torch.manual_seed(11)
     n = 9
