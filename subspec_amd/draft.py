@@ -120,9 +120,10 @@ class SubSpecSDDraftModel:
         ``max_depth - 1`` tree steps.  With ``prefix_len_dev`` no launch depends on the actual prefix length."""
         dev = self.decoder.device
         self._prefix_len_dev, self._prefix_bound = prefix_len_dev, prefix_len
+        pos32, rows32 = self._slot_tables(prefix_len, prefix_len_dev, rebuild=True)
         logits = self.decoder.tree_forward(root, torch.zeros(1, dtype=torch.long, device=dev),
                                            torch.ones(1, dtype=torch.int64, device=dev), prefix_len,
-                                           prefix_len_dev=prefix_len_dev)
+                                           prefix_len_dev=prefix_len_dev, positions32=pos32[0:1], rows32=rows32[0:1])
         self.levels = []
         self.level_state = {}                                                      # depth -> what speculate_once needs
         self.level_bits = self._own_bits(dev)[0:1].clone()                         # root: slot 0 (no host value involved)
@@ -187,6 +188,28 @@ class SubSpecSDDraftModel:
             self._own_bits_table = table = table.to(device)
         return table
 
+    def _slot_tables(self, prefix_len: int, prefix_len_dev: Optional[torch.Tensor], rebuild: bool = False):
+        """Rotary position and cache row of every tree slot, int32 [MAX_SLOTS] each, for the current prefix: slot 0 is
+        the root, slot s > 0 belongs to level 1 + (s - 1) // k.  Worked out once per speculation (two small launches);
+        a level takes its slice.  Per level it was five launches of a few microseconds each on the level's critical
+        path (fill, add, arange, two conversions)."""
+        k = self.draft_params.topk_len
+        dev = self.decoder.device
+        const = getattr(self, "_slot_const", None)
+        if const is None or const[0] != (k, str(dev)):
+            slots = torch.arange(MAX_SLOTS, dtype=torch.int32)
+            depth = torch.where(slots == 0, torch.zeros_like(slots), 1 + (slots - 1) // max(k, 1))
+            const = self._slot_const = ((k, str(dev)), depth.to(dev), slots.to(dev))
+        key = (k, int(prefix_len)) if prefix_len_dev is None else None      # a device-side prefix: rebuilt every time
+        held = getattr(self, "_slot_held", None)
+        if rebuild or key is None or held is None or held[0] != key:
+            if prefix_len_dev is None:
+                held = (key, const[1] + int(prefix_len), const[2] + int(prefix_len))
+            else:
+                held = (None, (const[1] + prefix_len_dev).to(torch.int32), (const[2] + prefix_len_dev).to(torch.int32))
+            self._slot_held = held
+        return held[1], held[2]
+
     def _expand(self, sampled_probs: torch.Tensor, parent_probs: torch.Tensor) -> None:
         k = self.draft_params.topk_len
         token_ids, child_probs, parent_indices = self.topk_sampling(sampled_probs, parent_probs, k)
@@ -207,13 +230,18 @@ class SubSpecSDDraftModel:
         total = self.first_slot + n
         if total > MAX_SLOTS:
             raise ValueError(f"draft tree exceeds the {MAX_SLOTS} tree slots of the attention mask")
-        depths = torch.full((n,), self.depth, dtype=torch.long, device=dev)
         bits = self.level_bits[:, 0].contiguous() if total <= 64 else self.level_bits[:, :(total + 63) // 64].contiguous()
         dyn = getattr(self, "_prefix_len_dev", None)
         # inside _grow_levels the prefix length may live on the device; prefix_len is then the bound the launches use
-        logits = self.decoder.tree_forward(self.token_ids[0], depths, bits,
-                                           self._prefix_bound if dyn is not None else self.prefix_len,
-                                           first_slot=self.first_slot, prefix_len_dev=dyn)
+        prefix = self._prefix_bound if dyn is not None else self.prefix_len
+        tables = {}
+        if n == self.draft_params.topk_len and self.first_slot == 1 + (self.depth - 1) * n:
+            # the regular tree (every level k nodes): positions and rows are slices of the speculation's tables
+            pos32, rows32 = self._slot_tables(prefix, dyn)
+            tables = dict(positions32=pos32[self.first_slot:total], rows32=rows32[self.first_slot:total])
+        depths = None if tables else torch.full((n,), self.depth, dtype=torch.long, device=dev)
+        logits = self.decoder.tree_forward(self.token_ids[0], depths, bits, prefix,
+                                           first_slot=self.first_slot, prefix_len_dev=dyn, **tables)
         self._expand(self._probs(logits).unsqueeze(0), self.parent_probs)
 
     def update_tree(self, cap: bool = False) -> Tree:

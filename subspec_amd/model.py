@@ -163,7 +163,8 @@ class Decoder:
         return self._native
 
     def _run_native_layers(self, x, positions, rows, anc_bits, prefix_len: int, slots: int,
-                           prefix_len_dev: Optional[torch.Tensor] = None) -> torch.Tensor:
+                           prefix_len_dev: Optional[torch.Tensor] = None, fresh: bool = False) -> torch.Tensor:
+        """``fresh``: ``x`` is a tensor of the caller's own making (the layers work in place and may keep it)."""
         cfg, cache = self.cfg, self.kv.cache
         n = x.shape[0]
         paged = not cache.contiguous
@@ -183,8 +184,8 @@ class Decoder:
         ws = self._native_ws.get("ws")
         if ws is None or ws.numel() < need:
             ws = self._native_ws["ws"] = torch.empty(need, dtype=torch.uint8, device=self.device)
-        x = x.contiguous().clone()
-        pos32, rows32 = positions.to(torch.int32), rows.to(torch.int32)
+        x = x if fresh and x.is_contiguous() else x.contiguous().clone()
+        pos32, rows32 = positions.to(torch.int32), rows.to(torch.int32)          # no copies when they are int32 already
         bits = anc_bits.to(torch.int64).contiguous()
         for i, w in enumerate(self._native_weights):
             ops.decoder_layer_(x, dims, w, pos32, rows32, bits, *layer_kv(i), ws)
@@ -270,9 +271,10 @@ class Decoder:
         x = self._run_layers(self.embed[token_ids], positions, positions, attn)
         return self.logits(x if all_logits else x[-1:])
 
-    def tree_forward(self, token_ids: torch.Tensor, depths: torch.Tensor, anc_bits: torch.Tensor, prefix_len: int,
+    def tree_forward(self, token_ids: torch.Tensor, depths: Optional[torch.Tensor], anc_bits: torch.Tensor, prefix_len: int,
                      first_slot: int = 0, n_tree_slots: Optional[int] = None,
-                     prefix_len_dev: Optional[torch.Tensor] = None) -> torch.Tensor:
+                     prefix_len_dev: Optional[torch.Tensor] = None,
+                     positions32: Optional[torch.Tensor] = None, rows32: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Forward of tree nodes occupying cache rows prefix_len+first_slot.. ; ``depths`` are the node
         depths (rotary position = prefix_len + depth), ``anc_bits`` int64 [n] bitsets over tree
         slots ([n, ceil(slots / 64)] words above 64 slots).  Up to 64 rows go through the one-call layers; a larger
@@ -281,16 +283,27 @@ class Decoder:
 
         ``prefix_len_dev`` (int64 device tensor of one element): the prefix length is taken from the device when the
         kernels run and ``prefix_len`` is only its upper bound -- nothing on the host side depends on the actual
-        value, so the call can be captured into a graph and replayed as the sequence grows (one-call layers only)."""
+        value, so the call can be captured into a graph and replayed as the sequence grows (one-call layers only).
+
+        ``positions32`` / ``rows32`` (int32 [n], both or neither): rotary positions and cache rows the caller has worked
+        out already -- a draft that grows a tree level by level derives them for all levels of a speculation at once
+        instead of with five small launches per level; ``depths`` is then unused (one-call layers only)."""
         n = token_ids.numel()
         slots = first_slot + n if n_tree_slots is None else n_tree_slots
         self.kv.cache.ensure(prefix_len + max(slots, first_slot + n))
         self._rope_tables(prefix_len + max(slots, first_slot + n) + 8)
         cfg = self.cfg
         native = self.use_native_layers and self.native_layers and n <= 64 and slots <= ops.L.MAX_TREE_NODES
-        if prefix_len_dev is not None:
-            if not native:
-                raise ValueError("a device-side prefix length needs the one-call decoder layers (at most 64 rows)")
+        if prefix_len_dev is not None and not native:
+            raise ValueError("a device-side prefix length needs the one-call decoder layers (at most 64 rows)")
+        if positions32 is not None and rows32 is not None:
+            if native:
+                return self.logits(self._run_native_layers(self.embed[token_ids], positions32, rows32, anc_bits, prefix_len,
+                                                           slots, prefix_len_dev=prefix_len_dev, fresh=True))
+            positions, rows = positions32.long(), rows32.long()
+        elif depths is None:
+            raise ValueError("tree_forward needs `depths`, or positions32 and rows32")
+        elif prefix_len_dev is not None:
             positions = depths.to(self.device) + prefix_len_dev
             rows = torch.arange(first_slot, first_slot + n, device=self.device) + prefix_len_dev
         else:
