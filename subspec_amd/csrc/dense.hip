@@ -14,8 +14,8 @@
 // wavefronts split K in groups of 64 and run as independent software pipelines (weights two groups
 // ahead in registers, activation block through a wavefront-private LDS stage), partial sums are
 // added in wavefront order at the end and split-K partials in split order by a second launch.
-// With the permutation above lane (ln, c) reads the 32 contiguous bytes of row ln, k = 64g + 16c ..
-// + 15: a wavefront's weight request covers whole 128-byte lines of 16 rows.
+// The weights are requested as whole 128-byte lines (rows 0..7 of a tile's 64-k block in one request, rows 8..15 in
+// the next), as streaming data, and pass through a wavefront-private LDS stage into the operand layout.
 #include "common.h"
 #include <algorithm>
 
@@ -51,9 +51,13 @@ __global__ __launch_bounds__(kDnThreads) void dense_gemm_kernel(
   __shared__ __attribute__((aligned(16))) unsigned char lds_raw[kStageBytes > kRedBytes ? kStageBytes : kRedBytes];
   uint16_t* const xstage = (uint16_t*)lds_raw;
   float* const red = (float*)lds_raw;
+  // a wavefront's weight block (16 rows x 128 bytes) on its way from the whole-line layout of the requests to the
+  // MFMA operand layout; 16-byte piece p of row r sits at p ^ (r / 2) % 8, which makes writes and reads conflict-free
+  __shared__ __attribute__((aligned(16))) uint16_t wstage_raw[4 * 1024];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int ln = lane & 15, c = lane >> 4;
+  uint16_t* const wst = wstage_raw + wave * 1024;
   const int G = K / kDnGroup;
   const int n_tiles = (int)(N / 16);
   const int ks = blockIdx.y;
@@ -88,7 +92,19 @@ __global__ __launch_bounds__(kDnThreads) void dense_gemm_kernel(
   uint16_t* const xl = xstage + wave * (2 * MT * 16 * kDnXlStride);  // this wavefront's two stages
   const int xl_write = (lane >> 3) * kDnXlStride + (lane & 7) * 8;
   const int xl_read = ln * kDnXlStride + c * 16;
-  const int w_lane = (ln * K + c * 16) * 2;                      // byte offset of this lane's 32 bytes inside a tile
+  // Weight requests cover whole 128-byte lines: one request fetches rows 0..7 of a tile's 64-k block (lane -> row
+  // lane / 8, 16-byte piece lane % 8), a second one rows 8..15, both as streaming data (every weight byte is read once
+  // per launch).  The MFMA B operand wants lane (ln, c) to hold pieces 2c and 2c + 1 of row ln, so a block passes
+  // through a wavefront-private LDS stage on its way to the matrix core.  Requests of 32 bytes per lane straight in
+  // operand layout (two half-line requests per line) cannot stream -- the line does not wait in the first-level cache
+  // for its second half -- and were 13 to 24 % slower (152064 x 3584 at 8 rows: 195 -> 169 us; 37888 x 3584 at 64
+  // rows with the SwiGLU output stage: 71.4 -> 63.0 us).
+  const int w_lane = ((lane >> 3) * K + (lane & 7) * 8) * 2;     // byte offset of this lane's piece of rows 0..7 inside a tile
+  const int w_lane2 = w_lane + 8 * K * 2;                        // ... of rows 8..15
+  const int wst_w0 = (lane >> 3) * 64 + (((lane & 7) ^ ((lane >> 4) & 7)) << 3);               // stage positions (elements)
+  const int wst_w1 = ((lane >> 3) + 8) * 64 + (((lane & 7) ^ ((((lane >> 3) + 8) >> 1) & 7)) << 3);
+  const int wst_r0 = ln * 64 + (((2 * c) ^ ((ln >> 1) & 7)) << 3), wst_r1 = ln * 64 + (((2 * c + 1) ^ ((ln >> 1) & 7)) << 3);
+  constexpr int kWAux = 2;                                       // cache policy of the weight requests: bit 1 = non-temporal
   int wofs[RT];                                                  // byte offset of (tile t, k = 0) from the first tile
 #pragma unroll
   for (int t = 0; t < RT; ++t) wofs[t] = tile_rel(min(t, ntl - 1)) * 16 * K * 2;
@@ -115,8 +131,8 @@ __global__ __launch_bounds__(kDnThreads) void dense_gemm_kernel(
 #define SUBSPEC_DN_FETCH_W(SLOT, J, T)                                                                  \
   {                                                                                                     \
     const int kc = wofs[T] + min(g_first + 4 * (J), G - 1) * (kDnGroup * 2);                            \
-    wbuf[SLOT][T][0] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, w_lane, kc, 0);                    \
-    wbuf[SLOT][T][1] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, w_lane + 16, kc, 0);               \
+    wbuf[SLOT][T][0] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, w_lane, kc, kWAux);                \
+    wbuf[SLOT][T][1] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, w_lane2, kc, kWAux);               \
   }
   // Step J works on LDS stage SLOT = J & 1.  Once its operands are in registers the stage is free:
   // the block of group J + 2 (requested kXSlots steps ago) is parked there and group J + 2 + kXSlots requested.
@@ -138,9 +154,12 @@ __global__ __launch_bounds__(kDnThreads) void dense_gemm_kernel(
     /* earlier, the new weights get registers of their own and a copy at the end of the loop body, which waits   */ \
     /* for EVERY request in flight.  (One tile per workgroup: a third slot instead, see wbuf.)                   */ \
     _Pragma("unroll") for (int t = 0; t < RT; ++t) {                                                    \
+      *(dn_u4*)(wst + wst_w0) = wbuf[WS][t][0];       /* whole-line layout -> operand layout */            \
+      *(dn_u4*)(wst + wst_w1) = wbuf[WS][t][1];                                                         \
+      const dn_u4 wb0 = *(const dn_u4*)(wst + wst_r0), wb1 = *(const dn_u4*)(wst + wst_r1);             \
       _Pragma("unroll") for (int mt = 0; mt < MT; ++mt) {                                               \
-        acc[t][mt] = dn_mfma32<DT>(xa[mt][0], wbuf[WS][t][0], acc[t][mt]);                              \
-        acc[t][mt] = dn_mfma32<DT>(xa[mt][1], wbuf[WS][t][1], acc[t][mt]);                              \
+        acc[t][mt] = dn_mfma32<DT>(xa[mt][0], wb0, acc[t][mt]);                                         \
+        acc[t][mt] = dn_mfma32<DT>(xa[mt][1], wb1, acc[t][mt]);                                         \
       }                                                                                                 \
       __builtin_amdgcn_sched_barrier(0);                                                                \
       SUBSPEC_DN_FETCH_W(WNEXT, (J) + 2, t);                                                            \
