@@ -266,14 +266,17 @@ __global__ __launch_bounds__(256) void dense_reduce_kernel(const float* __restri
 
 struct DnPlan { int wgs, row_tiles, splits, groups_per_split; };
 // Tiles per workgroup, measured with weights streamed from HBM (a different matrix every call): with few rows the
-// kernel only streams weights and more, smaller workgroups win (37888x3584, M = 8: 58.5 us at one tile per workgroup,
-// 65 us at four); at M = 64 every wavefront also fetches a [64 x 64] activation block per 64 k, which more tiles per
-// workgroup amortise (4608x3584, M = 64: 19.4 us at two tiles, 25.3 us at one).
+// kernel mostly streams weights and small workgroups win -- one tile, or two from 1024 tiles on, where a wavefront's
+// activation block is worth sharing (M = 8: 37888x3584 52.9 / 45.0 / 49.5 us at one / two / four tiles, 152064x3584
+// 197.9 / 167.3 / 170.0 us, 3584x3584 8.2 / 10.5 / 14.8 us); at M = 64 every wavefront also fetches a [64 x 64]
+// activation block per 64 k, which more tiles per workgroup amortise (4608x3584, M = 64: 16.1 us at two tiles, 25.4 us
+// at one; 37888x3584: 66.8 us at four, 77.1 at two, 120 at one).
 static DnPlan dn_plan(int64_t M, int64_t N, int64_t K) {
   const int G = (int)(K / kDnGroup);
   const int64_t tiles = N / 16, slots = M <= 16 ? 4096 : M <= 32 ? 1024 : 256;
   const int64_t want = (tiles + slots - 1) / slots;
   int row_tiles = want <= 1 ? 1 : want <= 2 ? 2 : 4;
+  if (M <= 16) row_tiles = tiles >= 1024 ? 2 : 1;
   // More than 32 rows over a long K (the down projection, 3584 x 18944): one tile per workgroup fetches four bytes
   // of activations for every byte of weights; four tiles and four K ranges keep as many workgroups with a quarter of
   // that (M = 64: 46.7 us with the reduction against 61.5 us).
