@@ -42,6 +42,24 @@ def test_dense_linear_matches_float64_product(dtype, N, K):
     assert torch.equal(ops.dense_linear(x, wd, None), ops.dense_linear(x, wd, None))
 
 
+def test_dense_linear_at_the_size_of_the_vocabulary_head():
+    """152064 x 3584 (the draft's lm_head): 9504 tiles, two per workgroup; fp32 reference (its error is far below the
+    bf16 rounding of the outputs)."""
+    g = torch.Generator().manual_seed(152064)
+    N, K = 152064, 3584
+    w = (torch.randn(N, K, generator=g) * 0.03).to(torch.bfloat16)
+    wd, wf = w.to(DEV), w.float()
+    for M in (1, 8, 16):
+        print("dense_linear head", M, flush=True)
+        x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+        got = ops.dense_linear(x.to(DEV), wd, None).cpu()
+        ref = x.float() @ wf.T
+        scale = ref.abs().amax().item()
+        assert got.shape == (M, N)
+        assert ((got.float() - ref).abs() <= 2.0 ** -7 * ref.abs() + 1e-3 * scale).all()
+        assert (got == ref.to(torch.bfloat16)).float().mean().item() >= 0.97
+
+
 def test_dense_linear_special_cases():
     # integer-valued operands: every product and partial sum is exact, so the result is exact whatever the order
     g = torch.Generator().manual_seed(2)
