@@ -16,7 +16,7 @@ HIPCC_FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     # MFMA results that feed vector ALU work stay in VGPRs instead of bouncing through AGPRs
     "-mllvm", "-amdgpu-mfma-vgpr-form=1",
-    "-Wno-unused-result",
+    "-Wno-unused-result", "-Wno-inline-asm",
 ]
 
 

@@ -34,6 +34,7 @@
 // algorithmic bytes per batch element = K+V rows actually attended + Q + O.
 #include "common.h"
 #include <algorithm>
+#include <stdlib.h>
 
 namespace subspec {
 
@@ -422,39 +423,714 @@ __global__ __launch_bounds__(256) void tree_attention_merge_kernel(
   *(uint2*)(out + (((int64_t)b * ap.n_rows + ap.row0 + row) * ap.hq + qh) * kAttnD + d4 * 4) = packed;
 }
 
+
+// ---------------------------------------------------------------------------------------------------------------
+// Windows of 17 to 64 query rows: the same algorithm on 32x32x16 matrix instructions.  A wavefront owns 32 rows of one
+// head.  S^T = K Q^T is two 32 x 32 accumulators per 64-key block (lane: query row lane % 32, sixteen keys
+// 32 t + 8 (r / 4) + 4 (lane / 32) + r % 4), so a row maximum is fifteen in-lane steps and ONE cross-lane step, and
+// registers 8 s .. 8 s + 7 of tile t are, packed, the B operand of the 16-key step (t, s) of O^T = V^T P^T.  A
+// 32 x 32 x 16 instruction occupies the matrix pipe for 32 cycles but the issue port for about 8 (the 16 x 16 x 32
+// form: 16 and 8), which leaves room for the softmax's vector instructions and the LDS operand reads of the other
+// wavefront of the SIMD: measured on this chip, one such instruction hides three fused multiply-adds, an exponential
+// and a 16-byte LDS read per lane, the 16 x 16 x 32 form only two multiply-adds.
+typedef float v16f __attribute__((ext_vector_type(16)));
+template <int DT>
+__device__ __forceinline__ v16f mfma32x32(uint4 a, uint4 b, v16f c) {
+  if constexpr (DT == SUBSPEC_BF16) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, a), __builtin_bit_cast(v8bf, b), c, 0, 0, 0);
+  } else {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, a), __builtin_bit_cast(v8h, b), c, 0, 0, 0);
+  }
+}
+constexpr int kKStride32 = kAttnD + 8;    // 272-byte rows: the 16-byte reads of 16 consecutive keys tile the 64 banks
+constexpr int kVStride32 = kAttnD + 32;   // 320-byte rows: a transposing read takes 64 bytes of each of 4 keys per 32 lanes
+constexpr int kTileFloats = 32 * kAttnD;  // fp32 partial O of one 32-row tile, stored [16 (d-tile, quad)][64 lanes][4]
+
+// WPH wavefronts per head (1: up to 32 rows, 2: up to 64), THREADS / 64 / WPH heads of one KV head per workgroup.
+template <int DT, bool PAGED, int WPH, int THREADS>
+__global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2))) void tree_attention32_kernel(
+    const uint16_t* __restrict__ q, const uint16_t* __restrict__ kc, const uint16_t* __restrict__ vc,
+    const uint64_t* __restrict__ anc, AttnParams ap, uint16_t* __restrict__ out, float* __restrict__ part_o,
+    float* __restrict__ part_ml) {
+  __shared__ __attribute__((aligned(16))) uint16_t Ks2[2][kKeyBlock * kKStride32];
+  __shared__ __attribute__((aligned(16))) uint16_t Vs2[2][kKeyBlock * kVStride32];
+  // ancestor bitsets of the window's rows (the heads of a workgroup share them).  Read from LDS inside the loop: a
+  // global load there would make the loop wait for EVERY request in flight, the prefetched keys included.
+  __shared__ uint64_t mask_s[kAttnRows][SUBSPEC_MAX_TREE_NODES / 64 + 1];
+  asm volatile("" ::"s"(ap.batch), "s"(ap.hq), "s"(ap.hkv), "s"(ap.n_rows), "s"(ap.n_slots), "s"(ap.seq_stride), "s"(ap.prefix),
+               "s"(ap.anc_batch_stride), "s"(ap.mask_words), "s"(ap.row0), "s"(ap.win_rows), "s"(ap.chunks), "s"(ap.chunk_keys),
+               "s"(ap.pairs_per_kv), "s"(ap.units), "s"(ap.scale_log2), "s"(ap.prefix_dev), "s"(ap.page_table),
+               "s"(ap.page_shift), "s"(ap.max_pages), "s"(ap.page_stride), "s"(ap.tok_stride), "s"(ap.v_delta));
+  asm volatile("" ::"s"(q), "s"(kc), "s"(vc), "s"(anc), "s"(out), "s"(part_o), "s"(part_ml));
+  const uint32_t lin = blockIdx.x;
+  const int xcd = (int)(lin % (uint32_t)kXcds);
+  const uint32_t slot = lin / (uint32_t)kXcds;
+  const int pair = (int)(slot % (uint32_t)ap.pairs_per_kv);
+  const uint32_t unit = (slot / (uint32_t)ap.pairs_per_kv) * (uint32_t)kXcds + (uint32_t)xcd;
+  if ((int64_t)unit >= ap.units) return;
+  const int chunk = (int)(unit % (uint32_t)ap.chunks);
+  const uint32_t bkv = unit / (uint32_t)ap.chunks;
+  const int kvh = (int)(bkv % (uint32_t)ap.hkv), b = (int)(bkv / (uint32_t)ap.hkv);
+  const int group = (int)((uint32_t)ap.hq / (uint32_t)ap.hkv);
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int lr = lane & 31, g = lane >> 5;              // query row of the lane inside its tile, half of the k range
+  constexpr int kHeadsPerWG = (THREADS / 64) / WPH;
+  const int head_in_group = pair * kHeadsPerWG + wave / WPH;
+  const bool head_ok = head_in_group < group;
+  const int qh = kvh * group + (head_ok ? head_in_group : 0);
+  const int bh = b * (int)ap.hq + qh;
+  const int n = (int)ap.n_rows;
+  const int64_t prefix = ap.prefix_dev ? min(max(*ap.prefix_dev, (int64_t)0), ap.prefix) : ap.prefix;
+  const int64_t kv_len = prefix + ap.n_slots;
+  const int tile = wave % WPH;
+  const int row = tile * 32 + lr;                       // row inside this launch's window
+  const bool row_ok = head_ok && row < ap.win_rows;
+  const int grow = ap.row0 + (row_ok ? row : 0);
+
+  // Q^T operands: B[k = 8 g + e][row] = Q[row][16 ks + 8 g + e]
+  uint4 qreg[kAttnD / 16];
+  {
+    const uint16_t* qp = q + ((int64_t)bh * n + grow) * kAttnD + g * 8;
+#pragma unroll
+    for (int ks = 0; ks < kAttnD / 16; ++ks) qreg[ks] = row_ok ? *(const uint4*)(qp + ks * 16) : make_uint4(0, 0, 0, 0);
+  }
+  for (int i = tid; i < kAttnRows * (SUBSPEC_MAX_TREE_NODES / 64 + 1); i += THREADS) {
+    const int r = i / (SUBSPEC_MAX_TREE_NODES / 64 + 1), w = i % (SUBSPEC_MAX_TREE_NODES / 64 + 1);
+    mask_s[r][w] = (r < ap.win_rows && w < ap.mask_words)
+                       ? anc[((int64_t)b * ap.anc_batch_stride + ap.row0 + r) * ap.mask_words + w] : 0ull;
+  }
+
+  v16f oacc[kAttnD / 32];
+#pragma unroll
+  for (int dt = 0; dt < kAttnD / 32; ++dt)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) oacc[dt][r] = 0.f;
+  float m_run = -INFINITY, l_run = 0.f;
+
+  const uint16_t* kbase = PAGED ? kc + (int64_t)kvh * kAttnD : kc + ((int64_t)b * ap.hkv + kvh) * ap.seq_stride * kAttnD;
+  const uint16_t* vbase = PAGED ? kbase + ap.v_delta : vc + ((int64_t)b * ap.hkv + kvh) * ap.seq_stride * kAttnD;
+  auto row_offset = [&](int64_t p) -> int64_t {
+    if constexpr (PAGED) {
+      const int page = min(max(ap.page_table[p >> ap.page_shift], 0), ap.max_pages - 1);
+      return (int64_t)page * ap.page_stride + (p & ((1 << ap.page_shift) - 1)) * ap.tok_stride;
+    } else {
+      return p * kAttnD;
+    }
+  };
+  const int64_t key0 = (int64_t)chunk * ap.chunk_keys;
+  const int64_t key1 = min(key0 + ap.chunk_keys, kv_len);
+
+  constexpr int KPT = 1024 / THREADS;                  // keys of a block per thread: 2 (512 threads), 4 (256), 8 (128)
+  constexpr int KSTEP = 64 / KPT;
+  // Two register sets: block j travels in set j % 2 and is written to LDS stage j % 2 one block ahead of its use, so the
+  // requests of TWO blocks are in flight while a block is multiplied (one block's worth per compute unit does not cover
+  // the memory latency).  Native vectors: arrays of HIP's uint4 struct would live in memory.
+  dec_u4 kst[2][KPT], vst[2][KPT];
+  const int skey = tid >> 4, sdc = tid & 15;
+#define SUBSPEC_ATTN32_FETCH(SET, KB)                                                            \
+  do {                                                                                           \
+    _Pragma("unroll") for (int i_ = 0; i_ < KPT; ++i_) {                                         \
+      const int64_t p_ = row_offset(min((KB) + i_ * KSTEP + skey, key1 - 1));                    \
+      kst[SET][i_] = *(const dec_u4*)(kbase + p_ + sdc * 8);                                     \
+      vst[SET][i_] = *(const dec_u4*)(vbase + p_ + sdc * 8);                                     \
+    }                                                                                            \
+  } while (0)
+#define SUBSPEC_ATTN32_STAGE(SET)                                                                \
+  do {                                                                                           \
+    _Pragma("unroll") for (int i_ = 0; i_ < KPT; ++i_) {                                         \
+      *(dec_u4*)(Ks2[SET] + (skey + i_ * KSTEP) * kKStride32 + sdc * 8) = kst[SET][i_];          \
+      *(dec_u4*)(Vs2[SET] + (skey + i_ * KSTEP) * kVStride32 + sdc * 8) = vst[SET][i_];          \
+    }                                                                                            \
+  } while (0)
+
+  // Every fetch and every stage is unconditional (rows beyond the chunk repeat its last row and are never multiplied):
+  // the counter that a wait names is fixed at compile time, and a request that is issued on one path only makes the
+  // compiler wait for ALL requests in flight wherever the paths join.
+  SUBSPEC_ATTN32_FETCH(0, key0);
+  SUBSPEC_ATTN32_FETCH(1, key0 + kKeyBlock);
+  SUBSPEC_ATTN32_STAGE(0);
+  SUBSPEC_ATTN32_FETCH(0, key0 + 2 * kKeyBlock);
+
+  // LDS addresses of the lane's operands.  K: key 32 t + lr, pieces of 16 bytes at 16 ks + 8 g.  V^T (transposing read,
+  // per 16 lanes: lane r supplies the 8 bytes of key r / 4 at d = 4 (r % 4) and receives four keys of d = r): keys
+  // 4 g + r / 4 of the 16-key step, d = 32 dt + 16 (lr / 16) + ...
+  const int koff = lr * kKStride32 + g * 8;
+  const int voff = (4 * g + ((lane & 15) >> 2)) * kVStride32 + (lr & 16) + 4 * (lane & 3);
+
+  for (int64_t kb2 = key0; kb2 < key1; kb2 += 2 * kKeyBlock) {
+#pragma unroll
+   for (int buf = 0; buf < 2; ++buf) {
+    const int64_t kb = kb2 + buf * kKeyBlock;
+    __syncthreads();                                   // stage `buf` is complete, and everyone has left the other stage
+    SUBSPEC_ATTN32_STAGE(buf ^ 1);
+    SUBSPEC_ATTN32_FETCH(buf ^ 1, kb + 3 * kKeyBlock);
+    if (kb >= key1) continue;                          // (uniform) odd number of blocks: the requests above keep every path's count equal
+    const uint16_t* Ks = Ks2[buf] + koff;
+    const uint16_t* Vs = Vs2[buf] + voff;
+
+    v16f sacc[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) sacc[t][r] = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < kAttnD / 16; ++ks) {
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        const uint4 a = *(const uint4*)(Ks + t * 32 * kKStride32 + ks * 16);
+        sacc[t] = mfma32x32<DT>(a, qreg[ks], sacc[t]);
+      }
+    }
+    const bool plain = kb + kKeyBlock <= prefix;
+    float mloc = -INFINITY;
+    if (plain) {
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int r = 0; r < 16; r += 2) mloc = fmaxf(fmaxf(sacc[t][r], sacc[t][r + 1]), mloc);
+    } else {
+      // a 64-key block touches at most two consecutive words of the row's bitset (a zero word follows the last)
+      const int word0 = min((int)(max(kb - prefix, (int64_t)0) >> 6), SUBSPEC_MAX_TREE_NODES / 64 - 1);
+      const uint64_t bits0 = row_ok ? mask_s[row][word0] : 0ull, bits1 = row_ok ? mask_s[row][word0 + 1] : 0ull;
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int64_t pos = kb + t * 32 + (r >> 2) * 8 + g * 4 + (r & 3);
+          const bool in_range = pos < kv_len;
+          const bool tree = pos >= prefix;
+          const int rel = tree ? (int)(pos - prefix) : 0;
+          const uint64_t word = (rel >> 6) == word0 ? bits0 : bits1;
+          const bool ok = in_range && (!tree || ((word >> (rel & 63)) & 1ull));
+          const float tv = ok ? sacc[t][r] : -INFINITY;
+          sacc[t][r] = tv;
+          mloc = fmaxf(mloc, tv);
+        }
+      }
+    }
+    mloc = fmaxf(mloc, __shfl_xor(mloc, 32, kWave));
+    const float m_new = fmaxf(m_run, mloc);
+    const float m_use = m_new == -INFINITY ? 0.f : m_new;
+    const float alpha = __builtin_amdgcn_exp2f((m_run - m_use) * ap.scale_log2);
+    m_run = m_new;
+    const float mneg = -m_use * ap.scale_log2;
+    if (__any(alpha != 1.0f)) {
+      l_run *= alpha;
+#pragma unroll
+      for (int dt = 0; dt < kAttnD / 32; ++dt) oacc[dt] *= alpha;
+    }
+    uint4 pb[2][2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+        float p[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          p[e] = __builtin_amdgcn_exp2f(fmaf(sacc[t][8 * s + e], ap.scale_log2, mneg));
+          l_run += p[e];
+        }
+        pb[t][s] = make_uint4(pack2<DT>(p[0], p[1]), pack2<DT>(p[2], p[3]), pack2<DT>(p[4], p[5]), pack2<DT>(p[6], p[7]));
+      }
+    }
+    // O^T += V^T P^T: four 32-wide d tiles, four 16-key steps; the A operand of step (t, s) holds, for the lane's d, the keys
+    // 32 t + 16 s + 4 g + {0..3} and 32 t + 16 s + 8 + 4 g + {0..3}, in the order the accumulator registers of S^T hold them
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+#pragma unroll
+        for (int dt = 0; dt < kAttnD / 32; ++dt) {
+          const uint16_t* vp = Vs + (t * 32 + s * 16) * kVStride32 + dt * 32;
+          const uint2 lo = lds_read_tr16(vp), hi = lds_read_tr16(vp + 8 * kVStride32);
+          oacc[dt] = mfma32x32<DT>(make_uint4(lo.x, lo.y, hi.x, hi.y), pb[t][s], oacc[dt]);
+        }
+      }
+    }
+   }
+  }
+#undef SUBSPEC_ATTN32_FETCH
+#undef SUBSPEC_ATTN32_STAGE
+
+  float l = l_run + __shfl_xor(l_run, 32, kWave);
+  if (!head_ok || tile * 32 >= ap.win_rows) return;      // (wave-uniform) nothing of this tile is wanted
+  if (ap.chunks == 1) {
+    if (!row_ok) return;
+    const float inv = l > 0.f ? 1.0f / l : 0.f;
+    uint16_t* op = out + (((int64_t)b * n + ap.row0 + row) * ap.hq + qh) * kAttnD + g * 4;
+#pragma unroll
+    for (int dt = 0; dt < kAttnD / 32; ++dt)
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4)
+        *(uint2*)(op + dt * 32 + q4 * 8) = make_uint2(pack2<DT>(oacc[dt][4 * q4] * inv, oacc[dt][4 * q4 + 1] * inv),
+                                                      pack2<DT>(oacc[dt][4 * q4 + 2] * inv, oacc[dt][4 * q4 + 3] * inv));
+  } else {
+    // partial tile: every store instruction of the wavefront writes 1 KB of consecutive addresses
+    float* po = part_o + (((int64_t)bh * ap.chunks + chunk) * 2 + tile) * kTileFloats + lane * 4;
+#pragma unroll
+    for (int dt = 0; dt < kAttnD / 32; ++dt)
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4)
+        *(v4f*)(po + (dt * 4 + q4) * 256) = v4f{oacc[dt][4 * q4], oacc[dt][4 * q4 + 1], oacc[dt][4 * q4 + 2], oacc[dt][4 * q4 + 3]};
+    if (g == 0) {
+      const int64_t pslot = ((int64_t)bh * ap.chunks + chunk) * kAttnRows + row;
+      *(v2f_t*)(part_ml + pslot * 2) = v2f_t{m_run * ap.scale_log2, l};
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// The same tiles with the two wavefronts of every SIMD half a block apart ("ping-pong").  Left to themselves the eight
+// wavefronts of a workgroup run in step (they start together and meet at a barrier per block): all of them multiply,
+// then all of them evaluate the softmax, and the matrix pipe idles while the vector ALU works and the other way round
+// -- measured: 1.76 us per 64-key block and workgroup for 1.0 us of matrix work, vector and matrix time simply added.
+// Here a block is two phases separated by workgroup barriers, M (O^T += V^T P^T of the previous block, then S^T = K Q^T
+// of this one: matrix instructions and their LDS operand reads) and V (softmax of S^T: vector ALU only); wavefronts
+// 4..7 (group B, the second wavefront of each SIMD) enter the loop one barrier later than wavefronts 0..3 (group A), so
+// whenever one wavefront of a SIMD is in M the other is in V.
+// K / V blocks travel from memory straight into LDS (global_load_lds_dwordx4: no staging registers, no LDS write
+// instructions) through a ring of four stages, issued four phases (two blocks) before their first use.  The copies are
+// inline assembly ON PURPOSE: a wait names a count fixed at compile time, and for LDS-DMA requests it knows about the
+// compiler waits for all of them before every LDS read; the waits for these are placed by hand (group A at the end of
+// V, group B at the end of M: every odd global phase).  A stage's rows are unpadded (a DMA instruction writes 1 KB of
+// consecutive LDS, four rows); the 16-byte pieces of a row are XOR-swizzled instead, by choosing which piece of the
+// row each lane fetches: K piece p of row r sits at p ^ (r % 16) (the operand read of 16 consecutive rows then covers
+// all 64 banks), V piece p at p ^ 4 (r % 4) (the transposing read takes 64 bytes of each of 4 consecutive rows).
+constexpr int kPPStages = 4;
+constexpr int kPPStageBytes = kKeyBlock * kAttnD * 2;                 // 16 KB
+constexpr int kPPVOff = kPPStages * kPPStageBytes;                    // V ring behind the K ring
+constexpr int kPPMaskOff = 2 * kPPStages * kPPStageBytes;             // 128 KB
+constexpr int kPPMaskWords = SUBSPEC_MAX_TREE_NODES / 64 + 1;         // a zero word follows the last
+constexpr int kPPLdsBytes = kPPMaskOff + kAttnRows * kPPMaskWords * 8;
+
+__device__ __forceinline__ void pp_wait_vmcnt4() { asm volatile("s_waitcnt vmcnt(4)" ::: "memory"); }
+__device__ __forceinline__ void pp_dma16(uint32_t lds_base, const uint16_t* src) {
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_base), "v"(src) : "memory", "m0");
+}
+
+// The matrix work of an M phase as steps of one matrix instruction each.  MODE 2 (the steady state) alternates the two
+// products: even steps are O^T += V^T P^T of the previous block ((t, s) major, the four d tiles minor), odd steps
+// S^T = K Q^T of this one (d step major, the two key tiles minor), so an accumulator comes up again only every fourth
+// (S^T) or eighth (O^T) step -- two S^T accumulators used alternately wait for each other (measured: 43 cycles per
+// instruction instead of 33).  MODE 0 is S^T alone (the first block), MODE 1 O^T alone (after the last).  The LDS operand of
+// step k + kAhead is requested right after the instruction of step k has been issued, through a ring of operand registers;
+// scheduling fences keep the compiler from undoing the distance (left alone it requests every operand immediately before
+// its use and waits for it, with the matrix pipe idle meanwhile).  With `copy`, the wavefront's four K / V copy instructions
+// of the block two ahead are issued a quarter of the steps apart instead of in a row: a copy instruction waits for room in the
+// compute unit's memory pipeline, and that wait then falls into the shadow of a matrix instruction.
+struct PPAddr { uint32_t vst, kst, vx, kx; };
+// a wavefront's four copy instructions of one block: K rows 0..3, K rows 4..7, V rows 0..3, V rows 4..7 of its share
+struct PPCopy {
+  const uint16_t *k0, *k1, *v0, *v1;     // lane addresses less the row offsets
+  int r0, r1;                            // element offsets of the two row groups inside the chunk
+  uint32_t kdst, vdst;                   // LDS addresses of the wavefront's rows in the stage
+};
+__device__ __forceinline__ void pp_copy_issue(const PPCopy& cp, int c) {
+  if (c == 0) pp_dma16(cp.kdst, cp.k0 + cp.r0);
+  else if (c == 1) pp_dma16(cp.kdst + 1024, cp.k1 + cp.r1);
+  else if (c == 2) pp_dma16(cp.vdst, cp.v0 + cp.r0);
+  else pp_dma16(cp.vdst + 1024, cp.v1 + cp.r1);
+}
+template <int MODE> __device__ __forceinline__ constexpr bool pp_step_is_pv(int k) { return MODE == 1 || (MODE == 2 && (k & 1) == 0); }
+template <int MODE> __device__ __forceinline__ constexpr int pp_step_index(int k) { return MODE == 2 ? k >> 1 : k; }
+template <int DT, int MODE>
+__device__ __forceinline__ dec_u4 pp_load_step(int k, const PPAddr& ad) {
+  const int j = pp_step_index<MODE>(k);
+  if (pp_step_is_pv<MODE>(k)) {
+    const int ts = j >> 2, dt = j & 3;                   // ts = 2 t + s: keys 16 ts .. 16 ts + 15 of the block
+    const uint32_t va = ad.vst + (ad.vx ^ (uint32_t)(dt << 6)) + (uint32_t)(ts * 16 * 256);
+    const uint2 lo = lds_read_tr16((const uint16_t*)(__attribute__((address_space(3))) uint16_t*)(uintptr_t)va);
+    const uint2 hi = lds_read_tr16((const uint16_t*)(__attribute__((address_space(3))) uint16_t*)(uintptr_t)(va + 8 * 256));
+    return dec_u4{lo.x, lo.y, hi.x, hi.y};
+  } else {
+    const int ks = j >> 1, t = j & 1;
+    const uint32_t ka = ad.kst + (ad.kx ^ (uint32_t)(ks << 5)) + (uint32_t)(t * 32 * 256);
+    return *(const dec_u4*)(__attribute__((address_space(3))) dec_u4*)(uintptr_t)ka;
+  }
+}
+template <int DT, int MODE>
+__device__ __forceinline__ void pp_matrix_phase(const PPAddr& ad, const PPCopy& cp, bool copy, v16f (&oacc)[4], v16f (&sacc)[2],
+                                                const uint4 (&pb)[2][2], const uint4 (&qreg)[8]) {
+  constexpr int kSteps = MODE == 2 ? 32 : 16;
+  constexpr int kAhead = 4;
+  dec_u4 ring[kAhead];
+#pragma unroll
+  for (int k = 0; k < kAhead; ++k) ring[k] = pp_load_step<DT, MODE>(k, ad);
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int k = 0; k < kSteps; ++k) {
+    const uint4 a = __builtin_bit_cast(uint4, ring[k % kAhead]);
+    const int j = pp_step_index<MODE>(k);
+    if (pp_step_is_pv<MODE>(k)) {
+      const int ts = j >> 2, dt = j & 3;
+      oacc[dt] = mfma32x32<DT>(a, pb[ts >> 1][ts & 1], oacc[dt]);
+    } else {
+      const int ks = j >> 1, t = j & 1;
+      if (ks == 0) {
+        v16f z;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) z[r] = 0.f;
+        sacc[t] = mfma32x32<DT>(a, qreg[0], z);
+      } else {
+        sacc[t] = mfma32x32<DT>(a, qreg[ks], sacc[t]);
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    if (k + kAhead < kSteps) ring[k % kAhead] = pp_load_step<DT, MODE>(k + kAhead, ad);
+    if (k % (kSteps / 4) == 1 && copy) pp_copy_issue(cp, k / (kSteps / 4));       // (uniform)
+    __builtin_amdgcn_sched_barrier(0);
+  }
+}
+
+// Online-softmax step of one 64-key block on the S^T accumulators (vector ALU only): masks the tree part, moves the running
+// maximum and sum, rescales O when a maximum moved, leaves P^T packed as the B operands of the next phase's O^T += V^T P^T.
+// Four partial sums and two partial maxima: the wavefront issues in the gaps the other wavefront's matrix instructions
+// leave, and a single dependent chain would wait for its own previous result in every one of them.
+struct PPRow { int64_t prefix, kv_len; const uint64_t* mask_row; float scale_log2; int g; bool row_ok; };
+template <int DT>
+__device__ __forceinline__ void pp_softmax_phase(int64_t kb, const PPRow& rw, v16f (&sacc)[2], v16f (&oacc)[4], uint4 (&pb)[2][2],
+                                                 float& m_run, float& l_run) {
+  const bool plain = kb + kKeyBlock <= rw.prefix;
+  float mloc = -INFINITY;
+  if (plain) {
+    float mt[2] = {-INFINITY, -INFINITY};
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int r = 0; r < 16; r += 2) mt[t] = fmaxf(fmaxf(sacc[t][r], sacc[t][r + 1]), mt[t]);
+    mloc = fmaxf(mt[0], mt[1]);
+  } else {
+    // a 64-key block touches at most two consecutive words of the row's bitset (a zero word follows the last)
+    const int word0 = min((int)(max(kb - rw.prefix, (int64_t)0) >> 6), SUBSPEC_MAX_TREE_NODES / 64 - 1);
+    const uint64_t bits0 = rw.row_ok ? rw.mask_row[word0] : 0ull, bits1 = rw.row_ok ? rw.mask_row[word0 + 1] : 0ull;
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int64_t pos = kb + t * 32 + (r >> 2) * 8 + rw.g * 4 + (r & 3);
+        const bool in_range = pos < rw.kv_len;
+        const bool tree = pos >= rw.prefix;
+        const int rel = tree ? (int)(pos - rw.prefix) : 0;
+        const uint64_t word = (rel >> 6) == word0 ? bits0 : bits1;
+        const bool ok = in_range && (!tree || ((word >> (rel & 63)) & 1ull));
+        const float tv = ok ? sacc[t][r] : -INFINITY;
+        sacc[t][r] = tv;
+        mloc = fmaxf(mloc, tv);
+      }
+    }
+  }
+  mloc = fmaxf(mloc, __shfl_xor(mloc, 32, kWave));
+  const float m_new = fmaxf(m_run, mloc);
+  const float m_use = m_new == -INFINITY ? 0.f : m_new;
+  const float alpha = __builtin_amdgcn_exp2f((m_run - m_use) * rw.scale_log2);
+  m_run = m_new;
+  const float mneg = -m_use * rw.scale_log2;
+  if (__any(alpha != 1.0f)) {
+    l_run *= alpha;
+#pragma unroll
+    for (int dt = 0; dt < kAttnD / 32; ++dt) oacc[dt] *= alpha;
+  }
+  float lsum[2][2];
+#pragma unroll
+  for (int t = 0; t < 2; ++t) {
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      float p[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) p[e] = __builtin_amdgcn_exp2f(fmaf(sacc[t][8 * s + e], rw.scale_log2, mneg));
+      lsum[t][s] = ((p[0] + p[1]) + (p[2] + p[3])) + ((p[4] + p[5]) + (p[6] + p[7]));
+      pb[t][s] = make_uint4(pack2<DT>(p[0], p[1]), pack2<DT>(p[2], p[3]), pack2<DT>(p[4], p[5]), pack2<DT>(p[6], p[7]));
+    }
+  }
+  l_run += (lsum[0][0] + lsum[0][1]) + (lsum[1][0] + lsum[1][1]);
+}
+
+#ifndef PP_GRP
+#define PP_GRP(W) (((W) >> 2) & 1)
+#endif
+#ifdef PP_TRACE
+__device__ long long pp_trace[4096 * 2 * 96];
+#define PP_T(IDX) do { if (lane == 0 && (wave == 0 || wave == (PP_GRP(1) ? 1 : PP_GRP(2) ? 2 : 4)) && (IDX) < 96) pp_trace[(blockIdx.x * 2 + (wave != 0)) * 96 + (IDX)] = clock64(); } while (0)
+#else
+#define PP_T(IDX) do {} while (0)
+#endif
+template <int DT, int WPH>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void tree_attention_pp_kernel(
+    const uint16_t* __restrict__ q, const uint16_t* __restrict__ kc, const uint16_t* __restrict__ vc,
+    const uint64_t* __restrict__ anc, AttnParams ap, uint16_t* __restrict__ out, float* __restrict__ part_o,
+    float* __restrict__ part_ml) {
+  __shared__ __attribute__((aligned(1024))) uint8_t lds[kPPLdsBytes];
+  asm volatile("" ::"s"(ap.batch), "s"(ap.hq), "s"(ap.hkv), "s"(ap.n_rows), "s"(ap.n_slots), "s"(ap.seq_stride), "s"(ap.prefix),
+               "s"(ap.anc_batch_stride), "s"(ap.mask_words), "s"(ap.row0), "s"(ap.win_rows), "s"(ap.chunks), "s"(ap.chunk_keys),
+               "s"(ap.pairs_per_kv), "s"(ap.units), "s"(ap.scale_log2), "s"(ap.prefix_dev));
+  asm volatile("" ::"s"(q), "s"(kc), "s"(vc), "s"(anc), "s"(out), "s"(part_o), "s"(part_ml));
+  const uint32_t lin = blockIdx.x;
+  const int xcd = (int)(lin % (uint32_t)kXcds);
+  const uint32_t slot = lin / (uint32_t)kXcds;
+  const int pair = (int)(slot % (uint32_t)ap.pairs_per_kv);
+  const uint32_t unit = (slot / (uint32_t)ap.pairs_per_kv) * (uint32_t)kXcds + (uint32_t)xcd;
+  if ((int64_t)unit >= ap.units) return;
+  const int chunk = (int)(unit % (uint32_t)ap.chunks);
+  const uint32_t bkv = unit / (uint32_t)ap.chunks;
+  const int kvh = (int)(bkv % (uint32_t)ap.hkv), b = (int)(bkv / (uint32_t)ap.hkv);
+  const int group = (int)((uint32_t)ap.hq / (uint32_t)ap.hkv);
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  PP_T(0);
+  const int lr = lane & 31, g = lane >> 5;
+  constexpr int kHeadsPerWG = 8 / WPH;
+  const int head_in_group = pair * kHeadsPerWG + wave / WPH;
+  const bool head_ok = head_in_group < group;
+  const int qh = kvh * group + (head_ok ? head_in_group : 0);
+  const int bh = b * (int)ap.hq + qh;
+  const int n = (int)ap.n_rows;
+  const int64_t prefix = ap.prefix_dev ? min(max(*ap.prefix_dev, (int64_t)0), ap.prefix) : ap.prefix;
+  const int64_t kv_len = prefix + ap.n_slots;
+  const int tile = wave % WPH;
+  const int row = tile * 32 + lr;
+  const bool live = head_ok && tile * 32 < ap.win_rows;     // (wave-uniform) this wavefront has rows to work on
+  const bool row_ok = head_ok && row < ap.win_rows;
+  const int grow = ap.row0 + (row_ok ? row : 0);
+  const bool grp_b = PP_GRP(wave) != 0;
+
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)lds;
+  const int64_t key0 = (int64_t)chunk * ap.chunk_keys;
+  const int64_t key1 = min(key0 + ap.chunk_keys, kv_len);
+  const int nkeys = (int)(key1 - key0);
+  const int nb = (nkeys + kKeyBlock - 1) / kKeyBlock;
+  const uint16_t* kbase = kc + (((int64_t)b * ap.hkv + kvh) * ap.seq_stride + key0) * kAttnD;
+  const uint16_t* vbase = vc + (((int64_t)b * ap.hkv + kvh) * ap.seq_stride + key0) * kAttnD;
+
+  // ---- everything that has to come out of memory before the first product is requested at once: Q rows, mask words,
+  //      then the first two K / V blocks; one wait covers all of it
+  uint4 qreg[kAttnD / 16];
+  {
+    const uint16_t* qp = q + ((int64_t)bh * n + grow) * kAttnD + g * 8;
+#pragma unroll
+    for (int ks = 0; ks < kAttnD / 16; ++ks) qreg[ks] = row_ok ? *(const uint4*)(qp + ks * 16) : make_uint4(0, 0, 0, 0);
+  }
+  uint64_t* mask_s = (uint64_t*)(lds + kPPMaskOff);
+  uint64_t mword[2];
+#pragma unroll
+  for (int u = 0; u < 2; ++u) {
+    const int i = tid + u * 512, r = i / kPPMaskWords, w = i % kPPMaskWords;
+    mword[u] = (i < kAttnRows * kPPMaskWords && r < ap.win_rows && w < ap.mask_words)
+                   ? anc[((int64_t)b * ap.anc_batch_stride + ap.row0 + r) * ap.mask_words + w] : 0ull;
+  }
+
+  // ---- copies: wavefront w brings rows 8 w .. 8 w + 7 of a block, K and V, two instructions of four rows each
+  const int crow = wave * 8 + (lane >> 4);                                       // row of the first instruction; + 4 for the second
+  const int kpiece0 = ((lane & 15) ^ (crow & 15)) * 8, kpiece1 = ((lane & 15) ^ ((crow + 4) & 15)) * 8;
+  const int vpiece = ((lane & 15) ^ (4 * (crow & 3))) * 8;                       // (crow + 4) % 4 == crow % 4
+  const uint32_t kdst = lds0 + wave * 2048, vdst = lds0 + kPPVOff + wave * 2048;
+  PPCopy cp;
+  cp.k0 = kbase + kpiece0; cp.k1 = kbase + kpiece1; cp.v0 = vbase + vpiece; cp.v1 = cp.v0;
+  // block J of the chunk -> stage J % 4 (rows past the chunk repeat its last row)
+#define SUBSPEC_PP_PLAN(J)                                                                     \
+  do {                                                                                         \
+    cp.r0 = min((J) * kKeyBlock + crow, nkeys - 1) * kAttnD;                                   \
+    cp.r1 = min((J) * kKeyBlock + crow + 4, nkeys - 1) * kAttnD;                               \
+    const uint32_t st_ = (uint32_t)((J) & (kPPStages - 1)) * kPPStageBytes;                    \
+    cp.kdst = kdst + st_; cp.vdst = vdst + st_;                                                \
+  } while (0)
+#define SUBSPEC_PP_ISSUE(J)                                                                    \
+  do {                                                                                         \
+    SUBSPEC_PP_PLAN(J);                                                                        \
+    pp_copy_issue(cp, 0); pp_copy_issue(cp, 1); pp_copy_issue(cp, 2); pp_copy_issue(cp, 3);    \
+  } while (0)
+  SUBSPEC_PP_ISSUE(0);
+  SUBSPEC_PP_ISSUE(1);
+
+  v16f oacc[kAttnD / 32], sacc[2];
+#pragma unroll
+  for (int dt = 0; dt < kAttnD / 32; ++dt)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) oacc[dt][r] = 0.f;
+#pragma unroll
+  for (int t = 0; t < 2; ++t)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) sacc[t][r] = 0.f;
+  uint4 pb[2][2] = {};
+  float m_run = -INFINITY, l_run = 0.f;
+
+  // operand addresses inside a stage (bytes).  K: key 32 t + lr, logical piece 2 ks + g.  V^T: the lane of a 16-lane group
+  // with index r supplies the 8 bytes of key 4 g + r / 4 (of the 16-key step's half) at d = 32 dt + 16 h + 4 (r % 4).
+  const int r16 = lane & 15, hh = (lane >> 4) & 1;
+  const uint32_t klane = lds0 + lr * 256;
+  const uint32_t vlane = lds0 + kPPVOff + (4 * g + (r16 >> 2)) * 256 + (2 * hh + ((r16 & 3) >> 1)) * 16 + (r16 & 1) * 8;
+  PPAddr ad;
+  ad.kx = (uint32_t)((g ^ (lr & 15)) << 4);
+  ad.vx = (uint32_t)((r16 >> 2) << 6);
+  PPRow rw{prefix, kv_len, mask_s + row * kPPMaskWords, ap.scale_log2, g, row_ok};
+#define SUBSPEC_PP_STAGES(I)                                                                   \
+  ad.vst = vlane + (uint32_t)(((I) - 1) & (kPPStages - 1)) * kPPStageBytes;                     \
+  ad.kst = klane + (uint32_t)((I) & (kPPStages - 1)) * kPPStageBytes
+
+  PP_T(1);
+  __builtin_amdgcn_s_waitcnt(0x0F70);                // the Q rows and mask words (and with them blocks 0 and 1)
+  PP_T(2);
+#pragma unroll
+  for (int u = 0; u < 2; ++u)
+    if (tid + u * 512 < kAttnRows * kPPMaskWords) mask_s[tid + u * 512] = mword[u];
+  __syncthreads();
+  PP_T(3);
+  if (grp_b) {
+    SUBSPEC_PP_ISSUE(2);
+    __syncthreads();
+  }
+  // ---- block 0: M is S^T only
+  if (!grp_b) SUBSPEC_PP_PLAN(2);
+  if (live) {
+    SUBSPEC_PP_STAGES(0);
+    pp_matrix_phase<DT, 0>(ad, cp, !grp_b, oacc, sacc, pb, qreg);
+  } else if (!grp_b) {
+    pp_copy_issue(cp, 0); pp_copy_issue(cp, 1); pp_copy_issue(cp, 2); pp_copy_issue(cp, 3);
+  }
+  if (grp_b) pp_wait_vmcnt4();
+  __syncthreads();
+  if (grp_b) SUBSPEC_PP_ISSUE(3);
+  if (live) pp_softmax_phase<DT>(key0, rw, sacc, oacc, pb, m_run, l_run);
+  if (!grp_b) pp_wait_vmcnt4();
+  __syncthreads();
+  PP_T(4);
+  for (int i = 1; i < nb; ++i) {
+    if (!grp_b) SUBSPEC_PP_PLAN(i + 2);
+    if (live) {
+      SUBSPEC_PP_STAGES(i);
+      pp_matrix_phase<DT, 2>(ad, cp, !grp_b, oacc, sacc, pb, qreg);
+    } else if (!grp_b) {
+      pp_copy_issue(cp, 0); pp_copy_issue(cp, 1); pp_copy_issue(cp, 2); pp_copy_issue(cp, 3);
+    }
+    PP_T(4 + 4 * i - 3);
+    if (grp_b) pp_wait_vmcnt4();
+    __syncthreads();
+    PP_T(4 + 4 * i - 2);
+    if (grp_b) SUBSPEC_PP_ISSUE(i + 3);
+    if (live) pp_softmax_phase<DT>(key0 + (int64_t)i * kKeyBlock, rw, sacc, oacc, pb, m_run, l_run);
+    PP_T(4 + 4 * i - 1);
+    if (!grp_b) pp_wait_vmcnt4();
+    __syncthreads();
+    PP_T(4 + 4 * i);
+  }
+  PP_T(80);
+  // ---- after the last block: M is O^T += V^T P^T only
+  if (live) {
+    SUBSPEC_PP_STAGES(nb);
+    pp_matrix_phase<DT, 1>(ad, cp, false, oacc, sacc, pb, qreg);
+  }
+  __syncthreads();
+  if (!grp_b) __syncthreads();
+#undef SUBSPEC_PP_STAGES
+#undef SUBSPEC_PP_PLAN
+#undef SUBSPEC_PP_ISSUE
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");     // no copy may still be on its way into LDS when the workgroup ends
+  PP_T(81);
+
+  float l = l_run + __shfl_xor(l_run, 32, kWave);
+  if (!live) return;
+  if (ap.chunks == 1) {
+    if (!row_ok) return;
+    const float inv = l > 0.f ? 1.0f / l : 0.f;
+    uint16_t* op = out + (((int64_t)b * n + ap.row0 + row) * ap.hq + qh) * kAttnD + g * 4;
+#pragma unroll
+    for (int dt = 0; dt < kAttnD / 32; ++dt)
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4)
+        *(uint2*)(op + dt * 32 + q4 * 8) = make_uint2(pack2<DT>(oacc[dt][4 * q4] * inv, oacc[dt][4 * q4 + 1] * inv),
+                                                      pack2<DT>(oacc[dt][4 * q4 + 2] * inv, oacc[dt][4 * q4 + 3] * inv));
+  } else {
+    float* po = part_o + (((int64_t)bh * ap.chunks + chunk) * 2 + tile) * kTileFloats + lane * 4;
+#pragma unroll
+    for (int dt = 0; dt < kAttnD / 32; ++dt)
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4)
+        *(v4f*)(po + (dt * 4 + q4) * 256) = v4f{oacc[dt][4 * q4], oacc[dt][4 * q4 + 1], oacc[dt][4 * q4 + 2], oacc[dt][4 * q4 + 3]};
+    if (g == 0) {
+      const int64_t pslot = ((int64_t)bh * ap.chunks + chunk) * kAttnRows + row;
+      *(v2f_t*)(part_ml + pslot * 2) = v2f_t{m_run * ap.scale_log2, l};
+    }
+  }
+#ifdef PP_TRACE
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  PP_T(82);
+#endif
+}
+
+// Merge for the tile layout above: one thread per four consecutive head dims of a row; blockIdx.x = (b, head, tile),
+// blockIdx.y = quarter of the tile's sixteen register quads.
+template <int DT>
+__global__ __launch_bounds__(256) void tree_attention32_merge_kernel(
+    const float* __restrict__ part_o, const float* __restrict__ part_ml, AttnParams ap, uint16_t* __restrict__ out) {
+  const int tile = blockIdx.x & 1, bh = blockIdx.x >> 1;
+  const int lane = threadIdx.x & 63, idx16 = blockIdx.y * 4 + (threadIdx.x >> 6);
+  const int row = tile * 32 + (lane & 31), g = lane >> 5;
+  if (row >= ap.win_rows) return;
+  const int b = bh / (int)ap.hq, qh = bh % (int)ap.hq;
+  const int64_t slot0 = (int64_t)bh * ap.chunks * kAttnRows + row;
+  const float* po = part_o + ((int64_t)bh * ap.chunks * 2 + tile) * kTileFloats + (idx16 * 64 + lane) * 4;
+  float m = -INFINITY;
+#pragma unroll 4
+  for (int c = 0; c < ap.chunks; ++c) m = fmaxf(m, part_ml[(slot0 + (int64_t)c * kAttnRows) * 2]);
+  v4f num = {0.f, 0.f, 0.f, 0.f};
+  float den = 0.f;
+#pragma unroll 4
+  for (int c = 0; c < ap.chunks; ++c) {
+    const v2f_t ml = *(const v2f_t*)(&part_ml[(slot0 + (int64_t)c * kAttnRows) * 2]);
+    const v4f oc = *(const v4f*)(po + (int64_t)c * 2 * kTileFloats);
+    const float w = ml[0] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(ml[0] - m);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) num[i] = fmaf(w, oc[i], num[i]);
+    den = fmaf(w, ml[1], den);
+  }
+  const float inv = den > 0.f ? 1.f / den : 0.f;
+  const int d0 = (idx16 >> 2) * 32 + (idx16 & 3) * 8 + g * 4;
+  *(uint2*)(out + (((int64_t)b * ap.n_rows + ap.row0 + row) * ap.hq + qh) * kAttnD + d0) =
+      make_uint2(pack2<DT>(num[0] * inv, num[1] * inv), pack2<DT>(num[2] * inv, num[3] * inv));
+}
+
 // Launch shape of one window of query rows.
-struct AttnPlan { int threads, rowt, wph, heads_per_wg, chunks; };
+struct AttnPlan { int threads, rowt, wph, heads_per_wg, chunks; bool mfma32; };
 static AttnPlan attn_plan(int64_t batch, int64_t hq, int64_t hkv, int64_t win_rows, int64_t kv_len) {
   AttnPlan pl;
   const int group = (int)(hq / hkv);
   const int64_t blocks = (kv_len + kKeyBlock - 1) / kKeyBlock;
-  if (win_rows <= 32) {
-    // a draft level: a wavefront is a whole head, eight heads share the staged keys
-    pl.threads = 512; pl.rowt = win_rows <= 16 ? 1 : 2; pl.wph = 1;
+  pl.mfma32 = win_rows > 16;
+  if (win_rows <= 16) {
+    // a draft level: a wavefront is a whole head (one 16-row tile), eight heads share the staged keys
+    pl.threads = 512; pl.rowt = 1; pl.wph = 1;
+  } else if (win_rows <= 32) {
+    // one 32-row tile per head, eight heads share the staged keys
+    pl.threads = 512; pl.rowt = 2; pl.wph = 1;
   } else if (batch * hq >= 128) {
-    // 33 to 64 rows, many (sequence, head) pairs: four heads share the staged keys (two wavefronts of 32 rows per head);
-    // the LDS traffic per head is less than half that of the one-head shape, which is what bounds this case
+    // 33 to 64 rows, many (sequence, head) pairs: four heads share the staged keys (two wavefronts of 32 rows per head)
     pl.threads = 512; pl.rowt = 2; pl.wph = 2;
   } else {
-    // 33 to 64 rows, few sequences: one head per 256-thread workgroup, so that the workgroups come from the heads
+    // 33 to 64 rows, few sequences: two heads per 256-thread workgroup, so that the workgroups come from the heads
     // and not from key chunks whose partial results would outweigh the keys
-    pl.threads = 256; pl.rowt = 1; pl.wph = 4;
+    pl.threads = 256; pl.rowt = 2; pl.wph = 2;
   }
   pl.heads_per_wg = (pl.threads / 64) / pl.wph;
   const int64_t wgs_per_chunk = batch * hkv * ((group + pl.heads_per_wg - 1) / pl.heads_per_wg);
-  // enough workgroups to cover the chip once, at least two key blocks per chunk ...
-  // enough workgroups to cover the chip once (three times with the small one-head workgroups, two or three of which
-  // share a compute unit), at least two key blocks per chunk ...
-  const int64_t target_wgs = pl.threads == 256 ? 768 : 256;
+  // enough workgroups to cover the chip once (twice with the small workgroups, two of which share a compute unit),
+  // at least two key blocks per chunk ...
+  const int64_t target_wgs = pl.threads == 256 ? 512 : 256;
   int64_t chunks = std::max<int64_t>(1, (target_wgs + wgs_per_chunk - 1) / wgs_per_chunk);
   if (win_rows <= 32) chunks = std::max<int64_t>(chunks, 1024 / std::max<int64_t>(1, batch * hq));   // few rows: short chunks, latency first
   chunks = std::min<int64_t>(chunks, std::max<int64_t>(1, blocks / 2));
   // ... and the partial results (fp32 rows x 128 per head and chunk) are priced against the K / V bytes (16-bit,
-  // 2 x kv_len x 128 per KV head): at most twice as many (config 3, one sequence: 29 MB of partials for 8.5 MB of keys
-  // before, 16.6 MB now; the same bytes again are read by the merge)
+  // 2 x kv_len x 128 per KV head): at most twice as many
   const int64_t by_bytes = std::max<int64_t>(1, 2 * (kv_len * hkv) / std::max<int64_t>(1, hq * win_rows));
   chunks = std::min<int64_t>(chunks, by_bytes);
   pl.chunks = (int)std::min<int64_t>(chunks, 64);
+  if (const char* e = getenv("SUBSPEC_ATTN_PLAN")) {     // tuning aid: "threads,wph,chunks" for windows of more than 32 rows
+    int t = 0, w = 0, c = 0;
+    if (win_rows > 32 && sscanf(e, "%d,%d,%d", &t, &w, &c) == 3 && (t == 512 || t == 256) && (w == 1 || w == 2) && c >= 1) {
+      pl.threads = t; pl.wph = 2; pl.heads_per_wg = (t / 64) / 2;
+      pl.chunks = (int)std::min<int64_t>(std::min<int64_t>(c, 64), std::max<int64_t>(1, blocks));
+    }
+  }
   return pl;
 }
 // the most partial slots any window of a call can need (the first window is the largest)
@@ -558,22 +1234,37 @@ static int tree_attention_impl(const char* what, const void* q, const void* k_ca
 #define SUBSPEC_ATTN_KERNEL(DT, PAGED, ROWT, WPH, THREADS)                                                          \
   hipLaunchKernelGGL((tree_attention_kernel<DT, PAGED, ROWT, WPH, THREADS>), grid, dim3(THREADS), 0, st, (const uint16_t*)q, \
                      (const uint16_t*)k_cache, (const uint16_t*)v_cache, anc_bits, ap, (uint16_t*)out, part_o, part_ml)
+#define SUBSPEC_ATTN32_KERNEL(DT, PAGED, WPH, THREADS)                                                             \
+  hipLaunchKernelGGL((tree_attention32_kernel<DT, PAGED, WPH, THREADS>), grid, dim3(THREADS), 0, st, (const uint16_t*)q, \
+                     (const uint16_t*)k_cache, (const uint16_t*)v_cache, anc_bits, ap, (uint16_t*)out, part_o, part_ml)
+#define SUBSPEC_ATTNPP_KERNEL(DT, WPH)                                                                             \
+  hipLaunchKernelGGL((tree_attention_pp_kernel<DT, WPH>), grid, dim3(512), 0, st, (const uint16_t*)q,              \
+                     (const uint16_t*)k_cache, (const uint16_t*)v_cache, anc_bits, ap, (uint16_t*)out, part_o, part_ml)
 #define SUBSPEC_ATTN_LAUNCH(DT, PAGED)                                                                             \
   do {                                                                                                             \
     {                                                                                                              \
       DominantKernelTimer timer(st);                                                                               \
-      if (pl.threads == 256) SUBSPEC_ATTN_KERNEL(DT, PAGED, 1, 4, 256);                                            \
-      else if (pl.wph == 2) SUBSPEC_ATTN_KERNEL(DT, PAGED, 2, 2, 512);                                             \
-      else if (pl.rowt == 1) SUBSPEC_ATTN_KERNEL(DT, PAGED, 1, 1, 512);                                            \
-      else SUBSPEC_ATTN_KERNEL(DT, PAGED, 2, 1, 512);                                                              \
+      if (!pl.mfma32) SUBSPEC_ATTN_KERNEL(DT, PAGED, 1, 1, 512);                                                   \
+      else if (pl.threads == 512 && !PAGED && !getenv("SUBSPEC_ATTN_NOPP")) {                                      \
+        if (pl.wph == 1) SUBSPEC_ATTNPP_KERNEL(DT, 1); else SUBSPEC_ATTNPP_KERNEL(DT, 2);                          \
+      }                                                                                                            \
+      else if (pl.wph == 1) SUBSPEC_ATTN32_KERNEL(DT, PAGED, 1, 512);                                              \
+      else if (pl.threads == 512) SUBSPEC_ATTN32_KERNEL(DT, PAGED, 2, 512);                                        \
+      else SUBSPEC_ATTN32_KERNEL(DT, PAGED, 2, 256);                                                               \
     }                                                                                                              \
-    if (ap.chunks > 1)                                                                                             \
-      hipLaunchKernelGGL((tree_attention_merge_kernel<DT>), merge_grid, dim3(merge_rows * 32), 0, st, part_o, part_ml, ap, \
-                         (uint16_t*)out);                                                                          \
+    if (ap.chunks > 1) {                                                                                           \
+      if (pl.mfma32)                                                                                               \
+        hipLaunchKernelGGL((tree_attention32_merge_kernel<DT>), dim3((unsigned)(batch * n_q_heads * 2), 4), dim3(256), 0, st, \
+                           part_o, part_ml, ap, (uint16_t*)out);                                                   \
+      else                                                                                                         \
+        hipLaunchKernelGGL((tree_attention_merge_kernel<DT>), merge_grid, dim3(merge_rows * 32), 0, st, part_o, part_ml, ap, \
+                           (uint16_t*)out);                                                                        \
+    }                                                                                                              \
   } while (0)
     if (dtype == SUBSPEC_BF16) { if (paged) SUBSPEC_ATTN_LAUNCH(SUBSPEC_BF16, true); else SUBSPEC_ATTN_LAUNCH(SUBSPEC_BF16, false); }
     else { if (paged) SUBSPEC_ATTN_LAUNCH(SUBSPEC_F16, true); else SUBSPEC_ATTN_LAUNCH(SUBSPEC_F16, false); }
 #undef SUBSPEC_ATTN_LAUNCH
+#undef SUBSPEC_ATTN32_KERNEL
 #undef SUBSPEC_ATTN_KERNEL
   }
   SUBSPEC_CHECK_HIP(hipGetLastError());
