@@ -444,7 +444,7 @@ __device__ __forceinline__ v16f mfma32x32(uint4 a, uint4 b, v16f c) {
 }
 constexpr int kKStride32 = kAttnD + 8;    // 272-byte rows: the 16-byte reads of 16 consecutive keys tile the 64 banks
 constexpr int kVStride32 = kAttnD + 32;   // 320-byte rows: a transposing read takes 64 bytes of each of 4 keys per 32 lanes
-constexpr int kTileFloats = 32 * kAttnD;  // fp32 partial O of one 32-row tile, stored [16 (d-tile, quad)][64 lanes][4]
+constexpr int kTileElems = 32 * kAttnD;   // partial O of one 32-row tile, 16-bit, stored [16 (d-tile, quad)][64 lanes][4]
 
 // WPH wavefronts per head (1: up to 32 rows, 2: up to 64), THREADS / 64 / WPH heads of one KV head per workgroup.
 template <int DT, bool PAGED, int WPH, int THREADS>
@@ -487,19 +487,6 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
   const int row = tile * 32 + lr;                       // row inside this launch's window
   const bool row_ok = head_ok && row < ap.win_rows;
   const int grow = ap.row0 + (row_ok ? row : 0);
-
-  // Q^T operands: B[k = 8 g + e][row] = Q[row][16 ks + 8 g + e]
-  uint4 qreg[kAttnD / 16];
-  {
-    const uint16_t* qp = q + ((int64_t)bh * n + grow) * kAttnD + g * 8;
-#pragma unroll
-    for (int ks = 0; ks < kAttnD / 16; ++ks) qreg[ks] = row_ok ? *(const uint4*)(qp + ks * 16) : make_uint4(0, 0, 0, 0);
-  }
-  for (int i = tid; i < kAttnRows * (SUBSPEC_MAX_TREE_NODES / 64 + 1); i += THREADS) {
-    const int r = i / (SUBSPEC_MAX_TREE_NODES / 64 + 1), w = i % (SUBSPEC_MAX_TREE_NODES / 64 + 1);
-    mask_s[r][w] = (r < ap.win_rows && w < ap.mask_words)
-                       ? anc[((int64_t)b * ap.anc_batch_stride + ap.row0 + r) * ap.mask_words + w] : 0ull;
-  }
 
   v16f oacc[kAttnD / 32];
 #pragma unroll
@@ -547,10 +534,32 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
   // Every fetch and every stage is unconditional (rows beyond the chunk repeat its last row and are never multiplied):
   // the counter that a wait names is fixed at compile time, and a request that is issued on one path only makes the
   // compiler wait for ALL requests in flight wherever the paths join.
+  // The longest transfer first, and nothing waits before everything is on its way: the first two key blocks, the Q rows
+  // (B operands: B[k = 8 g + e][row] = Q[row][16 ks + 8 g + e]), the mask words -- the latter only in chunks that reach the tree.
   SUBSPEC_ATTN32_FETCH(0, key0);
   SUBSPEC_ATTN32_FETCH(1, key0 + kKeyBlock);
+  uint4 qreg[kAttnD / 16];
+  {
+    const uint16_t* qp = q + ((int64_t)bh * n + grow) * kAttnD + g * 8;
+#pragma unroll
+    for (int ks = 0; ks < kAttnD / 16; ++ks) qreg[ks] = row_ok ? *(const uint4*)(qp + ks * 16) : make_uint4(0, 0, 0, 0);
+  }
+  constexpr int kMaskWords = SUBSPEC_MAX_TREE_NODES / 64 + 1, kMaskPerThread = (kAttnRows * kMaskWords + THREADS - 1) / THREADS;
+  uint64_t mword[kMaskPerThread];
+  const bool reaches_tree = key1 > prefix;             // (uniform)
+#pragma unroll
+  for (int u = 0; u < kMaskPerThread; ++u) {
+    const int i = tid + u * THREADS, r = i / kMaskWords, w = i % kMaskWords;
+    mword[u] = (reaches_tree && i < kAttnRows * kMaskWords && r < ap.win_rows && w < ap.mask_words)
+                   ? anc[((int64_t)b * ap.anc_batch_stride + ap.row0 + r) * ap.mask_words + w] : 0ull;
+  }
   SUBSPEC_ATTN32_STAGE(0);
   SUBSPEC_ATTN32_FETCH(0, key0 + 2 * kKeyBlock);
+  if (reaches_tree) {
+#pragma unroll
+    for (int u = 0; u < kMaskPerThread; ++u)
+      if (tid + u * THREADS < kAttnRows * kMaskWords) (&mask_s[0][0])[tid + u * THREADS] = mword[u];
+  }
 
   // LDS addresses of the lane's operands.  K: key 32 t + lr, pieces of 16 bytes at 16 ks + 8 g.  V^T (transposing read,
   // per 16 lanes: lane r supplies the 8 bytes of key r / 4 at d = 4 (r % 4) and receives four keys of d = r): keys
@@ -666,13 +675,16 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
         *(uint2*)(op + dt * 32 + q4 * 8) = make_uint2(pack2<DT>(oacc[dt][4 * q4] * inv, oacc[dt][4 * q4 + 1] * inv),
                                                       pack2<DT>(oacc[dt][4 * q4 + 2] * inv, oacc[dt][4 * q4 + 3] * inv));
   } else {
-    // partial tile: every store instruction of the wavefront writes 1 KB of consecutive addresses
-    float* po = part_o + (((int64_t)bh * ap.chunks + chunk) * 2 + tile) * kTileFloats + lane * 4;
+    // the chunk's own softmax-weighted average of V, in the 16-bit dtype (a convex combination of such averages is what the
+    // merge forms, so their rounding error does not grow); every store instruction writes 512 consecutive bytes
+    const float inv = l > 0.f ? 1.0f / l : 0.f;
+    uint16_t* po = (uint16_t*)part_o + (((int64_t)bh * ap.chunks + chunk) * 2 + tile) * kTileElems + lane * 4;
 #pragma unroll
     for (int dt = 0; dt < kAttnD / 32; ++dt)
 #pragma unroll
       for (int q4 = 0; q4 < 4; ++q4)
-        *(v4f*)(po + (dt * 4 + q4) * 256) = v4f{oacc[dt][4 * q4], oacc[dt][4 * q4 + 1], oacc[dt][4 * q4 + 2], oacc[dt][4 * q4 + 3]};
+        *(uint2*)(po + (dt * 4 + q4) * 256) = make_uint2(pack2<DT>(oacc[dt][4 * q4] * inv, oacc[dt][4 * q4 + 1] * inv),
+                                                         pack2<DT>(oacc[dt][4 * q4 + 2] * inv, oacc[dt][4 * q4 + 3] * inv));
     if (g == 0) {
       const int64_t pslot = ((int64_t)bh * ap.chunks + chunk) * kAttnRows + row;
       *(v2f_t*)(part_ml + pslot * 2) = v2f_t{m_run * ap.scale_log2, l};
@@ -690,7 +702,7 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
 // 4..7 (group B, the second wavefront of each SIMD) enter the loop one barrier later than wavefronts 0..3 (group A), so
 // whenever one wavefront of a SIMD is in M the other is in V.
 // K / V blocks travel from memory straight into LDS (global_load_lds_dwordx4: no staging registers, no LDS write
-// instructions) through a ring of four stages, issued four phases (two blocks) before their first use.  The copies are
+// instructions) through a ring of four stages; a wavefront issues its share of block i + 2 inside the M phase of block i.  The copies are
 // inline assembly ON PURPOSE: a wait names a count fixed at compile time, and for LDS-DMA requests it knows about the
 // compiler waits for all of them before every LDS read; the waits for these are placed by hand (group A at the end of
 // V, group B at the end of M: every odd global phase).  A stage's rows are unpadded (a DMA instruction writes 1 KB of
@@ -719,6 +731,12 @@ __device__ __forceinline__ void pp_dma16(uint32_t lds_base, const uint16_t* src)
 // its use and waits for it, with the matrix pipe idle meanwhile).  With `copy`, the wavefront's four K / V copy instructions
 // of the block two ahead are issued a quarter of the steps apart instead of in a row: a copy instruction waits for room in the
 // compute unit's memory pipeline, and that wait then falls into the shadow of a matrix instruction.
+// A wavefront on its own issues an instruction every five to six cycles, so the phase is as much a count of instructions
+// as of matrix cycles: the twelve operand addresses (8 d steps of K, 4 d tiles of V^T; the XOR swizzle keeps them from
+// being immediates) are formed once per phase, the key offsets are immediates.
+// The S^T accumulators do not start at zero but at -ref, the row's reference score (PPRef below), so the softmax does not
+// subtract.  (Q scaled by scale * log2(e) beforehand would save the multiplication as well, but rounds Q a second time:
+// 3 % error in the probabilities of rows whose scores reach the hundreds.  Not done.)
 struct PPAddr { uint32_t vst, kst, vx, kx; };
 // a wavefront's four copy instructions of one block: K rows 0..3, K rows 4..7, V rows 0..3, V rows 4..7 of its share
 struct PPCopy {
@@ -735,28 +753,40 @@ __device__ __forceinline__ void pp_copy_issue(const PPCopy& cp, int c) {
 template <int MODE> __device__ __forceinline__ constexpr bool pp_step_is_pv(int k) { return MODE == 1 || (MODE == 2 && (k & 1) == 0); }
 template <int MODE> __device__ __forceinline__ constexpr int pp_step_index(int k) { return MODE == 2 ? k >> 1 : k; }
 template <int DT, int MODE>
-__device__ __forceinline__ dec_u4 pp_load_step(int k, const PPAddr& ad) {
+__device__ __forceinline__ dec_u4 pp_load_step(int k, const uint32_t (&kaddr)[8], const uint32_t (&vaddr)[4]) {
   const int j = pp_step_index<MODE>(k);
   if (pp_step_is_pv<MODE>(k)) {
     const int ts = j >> 2, dt = j & 3;                   // ts = 2 t + s: keys 16 ts .. 16 ts + 15 of the block
-    const uint32_t va = ad.vst + (ad.vx ^ (uint32_t)(dt << 6)) + (uint32_t)(ts * 16 * 256);
+    const uint32_t va = vaddr[dt] + (uint32_t)(ts * 16 * 256);
     const uint2 lo = lds_read_tr16((const uint16_t*)(__attribute__((address_space(3))) uint16_t*)(uintptr_t)va);
     const uint2 hi = lds_read_tr16((const uint16_t*)(__attribute__((address_space(3))) uint16_t*)(uintptr_t)(va + 8 * 256));
     return dec_u4{lo.x, lo.y, hi.x, hi.y};
   } else {
     const int ks = j >> 1, t = j & 1;
-    const uint32_t ka = ad.kst + (ad.kx ^ (uint32_t)(ks << 5)) + (uint32_t)(t * 32 * 256);
+    const uint32_t ka = kaddr[ks] + (uint32_t)(t * 32 * 256);
     return *(const dec_u4*)(__attribute__((address_space(3))) dec_u4*)(uintptr_t)ka;
   }
 }
 template <int DT, int MODE>
 __device__ __forceinline__ void pp_matrix_phase(const PPAddr& ad, const PPCopy& cp, bool copy, v16f (&oacc)[4], v16f (&sacc)[2],
-                                                const uint4 (&pb)[2][2], const uint4 (&qreg)[8]) {
+                                                const v16f& cinit, const uint4 (&pb)[2][2], const uint4 (&qreg)[8]) {
   constexpr int kSteps = MODE == 2 ? 32 : 16;
   constexpr int kAhead = 4;
+  // the wavefront that multiplies goes first: between two wavefronts of a SIMD the older one wins every issue slot, and
+  // without this group B's matrix phases take a third longer than group A's
+  __builtin_amdgcn_s_setprio(1);
+  uint32_t kaddr[8], vaddr[4];
+  if (MODE != 1) {
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) kaddr[ks] = ad.kst + (ad.kx ^ (uint32_t)(ks << 5));
+  }
+  if (MODE != 0) {
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt) vaddr[dt] = ad.vst + (ad.vx ^ (uint32_t)(dt << 6));
+  }
   dec_u4 ring[kAhead];
 #pragma unroll
-  for (int k = 0; k < kAhead; ++k) ring[k] = pp_load_step<DT, MODE>(k, ad);
+  for (int k = 0; k < kAhead; ++k) ring[k] = pp_load_step<DT, MODE>(k, kaddr, vaddr);
   __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
   for (int k = 0; k < kSteps; ++k) {
@@ -767,40 +797,40 @@ __device__ __forceinline__ void pp_matrix_phase(const PPAddr& ad, const PPCopy& 
       oacc[dt] = mfma32x32<DT>(a, pb[ts >> 1][ts & 1], oacc[dt]);
     } else {
       const int ks = j >> 1, t = j & 1;
-      if (ks == 0) {
-        v16f z;
-#pragma unroll
-        for (int r = 0; r < 16; ++r) z[r] = 0.f;
-        sacc[t] = mfma32x32<DT>(a, qreg[0], z);
-      } else {
-        sacc[t] = mfma32x32<DT>(a, qreg[ks], sacc[t]);
-      }
+      sacc[t] = mfma32x32<DT>(a, qreg[ks], ks == 0 ? cinit : sacc[t]);
     }
     __builtin_amdgcn_sched_barrier(0);
-    if (k + kAhead < kSteps) ring[k % kAhead] = pp_load_step<DT, MODE>(k + kAhead, ad);
+    if (k + kAhead < kSteps) ring[k % kAhead] = pp_load_step<DT, MODE>(k + kAhead, kaddr, vaddr);
     if (k % (kSteps / 4) == 1 && copy) pp_copy_issue(cp, k / (kSteps / 4));       // (uniform)
     __builtin_amdgcn_sched_barrier(0);
   }
+  __builtin_amdgcn_s_setprio(0);
 }
 
-// Online-softmax step of one 64-key block on the S^T accumulators (vector ALU only): masks the tree part, moves the running
-// maximum and sum, rescales O when a maximum moved, leaves P^T packed as the B operands of the next phase's O^T += V^T P^T.
-// Four partial sums and two partial maxima: the wavefront issues in the gaps the other wavefront's matrix instructions
-// leave, and a single dependent chain would wait for its own previous result in every one of them.
+// Online-softmax step of one 64-key block on the S^T accumulators (vector ALU only).  The accumulators hold raw scores
+// relative to the row's REFERENCE score `ref`, which is not the running maximum but something within kPPSlack (in exp2
+// units) of it from below: the first block that shows the row a key sets it to that block's maximum, a later block moves it only when its
+// maximum exceeds it by more than kPPSlack (then O, the running sum and this block's arguments are rescaled -- rare once
+// the first blocks are through).  Probabilities are therefore at most 2^kPPSlack instead of at most 1, which costs neither
+// range nor precision in bf16 / fp16 x fp32, and the common case is 16 three-way maxima, 32 exponentials, 16 packed
+// conversions and 16 two-element dot products against ones for the row sum, besides the 32 multiplications by the scale.
+constexpr float kPPSlack = 8.0f;
 struct PPRow { int64_t prefix, kv_len; const uint64_t* mask_row; float scale_log2; int g; bool row_ok; };
+struct PPRef { float ref, l; bool have; };
 template <int DT>
-__device__ __forceinline__ void pp_softmax_phase(int64_t kb, const PPRow& rw, v16f (&sacc)[2], v16f (&oacc)[4], uint4 (&pb)[2][2],
-                                                 float& m_run, float& l_run) {
+__device__ __forceinline__ float pp_pair_sum(uint32_t packed, float acc) {
+  if constexpr (DT == SUBSPEC_BF16) return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(v2bf_t, packed), __builtin_bit_cast(v2bf_t, 0x3f803f80u), acc, false);
+  else return __builtin_amdgcn_fdot2(__builtin_bit_cast(v2h_t, packed), __builtin_bit_cast(v2h_t, 0x3c003c00u), acc, false);
+}
+__device__ __forceinline__ float pp_max_halves(float x) {          // maximum of lanes i and i ^ 32, in both
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+template <int DT>
+__device__ __forceinline__ void pp_softmax_phase(int64_t kb, const PPRow& rw, v16f (&sacc)[2], v16f (&oacc)[4], v16f& cinit,
+                                                 uint4 (&pb)[2][2], PPRef& rf) {
   const bool plain = kb + kKeyBlock <= rw.prefix;
-  float mloc = -INFINITY;
-  if (plain) {
-    float mt[2] = {-INFINITY, -INFINITY};
-#pragma unroll
-    for (int t = 0; t < 2; ++t)
-#pragma unroll
-      for (int r = 0; r < 16; r += 2) mt[t] = fmaxf(fmaxf(sacc[t][r], sacc[t][r + 1]), mt[t]);
-    mloc = fmaxf(mt[0], mt[1]);
-  } else {
+  if (!plain) {
     // a 64-key block touches at most two consecutive words of the row's bitset (a zero word follows the last)
     const int word0 = min((int)(max(kb - rw.prefix, (int64_t)0) >> 6), SUBSPEC_MAX_TREE_NODES / 64 - 1);
     const uint64_t bits0 = rw.row_ok ? rw.mask_row[word0] : 0ull, bits1 = rw.row_ok ? rw.mask_row[word0 + 1] : 0ull;
@@ -814,23 +844,32 @@ __device__ __forceinline__ void pp_softmax_phase(int64_t kb, const PPRow& rw, v1
         const int rel = tree ? (int)(pos - rw.prefix) : 0;
         const uint64_t word = (rel >> 6) == word0 ? bits0 : bits1;
         const bool ok = in_range && (!tree || ((word >> (rel & 63)) & 1ull));
-        const float tv = ok ? sacc[t][r] : -INFINITY;
-        sacc[t][r] = tv;
-        mloc = fmaxf(mloc, tv);
+        sacc[t][r] = ok ? sacc[t][r] : -INFINITY;
       }
     }
   }
-  mloc = fmaxf(mloc, __shfl_xor(mloc, 32, kWave));
-  const float m_new = fmaxf(m_run, mloc);
-  const float m_use = m_new == -INFINITY ? 0.f : m_new;
-  const float alpha = __builtin_amdgcn_exp2f((m_run - m_use) * rw.scale_log2);
-  m_run = m_new;
-  const float mneg = -m_use * rw.scale_log2;
-  if (__any(alpha != 1.0f)) {
-    l_run *= alpha;
+  float mt[2] = {-INFINITY, -INFINITY};
+#pragma unroll
+  for (int t = 0; t < 2; ++t)
+#pragma unroll
+    for (int r = 0; r < 16; r += 2) mt[t] = fmaxf(fmaxf(sacc[t][r], sacc[t][r + 1]), mt[t]);
+  const float mloc = pp_max_halves(fmaxf(mt[0], mt[1]));           // raw score units, relative to ref
+  const bool move = mloc > -INFINITY && (!rf.have || mloc * rw.scale_log2 > kPPSlack);
+  if (__any(move)) {
+    const float d = move ? mloc : 0.f;                              // the row's reference goes up (first time: anywhere) by d
+    const float alpha = __builtin_amdgcn_exp2f(-d * rw.scale_log2);
+    rf.ref += d;
+    rf.l *= alpha;
 #pragma unroll
     for (int dt = 0; dt < kAttnD / 32; ++dt) oacc[dt] *= alpha;
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) sacc[t][r] -= d;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) cinit[r] = -rf.ref;
   }
+  rf.have = rf.have || mloc > -INFINITY;
   float lsum[2][2];
 #pragma unroll
   for (int t = 0; t < 2; ++t) {
@@ -838,23 +877,14 @@ __device__ __forceinline__ void pp_softmax_phase(int64_t kb, const PPRow& rw, v1
     for (int s = 0; s < 2; ++s) {
       float p[8];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) p[e] = __builtin_amdgcn_exp2f(fmaf(sacc[t][8 * s + e], rw.scale_log2, mneg));
-      lsum[t][s] = ((p[0] + p[1]) + (p[2] + p[3])) + ((p[4] + p[5]) + (p[6] + p[7]));
+      for (int e = 0; e < 8; ++e) p[e] = __builtin_amdgcn_exp2f(sacc[t][8 * s + e] * rw.scale_log2);
       pb[t][s] = make_uint4(pack2<DT>(p[0], p[1]), pack2<DT>(p[2], p[3]), pack2<DT>(p[4], p[5]), pack2<DT>(p[6], p[7]));
+      lsum[t][s] = pp_pair_sum<DT>(pb[t][s].w, pp_pair_sum<DT>(pb[t][s].z, pp_pair_sum<DT>(pb[t][s].y, pp_pair_sum<DT>(pb[t][s].x, 0.f))));
     }
   }
-  l_run += (lsum[0][0] + lsum[0][1]) + (lsum[1][0] + lsum[1][1]);
+  rf.l += (lsum[0][0] + lsum[0][1]) + (lsum[1][0] + lsum[1][1]);
 }
 
-#ifndef PP_GRP
-#define PP_GRP(W) (((W) >> 2) & 1)
-#endif
-#ifdef PP_TRACE
-__device__ long long pp_trace[4096 * 2 * 96];
-#define PP_T(IDX) do { if (lane == 0 && (wave == 0 || wave == (PP_GRP(1) ? 1 : PP_GRP(2) ? 2 : 4)) && (IDX) < 96) pp_trace[(blockIdx.x * 2 + (wave != 0)) * 96 + (IDX)] = clock64(); } while (0)
-#else
-#define PP_T(IDX) do {} while (0)
-#endif
 template <int DT, int WPH>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void tree_attention_pp_kernel(
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ kc, const uint16_t* __restrict__ vc,
@@ -878,7 +908,6 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  PP_T(0);
   const int lr = lane & 31, g = lane >> 5;
   constexpr int kHeadsPerWG = 8 / WPH;
   const int head_in_group = pair * kHeadsPerWG + wave / WPH;
@@ -893,7 +922,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   const bool live = head_ok && tile * 32 < ap.win_rows;     // (wave-uniform) this wavefront has rows to work on
   const bool row_ok = head_ok && row < ap.win_rows;
   const int grow = ap.row0 + (row_ok ? row : 0);
-  const bool grp_b = PP_GRP(wave) != 0;
+  const bool grp_b = wave >= 4;                             // the second wavefront of each SIMD (wavefront w runs on SIMD w % 4)
 
   const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)lds;
   const int64_t key0 = (int64_t)chunk * ap.chunk_keys;
@@ -902,23 +931,6 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   const int nb = (nkeys + kKeyBlock - 1) / kKeyBlock;
   const uint16_t* kbase = kc + (((int64_t)b * ap.hkv + kvh) * ap.seq_stride + key0) * kAttnD;
   const uint16_t* vbase = vc + (((int64_t)b * ap.hkv + kvh) * ap.seq_stride + key0) * kAttnD;
-
-  // ---- everything that has to come out of memory before the first product is requested at once: Q rows, mask words,
-  //      then the first two K / V blocks; one wait covers all of it
-  uint4 qreg[kAttnD / 16];
-  {
-    const uint16_t* qp = q + ((int64_t)bh * n + grow) * kAttnD + g * 8;
-#pragma unroll
-    for (int ks = 0; ks < kAttnD / 16; ++ks) qreg[ks] = row_ok ? *(const uint4*)(qp + ks * 16) : make_uint4(0, 0, 0, 0);
-  }
-  uint64_t* mask_s = (uint64_t*)(lds + kPPMaskOff);
-  uint64_t mword[2];
-#pragma unroll
-  for (int u = 0; u < 2; ++u) {
-    const int i = tid + u * 512, r = i / kPPMaskWords, w = i % kPPMaskWords;
-    mword[u] = (i < kAttnRows * kPPMaskWords && r < ap.win_rows && w < ap.mask_words)
-                   ? anc[((int64_t)b * ap.anc_batch_stride + ap.row0 + r) * ap.mask_words + w] : 0ull;
-  }
 
   // ---- copies: wavefront w brings rows 8 w .. 8 w + 7 of a block, K and V, two instructions of four rows each
   const int crow = wave * 8 + (lane >> 4);                                       // row of the first instruction; + 4 for the second
@@ -942,6 +954,23 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   } while (0)
   SUBSPEC_PP_ISSUE(0);
   SUBSPEC_PP_ISSUE(1);
+  // ---- everything else that has to come out of memory before the first product, requested behind the first two K / V blocks
+  //      (the longest transfer first); one wait covers all of it
+  uint4 qreg[kAttnD / 16];
+  {
+    const uint16_t* qp = q + ((int64_t)bh * n + grow) * kAttnD + g * 8;
+#pragma unroll
+    for (int ks = 0; ks < kAttnD / 16; ++ks) qreg[ks] = row_ok ? *(const uint4*)(qp + ks * 16) : make_uint4(0, 0, 0, 0);
+  }
+  uint64_t* mask_s = (uint64_t*)(lds + kPPMaskOff);
+  uint64_t mword[2];
+#pragma unroll
+  for (int u = 0; u < 2; ++u) {
+    const int i = tid + u * 512, r = i / kPPMaskWords, w = i % kPPMaskWords;
+    mword[u] = (i < kAttnRows * kPPMaskWords && r < ap.win_rows && w < ap.mask_words)
+                   ? anc[((int64_t)b * ap.anc_batch_stride + ap.row0 + r) * ap.mask_words + w] : 0ull;
+  }
+
 
   v16f oacc[kAttnD / 32], sacc[2];
 #pragma unroll
@@ -953,7 +982,10 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
     for (int r = 0; r < 16; ++r) sacc[t][r] = 0.f;
   uint4 pb[2][2] = {};
-  float m_run = -INFINITY, l_run = 0.f;
+  v16f cinit;                                          // -ref in every register: what an S^T accumulator starts from
+#pragma unroll
+  for (int r = 0; r < 16; ++r) cinit[r] = 0.f;
+  PPRef rf{0.f, 0.f, false};
 
   // operand addresses inside a stage (bytes).  K: key 32 t + lr, logical piece 2 ks + g.  V^T: the lane of a 16-lane group
   // with index r supplies the 8 bytes of key 4 g + r / 4 (of the 16-key step's half) at d = 32 dt + 16 h + 4 (r % 4).
@@ -968,57 +1000,43 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   ad.vst = vlane + (uint32_t)(((I) - 1) & (kPPStages - 1)) * kPPStageBytes;                     \
   ad.kst = klane + (uint32_t)((I) & (kPPStages - 1)) * kPPStageBytes
 
-  PP_T(1);
   __builtin_amdgcn_s_waitcnt(0x0F70);                // the Q rows and mask words (and with them blocks 0 and 1)
-  PP_T(2);
 #pragma unroll
   for (int u = 0; u < 2; ++u)
     if (tid + u * 512 < kAttnRows * kPPMaskWords) mask_s[tid + u * 512] = mword[u];
   __syncthreads();
-  PP_T(3);
-  if (grp_b) {
-    SUBSPEC_PP_ISSUE(2);
-    __syncthreads();
-  }
+  if (grp_b) __syncthreads();
   // ---- block 0: M is S^T only
-  if (!grp_b) SUBSPEC_PP_PLAN(2);
+  SUBSPEC_PP_PLAN(2);
   if (live) {
     SUBSPEC_PP_STAGES(0);
-    pp_matrix_phase<DT, 0>(ad, cp, !grp_b, oacc, sacc, pb, qreg);
-  } else if (!grp_b) {
+    pp_matrix_phase<DT, 0>(ad, cp, true, oacc, sacc, cinit, pb, qreg);
+  } else {
     pp_copy_issue(cp, 0); pp_copy_issue(cp, 1); pp_copy_issue(cp, 2); pp_copy_issue(cp, 3);
   }
   if (grp_b) pp_wait_vmcnt4();
   __syncthreads();
-  if (grp_b) SUBSPEC_PP_ISSUE(3);
-  if (live) pp_softmax_phase<DT>(key0, rw, sacc, oacc, pb, m_run, l_run);
+  if (live) pp_softmax_phase<DT>(key0, rw, sacc, oacc, cinit, pb, rf);
   if (!grp_b) pp_wait_vmcnt4();
   __syncthreads();
-  PP_T(4);
   for (int i = 1; i < nb; ++i) {
-    if (!grp_b) SUBSPEC_PP_PLAN(i + 2);
+    SUBSPEC_PP_PLAN(i + 2);
     if (live) {
       SUBSPEC_PP_STAGES(i);
-      pp_matrix_phase<DT, 2>(ad, cp, !grp_b, oacc, sacc, pb, qreg);
-    } else if (!grp_b) {
+      pp_matrix_phase<DT, 2>(ad, cp, true, oacc, sacc, cinit, pb, qreg);
+    } else {
       pp_copy_issue(cp, 0); pp_copy_issue(cp, 1); pp_copy_issue(cp, 2); pp_copy_issue(cp, 3);
     }
-    PP_T(4 + 4 * i - 3);
     if (grp_b) pp_wait_vmcnt4();
     __syncthreads();
-    PP_T(4 + 4 * i - 2);
-    if (grp_b) SUBSPEC_PP_ISSUE(i + 3);
-    if (live) pp_softmax_phase<DT>(key0 + (int64_t)i * kKeyBlock, rw, sacc, oacc, pb, m_run, l_run);
-    PP_T(4 + 4 * i - 1);
+    if (live) pp_softmax_phase<DT>(key0 + (int64_t)i * kKeyBlock, rw, sacc, oacc, cinit, pb, rf);
     if (!grp_b) pp_wait_vmcnt4();
     __syncthreads();
-    PP_T(4 + 4 * i);
   }
-  PP_T(80);
   // ---- after the last block: M is O^T += V^T P^T only
   if (live) {
     SUBSPEC_PP_STAGES(nb);
-    pp_matrix_phase<DT, 1>(ad, cp, false, oacc, sacc, pb, qreg);
+    pp_matrix_phase<DT, 1>(ad, cp, false, oacc, sacc, cinit, pb, qreg);
   }
   __syncthreads();
   if (!grp_b) __syncthreads();
@@ -1026,9 +1044,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #undef SUBSPEC_PP_PLAN
 #undef SUBSPEC_PP_ISSUE
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");     // no copy may still be on its way into LDS when the workgroup ends
-  PP_T(81);
 
-  float l = l_run + __shfl_xor(l_run, 32, kWave);
+  const float l = rf.l + __shfl_xor(rf.l, 32, kWave);
   if (!live) return;
   if (ap.chunks == 1) {
     if (!row_ok) return;
@@ -1041,25 +1058,26 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         *(uint2*)(op + dt * 32 + q4 * 8) = make_uint2(pack2<DT>(oacc[dt][4 * q4] * inv, oacc[dt][4 * q4 + 1] * inv),
                                                       pack2<DT>(oacc[dt][4 * q4 + 2] * inv, oacc[dt][4 * q4 + 3] * inv));
   } else {
-    float* po = part_o + (((int64_t)bh * ap.chunks + chunk) * 2 + tile) * kTileFloats + lane * 4;
+    // the chunk's own softmax-weighted average of V, in the 16-bit dtype (a convex combination of such averages is what the
+    // merge forms, so their rounding error does not grow); every store instruction writes 512 consecutive bytes
+    const float inv = l > 0.f ? 1.0f / l : 0.f;
+    uint16_t* po = (uint16_t*)part_o + (((int64_t)bh * ap.chunks + chunk) * 2 + tile) * kTileElems + lane * 4;
 #pragma unroll
     for (int dt = 0; dt < kAttnD / 32; ++dt)
 #pragma unroll
       for (int q4 = 0; q4 < 4; ++q4)
-        *(v4f*)(po + (dt * 4 + q4) * 256) = v4f{oacc[dt][4 * q4], oacc[dt][4 * q4 + 1], oacc[dt][4 * q4 + 2], oacc[dt][4 * q4 + 3]};
+        *(uint2*)(po + (dt * 4 + q4) * 256) = make_uint2(pack2<DT>(oacc[dt][4 * q4] * inv, oacc[dt][4 * q4 + 1] * inv),
+                                                         pack2<DT>(oacc[dt][4 * q4 + 2] * inv, oacc[dt][4 * q4 + 3] * inv));
     if (g == 0) {
       const int64_t pslot = ((int64_t)bh * ap.chunks + chunk) * kAttnRows + row;
-      *(v2f_t*)(part_ml + pslot * 2) = v2f_t{m_run * ap.scale_log2, l};
+      *(v2f_t*)(part_ml + pslot * 2) = v2f_t{rf.have ? rf.ref * ap.scale_log2 : -INFINITY, l};
     }
   }
-#ifdef PP_TRACE
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  PP_T(82);
-#endif
 }
 
 // Merge for the tile layout above: one thread per four consecutive head dims of a row; blockIdx.x = (b, head, tile),
-// blockIdx.y = quarter of the tile's sixteen register quads.
+// blockIdx.y = quarter of the tile's sixteen register quads.  A chunk's tile is its normalised output, its weight
+// exp2(ref_c - max ref) * sum_c.
 template <int DT>
 __global__ __launch_bounds__(256) void tree_attention32_merge_kernel(
     const float* __restrict__ part_o, const float* __restrict__ part_ml, AttnParams ap, uint16_t* __restrict__ out) {
@@ -1069,20 +1087,28 @@ __global__ __launch_bounds__(256) void tree_attention32_merge_kernel(
   if (row >= ap.win_rows) return;
   const int b = bh / (int)ap.hq, qh = bh % (int)ap.hq;
   const int64_t slot0 = (int64_t)bh * ap.chunks * kAttnRows + row;
-  const float* po = part_o + ((int64_t)bh * ap.chunks * 2 + tile) * kTileFloats + (idx16 * 64 + lane) * 4;
+  const uint16_t* po = (const uint16_t*)part_o + ((int64_t)bh * ap.chunks * 2 + tile) * kTileElems + (idx16 * 64 + lane) * 4;
   float m = -INFINITY;
-#pragma unroll 4
+#pragma unroll 8
   for (int c = 0; c < ap.chunks; ++c) m = fmaxf(m, part_ml[(slot0 + (int64_t)c * kAttnRows) * 2]);
-  v4f num = {0.f, 0.f, 0.f, 0.f};
+  float num[4] = {0.f, 0.f, 0.f, 0.f};
   float den = 0.f;
-#pragma unroll 4
+#pragma unroll 8
   for (int c = 0; c < ap.chunks; ++c) {
     const v2f_t ml = *(const v2f_t*)(&part_ml[(slot0 + (int64_t)c * kAttnRows) * 2]);
-    const v4f oc = *(const v4f*)(po + (int64_t)c * 2 * kTileFloats);
-    const float w = ml[0] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(ml[0] - m);
+    const uint2 oc = *(const uint2*)(po + (int64_t)c * 2 * kTileElems);
+    const float w = ml[0] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(ml[0] - m) * ml[1];     // the chunk's share of the row sum
+    float f[4];
+    if constexpr (DT == SUBSPEC_BF16) {
+      f[0] = bf16_bits_to_float(oc.x & 0xffffu); f[1] = bf16_bits_to_float(oc.x >> 16);
+      f[2] = bf16_bits_to_float(oc.y & 0xffffu); f[3] = bf16_bits_to_float(oc.y >> 16);
+    } else {
+      f[0] = f16_bits_to_float(oc.x & 0xffffu); f[1] = f16_bits_to_float(oc.x >> 16);
+      f[2] = f16_bits_to_float(oc.y & 0xffffu); f[3] = f16_bits_to_float(oc.y >> 16);
+    }
 #pragma unroll
-    for (int i = 0; i < 4; ++i) num[i] = fmaf(w, oc[i], num[i]);
-    den = fmaf(w, ml[1], den);
+    for (int i = 0; i < 4; ++i) num[i] = fmaf(w, f[i], num[i]);
+    den += w;
   }
   const float inv = den > 0.f ? 1.f / den : 0.f;
   const int d0 = (idx16 >> 2) * 32 + (idx16 & 3) * 8 + g * 4;
@@ -1091,12 +1117,15 @@ __global__ __launch_bounds__(256) void tree_attention32_merge_kernel(
 }
 
 // Launch shape of one window of query rows.
-struct AttnPlan { int threads, rowt, wph, heads_per_wg, chunks; bool mfma32; };
+struct AttnPlan { int threads, rowt, wph, heads_per_wg, chunks; bool mfma32, pingpong; };
 static AttnPlan attn_plan(int64_t batch, int64_t hq, int64_t hkv, int64_t win_rows, int64_t kv_len) {
   AttnPlan pl;
   const int group = (int)(hq / hkv);
   const int64_t blocks = (kv_len + kKeyBlock - 1) / kKeyBlock;
   pl.mfma32 = win_rows > 16;
+  // the ping-pong kernel pays for its set-up over many blocks: (sequence, head) pairs enough to fill the chip with few key
+  // chunks.  One sequence never takes it, so that a request's attention over pages equals the contiguous one bit for bit.
+  pl.pingpong = pl.mfma32 && batch > 1 && batch * hq >= 128;
   if (win_rows <= 16) {
     // a draft level: a wavefront is a whole head (one 16-row tile), eight heads share the staged keys
     pl.threads = 512; pl.rowt = 1; pl.wph = 1;
@@ -1127,7 +1156,7 @@ static AttnPlan attn_plan(int64_t batch, int64_t hq, int64_t hkv, int64_t win_ro
   if (const char* e = getenv("SUBSPEC_ATTN_PLAN")) {     // tuning aid: "threads,wph,chunks" for windows of more than 32 rows
     int t = 0, w = 0, c = 0;
     if (win_rows > 32 && sscanf(e, "%d,%d,%d", &t, &w, &c) == 3 && (t == 512 || t == 256) && (w == 1 || w == 2) && c >= 1) {
-      pl.threads = t; pl.wph = 2; pl.heads_per_wg = (t / 64) / 2;
+      pl.threads = t; pl.wph = 2; pl.heads_per_wg = (t / 64) / 2; pl.pingpong = w == 1 && t == 512;
       pl.chunks = (int)std::min<int64_t>(std::min<int64_t>(c, 64), std::max<int64_t>(1, blocks));
     }
   }
@@ -1245,7 +1274,7 @@ static int tree_attention_impl(const char* what, const void* q, const void* k_ca
     {                                                                                                              \
       DominantKernelTimer timer(st);                                                                               \
       if (!pl.mfma32) SUBSPEC_ATTN_KERNEL(DT, PAGED, 1, 1, 512);                                                   \
-      else if (pl.threads == 512 && !PAGED && !getenv("SUBSPEC_ATTN_NOPP")) {                                      \
+      else if (pl.pingpong && !PAGED) {                                                                            \
         if (pl.wph == 1) SUBSPEC_ATTNPP_KERNEL(DT, 1); else SUBSPEC_ATTNPP_KERNEL(DT, 2);                          \
       }                                                                                                            \
       else if (pl.wph == 1) SUBSPEC_ATTN32_KERNEL(DT, PAGED, 1, 512);                                              \

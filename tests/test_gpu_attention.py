@@ -44,6 +44,53 @@ def test_small_shapes(dtype):
         _check(parents, q, k, v, P, f"small{seed}")
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_many_sequence_head_pairs(dtype):
+    """Windows of 17 to 64 rows with at least 128 (sequence, head) pairs take the kernel whose wavefronts alternate between
+    matrix and softmax phases and whose K / V blocks are copied straight into LDS: one, two, three and many 64-key blocks
+    per workgroup, one and several key chunks, prefixes that are no multiple of 64 (or empty), ragged last row tiles,
+    GQA groups of 1, 4, 7, 8 and 32 heads (workgroups with idle head slots), 17 to 32 rows (a wavefront is a whole head)."""
+    shapes = [(8, 16, 2, 64, 100, 200), (5, 28, 4, 40, 1000, 1100), (16, 8, 8, 33, 63, 128), (4, 32, 4, 20, 500, 600),
+              (3, 64, 8, 64, 0, 64), (2, 64, 2, 64, 4000, 4200), (32, 4, 1, 17, 7, 40), (6, 28, 4, 64, 1, 70),
+              (19, 7, 1, 48, 130, 200), (2, 64, 4, 32, 2500, 2560)]
+    for seed, (B, Hq, Hkv, n, P, S) in enumerate(shapes):
+        parents, q, k, v = _case(300 + seed, B, Hq, Hkv, n, P, S, dtype, depth=7)
+        k[:, :, P + n:] = 1e3                                          # stale rows beyond the tree must not be read
+        v[:, :, P + n:] = -1e3
+        _check(parents, q, k, v, P, f"pairs{seed}")
+
+
+def test_many_pairs_peaked_rows():
+    """Rows whose maximum moves late and far (a key far above everything before it, in the last chunk): the reference exponent
+    of such a row is raised after many blocks, and everything accumulated until then is rescaled."""
+    g = torch.Generator().manual_seed(77)
+    B, Hq, Hkv, n, P, S = 8, 16, 2, 64, 2048, 2112
+    parents, q, k, v = _case(77, B, Hq, Hkv, n, P, S, torch.bfloat16)
+    k[:, :, 1900] = 6 * q[:, ::8, 5]                                   # row 5 of every eighth head finds a near-copy of itself
+    k[:, :, 3] = -4 * q[:, ::8, 9]
+    q[:, :, 11] *= 30                                                  # scores of a few hundred for one row
+    q[:, :, 12] *= 0.0                                                 # and a row that is all ties
+    _check(parents, q, k, v, P, "peaked")
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_many_pairs_large_trees(dtype):
+    """Trees beyond 64 slots (two and more mask words per row) with many (sequence, head) pairs: every window of 64 rows."""
+    for seed, (B, n_slots, P, S, depth) in enumerate([(16, 128, 70, 256, 16), (16, 289, 200, 512, 48), (20, 100, 0, 128, 12)]):
+        g = torch.Generator().manual_seed(500 + seed)
+        parents, _, _ = W.random_tree(g, n=n_slots, max_depth=depth, max_children=6, vocab=1000, chain_depth=depth)
+        q = torch.randn(B, 8, n_slots, 128, generator=g).to(dtype)
+        k = torch.randn(B, 2, S, 128, generator=g).to(dtype)
+        v = torch.randn(B, 2, S, 128, generator=g).to(dtype)
+        k[:, :, P + n_slots:] = 1e3
+        print("attention many pairs, large tree", dtype, B, n_slots, P, flush=True)
+        ref = oa.tree_attention(q, k, v, parents, P)
+        anc = ops.ancestor_bits_tensor(parents, device=DEV)
+        out = ops.tree_attention(q.to(DEV), k.to(DEV), v.to(DEV), anc, P).float().cpu()
+        assert (out - ref).abs().amax().item() <= 1e-2 * ref.abs().amax().item()
+        assert torch.allclose(out, ref, rtol=1e-2, atol=2e-2)
+
+
 @pytest.mark.parametrize("B", [1, 8])
 def test_config3_qwen_geometry(B):
     parents, q, k, v = _case(100 + B, B, 28, 4, 64, 4096, 4160, torch.bfloat16)

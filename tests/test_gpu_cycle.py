@@ -253,22 +253,41 @@ def test_agreeing_draft_accepts_deep_paths():
             t = w[name + ".weight"]
             w[name + ".weight"] = quant.dequantize(*quant.quantize_int4_g64(t)).to(t.dtype)
 
+    prompt = torch.randint(0, CFG.vocab_size, (1, 32), generator=torch.Generator().manual_seed(4)).to(DEV)
+
     def run(depth):
         kv = create_kv_cache("static", max_cache_len=256, config=CFG, device=DEV, dtype=torch.bfloat16)
         target, draft, _ = build_models(CFG, kv, device=DEV, weights=weights)
         gen = SubSpecSDGenerator(target, None, SubSpecSDDraftModel(draft), DraftParams(temperature=0.2, max_depth=depth, topk_len=4))
-        prompt = torch.randint(0, CFG.vocab_size, (1, 32), generator=torch.Generator().manual_seed(4)).to(DEV)
         wandb_logger.clear_log_data()
         out = gen.generate(prompt, max_new_tokens=48, do_sample=False, past_key_values=kv)
-        return out[0, 32:].cpu(), dict(wandb_logger.log_data), kv
+        return out[0].cpu(), dict(wandb_logger.log_data), kv
+
+    def greedy_under_teacher_forcing(seq, tag):
+        """Every emitted token is the target's argmax at its prefix, or tied with it as far as bf16 logits can tell
+        (this toy model's logits tie EXACTLY in bf16 now and then, and which of two tied tokens wins depends on the
+        rounding of the window it was scored in: two correct runs may part ways at such a position)."""
+        kv = create_kv_cache("static", max_cache_len=256, config=CFG, device=DEV, dtype=torch.bfloat16)
+        target, _, _ = build_models(CFG, kv, device=DEV, weights=weights)
+        logits = target.prefill(seq[:-1].to(DEV), 0, all_logits=True).float().cpu()
+        scale, exact = logits.abs().amax().item(), 0
+        for t in range(31, seq.numel() - 1):
+            tok = int(seq[t + 1])
+            if tok == int(logits[t].argmax()):
+                exact += 1
+            else:
+                assert float(logits[t].max() - logits[t, tok]) <= 2e-2 * scale, (tag, t)
+        assert exact >= 0.85 * (seq.numel() - 32), (tag, exact)
 
     deep, log, kv = run(4)
     assert log["avg_sampled"] >= 3.0, log["avg_sampled"]            # at most 5 per cycle
     assert kv.get_seq_length() == 32 + 48 - 1
     shallow, log1, _ = run(1)
     assert log1["avg_sampled"] <= 2.0
-    agree = (deep == shallow).float().mean().item()
-    assert agree >= 0.9, agree                                      # bf16 near-ties may flip a token late in the sequence
+    greedy_under_teacher_forcing(deep, "depth 4")
+    greedy_under_teacher_forcing(shallow, "depth 1")
+    agree = int((deep[32:] == shallow[32:]).long().cumprod(0).sum())
+    assert agree >= 8, agree                                        # the runs may only part ways at a tie
 
 
 def _letter_tokenizer():
