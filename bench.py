@@ -49,7 +49,11 @@ def parse():
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="lower bound of CPU-baseline work")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-e2e", action="store_true", help="default workload: leave out the bounded config-5 end-to-end block")
-    ap.add_argument("--e2e-tokens", type=int, default=32, help="default workload: new tokens of each config-5 run in the e2e block")
+    ap.add_argument("--e2e-tokens", type=int, default=256,
+                    help="default workload: new tokens of the config-5 runs of the e2e block that stream layers 14-27 with random "
+                         "weights (256 is what BASELINE config 5 names: about 30 s per run)")
+    ap.add_argument("--e2e-tokens-other", type=int, default=32,
+                    help="default workload: new tokens of the other runs of the e2e block (all layers resident; agreeing draft)")
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="also run three plain copies of the logits tensor (known size) so that hardware byte counters "
                          "collected by rocprofv3 --pmc can be scaled")
@@ -233,7 +237,7 @@ def e2e_runs(args, runs, new_tokens, say=lambda *_: None):
     """BASELINE config 5: random-init Qwen2.5-7B-shaped decoder, target bf16 with layers 14-27 streamed from pinned host
     memory every forward, substitute draft int4 g64 resident, depth-8 / k-8 tree capped at 64 nodes, prompt 2048 random
     ids; exact and lossy verification.  `runs`: (keep_layers, agreeing_draft) pairs, each generated with both
-    verification methods.  Returns one JSON-ready line per generation."""
+    verification methods; a run may carry its own token count as a third element.  Returns one JSON-ready line per generation."""
     import torch
     from subspec_amd.cache import create_kv_cache
     from subspec_amd.draft import SubSpecSDDraftModel
@@ -246,7 +250,10 @@ def e2e_runs(args, runs, new_tokens, say=lambda *_: None):
     dev = "cuda:0"
     lines = []
     base = None
-    for keep_layers, agreeing in runs:
+    default_tokens = new_tokens
+    for run in runs:
+        keep_layers, agreeing = run[0], run[1]
+        new_tokens = run[2] if len(run) > 2 else default_tokens
         t0 = time.perf_counter()
         if args.checkpoint:
             cfg, weights = load_hf_checkpoint(args.checkpoint, device=dev)
@@ -327,10 +334,12 @@ def e2e_block(args):
     keys = ("verify_method", "resident_target_layers", "agreeing_draft", "n_iter", "n_tokens", "tokens_per_cycle", "avg_draft_s",
             "avg_target_s", "avg_verify_s", "cycle_tokens_per_s", "elapsed_s", "host_to_device_GB", "host_to_device_GB_per_s")
     out = {"workload": f"BASELINE config 5, Qwen2.5-7B shape (28 layers, hidden 3584, 28/4 heads, FFN 18944, vocab 152064), int4 g64 "
-                       f"draft, depth 8, k 8, <=64 nodes, prompt 2048, {args.e2e_tokens} new tokens; tokens_per_s = new tokens / "
+                       f"draft, depth 8, k 8, <=64 nodes, prompt 2048, {args.e2e_tokens} new tokens with layers 14-27 streamed and random "
+                       f"weights, {args.e2e_tokens_other} in the other runs; tokens_per_s = new tokens / "
                        "whole generate() including the prefill, cycle_tokens_per_s = tokens per cycle / (draft + target + verify)",
            "runs": []}
-    for line in e2e_runs(args, [(14, False), (28, False), (14, True)], args.e2e_tokens):
+    for line in e2e_runs(args, [(14, False, args.e2e_tokens), (28, False, args.e2e_tokens_other), (14, True, args.e2e_tokens_other)],
+                         args.e2e_tokens):
         out["runs"].append(dict({"tokens_per_s": line["value"]}, **{k: line["config"][k] for k in keys}))
     return out
 
