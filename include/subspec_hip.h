@@ -119,7 +119,9 @@ int subspec_tree_verify(const void* logits, int dtype, int64_t batch, int64_t ro
  * bytes = 6 MiB of device memory per GPU, held until the process ends).  The call allocates nothing.
  * batch * rows beyond SUBSPEC_TREE_VERIFY_STATIC_MAX_ROWS is rejected with SUBSPEC_ERR_LIMIT.  All calls
  * on one GPU share that GPU's array: calls that overlap on one GPU (different streams or threads) race;
- * calls in stream order do not.  Nothing in the array needs to start at zero. */
+ * calls in stream order do not.  Nothing in the array needs to start at zero.  The FIRST call on a device looks up the
+ * array's address (hipGetSymbolAddress, which may load the code object): make it outside a graph capture; every later
+ * call on that device only launches kernels. */
 #define SUBSPEC_TREE_VERIFY_STATIC_MAX_ROWS 2048
 
 int subspec_tree_verify_static(const void* logits, int dtype, int64_t batch, int64_t rows, int64_t vocab,

@@ -185,9 +185,9 @@ class Tree:
         self._rebuild(list(range(n)))
         # The frontier stays what it was, minus the nodes cut off, IN ITS ORDER: a level added later names its parents
         # by position in the previous level, and those positions must keep their meaning (a parent that was cut off
-        # is refused by add_nodes).  Shallower nodes that lost all their children do not become expandable.
-        if frontier:
-            self.available_leaves = frontier
+        # is refused by add_nodes).  Shallower nodes that lost all their children do not become expandable: when the
+        # whole last level is cut off the frontier is empty, and a later add_nodes raises instead of re-parenting.
+        self.available_leaves = frontier
         return torch.arange(self.current_size)
 
     # ------------------------------------------------------------------ export

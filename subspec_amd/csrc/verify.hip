@@ -595,9 +595,12 @@ __global__ __launch_bounds__(kTailThreads) void tree_accept_kernel(
   }
   __syncthreads();
   // Sliced rows of a run without the entropy gate come without the exact pass.  A row whose rounded probabilities
-  // may tie with the maximum (a maximum below 2 in magnitude, or a subnormal rounded maximum: not what a language
-  // model's logits look like) is scanned here by the whole wavefront: first index whose rounded probability equals
-  // the rounded maximum, as row_exact_body finds it.  Slow (a row per pass), and next to never taken.
+  // may tie with the maximum (a maximum below 2 in magnitude, or a subnormal rounded maximum) is resolved here by the
+  // whole wavefront: first index whose rounded probability equals the rounded maximum, as row_exact_body finds it.
+  // Only slices that can hold such an index are read: exp(x - m) must lie within the dtype's relative spacing at the
+  // rounded maximum of 1, i.e. the slice's own maximum within `delta` of the row's, and the slice must not lie behind the
+  // first index of the maximum logit (which ties with itself).  For rows as a language model emits them that is the one
+  // slice holding the maximum (64 steps), where a scan of the whole row would cost the launch a millisecond per tree.
   if (vp.ties_in_accept) {
 #pragma unroll
     for (int s = 0; s < kSlots; ++s) {
@@ -607,14 +610,30 @@ __global__ __launch_bounds__(kTailThreads) void tree_accept_kernel(
         pending &= pending - 1;
         const int r = s * kWave + src;
         const float m = sm_m[r], S = sm_S[r], pmax = __shfl(tie_pmax[s], src, kWave);
-        const int64_t base = ((int64_t)b * rows + r) * vp.vocab;
+        const int first_idx = sm_tgt[r];
+        const int64_t grow = (int64_t)b * rows + r;
+        const int64_t base = grow * vp.vocab;
+        // relative spacing of the dtype at 1 / S (twice over, for the rounding of the exponential itself)
+        const float spacing_normal = DT == SUBSPEC_BF16 ? 0.015625f : DT == SUBSPEC_F16 ? 0.001953125f : 2.4e-7f;
+        const float spacing_sub = DT == SUBSPEC_F16 ? 1.2e-7f : DT == SUBSPEC_BF16 ? 1.9e-40f : 3e-45f;   // twice 2^-24 / 2^-133 / 2^-149
+        const float rel = fmaxf(spacing_normal, spacing_sub * S);
+        const float delta = rel < 0.5f ? -logf(1.0f - rel) : INFINITY;
         int tie = 0x7fffffff;
-        for (int64_t i = lane; i < vp.vocab && tie == 0x7fffffff; i += kWave)
-          if (rounded_prob<DT>(load_warped<DT>(logits, base + i, vp), m, S) == pmax) tie = (int)i;
-        tie = wave_min_i(tie);
+        for (int c = 0; c < vp.splits && tie == 0x7fffffff; ++c) {                     // uniform
+          const int64_t c0 = (int64_t)c * vp.chunk;
+          if (c0 > first_idx) break;
+          if (!(part1[grow * vp.splits + c].m >= m - delta)) continue;
+          const int64_t c1 = min(c0 + vp.chunk, vp.vocab);
+          for (int64_t i0 = c0; i0 < c1 && tie == 0x7fffffff; i0 += kWave) {             // uniform
+            const int64_t i = i0 + lane;
+            int hit = 0x7fffffff;
+            if (i < c1 && rounded_prob<DT>(load_warped<DT>(logits, base + i, vp), m, S) == pmax) hit = (int)i;
+            tie = wave_min_i(hit);
+          }
+        }
         if (lane == src && tie != 0x7fffffff) {
           sm_tgt[r] = tie;
-          node_target[(int64_t)b * rows + r] = tie;
+          node_target[grow] = tie;
         }
       }
     }

@@ -47,6 +47,7 @@ class SubSpecSDDraftModel:
         self.capture_graphs = False
         self.graph_bucket = 256                   # a graph serves prefixes up to the next multiple of this
         self.graph_warmup = 2                     # eager speculations before the first capture (library handles, tables)
+        self.max_graphs = 8                       # captured buckets kept (each pins its level tensors and a workspace)
         self._graphs = {}
         self._eager_speculations = 0
         self.graph_replays = 0
@@ -78,6 +79,8 @@ class SubSpecSDDraftModel:
         return self
 
     def set_past_key_values(self, past_key_values) -> None:
+        if past_key_values is not self.past_key_values:
+            self._graphs.clear()                  # a captured graph holds the addresses of the cache it was recorded over
         self.past_key_values = past_key_values
         if past_key_values is not None:
             from .hf_model import as_decoder
@@ -153,19 +156,39 @@ class SubSpecSDDraftModel:
         return bound if bound >= self.prefix_len else None
 
     def _replay_levels(self, root: torch.Tensor, bound: int) -> None:
-        key = (bound, self.draft_params.max_depth, self.draft_params.topk_len, float(self.draft_params.temperature))
+        """A captured graph is bound to the memory its kernels were recorded over: the KV cache storage, the decoder's
+        layer workspace, the rotary tables, the weights.  The cache storage and the decoder are part of a graph's
+        identity (another cache, or a cache whose storage moved, never replays it), and every entry owns its workspace and
+        keeps the tensors of its capture alive, so an eager call that replaces the decoder's workspace cannot pull
+        memory from under a graph."""
+        dec = self.decoder
+        cache = dec.kv.cache
+        key = (bound, self.draft_params.max_depth, self.draft_params.topk_len, float(self.draft_params.temperature),
+               id(dec), int(cache.data.data_ptr()))
         entry = self._graphs.get(key)
         if entry is None:
-            dev = self.decoder.device
+            dev = dec.device
             self._own_bits(dev)                                                    # tables are built outside the capture
-            self.decoder.kv.cache.ensure(bound + 1 + (self.draft_params.max_depth - 1) * self.draft_params.topk_len)
+            cache.ensure(bound + 1 + (self.draft_params.max_depth - 1) * self.draft_params.topk_len)
+            dec._rope_tables(bound + 1 + (self.draft_params.max_depth - 1) * self.draft_params.topk_len + 8)
+            if len(self._graphs) >= self.max_graphs:                               # oldest bucket out
+                self._graphs.pop(next(iter(self._graphs)))
             entry = {"root": torch.zeros(1, dtype=torch.long, device=dev),
-                     "prefix": torch.zeros(1, dtype=torch.int64, device=dev), "graph": torch.cuda.CUDAGraph()}
+                     "prefix": torch.zeros(1, dtype=torch.int64, device=dev), "graph": torch.cuda.CUDAGraph(),
+                     "cache_data": cache.data, "rope": (dec.cos, dec.sin)}
             entry["root"].copy_(root)
             entry["prefix"].fill_(self.prefix_len)
+            shared_ws = dec._native_ws.pop("ws", None) if dec.native_layers else None
             torch.cuda.synchronize()
-            with torch.cuda.graph(entry["graph"]):
-                self._grow_levels(entry["root"], bound, entry["prefix"])
+            try:
+                with torch.cuda.graph(entry["graph"]):
+                    self._grow_levels(entry["root"], bound, entry["prefix"])
+                entry["ws"] = dec._native_ws.get("ws")                             # allocated under the capture: the graph's own
+            finally:
+                if shared_ws is not None:
+                    dec._native_ws["ws"] = shared_ws
+                else:
+                    dec._native_ws.pop("ws", None)
             entry["state"] = {name: getattr(self, name) for name in self._STATE}
             self._graphs[key] = entry
         entry["root"].copy_(root)

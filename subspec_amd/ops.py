@@ -98,11 +98,13 @@ def tree_verify(
         need = lib.subspec_tree_verify_workspace(B, rows, V, _dtype_code(logits))
         workspace = torch.empty(need, dtype=torch.uint8, device=dev)
     if out is not None:
-        want = {"tokens": (B, n + 1), "contexts": (B, n + 1), "counts": (B, 4), "target": (B, rows),
-                "entropy": (B, rows), "child_prob": (B, rows)}
-        for key, shape in want.items():
-            if tuple(out[key].shape) != shape or out[key].device != dev or not out[key].is_contiguous():
-                raise ValueError(f"out[{key!r}] must be a contiguous {shape} tensor on {dev}")
+        want = {"tokens": ((B, n + 1), torch.int64), "contexts": ((B, n + 1), torch.int64), "counts": ((B, 4), torch.int32),
+                "target": ((B, rows), torch.int64), "entropy": ((B, rows), torch.float32), "child_prob": ((B, rows), torch.float32)}
+        for key, (shape, dtype) in want.items():
+            # the kernels write these element types: a narrower tensor of the right shape would be overrun
+            if (tuple(out[key].shape) != shape or out[key].dtype != dtype or out[key].device != dev
+                    or not out[key].is_contiguous()):
+                raise ValueError(f"out[{key!r}] must be a contiguous {dtype} tensor of shape {shape} on {dev}")
     out = out if out is not None else {
         "tokens": torch.empty((B, n + 1), dtype=torch.int64, device=dev),
         "contexts": torch.empty((B, n + 1), dtype=torch.int64, device=dev),

@@ -83,3 +83,54 @@ def test_cycle_with_graph_replay_emits_the_targets_tokens():
     # exact verification emits the target's greedy continuation whatever tree the draft proposes
     same = (outs[True] == outs[False]).float().mean().item()
     assert same >= 0.95, same
+
+
+def test_graphs_do_not_outlive_the_cache_they_were_captured_over():
+    """Two generations with the same draft model over two caches: a graph captured over the first cache holds the
+    addresses of its K / V rows and must not be replayed over the second; an eager speculation that needs a larger layer
+    workspace in between must not pull the workspace from under a captured graph."""
+    w = init_weights(CFG, 9, DEV)
+    prompt = torch.randint(0, CFG.vocab_size, (1, 40), generator=torch.Generator().manual_seed(4)).to(DEV)
+
+    def generate(gen, kv, n):
+        wandb_logger.clear_log_data()
+        out = gen.generate(prompt, max_new_tokens=n, do_sample=False, past_key_values=kv)[0].cpu()
+        return out
+
+    kv_ref = create_kv_cache("static", max_cache_len=512, config=CFG, device=DEV, dtype=torch.bfloat16)
+    target, draft, _ = build_models(CFG, kv_ref, device=DEV, weights=w)
+    plain = SubSpecSDGenerator(target, None, SubSpecSDDraftModel(draft), DraftParams(temperature=0.2, max_depth=4, topk_len=4),
+                               generator_kwargs=dict(verify_method="exact", draft_graph=False))
+    want = generate(plain, kv_ref, 40)
+
+    kv1 = create_kv_cache("static", max_cache_len=512, config=CFG, device=DEV, dtype=torch.bfloat16)
+    target, draft, _ = build_models(CFG, kv1, device=DEV, weights=w)
+    dm = SubSpecSDDraftModel(draft)
+    gen = SubSpecSDGenerator(target, None, dm, DraftParams(temperature=0.2, max_depth=4, topk_len=4),
+                             generator_kwargs=dict(verify_method="exact", draft_graph=True))
+    dm.graph_bucket = 32
+    first = generate(gen, kv1, 40)
+    assert dm.graph_replays > 0 and len(dm._graphs) >= 2
+    held = len(dm._graphs)
+    # a second cache: the graphs of the first are dropped, new ones are captured over the new storage
+    kv2 = create_kv_cache("static", max_cache_len=512, config=CFG, device=DEV, dtype=torch.bfloat16)
+    kv1.cache.data.fill_(float("nan"))                       # whatever still pointed at the old cache would show
+    second = generate(gen, kv2, 40)
+    assert all(e["cache_data"] is kv2.cache.data for e in dm._graphs.values())
+    # an eager call that needs more workspace than any graph (a 64-row window) between two replays over the same cache
+    kv2.reset()
+    draft.tree_forward(torch.zeros(64, dtype=torch.long, device=DEV), torch.zeros(64, dtype=torch.long, device=DEV),
+                       torch.ones(64, dtype=torch.int64, device=DEV), 100)
+    torch.cuda.synchronize()
+    kv2.reset()
+    third = generate(gen, kv2, 40)
+    for tag, got in (("first", first), ("second", second), ("third", third)):
+        same = (got == want).float().mean().item()
+        assert same >= 0.95, (tag, same)                     # exact verification: the target's tokens whatever the draft proposes
+    assert torch.equal(second, third)
+    # the number of captured buckets is bounded
+    dm.max_graphs = 2
+    dm._graphs.clear()
+    kv2.reset()
+    generate(gen, kv2, 60)
+    assert len(dm._graphs) <= 2 and held >= 2

