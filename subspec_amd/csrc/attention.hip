@@ -14,27 +14,26 @@
 //                                     (the node in slot j is the row's node or one of its ancestors);
 //                                     words = ceil(slots / 64), at most 8
 //   out      [B, n, Hq, D]
-// One workgroup (8 wavefronts) owns several query heads of one KV head and one chunk of the keys, so
-// a staged K/V tile feeds several heads' worth of matrix work.  With 33 to 64 query rows it owns
-// FOUR heads (256 rows): wavefront w takes 32 rows (two 16-row tiles) of head w/2.  With fewer rows
-// (17 to 32: two tiles, up to 16 -- one level of the draft tree --: one tile) a wavefront is a
-// whole head and the workgroup owns EIGHT heads, all of a 7:1 GQA group, so K/V are staged once per
-// KV head and no wavefront multiplies padding rows.  Scores are produced TRANSPOSED, S^T = K Q^T, with v_mfma_f32_16x16x32: the
-// accumulator then holds, per lane, four consecutive keys of one query, and two such tiles are
-// exactly the eight-key B operand of the second product O^T = V^T P^T (with the matching key
-// permutation applied to the V^T operand), so probabilities go from one MFMA to the next without
-// leaving registers and the row maximum / sum need only two cross-lane steps.  The ancestor bitset
-// of a lane's query sits in a register pair; prefix keys need no mask at all.  K and V are staged
-// row-major in LDS (V^T operands come from transposing LDS reads); the global loads of the next 64-key block are issued before the
-// current block is multiplied.  Workgroups that share a KV chunk get consecutive slots on the same
-// XCD (linear id modulo 8), so the chunk is fetched from HBM once and served from that XCD's L2.
-// When the keys are split over several workgroups the partial (O, max, sum) triples are merged by
-// tree_attention_merge_kernel.
-// HBM-bound at the benchmark sizes provided QK^T / PV run on the matrix cores:
-// algorithmic bytes per batch element = K+V rows actually attended + Q + O.
+// One workgroup owns several query heads of one KV head and one chunk of the keys, so a staged K/V block feeds
+// several heads' worth of matrix work; workgroups that share a KV chunk get consecutive slots on the same XCD (linear
+// id modulo 8), so the chunk is fetched from HBM once and served from that XCD's L2.  Scores are produced TRANSPOSED,
+// S^T = K Q^T: the accumulator then holds, per lane, keys of ONE query, the row maximum / sum need one or two cross-lane
+// steps, and packed accumulator registers are the B operand of the second product O^T = V^T P^T (with the matching key
+// permutation applied to the V^T operand, read from row-major V by transposing LDS reads), so probabilities go from one
+// MFMA to the next without leaving registers.  Prefix keys need no mask at all.  Three kernels, chosen by attn_plan:
+//   * tree_attention_kernel: windows of up to 16 rows (a level of the draft tree).  v_mfma_f32_16x16x32, a wavefront
+//     is a whole head (one 16-row tile), eight heads (a whole 7:1 GQA group) share the staged keys.
+//   * tree_attention32_kernel: 17 to 64 rows, one sequence or few (sequence, head) pairs, and every paged call.
+//     v_mfma_f32_32x32x16, a wavefront owns 32 rows of a head; K / V blocks travel through two register sets into two
+//     padded LDS stages, two blocks' requests in flight.
+//   * tree_attention_pp_kernel: 17 to 64 rows, several sequences with at least 128 (sequence, head) pairs (config 3,
+//     B = 8).  The same tiles; the two wavefronts of a SIMD alternate between a matrix phase and a softmax phase, K / V
+//     blocks are copied from memory straight into a ring of four LDS stages.
+// When the keys are split over several workgroups the per-chunk results are merged by a second launch.
+// Algorithmic bytes per batch element = K+V rows actually attended + Q + O; at config 3 the arithmetic intensity
+// (405 FLOP/B) is above the chip's ridge, so the bound that applies is the matrix pipe, not HBM.
 #include "common.h"
 #include <algorithm>
-#include <stdlib.h>
 
 namespace subspec {
 
@@ -1153,13 +1152,6 @@ static AttnPlan attn_plan(int64_t batch, int64_t hq, int64_t hkv, int64_t win_ro
   const int64_t by_bytes = std::max<int64_t>(1, 2 * (kv_len * hkv) / std::max<int64_t>(1, hq * win_rows));
   chunks = std::min<int64_t>(chunks, by_bytes);
   pl.chunks = (int)std::min<int64_t>(chunks, 64);
-  if (const char* e = getenv("SUBSPEC_ATTN_PLAN")) {     // tuning aid: "threads,wph,chunks" for windows of more than 32 rows
-    int t = 0, w = 0, c = 0;
-    if (win_rows > 32 && sscanf(e, "%d,%d,%d", &t, &w, &c) == 3 && (t == 512 || t == 256) && (w == 1 || w == 2) && c >= 1) {
-      pl.threads = t; pl.wph = 2; pl.heads_per_wg = (t / 64) / 2; pl.pingpong = w == 1 && t == 512;
-      pl.chunks = (int)std::min<int64_t>(std::min<int64_t>(c, 64), std::max<int64_t>(1, blocks));
-    }
-  }
   return pl;
 }
 // the most partial slots any window of a call can need (the first window is the largest)
