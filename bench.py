@@ -170,7 +170,8 @@ def bench_attention(args):
         # 3.82 GFLOP per sequence over 9.44 MB: at 405 FLOP/B the shape sits above the ridge (310 FLOP/B)
         _kernel_line("tree-masked GQA attention latency",
                      f"BASELINE config 3, B={B}: q [B,28,64,128], KV [B,4,4160,128] bf16, another cache every call ({copies} copies)",
-                     call_us, kernel_us, nbytes, B * 4 * 64 * 28 * 4160 * 128, "subspec::tree_attention_kernel", bound="mfma",
+                     call_us, kernel_us, nbytes, B * 4 * 64 * 28 * 4160 * 128,
+                     "subspec::tree_attention_pp_kernel" if B > 1 else "subspec::tree_attention32_kernel", bound="mfma",
                      extra={"batch": B})
         del ks, vs
     # the same sequence out of a paged pool (16-token pages in shuffled order)
@@ -183,7 +184,7 @@ def bench_attention(args):
     call_us, kernel_us = _time_us(lambda: ops.tree_attention_paged(q, layer, pages, anc, 4096, workspace=ws), args.steps, args.warmup)
     _kernel_line("tree-masked GQA attention latency, paged KV", "config 3 shape, B=1, KV pool [300,2,16,4,128] bf16, shuffled pages",
                  call_us, kernel_us, 2 * 4 * 4160 * 128 * 2 + 2 * 28 * 64 * 128 * 2, 4 * 64 * 28 * 4160 * 128,
-                 "subspec::tree_attention_kernel", bound="mfma", extra={"batch": 1, "page_len": page_len})
+                 "subspec::tree_attention32_kernel", bound="mfma", extra={"batch": 1, "page_len": page_len})
 
 
 def bench_int4(args):

@@ -574,6 +574,7 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
     SUBSPEC_ATTN32_STAGE(buf ^ 1);
     SUBSPEC_ATTN32_FETCH(buf ^ 1, kb + 3 * kKeyBlock);
     if (kb >= key1) continue;                          // (uniform) odd number of blocks: the requests above keep every path's count equal
+    if (!(head_ok && tile * 32 < ap.win_rows)) continue; // (wave-uniform) a head slot or row tile with nothing in it only helps with the staging
     const uint16_t* Ks = Ks2[buf] + koff;
     const uint16_t* Vs = Vs2[buf] + voff;
 
@@ -1077,7 +1078,11 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 // Merge for the tile layout above: one thread per four consecutive head dims of a row; blockIdx.x = (b, head, tile),
 // blockIdx.y = quarter of the tile's sixteen register quads.  A chunk's tile is its normalised output, its weight
 // exp2(ref_c - max ref) * sum_c.
-template <int DT>
+// With up to eight chunks (CMAX = 4 or 8, the compiled bound) every load of a thread -- the reference and sum of its row
+// and its four elements, of every chunk -- is issued before the first is used, so the launch pays ONE round trip to
+// memory instead of one for the maximum and one for the sums (config 3, B = 8: 6.1 -> 5.3 us); CMAX = 0 is the two-pass
+// form for more chunks, where that many loads up front cost more than they save.
+template <int DT, int CMAX>
 __global__ __launch_bounds__(256) void tree_attention32_merge_kernel(
     const float* __restrict__ part_o, const float* __restrict__ part_ml, AttnParams ap, uint16_t* __restrict__ out) {
   const int tile = blockIdx.x & 1, bh = blockIdx.x >> 1;
@@ -1087,27 +1092,53 @@ __global__ __launch_bounds__(256) void tree_attention32_merge_kernel(
   const int b = bh / (int)ap.hq, qh = bh % (int)ap.hq;
   const int64_t slot0 = (int64_t)bh * ap.chunks * kAttnRows + row;
   const uint16_t* po = (const uint16_t*)part_o + ((int64_t)bh * ap.chunks * 2 + tile) * kTileElems + (idx16 * 64 + lane) * 4;
-  float m = -INFINITY;
-#pragma unroll 8
-  for (int c = 0; c < ap.chunks; ++c) m = fmaxf(m, part_ml[(slot0 + (int64_t)c * kAttnRows) * 2]);
-  float num[4] = {0.f, 0.f, 0.f, 0.f};
-  float den = 0.f;
-#pragma unroll 8
-  for (int c = 0; c < ap.chunks; ++c) {
-    const v2f_t ml = *(const v2f_t*)(&part_ml[(slot0 + (int64_t)c * kAttnRows) * 2]);
-    const uint2 oc = *(const uint2*)(po + (int64_t)c * 2 * kTileElems);
-    const float w = ml[0] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(ml[0] - m) * ml[1];     // the chunk's share of the row sum
-    float f[4];
+  auto unpack4 = [](uint2 o, float* f) {
     if constexpr (DT == SUBSPEC_BF16) {
-      f[0] = bf16_bits_to_float(oc.x & 0xffffu); f[1] = bf16_bits_to_float(oc.x >> 16);
-      f[2] = bf16_bits_to_float(oc.y & 0xffffu); f[3] = bf16_bits_to_float(oc.y >> 16);
+      f[0] = bf16_bits_to_float(o.x & 0xffffu); f[1] = bf16_bits_to_float(o.x >> 16);
+      f[2] = bf16_bits_to_float(o.y & 0xffffu); f[3] = bf16_bits_to_float(o.y >> 16);
     } else {
-      f[0] = f16_bits_to_float(oc.x & 0xffffu); f[1] = f16_bits_to_float(oc.x >> 16);
-      f[2] = f16_bits_to_float(oc.y & 0xffffu); f[3] = f16_bits_to_float(oc.y >> 16);
+      f[0] = f16_bits_to_float(o.x & 0xffffu); f[1] = f16_bits_to_float(o.x >> 16);
+      f[2] = f16_bits_to_float(o.y & 0xffffu); f[3] = f16_bits_to_float(o.y >> 16);
+    }
+  };
+  float m = -INFINITY, den = 0.f;
+  float num[4] = {0.f, 0.f, 0.f, 0.f};
+  if constexpr (CMAX > 0) {
+    v2f_t ml[CMAX];
+    uint2 oc[CMAX];
+#pragma unroll
+    for (int c = 0; c < CMAX; ++c) {
+      const int cc = min(c, ap.chunks - 1);              // chunks past the count repeat the last one and get no weight
+      ml[c] = *(const v2f_t*)(&part_ml[(slot0 + (int64_t)cc * kAttnRows) * 2]);
+      oc[c] = *(const uint2*)(po + (int64_t)cc * 2 * kTileElems);
     }
 #pragma unroll
-    for (int i = 0; i < 4; ++i) num[i] = fmaf(w, f[i], num[i]);
-    den += w;
+    for (int c = 0; c < CMAX; ++c) m = fmaxf(m, ml[c][0]);
+#pragma unroll
+    for (int c = 0; c < CMAX; ++c) {
+      // the chunk's share of the row sum
+      const float w = (c >= ap.chunks || ml[c][0] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(ml[c][0] - m) * ml[c][1];
+      float f[4];
+      unpack4(oc[c], f);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) num[i] = fmaf(w, f[i], num[i]);
+      den += w;
+    }
+  } else {
+    // many chunks (one sequence cut into a dozen or more): two passes, eight chunks' requests in flight in each
+#pragma unroll 8
+    for (int c = 0; c < ap.chunks; ++c) m = fmaxf(m, part_ml[(slot0 + (int64_t)c * kAttnRows) * 2]);
+#pragma unroll 8
+    for (int c = 0; c < ap.chunks; ++c) {
+      const v2f_t ml = *(const v2f_t*)(&part_ml[(slot0 + (int64_t)c * kAttnRows) * 2]);
+      const uint2 o = *(const uint2*)(po + (int64_t)c * 2 * kTileElems);
+      const float w = ml[0] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(ml[0] - m) * ml[1];
+      float f[4];
+      unpack4(o, f);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) num[i] = fmaf(w, f[i], num[i]);
+      den += w;
+    }
   }
   const float inv = den > 0.f ? 1.f / den : 0.f;
   const int d0 = (idx16 >> 2) * 32 + (idx16 & 3) * 8 + g * 4;
@@ -1274,10 +1305,12 @@ static int tree_attention_impl(const char* what, const void* q, const void* k_ca
       else SUBSPEC_ATTN32_KERNEL(DT, PAGED, 2, 256);                                                               \
     }                                                                                                              \
     if (ap.chunks > 1) {                                                                                           \
-      if (pl.mfma32)                                                                                               \
-        hipLaunchKernelGGL((tree_attention32_merge_kernel<DT>), dim3((unsigned)(batch * n_q_heads * 2), 4), dim3(256), 0, st, \
-                           part_o, part_ml, ap, (uint16_t*)out);                                                   \
-      else                                                                                                         \
+      if (pl.mfma32) {                                                                                             \
+        const dim3 mg((unsigned)(batch * n_q_heads * 2), 4);                                                       \
+        if (ap.chunks <= 4) hipLaunchKernelGGL((tree_attention32_merge_kernel<DT, 4>), mg, dim3(256), 0, st, part_o, part_ml, ap, (uint16_t*)out); \
+        else if (ap.chunks <= 8) hipLaunchKernelGGL((tree_attention32_merge_kernel<DT, 8>), mg, dim3(256), 0, st, part_o, part_ml, ap, (uint16_t*)out); \
+        else hipLaunchKernelGGL((tree_attention32_merge_kernel<DT, 0>), mg, dim3(256), 0, st, part_o, part_ml, ap, (uint16_t*)out); \
+      } else                                                                                                         \
         hipLaunchKernelGGL((tree_attention_merge_kernel<DT>), merge_grid, dim3(merge_rows * 32), 0, st, part_o, part_ml, ap, \
                            (uint16_t*)out);                                                                        \
     }                                                                                                              \
