@@ -347,8 +347,8 @@ int subspec_int4_linear(const void* x, const uint32_t* wq, const uint32_t* sz, c
 int subspec_int4_gate_up_silu(const void* x, const uint32_t* wq, const uint32_t* sz, const void* bias, void* act,
                               int dtype, int64_t M, int64_t N, int64_t K, void* stream);
 
-/* The same for a dense 16-bit gate|up weight W [2F, K] row-major (gate rows first), as the target's layers hold it;
- * 2F * K * 2 bytes must stay below 2 GiB. */
+/* The same for a dense 16-bit gate|up weight W [2F, K] row-major (gate rows first), as the target's layers hold it:
+ * 1 <= M <= 384; up to 32 rows 2F * K * 2 bytes must stay below 2 GiB. */
 int subspec_dense_gate_up_silu(const void* x, const void* w, const void* bias, void* act, int dtype, int64_t M,
                                int64_t N, int64_t K, void* stream);
 
@@ -427,14 +427,16 @@ int subspec_int4_decoder_layer(const subspec_decoder_layer_dims* dims, const sub
                                void* k_cache, void* v_cache, void* workspace, size_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------------------------------
- * Dense 16-bit linear for few activation rows:  y[M, N] = x[M, K] * W[N, K]^T (+ bias), 1 <= M <= 64.
+ * Dense 16-bit linear for the rows of a tree:  y[M, N] = x[M, K] * W[N, K]^T (+ bias), 1 <= M <= 384.
  *
  * Replaces  the nn.Linear projections (q/k/v, o, gate/up, down) of the TARGET model's decoder layers in
  *           the tree-decoding forward: ClassicSDGeneratorBase._tree_decoding -> self.target_model(...)
- *           specdecodes/models/generators/classic_sd.py:75-109 (at most max_verify_tokens = 64 rows).
+ *           specdecodes/models/generators/classic_sd.py:75-109 (max_verify_tokens = 64 rows by default,
+ *           1 + 48 * 6 = 289 rows in configs/exp_offloading/subspec_sd_qwen_7b.yaml:16-19).
  *
  * x  device [M, K], w  device [N, K] row-major, bias [N] or NULL, y [M, N]: all bf16 or all fp16.
- * N % 16 == 0, K % 64 == 0; x and w 16-byte aligned.  Products accumulate in fp32 and are rounded once.
+ * N % 16 == 0 (N % 32 == 0 above 64 rows), K % 64 == 0; x and w 16-byte aligned.  Products accumulate in fp32 and
+ * are rounded once.
  * workspace  subspec_dense_linear_workspace(M, N, K) bytes (fp32 partials when K is split).
  */
 size_t subspec_dense_linear_workspace(int64_t M, int64_t N, int64_t K);
@@ -444,7 +446,8 @@ int subspec_dense_linear(const void* x, const void* w, const void* bias, void* y
 
 /* One decoder layer with dense 16-bit projections: same sequence of kernels, arguments, workspace
  * (subspec_int4_decoder_layer_workspace) and limits as subspec_int4_decoder_layer, for the target
- * model's layers (HF Qwen2DecoderLayer inside the forward named above); q|k|v and gate|up rows are
+ * model's layers (HF Qwen2DecoderLayer inside the forward named above), except that n_rows may reach 384 (a whole
+ * 289-node tree in one call; the projection widths must then be multiples of 32); q|k|v and gate|up rows are
  * stored fused.  Weight matrices are row-major [N, K] in the activation dtype. */
 typedef struct subspec_dense_layer_weights {
   const void* input_norm;   /* [hidden] */

@@ -33,7 +33,7 @@ def decoder_layer(x, w, k_cache, v_cache, positions, cache_rows, anc_bits, prefi
                   eps, theta):
     """x [n, H] fp32; w: dict of fp32 dense weights (qkv [Q+2KV, H] + bias, o, gate_up [2F, H], down) and norm
     weights; k_cache / v_cache [Hkv, S, D] fp32, updated in place at cache_rows; anc_bits: python ints
-    over tree slots.  Returns the new x."""
+    over tree slots (any number of slots).  Returns the new x."""
     n = x.shape[0]
     Q, KV = n_q_heads * head_dim, n_kv_heads * head_dim
     h = rms_norm(x, w["input_norm"], eps)
@@ -46,12 +46,27 @@ def decoder_layer(x, w, k_cache, v_cache, positions, cache_rows, anc_bits, prefi
     v_cache[:, cache_rows] = v.transpose(0, 1)
     rep = n_q_heads // n_kv_heads
     out = torch.zeros(n, n_q_heads, head_dim)
-    for i in range(n):
-        keys = list(range(prefix_len)) + [prefix_len + j for j in range(64) if (anc_bits[i] >> j) & 1]
+    if n <= 64:
+        for i in range(n):
+            keys = list(range(prefix_len)) + [prefix_len + j for j in range(int(anc_bits[i]).bit_length()) if (anc_bits[i] >> j) & 1]
+            for hq in range(n_q_heads):
+                kk, vv = k_cache[hq // rep, keys], v_cache[hq // rep, keys]
+                p = torch.softmax(kk @ q[i, hq] / head_dim ** 0.5, 0)
+                out[i, hq] = p @ vv
+    else:
+        # the same sums for many rows at once: scores of every row against prefix + slots, the keys a row may not see at
+        # -inf (tests/test_oracle_decoder.py holds this form against the loop above)
+        slots = max(int(b).bit_length() for b in anc_bits)
+        allowed = torch.zeros(n, prefix_len + slots, dtype=torch.bool)
+        allowed[:, :prefix_len] = True
+        for i in range(n):
+            for j in range(int(anc_bits[i]).bit_length()):
+                if (anc_bits[i] >> j) & 1:
+                    allowed[i, prefix_len + j] = True
         for hq in range(n_q_heads):
-            kk, vv = k_cache[hq // rep, keys], v_cache[hq // rep, keys]
-            p = torch.softmax(kk @ q[i, hq] / head_dim ** 0.5, 0)
-            out[i, hq] = p @ vv
+            kk, vv = k_cache[hq // rep, :prefix_len + slots], v_cache[hq // rep, :prefix_len + slots]
+            s = (q[:, hq] @ kk.T / head_dim ** 0.5).masked_fill(~allowed, float("-inf"))
+            out[:, hq] = torch.softmax(s, -1) @ vv
     x = x + out.reshape(n, Q) @ w["o"].T
     h = rms_norm(x, w["post_norm"], eps)
     gate, up = (h @ w["gate_up"].T).chunk(2, -1)

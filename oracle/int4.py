@@ -30,16 +30,15 @@ def unpack_tiled(wq: torch.Tensor, sz: torch.Tensor, N: int, K: int):
     to check that packing loses nothing."""
     G = K // 64
     w = wq.to(torch.int64) & 0xFFFFFFFF                 # [nt, g, c, r, j]
-    codes = torch.zeros(N, K, dtype=torch.uint8)
-    for nt in range(N // 16):
-        for g in range(G):
-            for c in range(4):
-                for j in range(2):
-                    word = w[nt, g, c, :, j]            # 16 rows
-                    for i in range(4):
-                        k = 64 * g + 16 * c + 8 * j + 2 * i
-                        codes[nt * 16:(nt + 1) * 16, k] = ((word >> (4 * i)) & 0xF).to(torch.uint8)
-                        codes[nt * 16:(nt + 1) * 16, k + 1] = ((word >> (16 + 4 * i)) & 0xF).to(torch.uint8)
+    codes = torch.zeros(N // 16, 16, G, 64, dtype=torch.uint8)   # [nt, r, g, k % 64]: row 16 nt + r, k = 64 g + ...
+    for c in range(4):
+        for j in range(2):
+            word = w[:, :, c, :, j].permute(0, 2, 1)    # [nt, r, g]: all tiles and groups at once
+            for i in range(4):
+                k = 16 * c + 8 * j + 2 * i
+                codes[:, :, :, k] = ((word >> (4 * i)) & 0xF).to(torch.uint8)
+                codes[:, :, :, k + 1] = ((word >> (16 + 4 * i)) & 0xF).to(torch.uint8)
+    codes = codes.reshape(N, K)
     b = sz.to(torch.int64) & 0xFFFFFFFF                 # [nt, g, r]
     s16 = (b & 0xFFFF).to(torch.int32).to(torch.int16) if False else (b & 0xFFFF)
     z16 = (b >> 16) & 0xFFFF

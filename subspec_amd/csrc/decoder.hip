@@ -128,6 +128,8 @@ __global__ __launch_bounds__(64) void rope_write_kernel(const uint16_t* __restri
   Elem<DT>::store(dst, i + half, o_hi);
 }
 
+// rows of one call: the int4 stack serves draft levels and post-verify windows, the dense stack also whole large trees
+constexpr int kInt4LayerMaxRows = 64, kDenseLayerMaxRows = 384;
 struct LayerPlan {
   size_t h, qkv, q, a, o, gu, act, sub, sub_bytes, total;
 };
@@ -144,10 +146,13 @@ static LayerPlan layer_plan(const subspec_decoder_layer_dims& s) {
   p.o = take(M * H * es);
   p.gu = take(M * 2 * F * es);
   p.act = take(M * F * es);
-  size_t sub = subspec_int4_linear_workspace(s.n_rows, Q + 2 * KV, H);
-  sub = std::max(sub, subspec_int4_linear_workspace(s.n_rows, H, Q));
-  sub = std::max(sub, subspec_int4_linear_workspace(s.n_rows, 2 * F, H));
-  sub = std::max(sub, subspec_int4_linear_workspace(s.n_rows, H, F));
+  size_t sub = 256;
+  if (s.n_rows <= kInt4LayerMaxRows) {                 // wider windows are dense only
+    sub = std::max(sub, subspec_int4_linear_workspace(s.n_rows, Q + 2 * KV, H));
+    sub = std::max(sub, subspec_int4_linear_workspace(s.n_rows, H, Q));
+    sub = std::max(sub, subspec_int4_linear_workspace(s.n_rows, 2 * F, H));
+    sub = std::max(sub, subspec_int4_linear_workspace(s.n_rows, H, F));
+  }
   sub = std::max(sub, subspec_dense_linear_workspace(s.n_rows, Q + 2 * KV, H));
   sub = std::max(sub, subspec_dense_linear_workspace(s.n_rows, H, Q));
   sub = std::max(sub, subspec_dense_linear_workspace(s.n_rows, 2 * F, H));
@@ -159,11 +164,12 @@ static LayerPlan layer_plan(const subspec_decoder_layer_dims& s) {
   return p;
 }
 
-static int check_dims(const subspec_decoder_layer_dims* s) {
+static int check_dims(const subspec_decoder_layer_dims* s, int max_rows) {
   if (!s) SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "decoder_layer: null dims");
   if (s->dtype != SUBSPEC_BF16 && s->dtype != SUBSPEC_F16)
     SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "decoder_layer: dtype %d not supported (bf16 / fp16 only)", s->dtype);
-  if (s->n_rows < 1 || s->n_rows > 64) SUBSPEC_FAIL(SUBSPEC_ERR_LIMIT, "decoder_layer: n_rows=%lld outside 1..64", (long long)s->n_rows);
+  if (s->n_rows < 1 || s->n_rows > max_rows)
+    SUBSPEC_FAIL(SUBSPEC_ERR_LIMIT, "decoder_layer: n_rows=%lld outside 1..%d", (long long)s->n_rows, max_rows);
   if (s->head_dim != 128) SUBSPEC_FAIL(SUBSPEC_ERR_LIMIT, "decoder_layer: head_dim=%lld (built for 128)", (long long)s->head_dim);
   if (s->hidden <= 0 || s->hidden % 64 != 0 || s->hidden > 8 * kNormThreads * kNormMaxPieces)
     SUBSPEC_FAIL(SUBSPEC_ERR_LIMIT, "decoder_layer: hidden=%lld must be a multiple of 64 and at most %d", (long long)s->hidden,
@@ -250,7 +256,7 @@ static int run_layer(const subspec_decoder_layer_dims& s, const LayerWeights& w,
     if ((rc = int4_gate_up_silu_ex(h, (const uint32_t*)w.gate_up.w, (const uint32_t*)w.gate_up.sz, nullptr, act, DT, M,
                                    2 * (int64_t)F, H, nullptr, 0.f, st)))
       return rc;
-  } else if (4 * (int64_t)F * H < ((int64_t)1 << 31)) {
+  } else if (M > 32 || 4 * (int64_t)F * H < ((int64_t)1 << 31)) {   // (up to 32 rows the pair kernel addresses the matrix through one 2 GiB descriptor)
     if ((rc = dense_gate_up_silu_ex(h, w.gate_up.w, nullptr, act, DT, M, 2 * (int64_t)F, H, st))) return rc;
   } else {
     if ((rc = project(w, w.gate_up, h, nullptr, nullptr, gu, DT, M, 2 * (int64_t)F, H, sub, p.sub_bytes, st))) return rc;
@@ -291,15 +297,18 @@ extern "C" int subspec_rms_norm(const void* x, const void* weight, void* y, int 
 }
 
 extern "C" size_t subspec_int4_decoder_layer_workspace(const subspec_decoder_layer_dims* dims) {
-  if (!dims || check_dims(dims) != SUBSPEC_OK) return 0;
+  if (!dims || check_dims(dims, kDenseLayerMaxRows) != SUBSPEC_OK) return 0;
   return layer_plan(*dims).total;
 }
 
 static int decoder_layer_entry(const subspec_decoder_layer_dims* dims, const LayerWeights& w, void* x, const int32_t* positions,
                                const int32_t* cache_rows, const uint64_t* anc_bits, void* k_cache, void* v_cache,
                                void* workspace, size_t workspace_bytes, void* stream) {
-  const int rc = check_dims(dims);
+  const int rc = check_dims(dims, w.dense ? kDenseLayerMaxRows : kInt4LayerMaxRows);
   if (rc != SUBSPEC_OK) return rc;
+  // the wide dense kernels take weight rows in tiles of 32
+  if (dims->n_rows > 64 && ((dims->n_q_heads + 2 * dims->n_kv_heads) * dims->head_dim % 32 != 0 || dims->hidden % 32 != 0))
+    SUBSPEC_FAIL(SUBSPEC_ERR_LIMIT, "decoder_layer: more than 64 rows need projection widths that are multiples of 32");
   if (!x || !positions || !cache_rows || !anc_bits || !k_cache || (!v_cache && !dims->page_indices))
     SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "decoder_layer: null pointer argument");
   if (!w.input_norm || !w.post_norm || !w.qkv.w || !w.o.w || !w.gate_up.w || !w.down.w ||

@@ -155,6 +155,7 @@ class Decoder:
             self._native = (bool(self.layers) and (all(packed) or not any(packed)) and self.dtype != torch.float32
                             and (self.kv.cache.contiguous or hasattr(self.kv.cache, "pool")))
             if self._native:
+                self._native_packed = packed[0]      # int4 layers: windows of at most 64 rows
                 make = ops.decoder_layer_weights if packed[0] else ops.dense_layer_weights
                 self._native_make = make
                 resident = min(self.first_streamed, len(self.layers))
@@ -277,9 +278,10 @@ class Decoder:
                      positions32: Optional[torch.Tensor] = None, rows32: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Forward of tree nodes occupying cache rows prefix_len+first_slot.. ; ``depths`` are the node
         depths (rotary position = prefix_len + depth), ``anc_bits`` int64 [n] bitsets over tree
-        slots ([n, ceil(slots / 64)] words above 64 slots).  Up to 64 rows go through the one-call layers; a larger
-        window (a whole large tree in the target) runs module by module, so that every weight matrix is read once
-        for all rows (library GEMMs) and only attention is split into launches of 64 rows.  Returns logits [n, V].
+        slots ([n, ceil(slots / 64)] words above 64 slots).  Up to 64 rows (int4 layers) or 384 rows (dense layers: a
+        whole 289-node tree in the target) go through the one-call layers, every weight matrix read once for all
+        rows; a larger window runs module by module on library GEMMs with only attention on this library's kernel.
+        Returns logits [n, V].
 
         ``prefix_len_dev`` (int64 device tensor of one element): the prefix length is taken from the device when the
         kernels run and ``prefix_len`` is only its upper bound -- nothing on the host side depends on the actual
@@ -293,9 +295,12 @@ class Decoder:
         self.kv.cache.ensure(prefix_len + max(slots, first_slot + n))
         self._rope_tables(prefix_len + max(slots, first_slot + n) + 8)
         cfg = self.cfg
-        native = self.use_native_layers and self.native_layers and n <= 64 and slots <= ops.L.MAX_TREE_NODES
+        native = self.use_native_layers and self.native_layers and slots <= ops.L.MAX_TREE_NODES
+        if native and n > 64:                        # dense layers only, projection widths in tiles of 32
+            native = (n <= 384 and not self._native_packed and cfg.q_size % 32 == 0 and cfg.kv_size % 32 == 0
+                      and cfg.hidden_size % 32 == 0)
         if prefix_len_dev is not None and not native:
-            raise ValueError("a device-side prefix length needs the one-call decoder layers (at most 64 rows)")
+            raise ValueError("a device-side prefix length needs the one-call decoder layers (at most 64 rows; 384 for dense layers)")
         if positions32 is not None and rows32 is not None:
             if native:
                 return self.logits(self._run_native_layers(self.embed[token_ids], positions32, rows32, anc_bits, prefix_len,

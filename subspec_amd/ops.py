@@ -573,7 +573,7 @@ def int4_gate_up_silu(x: torch.Tensor, wq: torch.Tensor, sz: torch.Tensor, inter
 
 
 def dense_gate_up_silu(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """``silu(gate) * up`` from a dense fused weight [2F, K] (gate rows first) in one launch: x [..., K] (at most 64
+    """``silu(gate) * up`` from a dense fused weight [2F, K] (gate rows first) in one launch: x [..., K] (at most 384
     rows) -> [..., F]."""
     dev = _require_gpu(x, weight)
     N, K = weight.shape
@@ -609,7 +609,8 @@ def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
 
 
 def dense_linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """``F.linear(x, weight, bias)`` for at most 64 rows of bf16 / fp16 activations: x [..., K], weight [N, K]."""
+    """``F.linear(x, weight, bias)`` for at most 384 rows of bf16 / fp16 activations: x [..., K], weight [N, K]
+    (N a multiple of 16; of 32 above 64 rows)."""
     dev = _require_gpu(x, weight)
     N, K = weight.shape
     if x.shape[-1] != K or x.dtype != weight.dtype:

@@ -108,9 +108,19 @@ def test_single_layer_against_float32_oracle():
 
 
 def test_rejects_bad_arguments():
-    dims = ops.decoder_layer_dims(torch.bfloat16, 65, 256, 512, 2, 1, 128, 256, 10, 8, 1e-6, 1e6)
+    dims = ops.decoder_layer_dims(torch.bfloat16, 385, 256, 512, 2, 1, 128, 1024, 10, 8, 1e-6, 1e6)
     with pytest.raises(ValueError):
         ops.decoder_layer_workspace(dims)
+    # the int4 stack takes windows of at most 64 rows (the dense stack up to 384)
+    kv, draft, _, _, _ = _setup(3, 20, 8)
+    dims = ops.decoder_layer_dims(torch.bfloat16, 65, CFG.hidden_size, CFG.intermediate_size, CFG.num_attention_heads,
+                                  CFG.num_key_value_heads, CFG.head_dim, 256, 10, 65, CFG.rms_norm_eps, CFG.rope_theta)
+    ws = torch.empty(ops.decoder_layer_workspace(dims), dtype=torch.uint8, device=DEV)
+    with pytest.raises(ValueError):
+        ops.int4_decoder_layer_(torch.zeros(65, CFG.hidden_size, dtype=torch.bfloat16, device=DEV), dims,
+                                ops.decoder_layer_weights(draft.layers[0]), torch.zeros(65, dtype=torch.int32, device=DEV),
+                                torch.zeros(65, dtype=torch.int32, device=DEV), torch.zeros(65, 2, dtype=torch.int64, device=DEV),
+                                kv.cache.k(0), kv.cache.v(0), ws)
     with pytest.raises(ValueError):
         ops.decoder_layer_dims(torch.float32, 8, 256, 512, 2, 1, 128, 256, 10, 8, 1e-6, 1e6)
     dims = ops.decoder_layer_dims(torch.bfloat16, 8, 256, 512, 2, 1, 64, 256, 10, 8, 1e-6, 1e6)    # head_dim 64

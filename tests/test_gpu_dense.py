@@ -1,4 +1,4 @@
-"""GPU: the dense 16-bit linear for few rows and the target's one-call decoder layer (through the C ABI).
+"""GPU: the dense 16-bit linear for the rows of a tree (1 to 384) and the target's one-call decoder layer (through the C ABI).
 
 Bar (floating point): fp32 accumulation in a different order than the reference product, one rounding
 to the activation dtype: |y - ref| <= 2^-7 |ref| + 1e-2 of the output scale for bf16 (2^-10 for
@@ -26,7 +26,9 @@ def test_dense_linear_matches_float64_product(dtype, N, K):
     w = (torch.randn(N, K, generator=g) * 0.05).to(dtype)
     bias = (torch.randn(N, generator=g) * 0.1).to(dtype)
     wd = w.to(DEV)
-    for M in (1, 5, 16, 17, 33, 64):
+    for M in (1, 5, 16, 17, 33, 64, 65, 130, 289, 384):
+        if M > 64 and N % 32:                        # more than 64 rows: weight tiles of 32 rows
+            continue
         print("dense_linear", dtype, N, K, M, flush=True)
         x = torch.randn(M, K, generator=g).to(dtype)
         for b in (None, bias):
@@ -75,7 +77,7 @@ def test_dense_linear_special_cases():
     # leading dimensions are kept
     y = ops.dense_linear(torch.zeros(2, 3, 256, dtype=torch.bfloat16, device=DEV), eye.to(DEV))
     assert y.shape == (2, 3, 256)
-    for bad in (dict(M=65, N=256, K=256), dict(M=4, N=250, K=256), dict(M=4, N=256, K=200)):
+    for bad in (dict(M=385, N=256, K=256), dict(M=4, N=250, K=256), dict(M=4, N=256, K=200), dict(M=65, N=48, K=256)):
         with pytest.raises(ValueError):
             ops.dense_linear(torch.zeros(bad["M"], bad["K"], dtype=torch.bfloat16, device=DEV),
                              torch.zeros(bad["N"], bad["K"], dtype=torch.bfloat16, device=DEV))
@@ -84,18 +86,19 @@ def test_dense_linear_special_cases():
 
 
 def _setup(seed, prefix, n, first_streamed=None):
-    kv = create_kv_cache("static", max_cache_len=256, config=CFG, device=DEV, dtype=torch.bfloat16)
+    kv = create_kv_cache("static", max_cache_len=max(256, prefix + n + 8), config=CFG, device=DEV, dtype=torch.bfloat16)
     target, draft, w = build_models(CFG, kv, seed=seed, device=DEV, first_streamed=first_streamed)
     g = torch.Generator().manual_seed(seed)
     prompt = torch.randint(0, CFG.vocab_size, (prefix,), generator=g).to(DEV)
     target.prefill(prompt, 0)
-    parents, _, depths = W.random_tree(g, n=n, max_depth=5, max_children=3, vocab=CFG.vocab_size, chain_depth=3)
+    parents, _, depths = W.random_tree(g, n=n, max_depth=5, max_children=3 if n <= 200 else 4, vocab=CFG.vocab_size, chain_depth=3)
     toks = torch.randint(0, CFG.vocab_size, (n,), generator=g).to(DEV)
     anc = ops.ancestor_bits_tensor(parents, device=DEV)
     return kv, target, toks, torch.tensor(depths, device=DEV), anc
 
 
-@pytest.mark.parametrize("n,prefix,first_streamed", [(1, 17, None), (9, 40, None), (33, 100, 1), (64, 130, None)])
+@pytest.mark.parametrize("n,prefix,first_streamed", [(1, 17, None), (9, 40, None), (33, 100, 1), (64, 130, None),
+                                                     (65, 70, None), (200, 300, 1), (289, 130, None), (384, 64, None)])
 def test_target_native_layers_match_module_path(n, prefix, first_streamed):
     print("dense decoder layer stack", n, prefix, first_streamed, flush=True)
     kv, target, toks, depths, anc = _setup(21 + n, prefix, n, first_streamed)
@@ -150,7 +153,8 @@ def test_dense_gate_up_projection_with_the_activation_in_its_output_stage(dtype)
     """As for the int4 twin: the fused launch against the plain projection followed by the activation on the values
     it stored; only the exponential may differ in its last place."""
     for seed, (F, K, M, bias) in enumerate([(16, 64, 1, False), (48, 192, 5, True), (1184, 128, 17, True), (18944, 3584, 8, False),
-                                            (18944, 3584, 64, False), (2048, 512, 33, True), (40000, 64, 3, False)]):
+                                            (18944, 3584, 64, False), (2048, 512, 33, True), (40000, 64, 3, False),
+                                            (2048, 512, 65, True), (18944, 3584, 289, False), (1184, 128, 384, True)]):
         print("dense gate|up + silu", dtype, F, K, M, bias, flush=True)
         g = torch.Generator().manual_seed(800 + seed)
         W = (torch.randn(2 * F, K, generator=g) * (2.0 / K ** 0.5)).to(dtype).to(DEV)

@@ -1,7 +1,7 @@
 """GPU: the decoder-layer path at the Qwen2.5-7B geometry of BASELINE config 5 -- hidden 3584, 28 query heads over
 4 KV heads (7:1 GQA), head_dim 128, FFN 18944, prefix 2048 -- instead of the small decoder the other cycle tests use.
 
-* one `subspec_int4_decoder_layer` and one `subspec_dense_decoder_layer` call, 8 and 64 tree rows, against the
+* one `subspec_int4_decoder_layer` (8 and 64 tree rows) and one `subspec_dense_decoder_layer` call (8 to 289 rows) against the
   float32 oracle layer (`oracle/decoder.py`) on the same (for the draft: dequantized) weights: residual stream and
   the K / V rows written, tolerance 2e-2 of the largest magnitude (bf16 intermediates, as for the small geometry);
 * rotary positions near 32k (the reference's `max_position_embeddings`) through the same entry point;
@@ -45,7 +45,11 @@ def _layer_case(seed, n, prefix, max_len, depth_base=0):
 
 
 def _oracle(cfg, wd, x0, kc, vc, positions, rows, anc, prefix):
-    bits = [int(b) & ((1 << 64) - 1) for b in anc.cpu().tolist()]
+    mask = (1 << 64) - 1
+    if anc.dim() == 1:
+        bits = [int(b) & mask for b in anc.cpu().tolist()]
+    else:                                            # more than 64 tree slots: several 64-bit words per row
+        bits = [sum((int(wd_) & mask) << (64 * i) for i, wd_ in enumerate(row)) for row in anc.cpu().tolist()]
     k, v = kc.float().clone(), vc.float().clone()
     want = od.decoder_layer(x0.float().cpu(), wd, k, v, positions.cpu().long(), rows.cpu().long(), bits, prefix,
                             cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim, cfg.rms_norm_eps, cfg.rope_theta)
@@ -68,10 +72,12 @@ def _dims(cfg, n, max_len, prefix):
                                   cfg.num_key_value_heads, cfg.head_dim, max_len, prefix, n, cfg.rms_norm_eps, cfg.rope_theta)
 
 
-@pytest.mark.parametrize("n", [8, 64])
+@pytest.mark.parametrize("n", [8, 64, 65, 289])
 def test_dense_target_layer_at_7b_geometry(n):
+    """65 and 289 rows (a whole depth-48, k-6 tree of the reference's offloading configuration, 1 + 48 * 6 nodes) take the
+    32 x 32 x 16 projections and several 64-row attention windows inside the same call."""
     print("7B geometry, dense layer, rows", n, flush=True)
-    max_len = PREFIX + 64
+    max_len = PREFIX + max(64, n)
     cfg, w, anc, x0, kc, vc, positions, rows = _layer_case(100 + n, n, PREFIX, max_len)
     dims = _dims(cfg, n, max_len, PREFIX)
     ws = torch.empty(ops.decoder_layer_workspace(dims), dtype=torch.uint8, device=DEV)

@@ -62,3 +62,31 @@ def test_attention_block_matches_the_attention_oracle():
     q = od.rope((h @ w["qkv"].T + w["qkv_bias"])[:, :Hq * D].reshape(n, Hq, D), pos, 1e4)
     ref = oa.tree_attention(q.transpose(0, 1)[None], kc[None], vc[None], parents, prefix)     # caches hold the new rows
     assert torch.allclose(y - x, ref.reshape(n, Hq * D)[:, :H], rtol=1e-4, atol=1e-5)
+
+
+def test_many_row_form_equals_the_row_loop():
+    """Above 64 rows the oracle evaluates attention for all rows at once (masked scores) instead of row by row; both forms
+    on the same 70-row tree (slots beyond 64 in use), the loop form run as two calls' worth of rows over the same cache."""
+    g = torch.Generator().manual_seed(7)
+    H, Hq, Hkv, D, F, n, prefix = 64, 4, 2, 32, 96, 70, 11
+    w = _weights(g, H, Hq * D, Hkv * D, F)
+    x = torch.randn(n, H, generator=g)
+    parents = [-1] + [int(torch.randint(max(0, i - 9), i, (1,), generator=g)) for i in range(1, n)]
+    bits, depth = [], []
+    for i, p in enumerate(parents):
+        bits.append((1 << i) | (bits[p] if p >= 0 else 0))
+        depth.append(0 if p < 0 else depth[p] + 1)
+    assert max(b.bit_length() for b in bits) > 64
+    pos = torch.tensor([prefix + d for d in depth])
+    rows = torch.arange(prefix, prefix + n)
+    kc0, vc0 = torch.randn(Hkv, 96, D, generator=g), torch.randn(Hkv, 96, D, generator=g)
+    kc, vc = kc0.clone(), vc0.clone()
+    y = od.decoder_layer(x, w, kc, vc, pos, rows, bits, prefix, Hq, Hkv, D, 1e-6, 1e4)
+    # row loop: the K / V rows of all 70 nodes are in the cache already (kc, vc from the call above), so any window of at
+    # most 64 rows sees what it saw in the one call
+    parts = []
+    for lo, hi in ((0, 40), (40, 70)):
+        k2, v2 = kc.clone(), vc.clone()
+        parts.append(od.decoder_layer(x[lo:hi], w, k2, v2, pos[lo:hi], rows[lo:hi], bits[lo:hi], prefix, Hq, Hkv, D, 1e-6, 1e4))
+        assert torch.allclose(k2, kc, atol=1e-6) and torch.allclose(v2, vc, atol=1e-6)
+    assert torch.allclose(torch.cat(parts), y, rtol=1e-5, atol=1e-5)
