@@ -214,8 +214,9 @@ def bench_int4(args):
 
 
 def bench_dense(args):
-    """The target model's projections in the tree-decoding forward (bf16, at most 64 rows), next to the
-    library GEMM (torch F.linear) on the same operands; weights streamed from HBM as in bench_int4."""
+    """The target model's projections in the tree-decoding forward (bf16; 8 and 64 rows, and the 289 rows of a depth-48,
+    k-6 tree), next to the library GEMM (torch F.linear) on the same operands; weights streamed from HBM as in
+    bench_int4."""
     import torch
     import torch.nn.functional as F
     from subspec_amd import ops
@@ -223,14 +224,15 @@ def bench_dense(args):
     for N, K in ((4608, 3584), (3584, 3584), (37888, 3584), (3584, 18944)):
         copies = max(2, COLD_BYTES // (N * K * 2) + 1)
         wl = [(torch.randn(N, K, device=dev) * 0.02).to(torch.bfloat16) for _ in range(copies)]
-        for M in (8, 64):
+        for M in (8, 64, 289):
             x = torch.randn(M, K, device=dev).to(torch.bfloat16)
             steps = max(args.steps, copies)
             call_us, kernel_us = _time_us(_rotating(lambda i: ops.dense_linear(x, wl[i]), copies), steps, args.warmup)
             lib_us, _ = _time_us(_rotating(lambda i: F.linear(x, wl[i]), copies), steps, args.warmup)
             _kernel_line("dense 16-bit linear latency", f"target layer projection {K}->{N}, M={M}, bf16, weights streamed from "
                          f"HBM (rotating over {copies} copies)", call_us, kernel_us, N * K * 2 + M * (K + N) * 2, 2 * M * N * K,
-                         "subspec::dense_gemm_kernel", extra={"N": N, "K": K, "M": M, "library_gemm_call_us": round(lib_us, 2)})
+                         "subspec::dense_gemm_kernel" if M <= 32 else "subspec::dense_wide_kernel",
+                         extra={"N": N, "K": K, "M": M, "library_gemm_call_us": round(lib_us, 2)})
         del wl
 
 
@@ -255,6 +257,7 @@ def e2e_runs(args, runs, new_tokens, say=lambda *_: None):
     for run in runs:
         keep_layers, agreeing = run[0], run[1]
         new_tokens = run[2] if len(run) > 2 else default_tokens
+        tree = run[3] if len(run) > 3 else None             # (depth, k, node cap or None) of this run's draft tree
         t0 = time.perf_counter()
         if args.checkpoint:
             cfg, weights = load_hf_checkpoint(args.checkpoint, device=dev)
@@ -278,9 +281,12 @@ def e2e_runs(args, runs, new_tokens, say=lambda *_: None):
             v2 = args.generator == "v2"
             depth = args.tree_depth or (7 if v2 else 8)
             cap = args.max_verify_tokens or None
+            tree_k = args.tree_k
+            if tree is not None:
+                depth, tree_k, cap = tree
             gen = (SubSpecSDGeneratorV2 if v2 else SubSpecSDGenerator)(
                 target, None, SubSpecSDDraftModel(draft),
-                DraftParams(temperature=0.2, max_depth=depth, topk_len=args.tree_k, max_verify_tokens=cap),
+                DraftParams(temperature=0.2, max_depth=depth, topk_len=tree_k, max_verify_tokens=cap),
                 generator_kwargs=dict(verify_method=method, verify_kwargs=vk, draft_graph=bool(getattr(args, "draft_graph", False)),
                                       **(dict(postspec_steps=args.postspec_steps) if v2 else {})))
             kv.reset()
@@ -299,10 +305,11 @@ def e2e_runs(args, runs, new_tokens, say=lambda *_: None):
                 "config": {"workload": f"BASELINE config 5: {'checkpoint' if args.checkpoint else 'Qwen2.5-7B shape'}, "
                                        + ("all layers resident" if keep_layers >= cfg.num_hidden_layers else
                                           f"layers {keep_layers}-{cfg.num_hidden_layers - 1} streamed")
-                                       + f", int4 draft, depth {depth}, k {args.tree_k}, "
-                                       + (f"<={cap} nodes" if cap else f"{1 + depth * args.tree_k} nodes") + f", prompt 2048, {new_tokens} new tokens, verify {method}"
+                                       + f", int4 draft, depth {depth}, k {tree_k}, "
+                                       + (f"<={cap} nodes" if cap else f"{1 + depth * tree_k} nodes") + f", prompt 2048, {new_tokens} new tokens, verify {method}"
                                        + (", post-speculating driver" if v2 else ""),
                            "verify_method": method, "generator": args.generator,
+                           "tree": f"depth {depth}, k {tree_k}, " + (f"<={cap} nodes" if cap else f"{1 + depth * tree_k} nodes"),
                            "draft_graph_replays": gen.draft_model.graph_replays, "resident_target_layers": min(keep_layers, cfg.num_hidden_layers),
                            "ring_slabs": (target.streamer.n_slabs if target.streamer is not None else 0),
                            "agreeing_draft": bool(agreeing),
@@ -332,14 +339,18 @@ def e2e_block(args):
     """The bounded config-5 runs the default line carries: `--e2e-tokens` new tokens after the 2048-token prompt, layers
     14-27 streamed (the configuration BASELINE names) and all layers resident, random weights, exact and lossy; plus
     the streamed cycle with a draft that agrees with its target (the high-acceptance end random weights cannot show)."""
-    keys = ("verify_method", "resident_target_layers", "agreeing_draft", "n_iter", "n_tokens", "tokens_per_cycle", "avg_draft_s",
+    keys = ("verify_method", "resident_target_layers", "agreeing_draft", "tree", "n_iter", "n_tokens", "tokens_per_cycle", "avg_draft_s",
             "avg_target_s", "avg_verify_s", "cycle_tokens_per_s", "elapsed_s", "host_to_device_GB", "host_to_device_GB_per_s")
     out = {"workload": f"BASELINE config 5, Qwen2.5-7B shape (28 layers, hidden 3584, 28/4 heads, FFN 18944, vocab 152064), int4 g64 "
                        f"draft, depth 8, k 8, <=64 nodes, prompt 2048, {args.e2e_tokens} new tokens with layers 14-27 streamed and random "
-                       f"weights, {args.e2e_tokens_other} in the other runs; tokens_per_s = new tokens / "
+                       f"weights, {args.e2e_tokens_other} in the other runs (the last of them with the depth-48, k-6, 289-node tree); "
+                       "tokens_per_s = new tokens / "
                        "whole generate() including the prefill, cycle_tokens_per_s = tokens per cycle / (draft + target + verify)",
            "runs": []}
-    for line in e2e_runs(args, [(14, False, args.e2e_tokens), (28, False, args.e2e_tokens_other), (14, True, args.e2e_tokens_other)],
+    # the last run: the tree of the reference's offloading configuration (depth 48, k 6, all 289 nodes verified in one
+    # target forward; configs/exp_offloading/subspec_sd_qwen_7b.yaml:16-19), all layers resident
+    for line in e2e_runs(args, [(14, False, args.e2e_tokens), (28, False, args.e2e_tokens_other), (14, True, args.e2e_tokens_other),
+                                (28, False, args.e2e_tokens_other, (48, 6, None))],
                          args.e2e_tokens):
         out["runs"].append(dict({"tokens_per_s": line["value"]}, **{k: line["config"][k] for k in keys}))
     return out
