@@ -75,7 +75,8 @@ __device__ __forceinline__ uint2 lds_read_tr16(const uint16_t* p) {
 struct AttnParams {
   int64_t batch, hq, hkv, n_rows, n_slots, seq_stride, prefix, anc_batch_stride;
   int mask_words;              // 64-bit words per ancestor bitset: ceil(n_slots / 64)
-  int row0, win_rows;          // this launch covers query rows row0 .. row0 + win_rows - 1 (win_rows <= 64) of n_rows
+  int row0, win_rows;          // this launch covers query rows row0 .. row0 + win_rows - 1 (win_rows <= 64) of n_rows ...
+  int windows;                 // ... or `windows` > 1 windows of 64 rows from row0 on (32-row kernels): see attn_window
   int chunks;
   int64_t chunk_keys;          // multiple of kKeyBlock
   int pairs_per_kv;            // workgroups (groups of 4 or 8 query heads) per KV head
@@ -90,6 +91,16 @@ struct AttnParams {
   int page_shift, max_pages;
   int64_t page_stride, tok_stride, v_delta;   // elements
 };
+
+// Several windows of 64 query rows in one launch (a tree of more than 64 rows in the target): the windows of a sequence
+// read the same keys, so they are laid out as further batch entries -- virtual entry vb = window * batch + b -- that share
+// the cache of sequence b; split-KV partials are kept per virtual entry.
+struct AttnWindow { int b, row0, win_rows; };
+__device__ __forceinline__ AttnWindow attn_window(const AttnParams& ap, int vb) {
+  const int w = vb / (int)ap.batch;
+  const int row0 = ap.row0 + w * kAttnRows;
+  return AttnWindow{vb - w * (int)ap.batch, row0, ap.windows > 1 ? min((int)ap.n_rows - row0, kAttnRows) : ap.win_rows};
+}
 
 // THREADS = 512: eight wavefronts; 256: four wavefronts, each 16 rows of ONE head (ROWT = 1, WPH = 4) -- with 33 to 64
 // query rows and few sequences this shape gets its workgroups from the heads instead of from key chunks, so the
@@ -469,7 +480,9 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
   if ((int64_t)unit >= ap.units) return;
   const int chunk = (int)(unit % (uint32_t)ap.chunks);
   const uint32_t bkv = unit / (uint32_t)ap.chunks;
-  const int kvh = (int)(bkv % (uint32_t)ap.hkv), b = (int)(bkv / (uint32_t)ap.hkv);
+  const int kvh = (int)(bkv % (uint32_t)ap.hkv), vb = (int)(bkv / (uint32_t)ap.hkv);
+  const AttnWindow aw = attn_window(ap, vb);          // (sequence, window of 64 query rows) of this unit
+  const int b = aw.b;
   const int group = (int)((uint32_t)ap.hq / (uint32_t)ap.hkv);
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -478,14 +491,14 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
   const int head_in_group = pair * kHeadsPerWG + wave / WPH;
   const bool head_ok = head_in_group < group;
   const int qh = kvh * group + (head_ok ? head_in_group : 0);
-  const int bh = b * (int)ap.hq + qh;
+  const int bh = b * (int)ap.hq + qh, vbh = vb * (int)ap.hq + qh;   // q / out rows; partial slots
   const int n = (int)ap.n_rows;
   const int64_t prefix = ap.prefix_dev ? min(max(*ap.prefix_dev, (int64_t)0), ap.prefix) : ap.prefix;
   const int64_t kv_len = prefix + ap.n_slots;
   const int tile = wave % WPH;
   const int row = tile * 32 + lr;                       // row inside this launch's window
-  const bool row_ok = head_ok && row < ap.win_rows;
-  const int grow = ap.row0 + (row_ok ? row : 0);
+  const bool row_ok = head_ok && row < aw.win_rows;
+  const int grow = aw.row0 + (row_ok ? row : 0);
 
   v16f oacc[kAttnD / 32];
 #pragma unroll
@@ -549,8 +562,8 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
 #pragma unroll
   for (int u = 0; u < kMaskPerThread; ++u) {
     const int i = tid + u * THREADS, r = i / kMaskWords, w = i % kMaskWords;
-    mword[u] = (reaches_tree && i < kAttnRows * kMaskWords && r < ap.win_rows && w < ap.mask_words)
-                   ? anc[((int64_t)b * ap.anc_batch_stride + ap.row0 + r) * ap.mask_words + w] : 0ull;
+    mword[u] = (reaches_tree && i < kAttnRows * kMaskWords && r < aw.win_rows && w < ap.mask_words)
+                   ? anc[((int64_t)b * ap.anc_batch_stride + aw.row0 + r) * ap.mask_words + w] : 0ull;
   }
   SUBSPEC_ATTN32_STAGE(0);
   SUBSPEC_ATTN32_FETCH(0, key0 + 2 * kKeyBlock);
@@ -574,7 +587,7 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
     SUBSPEC_ATTN32_STAGE(buf ^ 1);
     SUBSPEC_ATTN32_FETCH(buf ^ 1, kb + 3 * kKeyBlock);
     if (kb >= key1) continue;                          // (uniform) odd number of blocks: the requests above keep every path's count equal
-    if (!(head_ok && tile * 32 < ap.win_rows)) continue; // (wave-uniform) a head slot or row tile with nothing in it only helps with the staging
+    if (!(head_ok && tile * 32 < aw.win_rows)) continue; // (wave-uniform) a head slot or row tile with nothing in it only helps with the staging
     const uint16_t* Ks = Ks2[buf] + koff;
     const uint16_t* Vs = Vs2[buf] + voff;
 
@@ -663,11 +676,11 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
 #undef SUBSPEC_ATTN32_STAGE
 
   float l = l_run + __shfl_xor(l_run, 32, kWave);
-  if (!head_ok || tile * 32 >= ap.win_rows) return;      // (wave-uniform) nothing of this tile is wanted
+  if (!head_ok || tile * 32 >= aw.win_rows) return;      // (wave-uniform) nothing of this tile is wanted
   if (ap.chunks == 1) {
     if (!row_ok) return;
     const float inv = l > 0.f ? 1.0f / l : 0.f;
-    uint16_t* op = out + (((int64_t)b * n + ap.row0 + row) * ap.hq + qh) * kAttnD + g * 4;
+    uint16_t* op = out + (((int64_t)b * n + aw.row0 + row) * ap.hq + qh) * kAttnD + g * 4;
 #pragma unroll
     for (int dt = 0; dt < kAttnD / 32; ++dt)
 #pragma unroll
@@ -678,7 +691,7 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
     // the chunk's own softmax-weighted average of V, in the 16-bit dtype (a convex combination of such averages is what the
     // merge forms, so their rounding error does not grow); every store instruction writes 512 consecutive bytes
     const float inv = l > 0.f ? 1.0f / l : 0.f;
-    uint16_t* po = (uint16_t*)part_o + (((int64_t)bh * ap.chunks + chunk) * 2 + tile) * kTileElems + lane * 4;
+    uint16_t* po = (uint16_t*)part_o + (((int64_t)vbh * ap.chunks + chunk) * 2 + tile) * kTileElems + lane * 4;
 #pragma unroll
     for (int dt = 0; dt < kAttnD / 32; ++dt)
 #pragma unroll
@@ -686,7 +699,7 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
         *(uint2*)(po + (dt * 4 + q4) * 256) = make_uint2(pack2<DT>(oacc[dt][4 * q4] * inv, oacc[dt][4 * q4 + 1] * inv),
                                                          pack2<DT>(oacc[dt][4 * q4 + 2] * inv, oacc[dt][4 * q4 + 3] * inv));
     if (g == 0) {
-      const int64_t pslot = ((int64_t)bh * ap.chunks + chunk) * kAttnRows + row;
+      const int64_t pslot = ((int64_t)vbh * ap.chunks + chunk) * kAttnRows + row;
       *(v2f_t*)(part_ml + pslot * 2) = v2f_t{m_run * ap.scale_log2, l};
     }
   }
@@ -903,7 +916,9 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   if ((int64_t)unit >= ap.units) return;
   const int chunk = (int)(unit % (uint32_t)ap.chunks);
   const uint32_t bkv = unit / (uint32_t)ap.chunks;
-  const int kvh = (int)(bkv % (uint32_t)ap.hkv), b = (int)(bkv / (uint32_t)ap.hkv);
+  const int kvh = (int)(bkv % (uint32_t)ap.hkv), vb = (int)(bkv / (uint32_t)ap.hkv);
+  const AttnWindow aw = attn_window(ap, vb);          // (sequence, window of 64 query rows) of this unit
+  const int b = aw.b;
   const int group = (int)((uint32_t)ap.hq / (uint32_t)ap.hkv);
 
   const int tid = threadIdx.x, lane = tid & 63;
@@ -913,15 +928,15 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   const int head_in_group = pair * kHeadsPerWG + wave / WPH;
   const bool head_ok = head_in_group < group;
   const int qh = kvh * group + (head_ok ? head_in_group : 0);
-  const int bh = b * (int)ap.hq + qh;
+  const int bh = b * (int)ap.hq + qh, vbh = vb * (int)ap.hq + qh;   // q / out rows; partial slots
   const int n = (int)ap.n_rows;
   const int64_t prefix = ap.prefix_dev ? min(max(*ap.prefix_dev, (int64_t)0), ap.prefix) : ap.prefix;
   const int64_t kv_len = prefix + ap.n_slots;
   const int tile = wave % WPH;
   const int row = tile * 32 + lr;
-  const bool live = head_ok && tile * 32 < ap.win_rows;     // (wave-uniform) this wavefront has rows to work on
-  const bool row_ok = head_ok && row < ap.win_rows;
-  const int grow = ap.row0 + (row_ok ? row : 0);
+  const bool live = head_ok && tile * 32 < aw.win_rows;     // (wave-uniform) this wavefront has rows to work on
+  const bool row_ok = head_ok && row < aw.win_rows;
+  const int grow = aw.row0 + (row_ok ? row : 0);
   const bool grp_b = wave >= 4;                             // the second wavefront of each SIMD (wavefront w runs on SIMD w % 4)
 
   const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)lds;
@@ -967,8 +982,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
   for (int u = 0; u < 2; ++u) {
     const int i = tid + u * 512, r = i / kPPMaskWords, w = i % kPPMaskWords;
-    mword[u] = (i < kAttnRows * kPPMaskWords && r < ap.win_rows && w < ap.mask_words)
-                   ? anc[((int64_t)b * ap.anc_batch_stride + ap.row0 + r) * ap.mask_words + w] : 0ull;
+    mword[u] = (i < kAttnRows * kPPMaskWords && r < aw.win_rows && w < ap.mask_words)
+                   ? anc[((int64_t)b * ap.anc_batch_stride + aw.row0 + r) * ap.mask_words + w] : 0ull;
   }
 
 
@@ -1050,7 +1065,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   if (ap.chunks == 1) {
     if (!row_ok) return;
     const float inv = l > 0.f ? 1.0f / l : 0.f;
-    uint16_t* op = out + (((int64_t)b * n + ap.row0 + row) * ap.hq + qh) * kAttnD + g * 4;
+    uint16_t* op = out + (((int64_t)b * n + aw.row0 + row) * ap.hq + qh) * kAttnD + g * 4;
 #pragma unroll
     for (int dt = 0; dt < kAttnD / 32; ++dt)
 #pragma unroll
@@ -1061,7 +1076,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     // the chunk's own softmax-weighted average of V, in the 16-bit dtype (a convex combination of such averages is what the
     // merge forms, so their rounding error does not grow); every store instruction writes 512 consecutive bytes
     const float inv = l > 0.f ? 1.0f / l : 0.f;
-    uint16_t* po = (uint16_t*)part_o + (((int64_t)bh * ap.chunks + chunk) * 2 + tile) * kTileElems + lane * 4;
+    uint16_t* po = (uint16_t*)part_o + (((int64_t)vbh * ap.chunks + chunk) * 2 + tile) * kTileElems + lane * 4;
 #pragma unroll
     for (int dt = 0; dt < kAttnD / 32; ++dt)
 #pragma unroll
@@ -1069,7 +1084,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         *(uint2*)(po + (dt * 4 + q4) * 256) = make_uint2(pack2<DT>(oacc[dt][4 * q4] * inv, oacc[dt][4 * q4 + 1] * inv),
                                                          pack2<DT>(oacc[dt][4 * q4 + 2] * inv, oacc[dt][4 * q4 + 3] * inv));
     if (g == 0) {
-      const int64_t pslot = ((int64_t)bh * ap.chunks + chunk) * kAttnRows + row;
+      const int64_t pslot = ((int64_t)vbh * ap.chunks + chunk) * kAttnRows + row;
       *(v2f_t*)(part_ml + pslot * 2) = v2f_t{rf.have ? rf.ref * ap.scale_log2 : -INFINITY, l};
     }
   }
@@ -1085,13 +1100,15 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 template <int DT, int CMAX>
 __global__ __launch_bounds__(256) void tree_attention32_merge_kernel(
     const float* __restrict__ part_o, const float* __restrict__ part_ml, AttnParams ap, uint16_t* __restrict__ out) {
-  const int tile = blockIdx.x & 1, bh = blockIdx.x >> 1;
+  const int tile = blockIdx.x & 1, vbh = blockIdx.x >> 1;
   const int lane = threadIdx.x & 63, idx16 = blockIdx.y * 4 + (threadIdx.x >> 6);
   const int row = tile * 32 + (lane & 31), g = lane >> 5;
-  if (row >= ap.win_rows) return;
-  const int b = bh / (int)ap.hq, qh = bh % (int)ap.hq;
-  const int64_t slot0 = (int64_t)bh * ap.chunks * kAttnRows + row;
-  const uint16_t* po = (const uint16_t*)part_o + ((int64_t)bh * ap.chunks * 2 + tile) * kTileElems + (idx16 * 64 + lane) * 4;
+  const int vb = vbh / (int)ap.hq, qh = vbh % (int)ap.hq;
+  const AttnWindow aw = attn_window(ap, vb);
+  const int b = aw.b;
+  if (row >= aw.win_rows) return;
+  const int64_t slot0 = (int64_t)vbh * ap.chunks * kAttnRows + row;
+  const uint16_t* po = (const uint16_t*)part_o + ((int64_t)vbh * ap.chunks * 2 + tile) * kTileElems + (idx16 * 64 + lane) * 4;
   auto unpack4 = [](uint2 o, float* f) {
     if constexpr (DT == SUBSPEC_BF16) {
       f[0] = bf16_bits_to_float(o.x & 0xffffu); f[1] = bf16_bits_to_float(o.x >> 16);
@@ -1142,20 +1159,20 @@ __global__ __launch_bounds__(256) void tree_attention32_merge_kernel(
   }
   const float inv = den > 0.f ? 1.f / den : 0.f;
   const int d0 = (idx16 >> 2) * 32 + (idx16 & 3) * 8 + g * 4;
-  *(uint2*)(out + (((int64_t)b * ap.n_rows + ap.row0 + row) * ap.hq + qh) * kAttnD + d0) =
+  *(uint2*)(out + (((int64_t)b * ap.n_rows + aw.row0 + row) * ap.hq + qh) * kAttnD + d0) =
       make_uint2(pack2<DT>(num[0] * inv, num[1] * inv), pack2<DT>(num[2] * inv, num[3] * inv));
 }
 
 // Launch shape of one window of query rows.
 struct AttnPlan { int threads, rowt, wph, heads_per_wg, chunks; bool mfma32, pingpong; };
-static AttnPlan attn_plan(int64_t batch, int64_t hq, int64_t hkv, int64_t win_rows, int64_t kv_len) {
+static AttnPlan attn_plan(int64_t batch, int64_t hq, int64_t hkv, int64_t win_rows, int64_t kv_len, bool one_sequence) {
   AttnPlan pl;
   const int group = (int)(hq / hkv);
   const int64_t blocks = (kv_len + kKeyBlock - 1) / kKeyBlock;
   pl.mfma32 = win_rows > 16;
   // the ping-pong kernel pays for its set-up over many blocks: (sequence, head) pairs enough to fill the chip with few key
   // chunks.  One sequence never takes it, so that a request's attention over pages equals the contiguous one bit for bit.
-  pl.pingpong = pl.mfma32 && batch > 1 && batch * hq >= 128;
+  pl.pingpong = pl.mfma32 && !one_sequence && batch * hq >= 128;
   if (win_rows <= 16) {
     // a draft level: a wavefront is a whole head (one 16-row tile), eight heads share the staged keys
     pl.threads = 512; pl.rowt = 1; pl.wph = 1;
@@ -1185,12 +1202,16 @@ static AttnPlan attn_plan(int64_t batch, int64_t hq, int64_t hkv, int64_t win_ro
   pl.chunks = (int)std::min<int64_t>(chunks, 64);
   return pl;
 }
-// the most partial slots any window of a call can need (the first window is the largest)
-static int attn_chunks_bound(int64_t batch, int64_t hq, int64_t hkv, int64_t n_rows, int64_t kv_len) {
-  int c = 1;
-  for (int64_t rows : {std::min<int64_t>(n_rows, kAttnRows), (int64_t)(n_rows % kAttnRows ? n_rows % kAttnRows : kAttnRows)})
-    c = std::max(c, attn_plan(batch, hq, hkv, rows, kv_len).chunks);
-  return c;
+// One call = one launch (pair): up to 64 query rows are one window; more rows are ceil(n_rows / 64) windows laid out as
+// further batch entries (attn_window), planned like that many sequences of 64 rows.
+struct AttnLaunch { int windows, win_rows; int64_t vbatch; AttnPlan pl; };
+static AttnLaunch attn_launch(int64_t batch, int64_t hq, int64_t hkv, int64_t n_rows, int64_t kv_len) {
+  AttnLaunch al;
+  al.windows = (int)((n_rows + kAttnRows - 1) / kAttnRows);
+  al.win_rows = (int)std::min<int64_t>(n_rows, kAttnRows);
+  al.vbatch = batch * al.windows;
+  al.pl = attn_plan(al.vbatch, hq, hkv, al.win_rows, kv_len, batch == 1);
+  return al;
 }
 
 }  // namespace subspec
@@ -1206,10 +1227,10 @@ static size_t attn_partial_bytes(int64_t batch, int64_t hq, int chunks, size_t* 
 extern "C" size_t subspec_tree_attention_workspace(int64_t batch, int64_t n_q_heads, int64_t n_kv_heads, int64_t n_rows,
                                                    int64_t prefix_len, int64_t n_tree_slots) {
   if (batch <= 0 || n_q_heads <= 0 || n_kv_heads <= 0 || n_q_heads % n_kv_heads != 0 || n_rows <= 0) return 256;
-  const int chunks = attn_chunks_bound(batch, n_q_heads, n_kv_heads, n_rows, prefix_len + n_tree_slots);
-  if (chunks == 1) return 256;
+  const AttnLaunch al = attn_launch(batch, n_q_heads, n_kv_heads, n_rows, prefix_len + n_tree_slots);
+  if (al.pl.chunks == 1) return 256;
   size_t o_bytes;
-  return attn_partial_bytes(batch, n_q_heads, chunks, &o_bytes);
+  return attn_partial_bytes(al.vbatch, n_q_heads, al.pl.chunks, &o_bytes);
 }
 
 static int tree_attention_impl(const char* what, const void* q, const void* k_cache, const void* v_cache, void* out, int dtype,
@@ -1232,7 +1253,9 @@ static int tree_attention_impl(const char* what, const void* q, const void* k_ca
   if (prefix_len < 0 || prefix_len + n_tree_slots > kv_seq_stride)
     SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "%s: prefix_len=%lld + n_tree_slots=%lld exceeds the cache length %lld", what,
                  (long long)prefix_len, (long long)n_tree_slots, (long long)kv_seq_stride);
-  if (batch * n_q_heads > 65535) SUBSPEC_FAIL(SUBSPEC_ERR_LIMIT, "%s: batch*heads=%lld too large", what, (long long)(batch * n_q_heads));
+  if (batch * n_q_heads * ((n_rows + kAttnRows - 1) / kAttnRows) > 65535)
+    SUBSPEC_FAIL(SUBSPEC_ERR_LIMIT, "%s: batch*heads*windows=%lld too large", what,
+                 (long long)(batch * n_q_heads * ((n_rows + kAttnRows - 1) / kAttnRows)));
   if ((uintptr_t)q % 8 || (uintptr_t)k_cache % 16 || (uintptr_t)v_cache % 16 || (uintptr_t)out % 8)
     SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "%s: q/out must be 8-byte and k/v 16-byte aligned", what);
   AttnParams ap;
@@ -1259,10 +1282,12 @@ static int tree_attention_impl(const char* what, const void* q, const void* k_ca
   const int group = (int)(n_q_heads / n_kv_heads);
   float* part_o = nullptr;
   float* part_ml = nullptr;
-  const int chunks_bound = attn_chunks_bound(batch, n_q_heads, n_kv_heads, n_rows, kv_len);
-  if (chunks_bound > 1) {
+  const AttnLaunch al = attn_launch(batch, n_q_heads, n_kv_heads, n_rows, kv_len);
+  const AttnPlan& pl = al.pl;
+  const int64_t vbatch = al.vbatch;
+  if (pl.chunks > 1) {
     size_t o_bytes;
-    const size_t need = attn_partial_bytes(batch, n_q_heads, chunks_bound, &o_bytes);
+    const size_t need = attn_partial_bytes(vbatch, n_q_heads, pl.chunks, &o_bytes);
     if (!workspace || workspace_bytes < need)
       SUBSPEC_FAIL(SUBSPEC_ERR_WORKSPACE, "%s: workspace of %zu bytes is smaller than the %zu required", what,
                    workspace_bytes, need);
@@ -1271,17 +1296,16 @@ static int tree_attention_impl(const char* what, const void* q, const void* k_ca
     part_ml = (float*)((char*)workspace + o_bytes);
   }
   hipStream_t st = (hipStream_t)stream;
-  // more than 64 query rows: one launch (pair) per window of 64, in stream order, sharing the partial buffers
-  for (int64_t row0 = 0; row0 < n_rows; row0 += kAttnRows) {
-    ap.row0 = (int)row0;
-    ap.win_rows = (int)std::min<int64_t>(n_rows - row0, kAttnRows);
-    const AttnPlan pl = attn_plan(batch, n_q_heads, n_kv_heads, ap.win_rows, kv_len);
+  {
+    ap.row0 = 0;
+    ap.win_rows = al.win_rows;
+    ap.windows = al.windows;
     ap.chunk_keys = (blocks + pl.chunks - 1) / pl.chunks * kKeyBlock;
     ap.chunks = (int)((kv_len + ap.chunk_keys - 1) / ap.chunk_keys);
-    ap.units = batch * n_kv_heads * ap.chunks;
+    ap.units = vbatch * n_kv_heads * ap.chunks;
     ap.pairs_per_kv = (group + pl.heads_per_wg - 1) / pl.heads_per_wg;
     const dim3 grid((unsigned)((ap.units + kXcds - 1) / kXcds * kXcds * ap.pairs_per_kv));
-    const int64_t merge_rows = batch * n_q_heads * ap.win_rows / 8 >= 1024 ? 8 : 2;   // rows per merge workgroup
+    const int64_t merge_rows = batch * n_q_heads * ap.win_rows / 8 >= 1024 ? 8 : 2;   // rows per merge workgroup (one window only)
     const dim3 merge_grid((unsigned)((ap.win_rows + merge_rows - 1) / merge_rows), (unsigned)(batch * n_q_heads));
 #define SUBSPEC_ATTN_KERNEL(DT, PAGED, ROWT, WPH, THREADS)                                                          \
   hipLaunchKernelGGL((tree_attention_kernel<DT, PAGED, ROWT, WPH, THREADS>), grid, dim3(THREADS), 0, st, (const uint16_t*)q, \
@@ -1306,7 +1330,7 @@ static int tree_attention_impl(const char* what, const void* q, const void* k_ca
     }                                                                                                              \
     if (ap.chunks > 1) {                                                                                           \
       if (pl.mfma32) {                                                                                             \
-        const dim3 mg((unsigned)(batch * n_q_heads * 2), 4);                                                       \
+        const dim3 mg((unsigned)(vbatch * n_q_heads * 2), 4);                                                      \
         if (ap.chunks <= 4) hipLaunchKernelGGL((tree_attention32_merge_kernel<DT, 4>), mg, dim3(256), 0, st, part_o, part_ml, ap, (uint16_t*)out); \
         else if (ap.chunks <= 8) hipLaunchKernelGGL((tree_attention32_merge_kernel<DT, 8>), mg, dim3(256), 0, st, part_o, part_ml, ap, (uint16_t*)out); \
         else hipLaunchKernelGGL((tree_attention32_merge_kernel<DT, 0>), mg, dim3(256), 0, st, part_o, part_ml, ap, (uint16_t*)out); \

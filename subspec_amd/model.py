@@ -239,15 +239,16 @@ class Decoder:
         return state["x"]
 
     def logits(self, x: torch.Tensor) -> torch.Tensor:
-        """Final norm and the language-model head (HuggingFace ``lm_head`` inside the draft forward,
-        specdecodes/models/draft_models/classic_sd.py:10-16).  A draft level (at most 16 rows) streams the 1.09 GB head
-        through the library's own dense kernel (152064 x 3584 bf16, 8 rows: 208 us = 0.66 of 8 TB/s against 225 us for
-        the vendor GEMM); wider inputs keep the vendor GEMM, which wins from about 32 rows up."""
+        """Final norm and the language-model head (HuggingFace ``lm_head`` inside the draft and target forwards,
+        specdecodes/models/draft_models/classic_sd.py:10-16, generators/classic_sd.py:102-109).  Up to 64 rows the
+        1.09 GB head streams through the dense kernels of this package (152064 x 3584 bf16: 170 us at 8 rows, 198 us at 32
+        against 232 / 255 us for the vendor GEMM; 204 us at 64 rows, where the two are level); wider inputs keep the
+        vendor GEMM (128 rows: 236 against 261 us)."""
         h = rms_norm(x, self.norm, self.cfg.rms_norm_eps)
         rows = h.numel() // h.shape[-1]
         V, H = self.lm_head.shape
-        if (h.is_cuda and rows <= 16 and h.dtype in (torch.bfloat16, torch.float16) and V % 16 == 0 and H % 64 == 0
-                and V * H * 2 < (1 << 31) and self.lm_head.is_contiguous()):
+        if (h.is_cuda and rows <= 64 and h.dtype in (torch.bfloat16, torch.float16) and H % 64 == 0
+                and (V % 32 == 0 if rows > 32 else V % 16 == 0 and V * H * 2 < (1 << 31)) and self.lm_head.is_contiguous()):
             return ops.dense_linear(h, self.lm_head)
         return F.linear(h, self.lm_head)
 
