@@ -222,7 +222,7 @@ int subspec_topk_expand(const void* probs, const void* parent_probs, int dtype, 
  *           flashinfer/attention_wrapper.py:116-151,288-316.
  *
  * q          device [batch, n_q_heads, n_rows, head_dim]      bf16 / fp16, head_dim = 128, n_rows <= SUBSPEC_MAX_TREE_NODES
- *            (64 rows per launch; more rows are further launches on the same stream)
+ *            (more than 64 rows: windows of 64 rows in the same launch, which share the keys)
  * k_cache    device [batch, n_kv_heads, kv_seq_stride, head_dim]  (HF static-cache layout); the K/V of
  * v_cache    the tree nodes must already sit in rows prefix_len .. prefix_len + n_tree_slots - 1
  * out        device [batch, n_rows, n_q_heads, head_dim]       (= [batch, n_rows, hidden])

@@ -281,7 +281,7 @@ def tree_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
     """``q`` [B, Hq, n, D], caches [B, Hkv, S, D] (tree K/V already written at rows prefix_len..),
     ``anc_bits`` int64 [n] (shared tree) or [B, n], with a trailing dimension of ceil(slots / 64) words when
     more than 64 tree slots are occupied: bit j = row may attend to tree slot j.  ``n_tree_slots`` (default n) is
-    the number of occupied tree slots (<= 512); n may be as large (64 rows per launch).  Returns [B, n, Hq * D]."""
+    the number of occupied tree slots (<= 512); n may be as large (windows of 64 rows inside one launch).  Returns [B, n, Hq * D]."""
     dev = _require_gpu(q, k_cache, v_cache, anc_bits)
     if q.dim() != 4 or k_cache.dim() != 4 or v_cache.shape != k_cache.shape:
         raise ValueError("expected q [B, Hq, n, D] and k/v caches [B, Hkv, S, D]")
