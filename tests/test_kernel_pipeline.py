@@ -158,6 +158,29 @@ def test_the_attention_kernels_keep_their_requests_in_flight(tmp_path):
         assert not stalled, "a full wait inside the block loop of: " + ", ".join(f"{k} (at {w})" for k, n, w in stalled)
 
 
+def test_the_wide_dense_kernel_waits_only_where_it_says(tmp_path):
+    """dense_wide_kernel copies weights and activations straight into LDS rings with requests the compiler does not know
+    about, and waits for them by hand: the weight wavefronts for all but the newest chunks of their ring, the activation
+    wavefronts likewise.  Any other wait for vector memory inside a K loop (the compiler adds one, for EVERY request, as
+    soon as it sees a request of its own there) would drain the rings once per chunk; accumulators in scratch memory
+    would do worse."""
+    asm = _assembly(os.path.join(build_mod.CSRC, "dense.hip"), tmp_path)
+    _recognised(asm, "dense_wide_kernel")
+    bodies = _kernel_bodies(asm, "dense_wide_kernel")
+    assert len(bodies) >= 12, "the parser found too few kernel variants"            # 3 shapes x SwiGLU or not x 2 dtypes
+    for kernel, lines in bodies.items():
+        assert not any("scratch_" in l for l in lines), f"{kernel} uses scratch memory"
+        # template arguments <DT, WM, MG, NTMAX, SW, SX, NWW, WPER, NXW, XPER, SILU> from the mangled name
+        args = [int(a) for a in re.findall(r"Li(\d+)E", kernel)]
+        assert len(args) >= 10, kernel
+        sw, sx, wper, xper = args[4], args[5], args[7], args[9]
+        expected = {(sw - 2) * wper, (sx - 2) * xper}
+        in_loop = [l for l in lines if "v_mfma" in l or "vmcnt" in l]
+        first, last = next(i for i, l in enumerate(in_loop) if "v_mfma" in l), max(i for i, l in enumerate(in_loop) if "v_mfma" in l)
+        waits = {int(m.group(1)) for l in in_loop[first:last] for m in [re.search(r"vmcnt\((\d+)\)", l)] if m}
+        assert waits and waits <= expected, f"{kernel}: waits {sorted(waits)} between its products, expected {sorted(expected)}"
+
+
 def test_no_hand_written_vector_instruction_sits_next_to_an_mfma():
     """With MFMA results kept in ordinary vector registers (-amdgpu-mfma-vgpr-form=1) the compiler inserts the wait
     states between an MFMA and the vector ALU instruction that reads its result, but only for instructions it emitted
