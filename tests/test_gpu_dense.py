@@ -20,7 +20,8 @@ CFG = DecoderConfig(num_hidden_layers=3, hidden_size=256, num_attention_heads=2,
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("N,K", [(16, 64), (256, 256), (4608, 3584), (3584, 18944), (37888, 3584), (1040, 448)])
+@pytest.mark.parametrize("N,K", [(16, 64), (256, 256), (4608, 3584), (3584, 18944), (37888, 3584), (1040, 448),
+                                 (32, 64), (96, 128), (1056, 448)])
 def test_dense_linear_matches_float64_product(dtype, N, K):
     g = torch.Generator().manual_seed(N + K)
     w = (torch.randn(N, K, generator=g) * 0.05).to(dtype)
