@@ -286,8 +286,11 @@ int int4_qkv_rope_ex(const void* x, const uint32_t* wq, const uint32_t* sz, cons
                      const KvRowMap& kv, int64_t n_q_heads, float rope_theta, const float* inv_freq, void* stream);
 int dense_gate_up_silu_ex(const void* x, const void* w, const void* bias, void* act, int dtype, int64_t M, int64_t N,
                           int64_t K, void* stream);
+// pending_splits != NULL: when K is split over workgroups the launch that sums the fp32 partials
+// (workspace: [splits][M][N]) is left to the caller's next kernel, *pending_splits = number of partials (then neither bias
+// nor residual has been applied and y is untouched); 1: y is complete
 int dense_linear_ex(const void* x, const void* w, const void* bias, const void* residual, void* y, int dtype, int64_t M,
-                    int64_t N, int64_t K, void* workspace, size_t workspace_bytes, void* stream);
+                    int64_t N, int64_t K, void* workspace, size_t workspace_bytes, void* stream, int* pending_splits = nullptr);
 
 
 }  // namespace subspec

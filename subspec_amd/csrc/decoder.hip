@@ -28,12 +28,16 @@ namespace subspec {
 
 // x[m] (+= delta[m], rounded, written back) ; y[m] = w * round(x * rsqrt(mean(x^2) + eps))
 // One workgroup per row; H % 8 == 0.  kMaxPieces 16-byte pieces per thread cover H <= 256 * 8 * kMaxPieces.
+// splits > 0: delta is not a 16-bit tensor yet but `splits` fp32 partial sums [splits][rows][H] of a projection whose K
+// was split over workgroups; they are summed in split order and rounded here (what the projection's own reduction
+// launch would have stored), which saves that launch.
 constexpr int kNormThreads = 256;
 constexpr int kNormMaxPieces = 8;
 template <int DT, bool kAdd>
 __global__ __launch_bounds__(kNormThreads) void add_rmsnorm_kernel(uint16_t* __restrict__ x, const uint16_t* __restrict__ delta,
                                                                    const uint16_t* __restrict__ w, uint16_t* __restrict__ y,
-                                                                   int H, float eps) {
+                                                                   int H, float eps, const float* __restrict__ partial = nullptr,
+                                                                   int splits = 0) {
   __shared__ float scratch[kNormThreads / kWave];
   const int m = blockIdx.x, tid = threadIdx.x, pieces = H / 8;
   dec_u4* xr = (dec_u4*)(x + (int64_t)m * H);
@@ -47,7 +51,19 @@ __global__ __launch_bounds__(kNormThreads) void add_rmsnorm_kernel(uint16_t* __r
       unpack8<DT>(xr[i], v[p]);
       if constexpr (kAdd) {
         float d[8];
-        unpack8<DT>(dr[i], d);
+        if (splits > 0) {
+#pragma unroll
+          for (int j = 0; j < 8; ++j) d[j] = 0.f;
+          for (int sp = 0; sp < splits; ++sp) {
+            const float4* pp = (const float4*)(partial + ((int64_t)sp * gridDim.x + m) * H) + 2 * i;
+            const float4 a = pp[0], b = pp[1];
+            d[0] += a.x; d[1] += a.y; d[2] += a.z; d[3] += a.w; d[4] += b.x; d[5] += b.y; d[6] += b.z; d[7] += b.w;
+          }
+#pragma unroll
+          for (int j = 0; j < 8; ++j) d[j] = Elem<DT>::round(d[j]);
+        } else {
+          unpack8<DT>(dr[i], d);
+        }
 #pragma unroll
         for (int j = 0; j < 8; ++j) v[p][j] = Elem<DT>::round(v[p][j] + d[j]);
         xr[i] = pack8<DT>(v[p]);
@@ -91,16 +107,35 @@ __global__ __launch_bounds__(256) void silu_mul_kernel(const uint16_t* __restric
 // Rotary embedding (rotate-half form, angle = position * theta^(-2i/D)) of the q and k heads of
 // qkv [M, (Hq + 2 Hkv) * D]; q goes to q_out [Hq, M, D], k and v to rows cache_rows[m] of the
 // layer's [Hkv, S, D] caches.  One wavefront per (row, head); lane i handles dims i and i + D/2.
+// splits > 0: qkv is still `splits` fp32 partial sums [splits][M][(Hq + 2 Hkv) * D] of the projection (K split over
+// workgroups) and `bias` its bias; sum, bias and the rounding to the activation dtype happen here instead of in a
+// reduction launch of their own.
 template <int DT>
 __global__ __launch_bounds__(64) void rope_write_kernel(const uint16_t* __restrict__ qkv, const int32_t* __restrict__ positions,
                                                         const int32_t* __restrict__ cache_rows, uint16_t* __restrict__ q_out,
                                                         KvRowMap kv, int M, int Hq, int Hkv, int D, float log2_theta,
-                                                        const float* __restrict__ inv_freq_table) {
+                                                        const float* __restrict__ inv_freq_table,
+                                                        const float* __restrict__ partial = nullptr, int splits = 0,
+                                                        const uint16_t* __restrict__ bias = nullptr) {
   const int m = blockIdx.x, hh = blockIdx.y, i = threadIdx.x;
   const int half = D / 2;
   if (i >= half) return;
-  const uint16_t* src = qkv + ((int64_t)m * (Hq + 2 * Hkv) + hh) * D;
-  const float lo = Elem<DT>::load(src, i), hi = Elem<DT>::load(src, i + half);
+  float lo, hi;
+  if (splits > 0) {
+    const int64_t width = (int64_t)(Hq + 2 * Hkv) * D, col = (int64_t)hh * D + i;
+    lo = hi = 0.f;
+    for (int sp = 0; sp < splits; ++sp) {
+      const float* pp = partial + ((int64_t)sp * M + m) * width + col;
+      lo += pp[0];
+      hi += pp[half];
+    }
+    lo = Elem<DT>::round(lo + (bias ? Elem<DT>::load(bias, col) : 0.f));
+    hi = Elem<DT>::round(hi + (bias ? Elem<DT>::load(bias, col + half) : 0.f));
+  } else {
+    const uint16_t* src = qkv + ((int64_t)m * (Hq + 2 * Hkv) + hh) * D;
+    lo = Elem<DT>::load(src, i);
+    hi = Elem<DT>::load(src, i + half);
+  }
   uint16_t* dst;
   if (hh < Hq) {
     dst = q_out + ((int64_t)hh * M + m) * D;
@@ -203,8 +238,10 @@ struct LayerWeights {
   bool dense;
 };
 static int project(const LayerWeights& w, const Projection& p, const void* x, const void* bias, const void* residual, void* y,
-                   int dtype, int64_t M, int64_t N, int64_t K, void* sub, size_t sub_bytes, hipStream_t st) {
-  if (w.dense) return dense_linear_ex(x, p.w, bias, residual, y, dtype, M, N, K, sub, sub_bytes, st);
+                   int dtype, int64_t M, int64_t N, int64_t K, void* sub, size_t sub_bytes, hipStream_t st,
+                   int* pending_splits = nullptr) {
+  if (pending_splits) *pending_splits = 1;
+  if (w.dense) return dense_linear_ex(x, p.w, bias, residual, y, dtype, M, N, K, sub, sub_bytes, st, pending_splits);
   return int4_linear_ex(x, (const uint32_t*)p.w, (const uint32_t*)p.sz, bias, residual, y, dtype, M, N, K, 64, sub, sub_bytes, st);
 }
 
@@ -234,9 +271,12 @@ static int run_layer(const subspec_decoder_layer_dims& s, const LayerWeights& w,
   } else {
     hipLaunchKernelGGL((add_rmsnorm_kernel<DT, false>), dim3(M), dim3(kNormThreads), 0, st, x, (const uint16_t*)nullptr,
                        (const uint16_t*)w.input_norm, h, H, s.rms_eps);
-    if ((rc = project(w, w.qkv, h, w.qkv_bias, nullptr, qkv, DT, M, Q + 2 * KV, H, sub, p.sub_bytes, st))) return rc;
+    // dense projections whose K is split leave the sum of their partials to the kernel that reads them next
+    int pending = 0;
+    if ((rc = project(w, w.qkv, h, w.qkv_bias, nullptr, qkv, DT, M, Q + 2 * KV, H, sub, p.sub_bytes, st, &pending))) return rc;
     hipLaunchKernelGGL((rope_write_kernel<DT>), dim3(M, Hq + 2 * Hkv), dim3(64), 0, st, qkv, positions, cache_rows, q, kv,
-                       M, Hq, Hkv, D, log2f(s.rope_theta), s.rope_inv_freq);
+                       M, Hq, Hkv, D, log2f(s.rope_theta), s.rope_inv_freq, (const float*)sub, pending > 1 ? pending : 0,
+                       (const uint16_t*)w.qkv_bias);
   }
   if ((rc = tree_attention_ex(q, k_cache, v_cache, a, DT, Hq, Hkv, M, s.n_tree_slots, s.kv_seq_stride, s.prefix_len,
                               s.prefix_len_dev, pg, anc_bits, 1.f / sqrtf((float)D), sub, p.sub_bytes, st)))
@@ -248,9 +288,10 @@ static int run_layer(const subspec_decoder_layer_dims& s, const LayerWeights& w,
                                    2 * (int64_t)F, H, w.post_norm, s.rms_eps, st)))
       return rc;
   } else {
-  if ((rc = project(w, w.o, a, nullptr, nullptr, o, DT, M, H, Q, sub, p.sub_bytes, st))) return rc;
+  int pending = 0;
+  if ((rc = project(w, w.o, a, nullptr, nullptr, o, DT, M, H, Q, sub, p.sub_bytes, st, &pending))) return rc;
   hipLaunchKernelGGL((add_rmsnorm_kernel<DT, true>), dim3(M), dim3(kNormThreads), 0, st, x, o, (const uint16_t*)w.post_norm, h, H,
-                     s.rms_eps);
+                     s.rms_eps, (const float*)sub, pending > 1 ? pending : 0);
   if (!w.dense) {
     // the activation sits in the output stage of the gate|up projection
     if ((rc = int4_gate_up_silu_ex(h, (const uint32_t*)w.gate_up.w, (const uint32_t*)w.gate_up.sz, nullptr, act, DT, M,

@@ -640,7 +640,8 @@ static int run_dense_silu(const void* x, const void* w, const void* bias, void* 
 
 template <int DT>
 static int run_dense(const void* x, const void* w, const void* bias, const void* residual, void* y, int64_t M, int64_t N,
-                     int64_t K, void* workspace, hipStream_t st) {
+                     int64_t K, void* workspace, hipStream_t st, int* pending_splits) {
+  if (pending_splits) *pending_splits = 1;
   if (wide_applies(M, N)) {
     const WidePlan pl = wide_plan(N, K, false);
     const WideParams p{(const uint16_t*)x, (const uint16_t*)w, (const uint16_t*)bias, (const uint16_t*)residual, (uint16_t*)y,
@@ -649,7 +650,8 @@ static int run_dense(const void* x, const void* w, const void* bias, const void*
       DominantKernelTimer timer(st);
       launch_wide<DT, false>(p, pl, st);
     }
-    if (pl.splits > 1)
+    if (pl.splits > 1 && pending_splits) *pending_splits = pl.splits;
+    else if (pl.splits > 1)
       hipLaunchKernelGGL((dense_reduce_kernel<DT>), dim3((unsigned)((M * N + 255) / 256)), dim3(256), 0, st, (const float*)workspace,
                          (const uint16_t*)bias, (const uint16_t*)residual, (uint16_t*)y, M, N, pl.splits);
     SUBSPEC_CHECK_HIP(hipGetLastError());
@@ -676,7 +678,8 @@ static int run_dense(const void* x, const void* w, const void* bias, const void*
   }
 #undef SUBSPEC_DN_LAUNCH_MT
 #undef SUBSPEC_DN_LAUNCH
-  if (pl.splits > 1)
+  if (pl.splits > 1 && pending_splits) *pending_splits = pl.splits;
+  else if (pl.splits > 1)
     hipLaunchKernelGGL((dense_reduce_kernel<DT>), dim3((unsigned)((M * N + 255) / 256)), dim3(256), 0, st, partial,
                        (const uint16_t*)bias, (const uint16_t*)residual, (uint16_t*)y, M, N, pl.splits);
   SUBSPEC_CHECK_HIP(hipGetLastError());
@@ -726,7 +729,7 @@ extern "C" int subspec_dense_gate_up_silu(const void* x, const void* w, const vo
 }
 
 int subspec::dense_linear_ex(const void* x, const void* w, const void* bias, const void* residual, void* y, int dtype, int64_t M,
-                             int64_t N, int64_t K, void* workspace, size_t workspace_bytes, void* stream) {
+                             int64_t N, int64_t K, void* workspace, size_t workspace_bytes, void* stream, int* pending_splits) {
   if (dtype != SUBSPEC_BF16 && dtype != SUBSPEC_F16)
     SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "dense_linear: dtype %d not supported (bf16 / fp16 only)", dtype);
   if (!x || !w || !y) SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "dense_linear: null pointer argument");
@@ -747,6 +750,6 @@ int subspec::dense_linear_ex(const void* x, const void* w, const void* bias, con
     if ((uintptr_t)workspace % 16) SUBSPEC_FAIL(SUBSPEC_ERR_ARG, "dense_linear: workspace must be 16-byte aligned");
   }
   hipStream_t st = (hipStream_t)stream;
-  if (dtype == SUBSPEC_BF16) return run_dense<SUBSPEC_BF16>(x, w, bias, residual, y, M, N, K, workspace, st);
-  return run_dense<SUBSPEC_F16>(x, w, bias, residual, y, M, N, K, workspace, st);
+  if (dtype == SUBSPEC_BF16) return run_dense<SUBSPEC_BF16>(x, w, bias, residual, y, M, N, K, workspace, st, pending_splits);
+  return run_dense<SUBSPEC_F16>(x, w, bias, residual, y, M, N, K, workspace, st, pending_splits);
 }
