@@ -45,6 +45,36 @@ def test_dense_linear_matches_float64_product(dtype, N, K):
     assert torch.equal(ops.dense_linear(x, wd, None), ops.dense_linear(x, wd, None))
 
 
+def test_dense_linear_ragged_shapes_above_32_rows():
+    """Row counts that leave row tiles partly empty, weight-tile counts that do not divide by the tiles of a workgroup,
+    K of one to many chunks, with and without K ranges; bias and the SwiGLU pair kernel on the same shapes."""
+    g = torch.Generator().manual_seed(77)
+    for case in range(24):
+        M = int(torch.randint(33, 385, (1,), generator=g))
+        N = 32 * int(torch.randint(1, 80, (1,), generator=g))
+        K = 64 * int(torch.randint(1, 40, (1,), generator=g))
+        dtype = torch.bfloat16 if case % 3 else torch.float16
+        print("dense_linear ragged", dtype, M, N, K, flush=True)
+        w = (torch.randn(N, K, generator=g) * (1.0 / K ** 0.5)).to(dtype)
+        x = torch.randn(M, K, generator=g).to(dtype)
+        b = (torch.randn(N, generator=g) * 0.1).to(dtype)
+        got = ops.dense_linear(x.to(DEV), w.to(DEV), b.to(DEV)).cpu()
+        ref = x.double() @ w.double().T + b.double()
+        rel = 2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -10
+        assert ((got.double() - ref).abs() <= rel * ref.abs() + 1e-3 * ref.abs().amax().item()).all(), (M, N, K)
+        assert (got == ref.to(dtype)).float().mean().item() >= 0.97, (M, N, K)
+        if N % 64 == 0:
+            F_ = N // 2
+            act = ops.dense_gate_up_silu(x.to(DEV), w.to(DEV), b.to(DEV)).cpu()
+            gate, up = got[:, :F_].float(), got[:, F_:].float()
+            want = ((gate / (1 + torch.exp(-gate))).to(dtype).float() * up).to(dtype)
+            # (the plain projection may have split K where the pair kernel does not: gate and up then differ in their
+            # last place here and there)
+            assert int((act != want).sum()) <= max(1, act.numel() // 100), (M, N, K)
+            ulp = 2.0 ** (-7 if dtype == torch.bfloat16 else -10)
+            assert ((act.float() - want.float()).abs() <= 4 * ulp * want.float().abs() + 1e-3 * want.float().abs().amax()).all(), (M, N, K)
+
+
 def test_dense_linear_at_the_size_of_the_vocabulary_head():
     """152064 x 3584 (the draft's lm_head): 9504 tiles, two per workgroup; fp32 reference (its error is far below the
     bf16 rounding of the outputs)."""
