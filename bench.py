@@ -84,7 +84,7 @@ def parse():
     ap.add_argument("--keep-layers", type=int, default=14, help="e2e workload: target layers kept resident; the rest stream")
     ap.add_argument("--ring-slabs", type=int, default=4,
                     help="e2e workload: device slabs of the streaming ring (layers the copies may run ahead of compute)")
-    ap.add_argument("--workload", default="verify-cycle", choices=["verify-cycle", "attention", "int4", "dense", "greedy", "sampling", "topk", "e2e"],
+    ap.add_argument("--workload", default="verify-cycle", choices=["verify-cycle", "attention", "int4", "dense", "greedy", "sampling", "topk", "e2e", "tree-forward"],
                     help="verify-cycle (default, BASELINE config 2) is the benchmark line; the others time one "
                          "kernel family of configs 1, 3 and 4 and print one JSON line per shape")
     return ap.parse_args()
@@ -329,6 +329,42 @@ def e2e_runs(args, runs, new_tokens, say=lambda *_: None):
     return lines
 
 
+def bench_tree_forward(args):
+    """One target forward over the rows of a whole draft tree, all 28 layers resident, prefix 2048: 64 rows (the default
+    verification window), 128, and the 289 rows of the reference's depth-48, k-6 tree
+    (configs/exp_offloading/subspec_sd_qwen_7b.yaml:16-19) -- through the one-call dense layers, and module by module on
+    library GEMMs with the same attention kernel."""
+    import torch
+    from subspec_amd import ops, workloads as W
+    from subspec_amd.cache import create_kv_cache
+    from subspec_amd.model import DecoderConfig, build_models
+    dev = "cuda:0"
+    cfg = DecoderConfig()
+    kv = create_kv_cache("static", max_cache_len=2048 + 400, config=cfg, device=dev, dtype=torch.bfloat16)
+    target, _, _ = build_models(cfg, kv, seed=0, device=dev, first_streamed=cfg.num_hidden_layers)
+    g = torch.Generator().manual_seed(0)
+    target.prefill(torch.randint(0, cfg.vocab_size, (2048,), generator=g).to(dev), 0)
+    weight_bytes = sum(t.numel() * 2 for w in target.layers for n_, t in w.items() if n_.endswith("_proj.weight"))
+    for n in (64, 128, 289):
+        parents, _, depths = W.random_tree(g, n=n, max_depth=48, max_children=6, vocab=cfg.vocab_size, chain_depth=8)
+        toks = torch.randint(0, cfg.vocab_size, (n,), generator=g).to(dev)
+        anc = ops.ancestor_bits_tensor(parents, device=dev)
+        d = torch.tensor(depths, device=dev)
+        times = {}
+        for native in (True, False):
+            target.use_native_layers = native
+            times[native], _ = _time_us(lambda: target.tree_forward(toks, d, anc, 2048), max(5, args.steps // 2), 2)
+        target.use_native_layers = True
+        flops = 2 * n * weight_bytes // 2
+        print(json.dumps({"metric": "target forward over the rows of a draft tree", "value": round(times[True] / 1e3, 3), "unit": "ms",
+                          "n_gpus": 1, "higher_is_better": False, "data": "synthetic", "dtype": "bf16",
+                          "config": {"workload": f"Qwen2.5-7B shape, 28 resident layers, prefix 2048, {n} tree rows, one-call dense layers",
+                                     "rows": n, "module_by_module_library_gemm_ms": round(times[False] / 1e3, 3),
+                                     "layer_weight_GB": round(weight_bytes / 1e9, 2),
+                                     "weights_over_time_TB_per_s": round(weight_bytes / (times[True] * 1e-6) / 1e12, 2),
+                                     "projection_TFLOP_per_s": round(flops / (times[True] * 1e-6) / 1e12, 1)}}), flush=True)
+
+
 def bench_e2e(args):
     for line in e2e_runs(args, [(args.keep_layers, args.agreeing_draft)], args.new_tokens,
                          say=lambda m: print(m, file=sys.stderr, flush=True)):
@@ -493,7 +529,7 @@ def main():
     L.lib()                                            # fail loudly when the HIP library is missing
     if args.workload != "verify-cycle":
         {"attention": bench_attention, "int4": bench_int4, "dense": bench_dense, "greedy": bench_greedy, "sampling": bench_sampling, "topk": bench_topk,
-         "e2e": bench_e2e}[args.workload](args)
+         "e2e": bench_e2e, "tree-forward": bench_tree_forward}[args.workload](args)
         return
     dev = torch.device("cuda:0")
     B, V, n, k = args.batch, args.vocab, 64, 16
