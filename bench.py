@@ -277,6 +277,7 @@ def e2e_runs(args, runs, new_tokens, say=lambda *_: None):
                                         n_slabs=getattr(args, "ring_slabs", 4))
         say(f"# models built in {time.perf_counter() - t0:.1f} s (resident target layers: {keep_layers}, agreeing draft: {agreeing})")
         prompt = torch.randint(0, cfg.vocab_size, (1, 2048), generator=torch.Generator().manual_seed(0)).to(dev)
+        warm = False
         for method, vk in (("exact", None), ("lossy", dict(threshold=0.3, window_size=6, threshold_method="entropy"))):
             v2 = args.generator == "v2"
             depth = args.tree_depth or (7 if v2 else 8)
@@ -289,6 +290,14 @@ def e2e_runs(args, runs, new_tokens, say=lambda *_: None):
                 DraftParams(temperature=0.2, max_depth=depth, topk_len=tree_k, max_verify_tokens=cap),
                 generator_kwargs=dict(verify_method=method, verify_kwargs=vk, draft_graph=bool(getattr(args, "draft_graph", False)),
                                       **(dict(postspec_steps=args.postspec_steps) if v2 else {})))
+            if not warm:
+                # one untimed prefill (a generation of one token): the first pass through the GEMM library in a new
+                # process selects and loads its kernels (290 ms against 42 ms for every later prefill of this prompt),
+                # which is no property of the cycle
+                kv.reset()
+                gen.generate(prompt, max_new_tokens=1, do_sample=False, past_key_values=kv)
+                torch.cuda.synchronize()
+                warm = True
             kv.reset()
             wandb_logger.clear_log_data()
             if target.streamer is not None:
