@@ -187,7 +187,8 @@ class SubSpecSDGenerator:
                     threshold=float(vk.get("threshold", 0.0)), window_size=int(vk.get("window_size", 1)),
                     threshold_method=str(vk.get("threshold_method", "prob") or "prob").strip().lower())
             input_ids = torch.cat([input_ids, sampled], dim=-1)
-            finished, input_ids, kept, prune_tokens = self._hit_stop(input_ids, sampled, max_length)
+            finished, input_ids, kept, prune_tokens = self._hit_stop(input_ids, sampled, max_length,
+                                                                     host_tokens=host[4:4 + emitted].tolist())
             if stream_callback is not None and kept.numel() > 0:
                 stream_callback(kept)
             past_key_values.seq_len += emitted
@@ -212,11 +213,12 @@ class SubSpecSDGenerator:
                 log[f"avg_{name}_time"] = (sum(a.elapsed_time(b) for a, b in pairs) / len(pairs) / 1e3) if pairs else 0.0
         return input_ids
 
-    def _hit_stop(self, input_ids, sampled_tokens, max_length: int):
+    def _hit_stop(self, input_ids, sampled_tokens, max_length: int, host_tokens=None):
         """Token-by-token stop check over the new block (generators/base.py:265-299): returns
-        (finished, input_ids cut after the stop, kept tokens, number of pruned tokens)."""
+        (finished, input_ids cut after the stop, kept tokens, number of pruned tokens).  ``host_tokens``: the same
+        tokens as a host-side list, when the caller has them (saves a device synchronisation per cycle)."""
         base = input_ids.shape[1] - sampled_tokens.shape[1]
-        toks = sampled_tokens[0].tolist()
+        toks = sampled_tokens[0].tolist() if host_tokens is None else list(host_tokens)
         for j, t in enumerate(toks):
             cur_len = base + j + 1
             stop = (max_length is not None and cur_len >= max_length) or \

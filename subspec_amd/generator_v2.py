@@ -192,7 +192,7 @@ class SubSpecSDGeneratorV2(SubSpecSDGenerator):
 
             sampled = tokens.view(1, -1).to(dev)
             input_ids = torch.cat([input_ids, sampled], dim=-1)
-            finished, input_ids, kept, prune_tokens = self._hit_stop(input_ids, sampled, max_length)
+            finished, input_ids, kept, prune_tokens = self._hit_stop(input_ids, sampled, max_length, host_tokens=tokens.tolist())
             if stream_callback is not None and kept.numel() > 0:
                 stream_callback(kept)
             if not is_prev_accepted or finished:
