@@ -24,6 +24,8 @@
 // M = 1-8, K > 2048: int4_rows8_kernel, the same MFMA arithmetic with nothing pipelined: every request of a
 //           wavefront is issued before its first wait.  This is the shape of a draft level (8 rows, one workgroup per
 //           compute unit), where a pipeline of a few groups is bound by round trips, not by bytes.
+//           A K of more than 56 groups over at least 128 tiles (the down projection): int4_rows8_long_kernel, one
+//           workgroup per tile over the whole of K, in rounds whose registers refill while they are used.
 // M = 2-64: int4_gemm_kernel, v_mfma_f32_16x16x32 with the activations as A and the weight tile as
 //           B operand; the 32 k of one MFMA step all come from one quantization group, so the raw
 //           accumulator of a group is scaled once.  The wavefronts of a workgroup split K, their
@@ -795,6 +797,125 @@ __global__ __launch_bounds__(kR8Threads) void int4_rows8_kernel(
   }
 }
 
+// ------------------------------------------------------------------ 1 <= M <= 8, a long K over at least 128 tiles
+// The down projection of a draft level (3584 x 18944: 296 groups) does not fit the K range of the kernel above, and
+// splitting K over workgroups costs fp32 partials and a second launch that is all latency (11.6 + 3.9 us).  Here one
+// workgroup owns one tile and ALL of K: wavefront w takes groups w, w + 8, ... in rounds of NG.  A round is the step
+// sequence of the kernel above against registers; what it adds is that the registers refill while they are used: the
+// activation blocks and (scale, zero) words of round r + 1 are requested when round r starts, and a step's weight
+// register is requested again for round r + 1 as soon as the step has taken its words, so NG weight requests per
+// wavefront stay in flight from the first round to the last.  3584 x 18944, 8 rows, weights from HBM: 14.5 us against
+// 12.3 + 3.8 us for the split form -- a launch, one round trip and 38 MB at 4.5 TB/s; a second set of weight registers
+// in flight two rounds ahead (15.8 us) and sixteen wavefronts of five groups per round (14.3 us) do not change that.  The eight partial tiles meet in LDS once, at the end, and
+// the output stage (bias, residual) runs in the same launch.
+template <int DT, int NW, int NG>
+__global__ __launch_bounds__(NW * 64) void int4_rows8_long_kernel(
+    const uint16_t* __restrict__ x, const uint2* __restrict__ wq, const uint32_t* __restrict__ sz,
+    const uint16_t* __restrict__ bias, const uint16_t* residual, uint16_t* y, int M, int64_t N, int K) {
+  asm volatile("" ::"s"(x), "s"(wq), "s"(sz), "s"(bias), "s"(residual), "s"(y), "s"(M), "s"(N), "s"(K));
+  static_assert(NW >= 8, "wavefront m finishes row m");
+  static_assert(NG <= 8, "two (scale, zero) requests per round cover eight steps");
+  constexpr int kStageBytes = NW * NG * 1024 + NW * 16;          // stages, one block of zeros per wavefront
+  constexpr int kRedBytes = NW * 32 * 16;                        // rows 0..7 of every wavefront's accumulators
+  __shared__ __attribute__((aligned(16))) unsigned char lds_raw[kStageBytes > kRedBytes ? kStageBytes : kRedBytes];
+  float* const red = (float*)lds_raw;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int ln = lane & 15, c = lane >> 4;
+  const int G = K / kGroup;
+  const int n_tiles = (int)(N / 16);
+  const int tile = blockIdx.x;
+  const int n_mine = wave < G ? (G - wave + NW - 1) / NW : 0;    // groups wave, wave + NW, ... of this wavefront
+  const int rounds = (n_mine + NG - 1) / NG;
+
+  const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)x, 0, M * K * 2, 0x00027000);
+  const __amdgpu_buffer_rsrc_t w_rsrc =
+      __builtin_amdgcn_make_buffer_rsrc((void*)wq, 0, (int)(n_tiles * (int64_t)G * 512), 0x00027000);
+  const __amdgpu_buffer_rsrc_t sz_rsrc =
+      __builtin_amdgcn_make_buffer_rsrc((void*)sz, 0, (int)(n_tiles * (int64_t)G * 64), 0x00027000);
+  const int prow = lane >> 3, ppiece = lane & 7;                 // the lane's row and 16-byte piece of an activation block
+  const int xg_off = (prow * K + ppiece * 8) * 2;                // rows past M read zeros (outside the descriptor)
+  const int wofs = tile * G;
+  const uint32_t kmask = 0x000f000fu | (uint32_t)(M >> 30), kmagic = I4<DT>::kMagic | ((uint32_t)xg_off >> 31);
+  const uint32_t one2 = DT == SUBSPEC_BF16 ? 0x3f803f80u : 0x3c003c00u;
+  const i4_u4 ones = i4_u4{one2, one2, one2, one2};
+  unsigned char* const stages = lds_raw + wave * (NG * 1024);
+  unsigned char* const zeros = lds_raw + NW * NG * 1024 + wave * 16;
+  // group of step J in round r; requests past the wavefront's last group repeat group G - 1 and are multiplied by zero
+  auto group_of = [&](int r, int J) { return min(wave + NW * (r * NG + J), G - 1); };
+
+  // ---- round 0: every request, activations first
+  i4_u4 xall[NG];
+#pragma unroll
+  for (int J = 0; J < NG; ++J) xall[J] = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, xg_off, group_of(0, J) * (kGroup * 2), 0);
+  __builtin_amdgcn_sched_barrier(0);
+  uint32_t szq[2];
+#pragma unroll
+  for (int h = 0; h < 2; ++h)
+    szq[h] = __builtin_amdgcn_raw_buffer_load_b32(sz_rsrc, ln * 4 + (wofs + group_of(0, min(4 * h + c, NG - 1))) * 64, 0, kStream);
+  i4_u2 wall[NG];
+#pragma unroll
+  for (int J = 0; J < NG; ++J) wall[J] = __builtin_amdgcn_raw_buffer_load_b64(w_rsrc, lane * 8, (wofs + group_of(0, J)) * 512, kStream);
+  __builtin_amdgcn_sched_barrier(0);
+  if (lane == 0) *(i4_u4*)zeros = i4_u4{0u, 0u, 0u, 0u};
+
+  i4_v4f acc = i4_v4f{0.f, 0.f, 0.f, 0.f};
+  const int rd0 = ln * 128 + (((2 * c) ^ ln) << 4), rd1 = ln * 128 + (((2 * c + 1) ^ ln) << 4);
+  for (int r = 0; r < rounds; ++r) {
+    // park this round's activation blocks (the wavefront's own stages: its reads of the last round are behind it)
+#pragma unroll
+    for (int J = 0; J < NG; ++J) *(i4_u4*)(stages + J * 1024 + prow * 128 + ((ppiece ^ prow) << 4)) = xall[J];
+    // the next round's activations and (scale, zero) words, ahead of the weight requests the steps below issue
+#pragma unroll
+    for (int J = 0; J < NG; ++J) xall[J] = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, xg_off, group_of(r + 1, J) * (kGroup * 2), 0);
+    uint32_t sz_next[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+      sz_next[h] = __builtin_amdgcn_raw_buffer_load_b32(sz_rsrc, ln * 4 + (wofs + group_of(r + 1, min(4 * h + c, NG - 1))) * 64, 0, kStream);
+    __builtin_amdgcn_sched_barrier(0);
+    const int live = n_mine - r * NG;                            // steps of this round with a group of their own
+#pragma unroll
+    for (int J = 0; J < NG; ++J) {
+      const i4_u4 xa0 = *(const i4_u4*)(ln < 8 ? stages + J * 1024 + rd0 : zeros);
+      const i4_u4 xa1 = *(const i4_u4*)(ln < 8 ? stages + J * 1024 + rd1 : zeros);
+      i4_v4f xs = i4_mfma32<DT>(xa0, ones, i4_v4f{0.f, 0.f, 0.f, 0.f});   // the group's activation sums, rows 4c + rr
+      xs = i4_mfma32<DT>(xa1, ones, xs);
+      const uint32_t w0 = wall[J].x, w1 = wall[J].y;
+      const i4_u4 b0 = i4_u4{code_pair(w0, 0, kmagic, kmask), code_pair(w0, 4, kmagic, kmask),
+                             code_pair(w0, 8, kmagic, kmask), code_pair(w0, 12, kmagic, kmask)};
+      const i4_u4 b1 = i4_u4{code_pair(w1, 0, kmagic, kmask), code_pair(w1, 4, kmagic, kmask),
+                             code_pair(w1, 8, kmagic, kmask), code_pair(w1, 12, kmagic, kmask)};
+      // the words are spent: the request for the next round goes into the SAME registers (issued while the old words
+      // were still wanted it would get others, and the copy back at the end of the round would wait for every request)
+      __builtin_amdgcn_sched_barrier(0);
+      wall[J] = __builtin_amdgcn_raw_buffer_load_b64(w_rsrc, lane * 8, (wofs + group_of(r + 1, J)) * 512, kStream);
+      __builtin_amdgcn_sched_barrier(0);
+      const uint32_t szw = (uint32_t)__shfl((int)szq[J >> 2], (J & 3) * 16 + ln, kWave);
+      const float sc = J < live ? f16_bits_to_float(szw & 0xffffu) : 0.f;
+      const float szo = -sc * (f16_bits_to_float(szw >> 16) + I4<DT>::kOffset);
+      i4_v4f raw = i4_mfma32<DT>(xa0, b0, i4_v4f{0.f, 0.f, 0.f, 0.f});
+      raw = i4_mfma32<DT>(xa1, b1, raw);
+#pragma unroll
+      for (int rr = 0; rr < 4; ++rr) acc[rr] = fmaf(sc, raw[rr], fmaf(szo, xs[rr], acc[rr]));
+    }
+    szq[0] = sz_next[0];
+    szq[1] = sz_next[1];
+  }
+
+  // ---- output stage: rows 0..7 of every wavefront's accumulators meet in LDS; wavefront m finishes row m
+  __syncthreads();                                               // every wavefront is done with its stages
+  if (lane < 32) *(i4_v4f*)(&red[(wave * 32 + lane) * 4]) = acc;
+  __syncthreads();
+  const int m = wave;
+  if (m >= M || c != 0) return;
+  float v = 0.f;
+#pragma unroll
+  for (int w = 0; w < NW; ++w) v += red[(w * 32 + (m >> 2) * 16 + ln) * 4 + (m & 3)];
+  const int64_t n0 = (int64_t)tile * 16 + ln;
+  if (bias) v += I4<DT>::to_float(bias[n0]);
+  store_linear_out<DT>(y, (int64_t)m * N + n0, v, residual);
+}
+
 template <int DT>
 __global__ __launch_bounds__(256) void int4_reduce_kernel(const float* __restrict__ partial,
                                                           const uint16_t* __restrict__ bias, const uint16_t* residual,
@@ -826,9 +947,13 @@ constexpr int kI4MaxRowTiles = 5;
 static int i4_row_tile_variant(int64_t need) { return need <= 1 ? 1 : need <= 2 ? 2 : need <= 3 ? 3 : kI4MaxRowTiles; }
 // Resident workgroups the launch is balanced for (register use allows 2 per SIMD row for M > 32).
 static int i4_slots(int64_t M) { return M > 32 ? 512 : 1024; }
+// One workgroup per tile over the whole of K (int4_rows8_long_kernel) instead of K ranges over workgroups: a K that
+// needs more than one range, and tiles enough to occupy half the chip.
+static bool i4_rows8_long(int64_t M, int64_t N, int G) { return M <= 8 && G > kR8Range && N / 16 >= 128; }
 static I4Plan i4_plan(int64_t M, int64_t N, int64_t K) {
   const int G = (int)(K / kGroup);
   const int64_t tiles = N / 16, slots = i4_slots(M);
+  if (i4_rows8_long(M, N, G)) return I4Plan{(int)tiles, 1, 1, G};
   if (i4_rows8_plain(M, G)) {
     // The 8-row kernel: K ranges of at most 56 groups, and as many tiles per workgroup (1, 2, 3 in one round; 4, 6, 8, 10
     // in rounds of two) as brings the launch down to one workgroup per compute unit.  (Qwen2.5-7B shapes inside the resident
@@ -950,6 +1075,10 @@ static int run_int4(const void* x, const uint32_t* wq, const uint32_t* sz, const
   } while (0)
     {
       DominantKernelTimer timer(st);
+      if (i4_rows8_long(M, N, (int)(K / kGroup))) {
+        hipLaunchKernelGGL((int4_rows8_long_kernel<DT, kR8Waves, 8>), dim3((unsigned)(N / 16)), dim3(kR8Threads), 0, st, (const uint16_t*)x,
+                           (const uint2*)wq, sz, (const uint16_t*)bias, (const uint16_t*)residual, (uint16_t*)y, (int)M, N, (int)K);
+      } else
       if (i4_rows8_plain(M, (int)(K / kGroup))) {
         switch (pl.row_tiles) {
           case 1: SUBSPEC_I4_ROWS8(1, 1); break;

@@ -95,10 +95,14 @@ def test_rows_up_to_8_long_k(dtype):
     """At most 8 rows and K > 2048 take the kernel that issues every request up front: every tile count per
     workgroup it is compiled for (1, 2, 3 in one round; 4, 6, 8, 10 in two), launches beyond one workgroup per
     compute unit, K ranges that are not multiples of 8 groups (dead steps), several K ranges, ragged last
-    workgroups, with and without bias."""
+    workgroups, with and without bias.  More than 56 groups over at least 128 tiles take the kernel that walks the
+    whole of K in one workgroup per tile: one round, a last round with dead steps, wavefronts with different round
+    counts, the tile count at its threshold; fewer tiles keep the K ranges over workgroups."""
     cases = [(16 * 7, 64 * 33, 3), (16 * 300, 64 * 40, 8), (16 * 601, 64 * 56, 5), (16 * 1000, 64 * 35, 2),
              (16 * 1501, 64 * 34, 8), (16 * 1900, 64 * 33, 1), (16 * 2400, 64 * 34, 7), (16 * 3001, 64 * 33, 8),
-             (16 * 9, 64 * 57, 8), (16 * 130, 64 * 120, 4), (16 * 224, 64 * 296, 6), (16 * 40, 64 * 1000, 8)]
+             (16 * 9, 64 * 57, 8), (16 * 130, 64 * 120, 4), (16 * 224, 64 * 296, 6), (16 * 40, 64 * 1000, 8),
+             (16 * 128, 64 * 57, 8), (16 * 128, 64 * 61, 1), (16 * 200, 64 * 129, 3), (16 * 129, 64 * 200, 8),
+             (16 * 127, 64 * 64, 8)]
     for i, (N, K, M) in enumerate(cases):
         _check(N, K, M, dtype, 1200 + i, bias=bool(i % 2))
 
