@@ -206,7 +206,8 @@ def bench_int4(args):
             nbytes = N * K // 2 + N * (K // 64) * 4 + M * (K + N) * 2
             _kernel_line("int4 g64 linear latency", f"BASELINE config 4: {K}->{N}, M={M}, bf16 activations, weights streamed "
                          f"from HBM (rotating over {copies} copies)", call_us, kernel_us, nbytes, 2 * M * N * K,
-                         "subspec::int4_rows8_kernel" if (M <= 8 and K > 2048) else
+                         "subspec::int4_rows8_long_kernel" if (M <= 8 and K > 3584 and N >= 2048) else
+                         "subspec::int4_rows8_kernel" if (M <= 16 and K > 2048) else
                          "subspec::int4_gemv_kernel" if M == 1 else "subspec::int4_gemm_kernel",
                          extra={"N": N, "K": K, "M": M, "same_weights_every_call_us": round(warm_us, 2),
                                 "same_weights_every_call_kernel_us": round(warm_kernel_us, 2)})

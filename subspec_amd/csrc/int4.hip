@@ -21,8 +21,8 @@
 //   sum_k (q_k - z) s x_k = s * (sum_k (off + q_k) x_k - (z + off) * sum_k x_k)    per group.
 // M = 1   : int4_gemv_kernel, v_dot2_f32 on (weight pair, activation pair); HBM-bound,
 //           algorithmic bytes = N*K/2 + N*(K/64)*4 (+ activations).  (K of at most 2048 only; longer K: next line.)
-// M = 1-8, K > 2048: int4_rows8_kernel, the same MFMA arithmetic with nothing pipelined: every request of a
-//           wavefront is issued before its first wait.  This is the shape of a draft level (8 rows, one workgroup per
+// M = 1-16, K > 2048: int4_rows8_kernel, the same MFMA arithmetic with nothing pipelined: every request of a
+//           wavefront is issued before its first wait.  This is the shape of a draft level (8 or 16 rows, one workgroup per
 //           compute unit), where a pipeline of a few groups is bound by round trips, not by bytes.
 //           A K of more than 56 groups over at least 128 tiles (the down projection): int4_rows8_long_kernel, one
 //           workgroup per tile over the whole of K, in rounds whose registers refill while they are used.
@@ -518,7 +518,7 @@ __global__ __launch_bounds__(kI4Threads) void int4_gemm_kernel(
   }
 }
 
-// ------------------------------------------------------------------ 1 <= M <= 8, at most 56 groups per workgroup
+// ------------------------------------------------------------------ 1 <= M <= 16, at most 56 groups per workgroup
 // Nothing is pipelined.  Eight wavefronts split the workgroup's K range by group (wavefront w: groups w, w + 8, ..., at
 // most kR8Groups of them); each issues EVERY request it will need before its first wait -- its gains, its activation
 // blocks, the (scale, zero) words of all its tiles, the weight words of its first RTR tiles -- parks the activation blocks
@@ -532,8 +532,9 @@ __global__ __launch_bounds__(kI4Threads) void int4_gemm_kernel(
 // 6.8 us of pure transfer in front of 9.7 us of steps, a first round of two 3 us (37888 x 3584: 22.9 -> 20.2 us per
 // call); rounds of one tile gain nothing more (14 requests per wavefront in flight cover the latency, 7 just do).
 //
-// LDS: a stage holds the 8 rows x 128 bytes of one group, 16-byte piece p of row r at position p ^ r (conflict-free
-// reads without padding); MFMA rows 8..15 read a block of zeros.  (scale, zero): a group's 16 words are 64 bytes, and one
+// LDS: a stage holds the 8 rows x 128 bytes of one group, 16-byte piece p of row r at position p ^ (r % 8) (conflict-free
+// reads without padding); MFMA rows 8..15 read a block of zeros.  R = 2 (9 to 16 rows): stages of 16 rows, every lane
+// fetches and parks two pieces (rows prow and prow + 8), and wavefront m finishes rows m and m + 8.  (scale, zero): a group's 16 words are 64 bytes, and one
 // request per (group, tile) would be half of all requests for a ninth of the bytes, so lane group c fetches the words
 // of steps c and 4 + c, two requests per tile, and a step picks its word up from lane group J % 4 with a cross-lane read.
 //
@@ -548,7 +549,7 @@ constexpr int kR8Waves = 8, kR8Groups = 7, kR8Threads = kR8Waves * 64;
 // wavefronts fetch each 128-byte line with two requests (a lane's 32 bytes are two 16-byte loads), and a streamed line
 // does not wait in the first-level cache for the second one.  A request of this kernel covers whole lines.
 constexpr int kStream = 2;
-template <int DT, int RTR, int NR, int EPI, bool NORM>
+template <int DT, int RTR, int NR, int EPI, bool NORM, int R = 1>
 __global__ __launch_bounds__(kR8Threads) void int4_rows8_kernel(
     const uint16_t* __restrict__ x, const uint2* __restrict__ wq, const uint32_t* __restrict__ sz,
     const uint16_t* __restrict__ bias, const uint16_t* residual, uint16_t* y, float* __restrict__ partial, int M, int64_t N,
@@ -567,11 +568,13 @@ __global__ __launch_bounds__(kR8Threads) void int4_rows8_kernel(
   constexpr int RT = RTR * NR, NW = kR8Waves, NG = kR8Groups;
   static_assert(NG <= 8, "two (scale, zero) requests per tile cover eight steps");
   static_assert(NG * 8 <= 64, "one gain piece per lane");
-  constexpr int kStageBytes = NW * NG * (1024 + 128) + NW * 16;   // stages, gains, one block of zeros per wavefront
-  constexpr int kRedBytes = RT * NW * 32 * 16;                     // rows 0..7 of every wavefront's accumulators
+  static_assert(R == 1 || R == 2, "8 or 16 activation rows");
+  constexpr int kStage = R * 1024;                               // a group's activation block: 8 R rows x 128 bytes
+  constexpr int kStageBytes = NW * NG * (kStage + 128) + NW * 16;  // stages, gains, one block of zeros per wavefront
+  constexpr int kRedBytes = RT * NW * 32 * R * 16;                 // rows 0..8 R - 1 of every wavefront's accumulators
   __shared__ __attribute__((aligned(16))) unsigned char lds_raw[kStageBytes > kRedBytes ? kStageBytes : kRedBytes];
-  __shared__ float sq_s[NORM ? NW * 8 : 1];                      // NORM: per wavefront, per row: sum of squares over its groups
-  __shared__ float rstd_s[NORM ? 8 : 1];
+  __shared__ float sq_s[NORM ? NW * 8 * R : 1];                  // NORM: per wavefront, per row: sum of squares over its groups
+  __shared__ float rstd_s[NORM ? 8 * R : 1];
   float* const red = (float*)lds_raw;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -615,9 +618,9 @@ __global__ __launch_bounds__(kR8Threads) void int4_rows8_kernel(
   const uint32_t one2 = DT == SUBSPEC_BF16 ? 0x3f803f80u : 0x3c003c00u;
   const i4_u4 ones = i4_u4{one2, one2, one2, one2};
 
-  unsigned char* const stages = lds_raw + wave * (NG * 1024);
-  unsigned char* const gains = lds_raw + NW * NG * 1024 + wave * (NG * 128);
-  unsigned char* const zeros = lds_raw + NW * NG * (1024 + 128) + wave * 16;
+  unsigned char* const stages = lds_raw + wave * (NG * kStage);
+  unsigned char* const gains = lds_raw + NW * NG * kStage + wave * (NG * 128);
+  unsigned char* const zeros = lds_raw + NW * NG * (kStage + 128) + wave * 16;
 
   // ---- every request
   i4_u4 gpiece;
@@ -626,10 +629,12 @@ __global__ __launch_bounds__(kR8Threads) void int4_rows8_kernel(
     const int q = min(lane, NG * 8 - 1);
     gpiece = __builtin_amdgcn_raw_buffer_load_b128(g_rsrc, (q & 7) * 16, min(g_first + NW * (q >> 3), G - 1) * (kGroup * 2), 0);
   }
-  i4_u4 xall[NG];
+  i4_u4 xall[NG][R];                                             // R = 2: rows prow and prow + 8
 #pragma unroll
   for (int J = 0; J < NG; ++J)
-    xall[J] = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, xg_off, min(g_first + NW * J, G - 1) * (kGroup * 2), 0);
+#pragma unroll
+    for (int h = 0; h < R; ++h)
+      xall[J][h] = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, xg_off + h * 8 * K * 2, min(g_first + NW * J, G - 1) * (kGroup * 2), 0);
   // the activation requests stay ahead of all others: a wait for a block that was requested after the weights would
   // be a wait for the weights
   __builtin_amdgcn_sched_barrier(0);
@@ -654,37 +659,42 @@ __global__ __launch_bounds__(kR8Threads) void int4_rows8_kernel(
   if constexpr (NORM) {
     if (lane < NG * 8) *(i4_u4*)(gains + lane * 16) = gpiece;
   }
-  float sq = 0.f;                                                // NORM: squares of row prow over this wavefront's groups
+  float sq[R];                                                   // NORM: squares of rows prow (+ 8) over this wavefront's groups
+#pragma unroll
+  for (int h = 0; h < R; ++h) sq[h] = 0.f;
   (void)sq;
 #pragma unroll
   for (int J = 0; J < NG; ++J) {
-    i4_u4 piece = xall[J];
-    if constexpr (NORM) {
-      float f_[8], g_[8];
-      unpack8<DT>(piece, f_);
-      unpack8<DT>(*(const i4_u4*)(gains + (J * 8 + ppiece) * 16), g_);
-      float ss_ = 0.f;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) { ss_ = fmaf(f_[e], f_[e], ss_); f_[e] *= g_[e]; }
-      sq += J < nj ? ss_ : 0.f;
-      piece = pack8<DT>(f_);
+    for (int h = 0; h < R; ++h) {
+      i4_u4 piece = xall[J][h];
+      if constexpr (NORM) {
+        float f_[8], g_[8];
+        unpack8<DT>(piece, f_);
+        unpack8<DT>(*(const i4_u4*)(gains + (J * 8 + ppiece) * 16), g_);
+        float ss_ = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) { ss_ = fmaf(f_[e], f_[e], ss_); f_[e] *= g_[e]; }
+        sq[h] += J < nj ? ss_ : 0.f;
+        piece = pack8<DT>(f_);
+      }
+      *(i4_u4*)(stages + J * kStage + (prow + 8 * h) * 128 + ((ppiece ^ prow) << 4)) = piece;
     }
-    *(i4_u4*)(stages + J * 1024 + prow * 128 + ((ppiece ^ prow) << 4)) = piece;
   }
 
   // ---- the steps: round r takes tiles r RTR .. r RTR + RTR - 1; a dead step or tile multiplies by a zero scale
   i4_v4f acc[RT];
 #pragma unroll
   for (int t = 0; t < RT; ++t) acc[t] = i4_v4f{0.f, 0.f, 0.f, 0.f};
-  const int rd0 = ln * 128 + (((2 * c) ^ ln) << 4), rd1 = ln * 128 + (((2 * c + 1) ^ ln) << 4);
+  const int rd0 = ln * 128 + (((2 * c) ^ (ln & 7)) << 4), rd1 = ln * 128 + (((2 * c + 1) ^ (ln & 7)) << 4);
   i4_v4f xsum[NG];
 #pragma unroll
   for (int r = 0; r < NR; ++r) {
 #pragma unroll
     for (int J = 0; J < NG; ++J) {
       const bool step_live = J < nj;
-      const i4_u4 xa0 = *(const i4_u4*)(ln < 8 ? stages + J * 1024 + rd0 : zeros);
-      const i4_u4 xa1 = *(const i4_u4*)(ln < 8 ? stages + J * 1024 + rd1 : zeros);
+      const i4_u4 xa0 = *(const i4_u4*)((R == 2 || ln < 8) ? stages + J * kStage + rd0 : zeros);
+      const i4_u4 xa1 = *(const i4_u4*)((R == 2 || ln < 8) ? stages + J * kStage + rd1 : zeros);
       if (r == 0) {                                              // the group's activation sums, rows 4c + rr: kept for all rounds
         xsum[J] = i4_mfma32<DT>(xa0, ones, i4_v4f{0.f, 0.f, 0.f, 0.f});
         xsum[J] = i4_mfma32<DT>(xa1, ones, xsum[J]);
@@ -718,32 +728,37 @@ __global__ __launch_bounds__(kR8Threads) void int4_rows8_kernel(
   // ---- output stage
   if constexpr (NORM) {
     // the eight lanes that share a row hold its squares over different k; one value per (wavefront, row) goes to LDS
-    float v = sq;
-    v += __shfl_xor(v, 1, kWave);
-    v += __shfl_xor(v, 2, kWave);
-    v += __shfl_xor(v, 4, kWave);
-    if (ppiece == 0) sq_s[wave * 8 + prow] = v;
+#pragma unroll
+    for (int h = 0; h < R; ++h) {
+      float v = sq[h];
+      v += __shfl_xor(v, 1, kWave);
+      v += __shfl_xor(v, 2, kWave);
+      v += __shfl_xor(v, 4, kWave);
+      if (ppiece == 0) sq_s[wave * 8 * R + prow + 8 * h] = v;
+    }
   }
   __syncthreads();                                               // every wavefront is done with its stages
   if constexpr (NORM) {
-    if (tid < 8) {
+    if (tid < 8 * R) {
       float ss = 0.f;
 #pragma unroll
-      for (int w = 0; w < NW; ++w) ss += sq_s[w * 8 + tid];
+      for (int w = 0; w < NW; ++w) ss += sq_s[w * 8 * R + tid];
       rstd_s[tid] = rsqrtf(ss / (float)K + fz.norm_eps);
     }
   }
-  if (lane < 32) {                                               // accumulator rows 4c + rr: lane groups 0 and 1 hold rows 0..7
+  if (lane < 32 * R) {                                           // accumulator rows 4c + rr: lane groups 0 and 1 hold rows 0..7
 #pragma unroll
-    for (int t = 0; t < RT; ++t) *(i4_v4f*)(&red[((t * NW + wave) * 32 + lane) * 4]) = acc[t];
+    for (int t = 0; t < RT; ++t) *(i4_v4f*)(&red[((t * NW + wave) * (32 * R) + lane) * 4]) = acc[t];
   }
   __syncthreads();
-  const int m = wave;                                            // this wavefront's row
+#pragma unroll
+  for (int mi = 0; mi < R; ++mi) {
+  const int m = wave + 8 * mi;                                   // this wavefront's row(s): wave, wave + 8
   if (m >= M) return;
   auto summed = [&](int t) {
     float v = 0.f;
 #pragma unroll
-    for (int w = 0; w < NW; ++w) v += red[((t * NW + w) * 32 + (m >> 2) * 16 + ln) * 4 + (m & 3)];
+    for (int w = 0; w < NW; ++w) v += red[((t * NW + w) * (32 * R) + (m >> 2) * 16 + ln) * 4 + (m & 3)];
     if constexpr (NORM) v *= rstd_s[m];
     return v;
   };
@@ -794,6 +809,7 @@ __global__ __launch_bounds__(kR8Threads) void int4_rows8_kernel(
         Elem<DT>::store(dst, d + 16, second_raw);
       }
     }
+  }
   }
 }
 
@@ -932,12 +948,13 @@ struct I4Plan { int wgs, row_tiles, splits, groups_per_split; };
 // The 8-row kernel takes K ranges (groups per workgroup) long enough that the pipelined loop would pay several round
 // trips and short enough for its registers and LDS stages.  Its workgroups hold 63 KB of LDS, two per compute unit.
 constexpr int kR8Range = kR8Waves * kR8Groups;
-static bool i4_rows8_plain(int64_t M, int G) { return M <= 8 && G > 32; }
+constexpr int kR8MaxRows = 16;                                  // 8 rows per block of the kernel's R parameter
+static bool i4_rows8_plain(int64_t M, int G) { return M <= kR8MaxRows && G > 32; }
 // Tile pairs per workgroup of a paired 8-row launch, 0 if it should not be one: one pair while that fits the 512
 // resident workgroups; beyond that whole compute units' worth -- ceil(pairs / 256) pairs each, 3 to 5, in rounds of
 // one pair, so that no compute unit gets a second workgroup while others have one.
 static int i4_rows8_pairs(int64_t M, int G, int64_t pairs) {
-  if (!(M <= 8 && G > 32 && G <= kR8Range)) return 0;
+  if (!(M <= kR8MaxRows && G > 32 && G <= kR8Range)) return 0;
   if (pairs <= 512) return 1;
   const int64_t p = (pairs + 255) / 256;
   return p <= 5 ? (int)std::max<int64_t>(p, 3) : 0;
@@ -1011,10 +1028,12 @@ static int run_int4_paired(const void* x, const uint32_t* wq, const uint32_t* sz
   const int p8_plan = i4_rows8_pairs(M, G, pairs);
   if (const int p8 = (EPI == kEpiRope && p8_plan > 1) ? 0 : p8_plan) {
     const dim3 grid8((unsigned)((pairs + p8 - 1) / p8), 1);
-#define SUBSPEC_I4_ROWS8(RTR, NR, NORM)                                                                            \
-  hipLaunchKernelGGL((int4_rows8_kernel<DT, RTR, NR, EPI, NORM>), grid8, dim3(kR8Threads), 0, st, (const uint16_t*)x, \
+#define SUBSPEC_I4_ROWS8_R(RTR, NR, NORM, R)                                                                       \
+  hipLaunchKernelGGL((int4_rows8_kernel<DT, RTR, NR, EPI, NORM, R>), grid8, dim3(kR8Threads), 0, st, (const uint16_t*)x, \
                      (const uint2*)wq, sz, (const uint16_t*)bias, (const uint16_t*)nullptr, (uint16_t*)out, (float*)nullptr,   \
                      (int)M, N, (int)K, 1, kR8Range, fz)
+#define SUBSPEC_I4_ROWS8(RTR, NR, NORM)                                                                            \
+  do { if (M <= 8) SUBSPEC_I4_ROWS8_R(RTR, NR, NORM, 1); else SUBSPEC_I4_ROWS8_R(RTR, NR, NORM, 2); } while (0)
 #define SUBSPEC_I4_ROWS8_P(NORM)                                                                                   \
   do {                                                                                                             \
     if (p8 == 1) SUBSPEC_I4_ROWS8(2, 1, NORM);                                                                     \
@@ -1026,6 +1045,7 @@ static int run_int4_paired(const void* x, const uint32_t* wq, const uint32_t* sz
     if (norm) SUBSPEC_I4_ROWS8_P(true); else SUBSPEC_I4_ROWS8_P(false);
 #undef SUBSPEC_I4_ROWS8_P
 #undef SUBSPEC_I4_ROWS8
+#undef SUBSPEC_I4_ROWS8_R
   } else
   if (M <= 16) { if (norm) SUBSPEC_I4_PAIRED_RT(1, true); else SUBSPEC_I4_PAIRED_RT(1, false); }
   else if (M <= 32) { if (norm) SUBSPEC_I4_PAIRED_RT(2, true); else SUBSPEC_I4_PAIRED_RT(2, false); }
@@ -1062,10 +1082,12 @@ static int run_int4(const void* x, const uint32_t* wq, const uint32_t* sz, const
   hipLaunchKernelGGL((int4_gemm_kernel<DT, MT, RT>), grid, dim3(kI4Threads), 0, st, (const uint16_t*)x,            \
                      (const uint2*)wq, sz, (const uint16_t*)bias, (const uint16_t*)residual, (uint16_t*)y, partial, (int)M, N, (int)K, \
                      pl.splits, pl.groups_per_split, I4Fused{})
-#define SUBSPEC_I4_ROWS8(RTR, NR)                                                                                  \
-  hipLaunchKernelGGL((int4_rows8_kernel<DT, RTR, NR, kEpiPlain, false>), grid, dim3(kR8Threads), 0, st, (const uint16_t*)x, \
+#define SUBSPEC_I4_ROWS8_R(RTR, NR, R)                                                                             \
+  hipLaunchKernelGGL((int4_rows8_kernel<DT, RTR, NR, kEpiPlain, false, R>), grid, dim3(kR8Threads), 0, st, (const uint16_t*)x, \
                      (const uint2*)wq, sz, (const uint16_t*)bias, (const uint16_t*)residual, (uint16_t*)y, partial, (int)M, N, (int)K, \
                      pl.splits, pl.groups_per_split, I4Fused{})
+#define SUBSPEC_I4_ROWS8(RTR, NR)                                                                                  \
+  do { if (M <= 8) SUBSPEC_I4_ROWS8_R(RTR, NR, 1); else SUBSPEC_I4_ROWS8_R(RTR, NR, 2); } while (0)
 #define SUBSPEC_I4_LAUNCH_MT(MT)                                                                                   \
   do {                                                                                                             \
     if (pl.row_tiles == 1) SUBSPEC_I4_LAUNCH(MT, 1);                                                               \
@@ -1095,6 +1117,7 @@ static int run_int4(const void* x, const uint32_t* wq, const uint32_t* sz, const
       else SUBSPEC_I4_LAUNCH_MT(4);
     }
 #undef SUBSPEC_I4_ROWS8
+#undef SUBSPEC_I4_ROWS8_R
 #undef SUBSPEC_I4_LAUNCH_MT
 #undef SUBSPEC_I4_LAUNCH
     if (pl.splits > 1)

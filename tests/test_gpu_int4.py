@@ -91,8 +91,8 @@ def test_random_shape_sweep():
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-def test_rows_up_to_8_long_k(dtype):
-    """At most 8 rows and K > 2048 take the kernel that issues every request up front: every tile count per
+def test_rows_up_to_16_long_k(dtype):
+    """At most 16 rows and K > 2048 take the kernel that issues every request up front: every tile count per
     workgroup it is compiled for (1, 2, 3 in one round; 4, 6, 8, 10 in two), launches beyond one workgroup per
     compute unit, K ranges that are not multiples of 8 groups (dead steps), several K ranges, ragged last
     workgroups, with and without bias.  More than 56 groups over at least 128 tiles take the kernel that walks the
@@ -105,6 +105,10 @@ def test_rows_up_to_8_long_k(dtype):
              (16 * 127, 64 * 64, 8)]
     for i, (N, K, M) in enumerate(cases):
         _check(N, K, M, dtype, 1200 + i, bias=bool(i % 2))
+    # 9 to 16 rows: the same kernel with activation blocks of 16 rows, every tile count again (and one shape whose
+    # long K stays split over workgroups at these row counts)
+    for i, (N, K, _) in enumerate(cases[:12]):
+        _check(N, K, 9 + (5 * i) % 8, dtype, 1300 + i, bias=bool(i % 2))
 
 
 def test_quantizer_default_refines_zero_points():
@@ -144,7 +148,10 @@ def test_gate_up_projection_with_the_activation_in_its_output_stage(dtype):
                                             (40000, 64, 3, False),
                                             # 8 rows, K > 2048: one, three, four and five tile pairs per workgroup
                                             (16 * 500, 2112, 8, True), (9728, 2112, 8, False), (14336, 2240, 5, True),
-                                            (16 * 1190, 2176, 1, False), (16 * 1500, 2112, 8, False)]):
+                                            (16 * 1190, 2176, 1, False), (16 * 1500, 2112, 8, False),
+                                            # 9 to 16 rows, K > 2048: the same tile counts with 16-row activation blocks
+                                            (16 * 500, 2112, 16, True), (9728, 2112, 9, False), (14336, 2240, 13, True),
+                                            (16 * 1190, 2176, 12, False), (18944, 3584, 16, False)]):
         print("gate|up + silu", dtype, F, K, M, bias, flush=True)
         g = torch.Generator().manual_seed(700 + seed)
         W = torch.randn(2 * F, K, generator=g) * (2.0 / K ** 0.5)
@@ -160,8 +167,8 @@ def test_gate_up_projection_with_the_activation_in_its_output_stage(dtype):
         assert got.shape == (M, F) and got.dtype == dtype
         differing = int((got != want).sum())
         # more than five tile pairs per compute unit: the fused launch stays on the four-wavefront kernel while the
-        # plain projection of 8 rows takes the eight-wavefront one, so the partial sums are grouped differently
-        same_grouping = not (M <= 8 and K > 2048 and F // 16 > 1280)
+        # plain projection of up to 16 rows takes the eight-wavefront one, so the partial sums are grouped differently
+        same_grouping = not (M <= 16 and K > 2048 and F // 16 > 1280)
         if same_grouping:
             assert differing <= max(1, got.numel() // 1000), (F, K, M, differing)
         ulp = 2.0 ** (-7 if dtype == torch.bfloat16 else -10)

@@ -93,7 +93,7 @@ def test_dense_target_layer_at_7b_geometry(n):
     _check(x, kd[0], vd[0], want, k, v, PREFIX, n, ("dense", n))
 
 
-@pytest.mark.parametrize("n,prefix,depth_base", [(8, PREFIX, 0), (64, PREFIX, 0), (8, 40, 32000)])
+@pytest.mark.parametrize("n,prefix,depth_base", [(8, PREFIX, 0), (64, PREFIX, 0), (8, 40, 32000), (13, PREFIX, 0), (16, 300, 0)])
 def test_int4_draft_layer_at_7b_geometry(n, prefix, depth_base):
     """depth_base = 32000: rotary positions near 32k through the same kernels (the angle is formed in fp32 from the
     position and the inverse frequency; the oracle's table is the eager formula)."""
