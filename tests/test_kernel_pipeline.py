@@ -138,6 +138,24 @@ def test_the_8_row_kernel_keeps_its_requests_in_order_and_its_registers(tmp_path
         assert waits and min(waits) >= 4, f"{kernel}: the first step waits for (nearly) every request: {sorted(set(waits))}"
 
 
+def test_the_long_k_8_row_kernel_refills_its_registers_without_draining_them(tmp_path):
+    """int4_rows8_long_kernel requests a step's weight words for the next round into the registers the step has just
+    emptied.  Requested while the old words are still wanted they land in other registers, and the copy back at the
+    end of the round waits for every request in flight -- a round trip per round that no result shows.  The loop must
+    therefore hold no full wait, every wait inside it must leave at least the other steps' requests outstanding, and
+    nothing may live in scratch memory."""
+    asm = _assembly(os.path.join(build_mod.CSRC, "int4.hip"), tmp_path)
+    _recognised(asm, "int4_rows8_long_kernel")
+    bodies = _kernel_bodies(asm, "int4_rows8_long_kernel")
+    assert len(bodies) >= 2, "the parser found too few kernel variants"
+    for kernel, lines in bodies.items():
+        assert not any("scratch_" in l for l in lines), f"{kernel} uses scratch memory"
+    loops = [l for l in _loops_with_full_waits(asm, "int4_rows8_long_kernel") if l[1] >= 100]
+    assert len({l[0] for l in loops}) >= 2, "the parser found no round loop"
+    stalled = [(k, n, w) for k, n, w in loops if w]
+    assert not stalled, "a full wait inside the round loop of: " + ", ".join(f"{k} (at {w})" for k, n, w in stalled)
+
+
 def test_the_attention_kernels_keep_their_requests_in_flight(tmp_path):
     """The 32 x 32 attention kernels keep K / V requests of later blocks on their way while a block is multiplied: the
     ping-pong kernel through copies into LDS that it waits for by hand (vmcnt(4): the newest block stays outstanding),
