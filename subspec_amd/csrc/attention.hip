@@ -412,19 +412,42 @@ __global__ __launch_bounds__(256) void tree_attention_merge_kernel(
   const int d4 = threadIdx.x & 31;
   const int64_t slot0 = (int64_t)bh * ap.chunks * kAttnRows + row;     // chunk c: slot0 + c * kAttnRows
   float m = -INFINITY;
-#pragma unroll 8
-  for (int c = 0; c < ap.chunks; ++c) m = fmaxf(m, part_ml[(slot0 + (int64_t)c * kAttnRows) * 2]);
   v4f num = {0.f, 0.f, 0.f, 0.f};
   float den = 0.f;
-#pragma unroll 8
-  for (int c = 0; c < ap.chunks; ++c) {
-    const int64_t slot = slot0 + (int64_t)c * kAttnRows;
-    const v2f_t ml = *(const v2f_t*)(&part_ml[slot * 2]);
-    const v4f oc = *(const v4f*)(&part_o[slot * kAttnD + d4 * 4]);
-    const float w = ml[0] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(ml[0] - m);
+  constexpr int kUpFront = 24;
+  if (ap.chunks <= kUpFront) {
+    // the usual case (a draft level has 12 to 18 chunks at prefixes of 2000 to 2400): every load of the launch is issued before the
+    // first wait -- one round trip instead of two (the maxima first, then the rows); the sums run in the same order
+    v2f_t ml[kUpFront];
+    v4f oc[kUpFront];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) num[i] = fmaf(w, oc[i], num[i]);
-    den = fmaf(w, ml[1], den);
+    for (int c = 0; c < kUpFront; ++c) {
+      const int64_t slot = slot0 + (int64_t)min(c, (int)ap.chunks - 1) * kAttnRows;
+      ml[c] = *(const v2f_t*)(&part_ml[slot * 2]);
+      oc[c] = *(const v4f*)(&part_o[slot * kAttnD + d4 * 4]);
+    }
+#pragma unroll
+    for (int c = 0; c < kUpFront; ++c) m = fmaxf(m, ml[c][0]);         // slots past the last chunk repeat it
+#pragma unroll
+    for (int c = 0; c < kUpFront; ++c) {
+      const float w = (c >= ap.chunks || ml[c][0] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(ml[c][0] - m);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) num[i] = fmaf(w, oc[c][i], num[i]);
+      den = fmaf(w, ml[c][1], den);
+    }
+  } else {
+#pragma unroll 8
+    for (int c = 0; c < ap.chunks; ++c) m = fmaxf(m, part_ml[(slot0 + (int64_t)c * kAttnRows) * 2]);
+#pragma unroll 8
+    for (int c = 0; c < ap.chunks; ++c) {
+      const int64_t slot = slot0 + (int64_t)c * kAttnRows;
+      const v2f_t ml = *(const v2f_t*)(&part_ml[slot * 2]);
+      const v4f oc = *(const v4f*)(&part_o[slot * kAttnD + d4 * 4]);
+      const float w = ml[0] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(ml[0] - m);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) num[i] = fmaf(w, oc[i], num[i]);
+      den = fmaf(w, ml[1], den);
+    }
   }
   const float inv = den > 0.f ? 1.f / den : 0.f;
   uint2 packed;

@@ -652,6 +652,53 @@ __global__ __launch_bounds__(kR8Threads) void int4_rows8_kernel(
 #pragma unroll
     for (int tt = 0; tt < RTR; ++tt)
       wall[J][tt] = __builtin_amdgcn_raw_buffer_load_b64(w_rsrc, lane * 8, (wofs[tt] + min(g_first + NW * J, G - 1)) * 512, kStream);
+  // What the output stage adds to this thread's elements (wavefront w finishes rows w and w + 8, lane group c the items
+  // c, c + 4, ...): requested here, behind everything else, so that the output stage does not end in a round trip of its own.
+  constexpr int kItems = PAIRED ? RT / 2 : RT;
+  constexpr int kOut = (kItems + 3) / 4;
+  // (The 16-bit words are kept as they come and converted where they are used: an instruction that touches a loaded
+  // value here would wait for every request issued before it.  Elements this thread does not own repeat one it may read.)
+  uint32_t res_pre[kOut][R], bias_pre[kOut];
+#pragma unroll
+  for (int io = 0; io < kOut; ++io) {
+    bias_pre[io] = 0u;
+#pragma unroll
+    for (int mi = 0; mi < R; ++mi) res_pre[io][mi] = 0u;
+  }
+  uint32_t bias1_pre[kOut];                                      // paired tiles: the second tile's bias
+  int pos_pre[R], crow_pre[R];                                   // rotary: position and cache row of the thread's rows
+#pragma unroll
+  for (int io = 0; io < kOut; ++io) bias1_pre[io] = 0u;
+#pragma unroll
+  for (int mi = 0; mi < R; ++mi) { pos_pre[mi] = 0; crow_pre[mi] = 0; }
+  (void)bias1_pre; (void)pos_pre; (void)crow_pre;
+  if constexpr (!PAIRED) {
+#pragma unroll
+    for (int io = 0; io < kOut; ++io) {
+      const int64_t n0 = (int64_t)tile_of(min(io * 4 + c, ntl - 1)) * 16 + ln;
+      if (bias) bias_pre[io] = bias[n0];                          // (uniform)
+      if (residual) {                                             // (uniform)
+#pragma unroll
+        for (int mi = 0; mi < R; ++mi) res_pre[io][mi] = residual[(int64_t)min(wave + 8 * mi, M - 1) * N + n0];
+      }
+    }
+  } else {
+    if (bias) {                                                   // (uniform)
+#pragma unroll
+      for (int io = 0; io < kOut; ++io) {
+        const int t0 = 2 * min(io * 4 + c, ntl / 2 - 1);
+        bias_pre[io] = bias[(int64_t)tile_of(t0) * 16 + ln];
+        bias1_pre[io] = bias[(int64_t)tile_of(t0 + 1) * 16 + ln];
+      }
+    }
+    if constexpr (ROPE) {
+#pragma unroll
+      for (int mi = 0; mi < R; ++mi) {
+        pos_pre[mi] = fz.positions[min(wave + 8 * mi, M - 1)];
+        crow_pre[mi] = fz.cache_rows[min(wave + 8 * mi, M - 1)];
+      }
+    }
+  }
 
   __builtin_amdgcn_sched_barrier(0);
   // ---- park the activation blocks
@@ -762,21 +809,26 @@ __global__ __launch_bounds__(kR8Threads) void int4_rows8_kernel(
     if constexpr (NORM) v *= rstd_s[m];
     return v;
   };
-  constexpr int kItems = PAIRED ? RT / 2 : RT;                   // lane group c takes items c, c + 4, ...
 #pragma unroll
-  for (int i0 = 0; i0 < kItems; i0 += 4) {
+  for (int i0 = 0; i0 < kItems; i0 += 4) {                       // lane group c takes items c, c + 4, ...
     const int item = i0 + c;
     const int t0 = PAIRED ? 2 * item : item;
     if (item >= kItems || t0 >= ntl) continue;
     const int64_t n0 = (int64_t)tile_of(t0) * 16 + ln;
-    const float b0v = (splits == 1 && bias) ? I4<DT>::to_float(bias[n0]) : 0.f;
     const float v0 = summed(t0);
     if constexpr (!PAIRED) {
-      if (splits == 1) store_linear_out<DT>(y, (int64_t)m * N + n0, v0 + b0v, residual);
-      else partial[((int64_t)ks * M + m) * N + n0] = v0;
+      if (splits == 1) {                                         // out = round(round(v) + residual), as store_linear_out
+        asm volatile("" : "+v"(bias_pre[i0 / 4]), "+v"(res_pre[i0 / 4][mi]));
+        float v = v0 + (bias ? I4<DT>::to_float((uint16_t)bias_pre[i0 / 4]) : 0.f);
+        if (residual) v = Elem<DT>::round(v) + I4<DT>::to_float((uint16_t)res_pre[i0 / 4][mi]);
+        Elem<DT>::store(y, (int64_t)m * N + n0, v);
+      } else {
+        partial[((int64_t)ks * M + m) * N + n0] = v0;
+      }
     } else {
-      const int64_t n1 = (int64_t)tile_of(t0 + 1) * 16 + ln;
-      const float b1v = bias ? I4<DT>::to_float(bias[n1]) : 0.f;
+      asm volatile("" : "+v"(bias_pre[i0 / 4]), "+v"(bias1_pre[i0 / 4]), "+v"(pos_pre[mi]), "+v"(crow_pre[mi]));
+      const float b0v = bias ? I4<DT>::to_float((uint16_t)bias_pre[i0 / 4]) : 0.f;
+      const float b1v = bias ? I4<DT>::to_float((uint16_t)bias1_pre[i0 / 4]) : 0.f;
       const float first = Elem<DT>::round(v0 + b0v), second_raw = summed(t0 + 1) + b1v;
       const int u = unit0 + item;
       if constexpr (SILU) {
@@ -789,7 +841,7 @@ __global__ __launch_bounds__(kR8Threads) void int4_rows8_kernel(
         const int head = u >> 2, d = (u & 3) * 16 + ln;
         const float inv_freq = fz.inv_freq ? fz.inv_freq[d] : exp2f(-(float)(2 * d) / 128.f * fz.log2_theta);
         float sn, cs;
-        sincosf((float)fz.positions[m] * inv_freq, &sn, &cs);
+        sincosf((float)pos_pre[mi] * inv_freq, &sn, &cs);
         cs = Elem<DT>::round(cs);
         sn = Elem<DT>::round(sn);
         const float lo = first, hi = Elem<DT>::round(second_raw);
@@ -797,14 +849,14 @@ __global__ __launch_bounds__(kR8Threads) void int4_rows8_kernel(
         const float o_hi = Elem<DT>::round(hi * cs) + Elem<DT>::round(lo * sn);
         uint16_t *dst, *unused;
         if (head < fz.hq) dst = fz.q_out + ((int64_t)head * M + m) * 128;
-        else if (!kv_row_ptrs(fz.kv, head - fz.hq, fz.cache_rows[m], &dst, &unused)) continue;   // a row outside the layer's cache is dropped
+        else if (!kv_row_ptrs(fz.kv, head - fz.hq, crow_pre[mi], &dst, &unused)) continue;   // a row outside the layer's cache is dropped
         Elem<DT>::store(dst, d, o_lo);
         Elem<DT>::store(dst, d + 64, o_hi);
       } else {
         // two consecutive tiles of a value head: copied
         const int vt = 2 * (u - qk_units), kvh = vt >> 3, d = (vt & 7) * 16 + ln;
         uint16_t *dst, *unused;
-        if (!kv_row_ptrs(fz.kv, kvh, fz.cache_rows[m], &unused, &dst)) continue;
+        if (!kv_row_ptrs(fz.kv, kvh, crow_pre[mi], &unused, &dst)) continue;
         Elem<DT>::store(dst, d, first);
         Elem<DT>::store(dst, d + 16, second_raw);
       }
@@ -872,6 +924,14 @@ __global__ __launch_bounds__(NW * 64) void int4_rows8_long_kernel(
   i4_u2 wall[NG];
 #pragma unroll
   for (int J = 0; J < NG; ++J) wall[J] = __builtin_amdgcn_raw_buffer_load_b64(w_rsrc, lane * 8, (wofs + group_of(0, J)) * 512, kStream);
+  // what the output stage adds to this thread's element (wavefront m finishes row m, lane group 0 the sixteen columns):
+  // requested here, so that the output stage does not end in a round trip of its own
+  // (kept as the 16-bit words they are until then: an instruction that touches a loaded value here would wait for every
+  // request issued before it; wavefronts without a row repeat the last one)
+  const int64_t n_out = (int64_t)tile * 16 + ln;
+  uint32_t bias_pre = 0u, res_pre = 0u;
+  if (bias) bias_pre = bias[n_out];                                // (uniform)
+  if (residual) res_pre = residual[(int64_t)min(wave, M - 1) * N + n_out];
   __builtin_amdgcn_sched_barrier(0);
   if (lane == 0) *(i4_u4*)zeros = i4_u4{0u, 0u, 0u, 0u};
 
@@ -927,9 +987,10 @@ __global__ __launch_bounds__(NW * 64) void int4_rows8_long_kernel(
   float v = 0.f;
 #pragma unroll
   for (int w = 0; w < NW; ++w) v += red[(w * 32 + (m >> 2) * 16 + ln) * 4 + (m & 3)];
-  const int64_t n0 = (int64_t)tile * 16 + ln;
-  if (bias) v += I4<DT>::to_float(bias[n0]);
-  store_linear_out<DT>(y, (int64_t)m * N + n0, v, residual);
+  asm volatile("" : "+v"(bias_pre), "+v"(res_pre));
+  if (bias) v += I4<DT>::to_float((uint16_t)bias_pre);
+  if (residual) v = Elem<DT>::round(v) + I4<DT>::to_float((uint16_t)res_pre);   // out = round(round(v) + residual), as store_linear_out
+  Elem<DT>::store(y, (int64_t)m * N + n_out, v);
 }
 
 template <int DT>
