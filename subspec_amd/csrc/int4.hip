@@ -672,24 +672,25 @@ __global__ __launch_bounds__(kR8Threads) void int4_rows8_kernel(
 #pragma unroll
   for (int mi = 0; mi < R; ++mi) { pos_pre[mi] = 0; crow_pre[mi] = 0; }
   (void)bias1_pre; (void)pos_pre; (void)crow_pre;
+  // No branch around a request: one that is issued on one path only makes the compiler wait for ALL requests in flight
+  // where the paths join.  A tensor that is not there is replaced by the activations' first element.
+  const uint16_t* const bias_src = bias ? bias : x;
+  const uint16_t* const res_src = residual ? residual : x;
+  const int64_t bias_on = bias ? 1 : 0, res_on = residual ? 1 : 0;
   if constexpr (!PAIRED) {
 #pragma unroll
     for (int io = 0; io < kOut; ++io) {
       const int64_t n0 = (int64_t)tile_of(min(io * 4 + c, ntl - 1)) * 16 + ln;
-      if (bias) bias_pre[io] = bias[n0];                          // (uniform)
-      if (residual) {                                             // (uniform)
+      bias_pre[io] = bias_src[n0 * bias_on];
 #pragma unroll
-        for (int mi = 0; mi < R; ++mi) res_pre[io][mi] = residual[(int64_t)min(wave + 8 * mi, M - 1) * N + n0];
-      }
+      for (int mi = 0; mi < R; ++mi) res_pre[io][mi] = res_src[((int64_t)min(wave + 8 * mi, M - 1) * N + n0) * res_on];
     }
   } else {
-    if (bias) {                                                   // (uniform)
 #pragma unroll
-      for (int io = 0; io < kOut; ++io) {
-        const int t0 = 2 * min(io * 4 + c, ntl / 2 - 1);
-        bias_pre[io] = bias[(int64_t)tile_of(t0) * 16 + ln];
-        bias1_pre[io] = bias[(int64_t)tile_of(t0 + 1) * 16 + ln];
-      }
+    for (int io = 0; io < kOut; ++io) {
+      const int t0 = 2 * min(io * 4 + c, ntl / 2 - 1);
+      bias_pre[io] = bias_src[((int64_t)tile_of(t0) * 16 + ln) * bias_on];
+      bias1_pre[io] = bias_src[((int64_t)tile_of(t0 + 1) * 16 + ln) * bias_on];
     }
     if constexpr (ROPE) {
 #pragma unroll
@@ -929,9 +930,11 @@ __global__ __launch_bounds__(NW * 64) void int4_rows8_long_kernel(
   // (kept as the 16-bit words they are until then: an instruction that touches a loaded value here would wait for every
   // request issued before it; wavefronts without a row repeat the last one)
   const int64_t n_out = (int64_t)tile * 16 + ln;
-  uint32_t bias_pre = 0u, res_pre = 0u;
-  if (bias) bias_pre = bias[n_out];                                // (uniform)
-  if (residual) res_pre = residual[(int64_t)min(wave, M - 1) * N + n_out];
+  // (no branch around a request -- the compiler would wait for every request in flight where the paths join: a tensor
+  // that is not there is replaced by the activations' first element)
+  const uint32_t bias_pre = (bias ? bias : x)[bias ? n_out : 0];
+  const uint32_t res_pre_ld = (residual ? residual : x)[residual ? (int64_t)min(wave, M - 1) * N + n_out : 0];
+  uint32_t res_pre = res_pre_ld, bias_pre_v = bias_pre;
   __builtin_amdgcn_sched_barrier(0);
   if (lane == 0) *(i4_u4*)zeros = i4_u4{0u, 0u, 0u, 0u};
 
@@ -987,8 +990,8 @@ __global__ __launch_bounds__(NW * 64) void int4_rows8_long_kernel(
   float v = 0.f;
 #pragma unroll
   for (int w = 0; w < NW; ++w) v += red[(w * 32 + (m >> 2) * 16 + ln) * 4 + (m & 3)];
-  asm volatile("" : "+v"(bias_pre), "+v"(res_pre));
-  if (bias) v += I4<DT>::to_float((uint16_t)bias_pre);
+  asm volatile("" : "+v"(bias_pre_v), "+v"(res_pre));
+  if (bias) v += I4<DT>::to_float((uint16_t)bias_pre_v);
   if (residual) v = Elem<DT>::round(v) + I4<DT>::to_float((uint16_t)res_pre);   // out = round(round(v) + residual), as store_linear_out
   Elem<DT>::store(y, (int64_t)m * N + n_out, v);
 }
